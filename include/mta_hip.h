@@ -1,0 +1,107 @@
+/* C ABI of libmta_hip.so: Multi-Token-Attention forward kernels for AMD MI355X (gfx950).
+ *
+ * The reference (Gusanidas/multitokenatention_triton) has no FFI: its operators are
+ * Triton kernels launched from torch.autograd.Function.forward.  Each entry point
+ * below replaces one such launch site (cited per function) and is what a ctypes /
+ * cffi / pybind binding in the reference's operator files would call.
+ *
+ * Conventions
+ *  - All tensors are dense, row-major ("contiguous NCHW"), device pointers.
+ *  - The caller allocates and owns every buffer.  The library allocates nothing,
+ *    keeps no pointer after return, and fully defines the output (fill values
+ *    included), so outputs may be uninitialised memory.
+ *  - Work is only enqueued on `stream` (a hipStream_t; NULL = the null stream); no
+ *    entry point synchronises.
+ *  - Return value: 0 = ok; negative = MTA_ERR_* (argument rejected, nothing
+ *    launched); positive = hipError_t reported by the launch.
+ *  - dtype codes: MTA_F32, MTA_BF16, MTA_F16.  Accumulation is always fp32.
+ */
+#ifndef MTA_HIP_H
+#define MTA_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MTA_ABI_VERSION 1
+
+enum mta_dtype { MTA_F32 = 0, MTA_BF16 = 1, MTA_F16 = 2 };
+
+enum mta_error {
+    MTA_OK = 0,
+    MTA_ERR_NULL = -1,        /* a required pointer is NULL */
+    MTA_ERR_DTYPE = -2,       /* unknown dtype code */
+    MTA_ERR_SHAPE = -3,       /* a size is <= 0 or exceeds what the kernel indexes */
+    MTA_ERR_KERNEL_SIZE = -4, /* conv kernel R or S outside the supported range */
+    MTA_ERR_GROUP = -5,       /* group_size does not divide the head count */
+    MTA_ERR_ALIGN = -6,       /* pointer not aligned to its element size */
+    MTA_ERR_HEAD_DIM = -7,    /* head dim unsupported by the fused kernel */
+    MTA_ERR_DEVICE = -8       /* no usable gfx950 device / device query failed */
+};
+
+/* Largest conv kernel the entry points accept. */
+#define MTA_MAX_KERNEL_R 32
+#define MTA_MAX_KERNEL_S 63
+
+int mta_abi_version(void);
+const char *mta_strerror(int code);
+
+/* Depthwise (groups = channels) 2-D cross-correlation over an (N,C,H,W) score tensor:
+ *   y[n,c,p,q] = sum_{i<R, j<S} w[c,i,j] * xm[n,c, p+i-(R-1), q+j-(S-1)/2]
+ * xm = x with out-of-range taps read as 0 and, when causal, taps with col>row read
+ * as 0.  When causal every output with q>p is written as +0.0.
+ * Replaces Conv2dTritonFunction.forward + conv_fwd_kernel
+ * (convolution_2d_trit.py:302-333, 52-135).  w is (C,R,S). */
+int mta_conv2d_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H,
+                   int64_t W, int R, int S, int causal, int io_dtype, int w_dtype, void *stream);
+
+/* Same op with the input multiplied by `in_scale` as it is read (products are formed
+ * in fp32 and, for 16-bit I/O, rounded to the I/O dtype before the taps, which is what
+ * a separate elementwise scale in that dtype would produce).  Lets the caller fold
+ * the 1/sqrt(D) of mta_attention_triton.py:69-71 into the conv's load. */
+int mta_conv2d_scaled_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H,
+                          int64_t W, int R, int S, int causal, float in_scale, int io_dtype,
+                          int w_dtype, void *stream);
+
+/* Head mixing over axis 1 of an (N,C,P,Q) tensor, no transpose:
+ *   y[n,o,p,q] = sum_i w[o,i] * x[n,i,p,q]          (w is (C,C), row = output head)
+ * When causal every q>p is written as `fill` (0 or -inf) and never read.
+ * group_size = 0: w is dense.  group_size = G > 0: the caller promises w is zero
+ * outside its GxG diagonal blocks; only the blocks are read.
+ * Replaces TritonLinearHeadFunction.forward + linear_head_kernel_forward
+ * (triton_linear_head.py:283-319, 76-139). */
+int mta_headmix_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t P,
+                    int64_t Q, int group_size, int causal, float fill, int io_dtype, int w_dtype,
+                    void *stream);
+
+/* Fused head mixing + row softmax + head mixing over (N,C,P,Q), one pass:
+ *   s[o] = w1 ? sum_i w1[o,i] x[i] : x[o]      (fp32, rounded to the I/O dtype;
+ *                                               causal: q>p takes no part)
+ *   p[o] = softmax over q of s[o]              (fp32, rounded to the I/O dtype)
+ *   y[o] = w2 ? sum_i w2[o,i] p[i] : p[o]      (causal: q>p written as +0.0)
+ * w1 and/or w2 may be NULL (identity); both NULL is a plain causal row softmax.
+ * group_size as in mta_headmix_fwd and applies to both weights.
+ * Replaces the wpsm_triton -> F.softmax(scores.float()).type_as(xq) -> wposm_triton
+ * chain of mta_attention_triton.py:75-85 (the last link only when the post-softmax
+ * conv between them is the identity; otherwise pass w2 = NULL). */
+int mta_headmix_softmax_fwd(const void *x, const void *w1, const void *w2, void *y, int64_t N,
+                            int64_t C, int64_t P, int64_t Q, int group_size, int causal,
+                            int io_dtype, int w_dtype, void *stream);
+
+/* Fused conv-attention forward:
+ *   O = softmax( mask( conv( mask0(Q K^T) ) ) * scale ) V        per (batch, head)
+ * q,k,v,o are (B,H,S,D); w is (H,R,Sk).  mask0 zeroes col>row before the conv, mask
+ * sets col>row to -inf after it (both only when causal).  No S x S tensor is
+ * written.  Replaces TritonAttention.forward + _attn_fwd + qk_conv_fwd_kernel
+ * (conv_attention_triton.py:362-452, 167-356; qk_conv_kernel.py:11-184); the
+ * reference's second output (the QK scratch) has no counterpart. */
+int mta_conv_attn_fwd(const void *q, const void *k, const void *v, const void *w, void *o,
+                      int64_t B, int64_t H, int64_t S, int64_t D, int R, int Sk, int causal,
+                      float scale, int io_dtype, int w_dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MTA_HIP_H */

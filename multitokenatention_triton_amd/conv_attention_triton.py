@@ -1,0 +1,51 @@
+"""Fused conv-attention forward (HIP-backed).
+
+Mirrors TritonConvAttention (conv_attention_triton.py:476-502) and TritonAttention
+(:359-452) of the reference.  O = softmax(mask(conv(mask0(Q K^T))) * scale) V is computed
+by ``mta_conv_attn_fwd`` with score tiles kept in LDS.  The reference also returns the
+(B,H,S,S) QK scratch it fills in global memory; this build never materialises it and
+returns ``None`` in its place (the reference's own harness accepts that,
+compare_conv_attention2.py:171-187).
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from . import ops
+
+
+class TritonAttention(torch.autograd.Function):
+    """apply(Q, K, V, W, causal, softmax_scale) -> (O, None); Q,K,V are (B,H,S,D), W is (H,R,S)."""
+
+    @staticmethod
+    def forward(ctx, Q, K, V, W, causal, softmax_scale):
+        # shape checks of conv_attention_triton.py:369-370
+        assert W.shape[0] == Q.shape[1]
+        assert Q.shape[-1] == K.shape[-1] and K.shape[-1] == V.shape[-1]
+        out = ops.conv_attn_fwd(Q, K, V, W, causal, softmax_scale)
+        ctx.mark_non_differentiable(out)
+        return out, None
+
+    @staticmethod
+    def backward(ctx, dO, dQK):
+        raise NotImplementedError("the HIP build of TritonAttention is forward-only")
+
+
+class TritonConvAttention(nn.Module):
+    def __init__(self, channels, kernel_size, causal=False):
+        super().__init__()
+        self.channels = channels
+        self.kernel_size = tuple(kernel_size) if isinstance(kernel_size, (tuple, list)) else (kernel_size, kernel_size)
+        self.causal = causal
+        self.weight = nn.Parameter(torch.empty(channels, *self.kernel_size))
+        self._init_parameters()
+
+    def _init_parameters(self):
+        # the reference's default (conv_attention_triton.py:494-499): 1.0 at [R//2, S//2]
+        with torch.no_grad():
+            self.weight.zero_()
+            self.weight[:, self.kernel_size[0] // 2, self.kernel_size[1] // 2] = 1.0
+
+    def forward(self, Q, K, V, causal, softmax_scale):
+        return TritonAttention.apply(Q, K, V, self.weight, causal, softmax_scale)

@@ -1,0 +1,67 @@
+// Shared device/host helpers for the MTA forward kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mta_hip.h"
+
+namespace mta {
+
+// ---- 16-bit storage types (raw bits; arithmetic is always done in fp32) ----------
+struct bf16_t { uint16_t bits; };
+struct f16_t { _Float16 v; };
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16_t v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
+__device__ __forceinline__ float to_float(f16_t v) { return (float)v.v; }
+
+// round-to-nearest-even fp32 -> bf16 (NaN kept quiet), as torch does
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ T from_float(float v);
+template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return bf16_t{f32_to_bf16_bits(v)}; }
+template <> __device__ __forceinline__ f16_t from_float<f16_t>(float v) { return f16_t{(_Float16)v}; }
+
+// value of the I/O dtype nearest to v, as fp32 (models an intermediate stored in T)
+template <typename T> __device__ __forceinline__ float round_to(float v) { return to_float(from_float<T>(v)); }
+
+// read element `idx` of an array whose dtype is only known at run time (weights)
+__device__ __forceinline__ float load_any(const void *p, int dtype, int64_t idx)
+{
+    if (dtype == MTA_F32) return ((const float *)p)[idx];
+    if (dtype == MTA_BF16) return to_float(((const bf16_t *)p)[idx]);
+    return to_float(((const f16_t *)p)[idx]);
+}
+
+template <typename T> struct vec_of;  // elements per 16-byte vector
+template <> struct vec_of<float> { static constexpr int n = 4; };
+template <> struct vec_of<bf16_t> { static constexpr int n = 8; };
+template <> struct vec_of<f16_t> { static constexpr int n = 8; };
+
+template <typename T> struct alignas(16) pack16 { T v[vec_of<T>::n]; };
+
+// ---- host-side helpers --------------------------------------------------------------
+inline int dtype_size(int dt) { return dt == MTA_F32 ? 4 : (dt == MTA_BF16 || dt == MTA_F16) ? 2 : 0; }
+inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+inline int launch_status()
+{
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? MTA_OK : (int)e;
+}
+
+#define MTA_DISPATCH_IO(dt, ...)                                      \
+    do {                                                              \
+        if ((dt) == MTA_F32) { using io_t = float; __VA_ARGS__; }     \
+        else if ((dt) == MTA_BF16) { using io_t = mta::bf16_t; __VA_ARGS__; } \
+        else { using io_t = mta::f16_t; __VA_ARGS__; }                \
+    } while (0)
+
+}  // namespace mta

@@ -1,0 +1,161 @@
+// Head mixing over axis 1 of an (N,C,P,Q) score tensor, without a transpose.
+//
+//   y[n,o,p,q] = sum_i w[o,i] * x[n,i,p,q]
+//
+// Heads are P*Q elements apart, keys are contiguous.  Each lane owns one 16-byte
+// vector of consecutive keys q at a fixed (n,p) and walks the heads of its mixing
+// group, so every global access is a fully coalesced 16-byte-per-lane row segment
+// and the small GxG contraction happens inside the lane (no cross-lane traffic).
+// Causal: vectors wholly above the diagonal are never read and receive the fill
+// value; the vector that straddles the diagonal is masked per element.
+#include "common.hpp"
+
+namespace {
+using namespace mta;
+
+constexpr int NT = 256;
+
+template <typename T, int VEC> struct alignas(sizeof(T) * VEC) vecN { T v[VEC]; };
+
+// G heads mixed inside one lane, G known at compile time.
+template <typename T, int G, int VEC>
+__global__ __launch_bounds__(NT) void headmix_fixed(const T *__restrict__ x, const void *__restrict__ w,
+                                                    T *__restrict__ y, int C, int P, int Q, int causal,
+                                                    float fill, int w_dtype, int qchunks)
+{
+    __shared__ float wsm[G * G];
+    const int tid = threadIdx.x;
+    const int groups = C / G;
+    int64_t b = blockIdx.x;
+    const int qc = (int)(b % qchunks); b /= qchunks;
+    const int p = (int)(b % P); b /= P;
+    const int g = (int)(b % groups);
+    const int64_t n = b / groups;
+    const int q = (qc * NT + tid) * VEC;
+    const int64_t plane = (int64_t)P * Q;
+    const int64_t base = (n * C + (int64_t)g * G) * plane + (int64_t)p * Q + q;
+    using V = vecN<T, VEC>;
+    const bool chunk_above = causal && (qc * NT * VEC > p);  // uniform per workgroup
+
+    if (!chunk_above) {
+        for (int t = tid; t < G * G; t += NT)
+            wsm[t] = load_any(w, w_dtype, (int64_t)(g * G + t / G) * C + g * G + t % G);
+        __syncthreads();
+    }
+    if (q >= Q) return;
+    const T fill_t = from_float<T>(fill);
+    if (causal && q > p) {
+        V f;
+#pragma unroll
+        for (int u = 0; u < VEC; ++u) f.v[u] = fill_t;
+#pragma unroll
+        for (int o = 0; o < G; ++o) *reinterpret_cast<V *>(y + base + o * plane) = f;
+        return;
+    }
+    V xin[G];
+#pragma unroll
+    for (int i = 0; i < G; ++i) xin[i] = *reinterpret_cast<const V *>(x + base + i * plane);
+#pragma unroll
+    for (int o = 0; o < G; ++o) {
+        float acc[VEC];
+#pragma unroll
+        for (int u = 0; u < VEC; ++u) acc[u] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < G; ++i) {
+            const float wv = wsm[o * G + i];
+#pragma unroll
+            for (int u = 0; u < VEC; ++u) acc[u] = fmaf(wv, to_float(xin[i].v[u]), acc[u]);
+        }
+        V out;
+#pragma unroll
+        for (int u = 0; u < VEC; ++u) out.v[u] = (causal && q + u > p) ? fill_t : from_float<T>(acc[u]);
+        *reinterpret_cast<V *>(y + base + o * plane) = out;
+    }
+}
+
+// Any group size: one (output head, vector) per lane-iteration, inputs re-read per output head.
+template <typename T, int VEC>
+__global__ __launch_bounds__(NT) void headmix_any(const T *__restrict__ x, const void *__restrict__ w,
+                                                  T *__restrict__ y, int C, int G, int P, int Q, int causal,
+                                                  float fill, int w_dtype, int qchunks)
+{
+    const int tid = threadIdx.x;
+    const int groups = C / G;
+    int64_t b = blockIdx.x;
+    const int qc = (int)(b % qchunks); b /= qchunks;
+    const int p = (int)(b % P); b /= P;
+    const int g = (int)(b % groups);
+    const int64_t n = b / groups;
+    const int q = (qc * NT + tid) * VEC;
+    if (q >= Q) return;
+    const int64_t plane = (int64_t)P * Q;
+    const int64_t base = (n * C + (int64_t)g * G) * plane + (int64_t)p * Q + q;
+    using V = vecN<T, VEC>;
+    const T fill_t = from_float<T>(fill);
+    for (int o = 0; o < G; ++o) {
+        float acc[VEC];
+#pragma unroll
+        for (int u = 0; u < VEC; ++u) acc[u] = 0.0f;
+        if (!(causal && q > p)) {
+            for (int i = 0; i < G; ++i) {
+                const float wv = load_any(w, w_dtype, (int64_t)(g * G + o) * C + g * G + i);
+                const V xv = *reinterpret_cast<const V *>(x + base + i * plane);
+#pragma unroll
+                for (int u = 0; u < VEC; ++u) acc[u] = fmaf(wv, to_float(xv.v[u]), acc[u]);
+            }
+        }
+        V out;
+#pragma unroll
+        for (int u = 0; u < VEC; ++u) out.v[u] = (causal && q + u > p) ? fill_t : from_float<T>(acc[u]);
+        *reinterpret_cast<V *>(y + base + o * plane) = out;
+    }
+}
+
+template <typename T, int VEC>
+int launch(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t P, int64_t Q, int G, int causal,
+           float fill, int w_dtype, hipStream_t st)
+{
+    const int qchunks = (int)((Q + (int64_t)NT * VEC - 1) / ((int64_t)NT * VEC));
+    const int64_t blocks = N * (C / G) * P * qchunks;
+    if (blocks > 0x7fffffffLL) return MTA_ERR_SHAPE;
+    dim3 grid((unsigned)blocks);
+#define MTA_HM_CASE(g)                                                                                       \
+    if (G == g) {                                                                                            \
+        hipLaunchKernelGGL((headmix_fixed<T, g, VEC>), grid, dim3(NT), 0, st, (const T *)x, w, (T *)y, (int)C, \
+                           (int)P, (int)Q, causal, fill, w_dtype, qchunks);                                  \
+        return launch_status();                                                                              \
+    }
+    MTA_HM_CASE(1)
+    MTA_HM_CASE(2)
+    MTA_HM_CASE(4)
+    MTA_HM_CASE(8)
+    MTA_HM_CASE(16)
+    MTA_HM_CASE(32)
+#undef MTA_HM_CASE
+    hipLaunchKernelGGL((headmix_any<T, VEC>), grid, dim3(NT), 0, st, (const T *)x, w, (T *)y, (int)C, G, (int)P,
+                       (int)Q, causal, fill, w_dtype, qchunks);
+    return launch_status();
+}
+}  // namespace
+
+extern "C" int mta_headmix_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t P,
+                               int64_t Q, int group_size, int causal, float fill, int io_dtype, int w_dtype,
+                               void *stream)
+{
+    if (!x || !w || !y) return MTA_ERR_NULL;
+    if (!dtype_size(io_dtype) || !dtype_size(w_dtype)) return MTA_ERR_DTYPE;
+    if (N <= 0 || C <= 0 || P <= 0 || Q <= 0 || P > (1 << 24) || Q > (1 << 24) || C > 4096) return MTA_ERR_SHAPE;
+    if (group_size < 0 || (group_size > 0 && C % group_size != 0)) return MTA_ERR_GROUP;
+    if (!aligned_to(x, dtype_size(io_dtype)) || !aligned_to(y, dtype_size(io_dtype)) ||
+        !aligned_to(w, dtype_size(w_dtype)))
+        return MTA_ERR_ALIGN;
+    const int G = group_size > 0 ? group_size : (int)C;
+    hipStream_t st = (hipStream_t)stream;
+    MTA_DISPATCH_IO(io_dtype, {
+        constexpr int VEC = vec_of<io_t>::n;
+        const bool vec_ok = (Q % VEC == 0) && aligned_to(x, 16) && aligned_to(y, 16);
+        return vec_ok ? launch<io_t, VEC>(x, w, y, N, C, P, Q, G, causal, fill, w_dtype, st)
+                      : launch<io_t, 1>(x, w, y, N, C, P, Q, G, causal, fill, w_dtype, st);
+    });
+    return MTA_ERR_DTYPE;
+}

@@ -1,0 +1,265 @@
+// Fused  head-mix -> causal row softmax -> head-mix  over an (N,C,P,Q) score tensor.
+//
+// One workgroup owns one query row p of one mixing group (G heads) of one batch
+// entry.  The G x Q row segment is read once (only q <= p when causal), mixed with
+// w1 in fp32, kept in registers through the max / sum reductions, normalised, mixed
+// with w2 and written once.  This is one pass over the tensor where the unfused
+// pipeline makes three or four, and it removes the fp32 copy of the score tensor
+// that a float softmax of a 16-bit tensor would materialise.
+//
+// Rounding points of the unfused pipeline in a 16-bit dtype are reproduced: the
+// mixed scores and the probabilities are rounded to the I/O dtype before they are
+// used again.
+#include "common.hpp"
+
+namespace {
+using namespace mta;
+
+template <typename T, int VEC> struct alignas(sizeof(T) * VEC) vecN { T v[VEC]; };
+
+template <int NT> __device__ __forceinline__ float block_max(float v, float *red)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    constexpr int NW = NT / 64;
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) r = fmaxf(r, red[i]);
+    __syncthreads();
+    return r;
+}
+
+template <int NT> __device__ __forceinline__ float block_sum(float v, float *red)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    constexpr int NW = NT / 64;
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) r += red[i];
+    __syncthreads();
+    return r;
+}
+
+// Register-resident row: Q <= NT*VEC*NV.
+template <typename T, int G, int NV, int VEC, int NT>
+__global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, const void *__restrict__ w1,
+                                                      const void *__restrict__ w2, T *__restrict__ y, int C,
+                                                      int P, int Q, int causal, int w_dtype)
+{
+    __shared__ float w1s[G * G];
+    __shared__ float w2s[G * G];
+    __shared__ float red[NT / 64];
+    const int tid = threadIdx.x;
+    const int groups = C / G;
+    int64_t b = blockIdx.x;
+    const int p = (int)(b % P); b /= P;
+    const int g = (int)(b % groups);
+    const int64_t n = b / groups;
+    const int64_t plane = (int64_t)P * Q;
+    const int64_t base = (n * C + (int64_t)g * G) * plane + (int64_t)p * Q;
+    const int last = causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;  // last attended key
+    using V = vecN<T, VEC>;
+
+    for (int t = tid; t < G * G; t += NT) {
+        const int64_t widx = (int64_t)(g * G + t / G) * C + g * G + t % G;
+        w1s[t] = w1 ? load_any(w1, w_dtype, widx) : (t / G == t % G ? 1.0f : 0.0f);
+        w2s[t] = w2 ? load_any(w2, w_dtype, widx) : (t / G == t % G ? 1.0f : 0.0f);
+    }
+    __syncthreads();
+
+    float s[G][NV][VEC];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int q = (k * NT + tid) * VEC;
+        if (q <= last && q < Q) {
+            V xin[G];
+#pragma unroll
+            for (int i = 0; i < G; ++i) xin[i] = *reinterpret_cast<const V *>(x + base + i * plane + q);
+#pragma unroll
+            for (int o = 0; o < G; ++o) {
+#pragma unroll
+                for (int u = 0; u < VEC; ++u) {
+                    float acc;
+                    if (w1) {
+                        acc = 0.0f;
+#pragma unroll
+                        for (int i = 0; i < G; ++i) acc = fmaf(w1s[o * G + i], to_float(xin[i].v[u]), acc);
+                        acc = round_to<T>(acc);
+                    } else {
+                        acc = to_float(xin[o].v[u]);
+                    }
+                    s[o][k][u] = (q + u <= last) ? acc : -INFINITY;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int o = 0; o < G; ++o)
+#pragma unroll
+                for (int u = 0; u < VEC; ++u) s[o][k][u] = -INFINITY;
+        }
+    }
+
+#pragma unroll
+    for (int o = 0; o < G; ++o) {
+        float m = -INFINITY;
+#pragma unroll
+        for (int k = 0; k < NV; ++k)
+#pragma unroll
+            for (int u = 0; u < VEC; ++u) m = fmaxf(m, s[o][k][u]);
+        m = block_max<NT>(m, red);
+        float sum = 0.0f;
+#pragma unroll
+        for (int k = 0; k < NV; ++k)
+#pragma unroll
+            for (int u = 0; u < VEC; ++u) {
+                const float e = (s[o][k][u] == -INFINITY) ? 0.0f : __expf(s[o][k][u] - m);
+                s[o][k][u] = e;
+                sum += e;
+            }
+        sum = block_sum<NT>(sum, red);
+        const float inv = 1.0f / sum;
+#pragma unroll
+        for (int k = 0; k < NV; ++k)
+#pragma unroll
+            for (int u = 0; u < VEC; ++u) s[o][k][u] = round_to<T>(s[o][k][u] * inv);
+    }
+
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int q = (k * NT + tid) * VEC;
+        if (q >= Q) continue;
+#pragma unroll
+        for (int o = 0; o < G; ++o) {
+            V out;
+#pragma unroll
+            for (int u = 0; u < VEC; ++u) {
+                float acc;
+                if (w2) {
+                    acc = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < G; ++i) acc = fmaf(w2s[o * G + i], s[i][k][u], acc);
+                } else {
+                    acc = s[o][k][u];
+                }
+                out.v[u] = from_float<T>((q + u <= last) ? acc : 0.0f);
+            }
+            *reinterpret_cast<V *>(y + base + o * plane + q) = out;
+        }
+    }
+}
+
+// Any row length / any group size: three sweeps over the row, inputs re-read (and re-mixed)
+// in each; scalar accesses.  Correctness fallback for ragged or very long rows.
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) void mix_softmax_mix_any(const T *__restrict__ x, const void *__restrict__ w1,
+                                                          const void *__restrict__ w2, T *__restrict__ y, int C,
+                                                          int G, int P, int Q, int causal, int w_dtype)
+{
+    __shared__ float red[NT / 64];
+    extern __shared__ float stats[];  // [G] max, [G] 1/sum
+    const int tid = threadIdx.x;
+    const int groups = C / G;
+    int64_t b = blockIdx.x;
+    const int p = (int)(b % P); b /= P;
+    const int g = (int)(b % groups);
+    const int64_t n = b / groups;
+    const int64_t plane = (int64_t)P * Q;
+    const int64_t base = (n * C + (int64_t)g * G) * plane + (int64_t)p * Q;
+    const int last = causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;
+
+    auto mixed = [&](int o, int q) -> float {
+        if (!w1) return to_float(x[base + o * plane + q]);
+        float acc = 0.0f;
+        for (int i = 0; i < G; ++i)
+            acc = fmaf(load_any(w1, w_dtype, (int64_t)(g * G + o) * C + g * G + i), to_float(x[base + i * plane + q]), acc);
+        return round_to<T>(acc);
+    };
+    for (int o = 0; o < G; ++o) {
+        float m = -INFINITY;
+        for (int q = tid; q <= last; q += NT) m = fmaxf(m, mixed(o, q));
+        m = block_max<NT>(m, red);
+        float sum = 0.0f;
+        for (int q = tid; q <= last; q += NT) sum += __expf(mixed(o, q) - m);
+        sum = block_sum<NT>(sum, red);
+        if (tid == 0) { stats[o] = m; stats[G + o] = 1.0f / sum; }
+    }
+    __syncthreads();
+    for (int q = tid; q < Q; q += NT) {
+        for (int o = 0; o < G; ++o) {
+            float acc = 0.0f;
+            if (q <= last) {
+                if (w2) {
+                    for (int i = 0; i < G; ++i) {
+                        const float pr = round_to<T>(__expf(mixed(i, q) - stats[i]) * stats[G + i]);
+                        acc = fmaf(load_any(w2, w_dtype, (int64_t)(g * G + o) * C + g * G + i), pr, acc);
+                    }
+                } else {
+                    acc = round_to<T>(__expf(mixed(o, q) - stats[o]) * stats[G + o]);
+                }
+            }
+            y[base + o * plane + q] = from_float<T>(acc);
+        }
+    }
+}
+
+template <typename T, int G, int NV>
+int launch_fixed(const void *x, const void *w1, const void *w2, void *y, int64_t N, int64_t C, int64_t P,
+                 int64_t Q, int causal, int w_dtype, hipStream_t st)
+{
+    constexpr int VEC = vec_of<T>::n;
+    constexpr int NT = 256;
+    const int64_t blocks = N * (C / G) * P;
+    hipLaunchKernelGGL((mix_softmax_mix<T, G, NV, VEC, NT>), dim3((unsigned)blocks), dim3(NT), 0, st, (const T *)x,
+                       w1, w2, (T *)y, (int)C, (int)P, (int)Q, causal, w_dtype);
+    return launch_status();
+}
+
+template <typename T>
+int dispatch(const void *x, const void *w1, const void *w2, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
+             int G, int causal, int w_dtype, hipStream_t st)
+{
+    constexpr int VEC = vec_of<T>::n;
+    const bool vec_ok = (Q % VEC == 0) && aligned_to(x, 16) && aligned_to(y, 16);
+    const int64_t nv = (Q + 256 * VEC - 1) / (256 * VEC);
+    if (vec_ok) {
+#define MTA_RS_CASE(g, v)                                                                   \
+    if (G == g && nv <= v) return launch_fixed<T, g, v>(x, w1, w2, y, N, C, P, Q, causal, w_dtype, st);
+        MTA_RS_CASE(1, 1) MTA_RS_CASE(1, 2) MTA_RS_CASE(1, 4) MTA_RS_CASE(1, 8)
+        MTA_RS_CASE(2, 1) MTA_RS_CASE(2, 2) MTA_RS_CASE(2, 4)
+        MTA_RS_CASE(4, 1) MTA_RS_CASE(4, 2) MTA_RS_CASE(4, 4)
+        MTA_RS_CASE(8, 1) MTA_RS_CASE(8, 2)
+#undef MTA_RS_CASE
+    }
+    constexpr int NT = 256;
+    const int64_t blocks = N * (C / G) * P;
+    hipLaunchKernelGGL((mix_softmax_mix_any<T, NT>), dim3((unsigned)blocks), dim3(NT), sizeof(float) * 2 * G, st,
+                       (const T *)x, w1, w2, (T *)y, (int)C, G, (int)P, (int)Q, causal, w_dtype);
+    return launch_status();
+}
+}  // namespace
+
+extern "C" int mta_headmix_softmax_fwd(const void *x, const void *w1, const void *w2, void *y, int64_t N,
+                                       int64_t C, int64_t P, int64_t Q, int group_size, int causal,
+                                       int io_dtype, int w_dtype, void *stream)
+{
+    if (!x || !y) return MTA_ERR_NULL;
+    if (!dtype_size(io_dtype) || !dtype_size(w_dtype)) return MTA_ERR_DTYPE;
+    if (N <= 0 || C <= 0 || P <= 0 || Q <= 0 || P > (1 << 24) || Q > (1 << 24) || C > 4096) return MTA_ERR_SHAPE;
+    if (group_size < 0 || (group_size > 0 && C % group_size != 0)) return MTA_ERR_GROUP;
+    if (!aligned_to(x, dtype_size(io_dtype)) || !aligned_to(y, dtype_size(io_dtype)) ||
+        (w1 && !aligned_to(w1, dtype_size(w_dtype))) || (w2 && !aligned_to(w2, dtype_size(w_dtype))))
+        return MTA_ERR_ALIGN;
+    int G = group_size > 0 ? group_size : (int)C;
+    if (!w1 && !w2) G = 1;
+    if (N * (C / G) * P > 0x7fffffffLL) return MTA_ERR_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    MTA_DISPATCH_IO(io_dtype, return dispatch<io_t>(x, w1, w2, y, N, C, P, Q, G, causal, w_dtype, st));
+    return MTA_ERR_DTYPE;
+}

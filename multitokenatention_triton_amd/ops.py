@@ -1,0 +1,185 @@
+"""Tensor-level wrappers over the C ABI: torch supplies device memory and the stream,
+every computation happens in libmta_hip.so.  No fallback: a CPU tensor or a missing
+library raises.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+_DTYPE_CODE = {torch.float32: _lib.MTA_F32, torch.bfloat16: _lib.MTA_BF16, torch.float16: _lib.MTA_F16}
+
+
+def _code(t: torch.Tensor, what: str) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise TypeError(f"{what}: dtype {t.dtype} is not supported (float32, bfloat16, float16)") from None
+
+
+def _device_tensor(t: torch.Tensor, what: str) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{what} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{what} lives on {t.device}: the MTA kernels only run on an AMD GPU "
+                           "(there is no CPU path)")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _out_like(x: torch.Tensor, out: Optional[torch.Tensor]) -> torch.Tensor:
+    if out is None:
+        return torch.empty_like(x, memory_format=torch.contiguous_format)
+    if out.shape != x.shape or out.dtype != x.dtype or out.device != x.device or not out.is_contiguous():
+        raise ValueError("out must be a contiguous tensor with the input's shape, dtype and device")
+    return out
+
+
+def conv2d_causal(x: torch.Tensor, weight: torch.Tensor, causal: bool, in_scale: Optional[float] = None,
+                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Depthwise conv over (N,C,H,W) with a (C,R,S) kernel; see mta_conv2d_fwd in include/mta_hip.h."""
+    x = _device_tensor(x, "input")
+    weight = _device_tensor(weight.detach(), "weight")
+    if x.dim() != 4 or weight.dim() != 3:
+        raise ValueError(f"expected input (N,C,H,W) and weight (C,R,S), got {tuple(x.shape)} and {tuple(weight.shape)}")
+    n, c, h, w = x.shape
+    c_out, r, s = weight.shape
+    # same check and message as convolution_2d_trit.py:306
+    assert c == c_out, "This implementation assumes depthwise convolution (C_in == C_out)"
+    y = _out_like(x, out)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        if in_scale is None:
+            rc = lib.mta_conv2d_fwd(x.data_ptr(), weight.data_ptr(), y.data_ptr(), n, c, h, w, r, s, int(bool(causal)),
+                                    _code(x, "input"), _code(weight, "weight"), _stream(x))
+        else:
+            rc = lib.mta_conv2d_scaled_fwd(x.data_ptr(), weight.data_ptr(), y.data_ptr(), n, c, h, w, r, s,
+                                           int(bool(causal)), float(in_scale), _code(x, "input"),
+                                           _code(weight, "weight"), _stream(x))
+    _lib.check(rc, "mta_conv2d_fwd")
+    return y
+
+
+def headmix(x: torch.Tensor, weight: torch.Tensor, causal: bool = True, fill: float = 0.0,
+            group_size: Optional[int] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y[n,o,p,q] = sum_i W[o,i] x[n,i,p,q]; see mta_headmix_fwd in include/mta_hip.h."""
+    x = _device_tensor(x, "input")
+    weight = _device_tensor(weight.detach(), "weight")
+    if x.dim() != 4:
+        raise ValueError(f"expected input (N,C,P,Q), got {tuple(x.shape)}")
+    n, c, p, q = x.shape
+    l = weight.shape[0]
+    # same checks and messages as triton_linear_head.py:286-290
+    assert tuple(weight.shape) == (l, l), f"Weight must be square matrix, got {weight.shape}"
+    assert c == l, f"Channel dimension {c} must match weight dimension {l}"
+    y = _out_like(x, out)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().mta_headmix_fwd(x.data_ptr(), weight.data_ptr(), y.data_ptr(), n, c, p, q,
+                                         int(group_size or 0), int(bool(causal)), float(fill), _code(x, "input"),
+                                         _code(weight, "weight"), _stream(x))
+    _lib.check(rc, "mta_headmix_fwd")
+    return y
+
+
+def headmix_softmax(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optional[torch.Tensor], causal: bool = True,
+                    group_size: Optional[int] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """mix(w1) -> causal row softmax -> mix(w2) in one pass; see mta_headmix_softmax_fwd."""
+    x = _device_tensor(x, "input")
+    if x.dim() != 4:
+        raise ValueError(f"expected input (N,C,P,Q), got {tuple(x.shape)}")
+    n, c, p, q = x.shape
+    ws = []
+    for w in (w1, w2):
+        if w is not None:
+            w = _device_tensor(w.detach(), "weight")
+            assert tuple(w.shape) == (c, c), f"Weight must be ({c},{c}), got {tuple(w.shape)}"
+        ws.append(w)
+    present = [w for w in ws if w is not None]
+    if len(present) == 2 and present[0].dtype != present[1].dtype:
+        raise TypeError("w1 and w2 must share a dtype")
+    wcode = _code(present[0], "weight") if present else _lib.MTA_F32
+    y = _out_like(x, out)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().mta_headmix_softmax_fwd(
+            x.data_ptr(), ws[0].data_ptr() if ws[0] is not None else None,
+            ws[1].data_ptr() if ws[1] is not None else None, y.data_ptr(), n, c, p, q, int(group_size or 0),
+            int(bool(causal)), _code(x, "input"), wcode, _stream(x))
+    _lib.check(rc, "mta_headmix_softmax_fwd")
+    return y
+
+
+def conv_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, weight: torch.Tensor, causal: bool,
+                  softmax_scale: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """O = softmax(mask(conv(mask0(QK^T))) * scale) V for (B,H,S,D) inputs; see mta_conv_attn_fwd."""
+    q = _device_tensor(q, "Q")
+    k = _device_tensor(k, "K")
+    v = _device_tensor(v, "V")
+    weight = _device_tensor(weight.detach(), "W")
+    if q.dim() != 4 or q.shape != k.shape or q.shape != v.shape:
+        raise ValueError(f"Q, K, V must share a (B,H,S,D) shape, got {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}")
+    if not (q.dtype == k.dtype == v.dtype):
+        raise TypeError("Q, K, V must share a dtype")
+    b, h, s, d = q.shape
+    # same check as conv_attention_triton.py:369
+    assert weight.dim() == 3 and weight.shape[0] == h, "CHANNEL_DIM == NUM_HEADS"
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    o = _out_like(q, out)
+    with torch.cuda.device(q.device):
+        rc = _lib.load().mta_conv_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), weight.data_ptr(), o.data_ptr(),
+                                           b, h, s, d, weight.shape[1], weight.shape[2], int(bool(causal)),
+                                           float(softmax_scale), _code(q, "Q"), _code(weight, "W"), _stream(q))
+    _lib.check(rc, "mta_conv_attn_fwd")
+    return o
+
+
+# ---------------------------------------------------------------------------------------
+# weight structure probes (host side, cached per weight version; one device->host copy each)
+# ---------------------------------------------------------------------------------------
+_probe_cache: dict = {}
+
+
+def _cached(kind: str, w: torch.Tensor, fn):
+    key = (kind, w.data_ptr(), w._version, tuple(w.shape), w.dtype, str(w.device))
+    hit = _probe_cache.get(key)
+    if hit is None:
+        if len(_probe_cache) > 256:
+            _probe_cache.clear()
+        hit = fn(w.detach().float().cpu())
+        _probe_cache[key] = hit
+    return hit
+
+
+def block_diagonal_group(weight: torch.Tensor) -> int:
+    """Smallest G dividing H such that the (H,H) weight is zero outside its GxG diagonal blocks."""
+    def probe(w):
+        h = w.shape[0]
+        nz = w != 0
+        for g in range(1, h + 1):
+            if h % g:
+                continue
+            idx = torch.arange(h) // g
+            if not bool((nz & (idx[:, None] != idx[None, :])).any()):
+                return g
+        return h
+    return _cached("group", weight, probe)
+
+
+def is_identity_head_weight(weight: torch.Tensor) -> bool:
+    return _cached("eye", weight, lambda w: bool(torch.equal(w, torch.eye(w.shape[0]))))
+
+
+def is_identity_conv_kernel(weight: torch.Tensor) -> bool:
+    """True when the (C,R,S) kernel is exactly 1.0 at [R-1, S//2] and 0 elsewhere (a pass-through)."""
+    def probe(w):
+        ref = torch.zeros_like(w)
+        ref[:, -1, w.shape[-1] // 2] = 1.0
+        return bool(torch.equal(w, ref)) and (w.shape[-1] % 2 == 1)
+    return _cached("delta", weight, probe)

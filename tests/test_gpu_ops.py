@@ -1,0 +1,186 @@
+"""GPU parity of the standalone operators (through the C ABI) against the CPU oracle.
+
+Tolerances (written here once):
+  fp32 I/O : rtol 1e-4, atol 1e-5
+  bf16/fp16: atol 2e-2 plus one unit in the last place of the 16-bit format as rtol
+             (2^-7 for bf16, 2^-10 for fp16) -- an op output of magnitude m cannot be
+             pinned tighter than the oracle's own rounding of m.
+Causal fill patterns (+0.0 / -inf above the diagonal) are compared bit-exactly.
+"""
+import pytest
+import torch
+
+from oracle import mta_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DT = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+
+
+def tol(dtype):
+    if dtype == torch.float32:
+        return dict(rtol=1e-4, atol=1e-5)
+    return dict(rtol=2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10, atol=2e-2)
+
+
+def _randn(shape, seed, dtype, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (std * torch.randn(*shape, generator=g)).to(dtype)
+
+
+def _upper(p, q):
+    return torch.triu(torch.ones(p, q, dtype=torch.bool), 1)
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from multitokenatention_triton_amd import ops as _ops
+    return _ops
+
+
+CONV_CASES = [
+    # N, C, H(=W), R, S
+    (1, 2, 1, 3, 3), (1, 1, 7, 1, 1), (2, 3, 37, 3, 5), (1, 2, 64, 6, 11), (1, 2, 130, 6, 11),
+    (1, 1, 100, 4, 6), (1, 2, 96, 11, 15), (1, 1, 70, 2, 7), (1, 4, 256, 3, 5), (1, 1, 45, 32, 63),
+]
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv_parity(ops, case, causal, dt):
+    n, c, s, r, sk = case
+    dtype = DT[dt]
+    print(f"conv case={case} causal={causal} dt={dt}", flush=True)
+    x = _randn((n, c, s, s), 1, dtype)
+    if causal:
+        x = torch.tril(x)
+    w = _randn((c, r, sk), 2, dtype, 0.2)
+    want = O.depthwise_conv(x.float(), w.float(), causal)
+    want_rounded = want.to(dtype)
+    got = ops.conv2d_causal(x.cuda(), w.cuda(), causal).cpu()
+    assert got.dtype == dtype and got.shape == x.shape
+    torch.testing.assert_close(got.float(), want_rounded.float(), **tol(dtype))
+    if causal:
+        up = _upper(s, s)
+        assert (got[..., up] == 0).all() and not torch.signbit(got[..., up]).any()
+
+
+@pytest.mark.parametrize("wdt", ["f32", "bf16"])
+def test_conv_weight_dtype_and_scale(ops, wdt):
+    x = torch.tril(_randn((1, 2, 80, 80), 3, torch.bfloat16, 8.0))
+    w = _randn((2, 6, 11), 4, DT[wdt], 0.05)
+    scale = float(torch.rsqrt(torch.tensor(128.0)))
+    xs = x * torch.rsqrt(torch.tensor(128))          # bf16 result, as the reference computes it
+    want = O.depthwise_conv(xs.float(), w.float(), True).to(torch.bfloat16)
+    got = ops.conv2d_causal(x.cuda(), w.cuda(), True, in_scale=scale).cpu()
+    torch.testing.assert_close(got.float(), want.float(), **tol(torch.bfloat16))
+
+
+def test_conv_identity_tap_bit_exact(ops):
+    for dtype in (torch.float32, torch.bfloat16):
+        x = _randn((2, 3, 77, 77), 5, dtype)
+        w = O.identity_conv_kernel(3, 6, 11, dtype)
+        got = ops.conv2d_causal(x.cuda(), w.cuda(), True).cpu()
+        assert torch.equal(got, torch.tril(x) + 0.0)
+
+
+def test_conv_delta_is_shift(ops):
+    x = torch.tril(_randn((1, 1, 50, 50), 6, torch.float32))
+    for (i, j) in [(0, 0), (2, 4), (5, 10), (3, 5)]:
+        w = torch.zeros(1, 6, 11)
+        w[0, i, j] = 1.0
+        got = ops.conv2d_causal(x.cuda(), w.cuda(), True).cpu()
+        assert torch.equal(got, O.depthwise_conv(x, w, True))
+
+
+HM_CASES = [
+    # N, C, P, Q, group (None = dense)
+    (1, 4, 9, 9, None), (2, 4, 64, 64, 2), (1, 8, 40, 40, 4), (1, 6, 33, 33, None), (1, 6, 24, 24, 3),
+    (1, 16, 48, 48, None), (1, 32, 16, 16, 4), (1, 32, 24, 24, None), (2, 2, 300, 300, 1), (1, 4, 5, 2056, 2),
+]
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("causal,fill", [(True, 0.0), (True, float("-inf")), (False, 0.0)])
+@pytest.mark.parametrize("case", HM_CASES)
+def test_headmix_parity(ops, case, causal, fill, dt):
+    n, c, p, q, group = case
+    dtype = DT[dt]
+    print(f"headmix case={case} causal={causal} fill={fill} dt={dt}", flush=True)
+    x = _randn((n, c, p, q), 7, dtype)
+    g = torch.Generator().manual_seed(8)
+    if group:
+        w = O.block_diag_head_weight(c, group, 0.1, g, dtype)
+    else:
+        w = (torch.eye(c) + 0.1 * torch.randn(c, c, generator=g)).to(dtype)
+    want = O.head_linear(x.float(), w.float(), causal, fill).to(dtype)
+    got = ops.headmix(x.cuda(), w.cuda(), causal, fill, group_size=group).cpu()
+    if causal:
+        up = _upper(p, q)
+        if fill == 0.0:
+            assert (got[..., up] == 0).all() and not torch.signbit(got[..., up]).any()
+        else:
+            assert torch.isneginf(got[..., up]).all()
+        low = ~up
+        torch.testing.assert_close(got[..., low].float(), want[..., low].float(), **tol(dtype))
+    else:
+        torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+    if group:  # the group hint must not change the result of the dense contraction
+        dense = ops.headmix(x.cuda(), w.cuda(), causal, fill, group_size=None).cpu()
+        torch.testing.assert_close(dense.float().nan_to_num(neginf=-1e30), got.float().nan_to_num(neginf=-1e30),
+                                   **tol(dtype))
+
+
+def test_headmix_identity_and_permutation_bit_exact(ops):
+    x = _randn((1, 4, 31, 31), 9, torch.bfloat16)
+    got = ops.headmix(x.cuda(), torch.eye(4).cuda(), True, 0.0).cpu()
+    assert torch.equal(got, torch.tril(x) + 0.0)
+    perm = torch.tensor([2, 0, 3, 1])
+    wp = torch.zeros(4, 4)
+    wp[torch.arange(4), perm] = 1.0
+    got = ops.headmix(x.cuda(), wp.cuda(), True, 0.0).cpu()
+    assert torch.equal(got, torch.tril(x[:, perm]) + 0.0)
+
+
+MS_CASES = [
+    # N, C, P(=Q), group, use_w1, use_w2
+    (1, 4, 64, 2, True, True), (2, 4, 100, 4, True, False), (1, 8, 257, 4, False, True), (1, 2, 33, 1, False, False),
+    (1, 8, 2048, 4, True, True), (1, 3, 50, 3, True, True), (1, 8, 72, 8, True, True), (1, 4, 4096, 4, True, True),
+]
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("case", MS_CASES)
+def test_mix_softmax_mix_parity(ops, case, causal, dt):
+    n, c, s, group, use1, use2 = case
+    dtype = DT[dt]
+    print(f"mix_softmax_mix case={case} causal={causal} dt={dt}", flush=True)
+    x = _randn((n, c, s, s), 10, dtype, 2.0)
+    g = torch.Generator().manual_seed(11)
+    w1 = O.block_diag_head_weight(c, group, 0.1, g, dtype) if use1 else None
+    w2 = O.block_diag_head_weight(c, group, 0.1, g, dtype) if use2 else None
+    s2 = O.head_linear(x, w1, causal, float("-inf")) if use1 else (
+        x.masked_fill(_upper(s, s), float("-inf")) if causal else x)
+    p0 = torch.softmax(s2.float(), -1).to(dtype)
+    want = O.head_linear(p0, w2, causal, 0.0) if use2 else p0
+    got = ops.headmix_softmax(x.cuda(), w1.cuda() if use1 else None, w2.cuda() if use2 else None, causal,
+                              group_size=group).cpu()
+    if causal:
+        up = _upper(s, s)
+        assert (got[..., up] == 0).all() and not torch.signbit(got[..., up]).any()
+    t = tol(dtype)
+    torch.testing.assert_close(got.float(), want.float(), rtol=t["rtol"] * 2, atol=2e-3 if dtype != torch.float32 else 1e-6)
+
+
+def test_error_codes(ops):
+    x = torch.zeros(1, 2, 8, 8, device="cuda")
+    with pytest.raises(ValueError, match="kernel size"):
+        ops.conv2d_causal(x, torch.zeros(2, 40, 3, device="cuda"), True)
+    with pytest.raises(ValueError, match="group"):
+        ops.headmix(torch.zeros(1, 6, 8, 8, device="cuda"), torch.eye(6).cuda(), True, 0.0, group_size=4)
+    with pytest.raises(AssertionError):
+        ops.conv2d_causal(x, torch.zeros(3, 3, 3, device="cuda"), True)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.conv2d_causal(x.cpu(), torch.zeros(2, 3, 3), True)
