@@ -11,8 +11,14 @@ mta_attention_pytorch.py:58-83):
     post-softmax conv kernel is the identity tap -- the post-softmax head mixing run
     as one kernel (``mta_headmix_softmax_fwd``): one pass over the score tensor
     instead of four, and no fp32 copy of it;
-  * block-diagonal head-mixing weights are detected (once per weight version) and
-    only their blocks are applied.
+  * block-diagonal head-mixing weights are detected and only their blocks are applied.
+
+Weight structure (identity conv tap, identity / block-diagonal head weights) is probed on
+the host and remembered per parameter, keyed by the parameter's autograd version counter
+and storage address.  Optimizer steps, ``load_state_dict``, ``copy_`` under ``no_grad`` and
+this module's own reset/copy methods all move that counter.  A write through ``.data``
+does not: after one, call ``refresh_structure()`` (or construct the module with
+``weight_structure="dense"``, which never assumes any structure).
 """
 from __future__ import annotations
 
@@ -72,6 +78,9 @@ class MTAAttentionTriton(nn.Module):
         self.wposm_triton = TritonLinearHead(n_heads, causal=causal)
         # optional observer: called as hook(stage_name) right before each stage is enqueued
         self._stage_hook = None
+        # "auto": probe weight structure and pick specialised kernels; "dense": assume nothing
+        self.weight_structure = "auto"
+        self._structure = {}
 
     # ------------------------------------------------------------------ forward
     def _mark(self, name: str) -> None:
@@ -92,11 +101,11 @@ class MTAAttentionTriton(nn.Module):
         scores = ops.conv2d_causal(scores, self.mta_conv_triton.weight, self.causal, in_scale=scale)
 
         w_pre, w_post = self.wpsm_triton.weight, self.wposm_triton.weight
-        g_pre = 1 if ops.is_identity_head_weight(w_pre) else ops.block_diagonal_group(w_pre)
-        g_post = 1 if ops.is_identity_head_weight(w_post) else ops.block_diagonal_group(w_post)
-        post_conv_identity = ops.is_identity_conv_kernel(self.mta_conv_after_sm_triton.weight)
-        w1 = None if g_pre == 1 and ops.is_identity_head_weight(w_pre) else w_pre
-        w2 = None if g_post == 1 and ops.is_identity_head_weight(w_post) else w_post
+        pre_eye, g_pre = self._probe("wpsm", w_pre, _probe_head)
+        post_eye, g_post = self._probe("wposm", w_post, _probe_head)
+        post_conv_identity = self._probe("conv_post", self.mta_conv_after_sm_triton.weight, _probe_conv)
+        w1 = None if pre_eye else w_pre
+        w2 = None if post_eye else w_post
 
         if post_conv_identity and _lcm(g_pre, g_post) <= _FUSED_MAX_GROUP:
             self._mark("mix_softmax_mix")
@@ -123,6 +132,20 @@ class MTAAttentionTriton(nn.Module):
         output = torch.matmul(scores, xv)
         self._mark("end")
         return output.transpose(1, 2)
+
+    def _probe(self, name, weight, fn):
+        if self.weight_structure != "auto":
+            return (False, self.n_heads) if fn is _probe_head else False
+        key = (id(weight), weight._version, weight.data_ptr(), weight.dtype)
+        hit = self._structure.get(name)
+        if hit is None or hit[0] != key:
+            hit = (key, fn(weight))
+            self._structure[name] = hit
+        return hit[1]
+
+    def refresh_structure(self):
+        """Forget what was learnt about the weights' structure (needed after writes through ``.data``)."""
+        self._structure.clear()
 
     def _forward_with_mask(self, xq, xk, xv, mask):
         """use_mask=True: an explicit additive mask tensor drives the masking (mta_attention_triton.py:63-64,
@@ -206,6 +229,17 @@ class MTAAttentionTriton(nn.Module):
                 self.wpsm_triton.weight.copy_(mta_attention.wpsm.weight.data)
             if hasattr(mta_attention, "wposm"):
                 self.wposm_triton.weight.copy_(mta_attention.wposm.weight.data)
+
+
+def _probe_head(w):
+    """(is identity, block-diagonal group size)."""
+    if ops.is_identity_head_weight(w):
+        return True, 1
+    return False, ops.block_diagonal_group(w)
+
+
+def _probe_conv(w):
+    return ops.is_identity_conv_kernel(w)
 
 
 def _lcm(a: int, b: int) -> int:

@@ -141,45 +141,30 @@ def conv_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, weight: tor
 
 
 # ---------------------------------------------------------------------------------------
-# weight structure probes (host side, cached per weight version; one device->host copy each)
+# weight structure probes (host side: each call copies the small weight to the host once)
 # ---------------------------------------------------------------------------------------
-_probe_cache: dict = {}
-
-
-def _cached(kind: str, w: torch.Tensor, fn):
-    key = (kind, w.data_ptr(), w._version, tuple(w.shape), w.dtype, str(w.device))
-    hit = _probe_cache.get(key)
-    if hit is None:
-        if len(_probe_cache) > 256:
-            _probe_cache.clear()
-        hit = fn(w.detach().float().cpu())
-        _probe_cache[key] = hit
-    return hit
-
-
 def block_diagonal_group(weight: torch.Tensor) -> int:
     """Smallest G dividing H such that the (H,H) weight is zero outside its GxG diagonal blocks."""
-    def probe(w):
-        h = w.shape[0]
-        nz = w != 0
-        for g in range(1, h + 1):
-            if h % g:
-                continue
-            idx = torch.arange(h) // g
-            if not bool((nz & (idx[:, None] != idx[None, :])).any()):
-                return g
-        return h
-    return _cached("group", weight, probe)
+    w = weight.detach().float().cpu()
+    h = w.shape[0]
+    nz = w != 0
+    for g in range(1, h + 1):
+        if h % g:
+            continue
+        idx = torch.arange(h) // g
+        if not bool((nz & (idx[:, None] != idx[None, :])).any()):
+            return g
+    return h
 
 
 def is_identity_head_weight(weight: torch.Tensor) -> bool:
-    return _cached("eye", weight, lambda w: bool(torch.equal(w, torch.eye(w.shape[0]))))
+    w = weight.detach().float().cpu()
+    return bool(torch.equal(w, torch.eye(w.shape[0])))
 
 
 def is_identity_conv_kernel(weight: torch.Tensor) -> bool:
-    """True when the (C,R,S) kernel is exactly 1.0 at [R-1, S//2] and 0 elsewhere (a pass-through)."""
-    def probe(w):
-        ref = torch.zeros_like(w)
-        ref[:, -1, w.shape[-1] // 2] = 1.0
-        return bool(torch.equal(w, ref)) and (w.shape[-1] % 2 == 1)
-    return _cached("delta", weight, probe)
+    """True when the (C,R,S) kernel is exactly 1.0 at [R-1, S//2] and 0 elsewhere, S odd (a pass-through)."""
+    w = weight.detach().float().cpu()
+    ref = torch.zeros_like(w)
+    ref[:, -1, w.shape[-1] // 2] = 1.0
+    return bool(torch.equal(w, ref)) and (w.shape[-1] % 2 == 1)

@@ -183,7 +183,9 @@ def conv_attention_forward(Q, K, V, conv_weight, causal: bool = True,
         scores = scores.masked_fill(upper, 0)
     r, sk = conv_weight.shape[-2], conv_weight.shape[-1]
     pad_k = (sk - 1) // 2
-    padded = F.pad(scores, (pad_k, pad_k, r - 1, 0), value=0.0)
+    # reference: (pad_k, pad_k), key size odd.  For an even key size the right pad is
+    # sk-1-pad_k, the index arithmetic of qk_conv_kernel.py:126-129 (pad_k on the left).
+    padded = F.pad(scores, (pad_k, sk - 1 - pad_k, r - 1, 0), value=0.0)
     conv = F.conv2d(padded, conv_weight.to(Q.dtype).unsqueeze(1), padding=0, groups=h)
     if causal:
         conv = conv.masked_fill(upper, NEG_INF)
@@ -213,7 +215,7 @@ def conv_attention_rows(Q, K, V, conv_weight, row0: int, row1: int, causal: bool
     if causal:
         scores = scores.masked_fill(upper, 0)
     pad_k = (sk - 1) // 2
-    padded = F.pad(scores, (pad_k, pad_k, top_pad, 0), value=0.0)
+    padded = F.pad(scores, (pad_k, sk - 1 - pad_k, top_pad, 0), value=0.0)
     conv = F.conv2d(padded, conv_weight.to(Q.dtype).unsqueeze(1), padding=0, groups=h)
     if causal:
         conv = conv.masked_fill(upper[row0 - lo:], NEG_INF)

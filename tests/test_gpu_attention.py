@@ -1,0 +1,172 @@
+"""GPU parity of the two attention entry points against the CPU oracle.
+
+  MTAAttentionTriton.forward      vs oracle.mta_forward            (mta_attention_pytorch.py:58-83)
+  TritonConvAttention.forward     vs oracle.conv_attention_forward (conv_attention_pytorch.py:33-71)
+
+Tolerances: fp32 rtol 1e-4 / atol 1e-5; bf16 and fp16 atol 2e-2 (outputs are convex
+combinations of N(0,1) values, so |out| is O(1) and no rtol is added).
+"""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import mta_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def tol(dtype):
+    return dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=0.0, atol=2e-2)
+
+
+@pytest.fixture(scope="module")
+def pkg():
+    import multitokenatention_triton_amd as m
+    return m
+
+
+def _mta_module(pkg, h, r1, s1, r2, s2, w_pre, wpsm, w_post, wposm, dtype, causal=True):
+    cfg = pkg.MTAConfig(query_kernel_size=r1, key_kernel_size=s1, after_sm_query_kernel_size=r2,
+                        after_sm_key_kernel_size=s2)
+    mod = pkg.MTAAttentionTriton(h, cfg, dropout=0.0, causal=causal, use_mask=False)
+    with torch.no_grad():
+        mod.mta_conv_triton.weight.copy_(w_pre)
+        mod.wpsm_triton.weight.copy_(wpsm)
+        mod.mta_conv_after_sm_triton.weight.copy_(w_post)
+        mod.wposm_triton.weight.copy_(wposm)
+    return mod.to(dtype).cuda().eval()
+
+
+def _config_like(h, group, r1, s1, std, dtype, post="identity", seed=123):
+    g = torch.Generator().manual_seed(seed + 2)
+    w_pre = O.seeded_conv_weight(h, r1, s1, std, torch.float32, seed=seed + 1)
+    wpsm = O.block_diag_head_weight(h, group, 0.1, g)
+    wposm = O.block_diag_head_weight(h, group, 0.1, g)
+    if post == "identity":
+        w_post = O.identity_conv_kernel(h, 3, 3)
+    else:
+        w_post = O.seeded_conv_weight(h, 3, 3, 0.05, torch.float32, seed=seed + 3)
+    return [t.to(dtype) for t in (w_pre, wpsm, w_post, wposm)]
+
+
+def _oracle_mta(q, k, v, params):
+    w_pre, wpsm, w_post, wposm = params
+    return O.mta_forward(q, k, v, w_pre.unsqueeze(1), wpsm, w_post.unsqueeze(1), wposm)
+
+
+def test_mta_config1_fp32(pkg):
+    """BASELINE config 1: B1 H4 S256 D64 fp32, 3x5 conv + identity tap, head-mix groups of 2."""
+    print("mta config1 fp32", flush=True)
+    q, k, v = O.seeded_qkv(1, 4, 256, 64, torch.float32)
+    params = _config_like(4, 2, 3, 5, 0.1, torch.float32)
+    want = _oracle_mta(q, k, v, params)
+    mod = _mta_module(pkg, 4, 3, 5, 3, 3, *params, torch.float32)
+    got = mod(q.cuda(), k.cuda(), v.cuda(), None, None)
+    assert got.shape == (1, 256, 4, 64) and not got.is_contiguous()
+    torch.testing.assert_close(got.cpu(), want, **tol(torch.float32))
+
+
+@pytest.mark.parametrize("post", ["identity", "random"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_mta_general(pkg, dtype, post):
+    print(f"mta general {dtype} post={post}", flush=True)
+    q, k, v = O.seeded_qkv(2, 8, 200, 64, dtype)
+    params = _config_like(8, 4, 6, 11, 0.05, dtype, post=post)
+    want = _oracle_mta(q, k, v, params)
+    mod = _mta_module(pkg, 8, 6, 11, 3, 3, *params, dtype)
+    got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
+    torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+
+
+def test_mta_dense_head_weights(pkg):
+    print("mta dense", flush=True)
+    dtype = torch.float32
+    q, k, v = O.seeded_qkv(1, 16, 96, 64, dtype)
+    g = torch.Generator().manual_seed(5)
+    params = [O.seeded_conv_weight(16, 3, 3, 0.1, dtype), torch.eye(16) + 0.1 * torch.randn(16, 16, generator=g),
+              O.seeded_conv_weight(16, 3, 3, 0.1, dtype, seed=9), torch.eye(16) + 0.1 * torch.randn(16, 16, generator=g)]
+    want = _oracle_mta(q, k, v, params)
+    mod = _mta_module(pkg, 16, 3, 3, 3, 3, *params, dtype)
+    got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
+    torch.testing.assert_close(got, want, **tol(dtype))
+
+
+def test_mta_identity_weights_is_sdpa(pkg):
+    """The reference's own check (compare_mta_attention.py:21-27, 61-74): B2 H16 S128 D64 fp32, seed 123."""
+    print("mta identity", flush=True)
+    cfg = pkg.MTAConfig()
+    mod = pkg.MTAAttentionTriton(16, cfg, 0.0, True).cuda().eval()
+    mod.reset_mta_parameters()
+    q, k, v = O.seeded_qkv(2, 16, 128, 64, torch.float32, seed=123)
+    got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
+    want = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2)
+    torch.testing.assert_close(got, want, rtol=1e-3, atol=1e-5)  # the reference script's own bar
+    torch.testing.assert_close(got, want, **tol(torch.float32))
+
+
+def test_mta_use_mask_path(pkg):
+    print("mta use_mask", flush=True)
+    dtype = torch.float32
+    q, k, v = O.seeded_qkv(1, 4, 64, 64, dtype)
+    params = _config_like(4, 2, 3, 5, 0.1, dtype, post="random")
+    want = _oracle_mta(q, k, v, params)
+    cfg = pkg.MTAConfig(query_kernel_size=3, key_kernel_size=5)
+    mod = pkg.MTAAttentionTriton(4, cfg, 0.0, True, use_mask=True)
+    with torch.no_grad():
+        for dst, src in zip((mod.mta_conv_triton, mod.wpsm_triton, mod.mta_conv_after_sm_triton, mod.wposm_triton), params):
+            dst.weight.copy_(src)
+    mod = mod.cuda().eval()
+    got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
+    torch.testing.assert_close(got, want, **tol(dtype))
+
+
+CA_CASES = [
+    # B, H, S, D, R, Sk, causal, dtype
+    (2, 8, 128, 64, 3, 3, True, torch.float32),     # compare_conv_attention2.py:106-125 shape, seed 42
+    (1, 2, 300, 64, 6, 11, True, torch.float32),
+    (1, 2, 257, 128, 6, 11, True, torch.bfloat16),
+    (1, 3, 200, 128, 5, 7, False, torch.bfloat16),
+    (1, 2, 130, 64, 1, 1, True, torch.float16),
+    (1, 1, 64, 64, 2, 2, True, torch.float32),
+    (1, 2, 500, 128, 11, 15, True, torch.float32),
+    (1, 1, 1, 64, 3, 3, True, torch.float32),
+    (1, 2, 1000, 128, 6, 11, True, torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("case", CA_CASES)
+def test_conv_attention_parity(pkg, case):
+    b, h, s, d, r, sk, causal, dtype = case
+    print(f"conv_attention case={case}", flush=True)
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=42)
+    w = O.seeded_conv_weight(h, r, sk, 0.05, dtype)
+    want = O.conv_attention_forward(q, k, v, w, causal, None)
+    mod = pkg.TritonConvAttention(h, (r, sk), causal=causal)
+    with torch.no_grad():
+        mod.weight.copy_(w)
+    mod = mod.to(dtype).cuda()
+    got, qk = mod(q.cuda(), k.cuda(), v.cuda(), causal, d ** -0.5)
+    assert qk is None and got.shape == q.shape and got.is_contiguous()
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dtype))
+
+
+def test_conv_attention_identity_tap_is_sdpa(pkg):
+    print("conv_attention identity", flush=True)
+    q, k, v = O.seeded_qkv(2, 8, 128, 64, torch.float32, seed=42)
+    w = O.identity_conv_kernel(8, 3, 3)
+    for causal in (True, False):
+        got = pkg.ops.conv_attn_fwd(q.cuda(), k.cuda(), v.cuda(), w.cuda(), causal, None).cpu()
+        want = F.scaled_dot_product_attention(q, k, v, is_causal=causal)
+        torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-5)
+
+
+def test_conv_attention_row_slabs_long_sequence(pkg):
+    """S=4096 bf16 6x11: compare three row slabs with the slab form of the oracle."""
+    print("conv_attention slabs", flush=True)
+    dtype = torch.bfloat16
+    q, k, v = O.seeded_qkv(1, 2, 4096, 128, dtype)
+    w = O.seeded_conv_weight(2, 6, 11, 0.05, dtype)
+    got = pkg.ops.conv_attn_fwd(q.cuda(), k.cuda(), v.cuda(), w.cuda(), True, None).cpu()
+    for r0, r1 in [(0, 128), (2040, 2170), (3968, 4096)]:
+        want = O.conv_attention_rows(q, k, v, w, r0, r1, True, None)
+        torch.testing.assert_close(got[:, :, r0:r1].float(), want.float(), **tol(dtype))
