@@ -1,0 +1,230 @@
+#!/usr/bin/env python3
+"""Benchmark of the MTA forward path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extras]
+
+A step is one full Multi-Token-Attention forward (MTAAttentionTriton.forward) at the
+configuration the headline metric is quoted on: B=2, H=16, S=4096, D=128, bf16, causal,
+6x11 pre-softmax conv (N(0,0.05) + identity tap), identity pre-softmax head weights,
+identity 3x3 post-softmax conv, post-softmax head mixing in groups of 4 (I + N(0,0.1)).
+Inputs are synthetic, seeded, and resident in HBM before the timed region.  Prints ONE
+JSON line.  `value` is the latency of one forward in ms.
+
+The `roofline` object is for the slowest hand-written kernel of the step; its duration
+is measured live with events recorded on the stream the kernels run on.  `kernels` adds
+the standalone operators at their own configurations (conv alone, head-mix alone, fused
+conv-attention).  `cpu_baseline` times the oracle (a torch restatement of the
+reference's PyTorch module) on the host cores, on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
+MFMA_BF16_PEAK_TF = 2500.0  # MI355X dense bf16, published
+
+
+def tri(s: int) -> int:
+    return s * (s + 1) // 2
+
+
+def score_pass_bytes(b, h, s, esize):
+    """Algorithmic bytes of one causal pass over a (B,H,S,S) tensor: read the lower triangle, write everything."""
+    return b * h * (tri(s) + s * s) * esize
+
+
+def build_c4(torch, mta, O, device, b=2, h=16, s=4096, d=128, dtype=None, nsets=3):
+    dtype = dtype or torch.bfloat16
+    g = torch.Generator().manual_seed(125)
+    cfg = mta.MTAConfig(query_kernel_size=6, key_kernel_size=11)
+    mod = mta.MTAAttentionTriton(h, cfg, dropout=0.0, causal=True).to(dtype)
+    with torch.no_grad():
+        mod.mta_conv_triton.weight.copy_(O.seeded_conv_weight(h, 6, 11, 0.05, dtype))
+        mod.wpsm_triton.weight.copy_(torch.eye(h))
+        mod.mta_conv_after_sm_triton.weight.copy_(O.identity_conv_kernel(h, 3, 3, dtype))
+        mod.wposm_triton.weight.copy_(O.block_diag_head_weight(h, 4, 0.1, g, dtype))
+    mod = mod.to(device).eval()
+    sets = [tuple(t.to(device) for t in O.seeded_qkv(b, h, s, d, dtype, seed=123 + i)) for i in range(nsets)]
+    return mod, sets
+
+
+def time_steps(torch, fn, nsets, warmup, steps):
+    for i in range(warmup):
+        fn(i % nsets)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        fn(i % nsets)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def stage_breakdown(torch, mod, sets, steps):
+    """Average duration of each stage of forward(), from events on the kernels' own stream."""
+    marks = []
+    mod._stage_hook = lambda name: marks.append((name, _record(torch)))
+    per_step = []
+    for i in range(steps):
+        marks.clear()
+        mod(*sets[i % len(sets)], None, None)
+        per_step.append(list(marks))
+    torch.cuda.synchronize()
+    mod._stage_hook = None
+    acc = {}
+    for m in per_step:
+        for (name, ev), (_, nxt) in zip(m[:-1], m[1:]):
+            acc.setdefault(name, []).append(ev.elapsed_time(nxt))
+    return {k: sum(v) / len(v) for k, v in acc.items()}
+
+
+def _record(torch):
+    ev = torch.cuda.Event(enable_timing=True)
+    ev.record()  # on the current stream, the one ops.py hands to the library
+    return ev
+
+
+def bench_kernels(torch, mta, O, device, steps, warmup):
+    """Standalone operators at their own BASELINE configurations."""
+    out = {}
+    bf16 = torch.bfloat16
+    g = torch.Generator().manual_seed(7)
+    # conv alone: (2,16,2048,2048) bf16, 6x11 N(0,0.05), causal
+    n, c, s = 2, 16, 2048
+    w = O.seeded_conv_weight(c, 6, 11, 0.05, bf16, identity_tap=False).to(device)
+    xs = [torch.tril(torch.randn(n, c, s, s, generator=g).to(bf16)).to(device) for _ in range(3)]
+    ys = [torch.empty_like(x) for x in xs]
+    ms = time_steps(torch, lambda i: mta.ops.conv2d_causal(xs[i], w, True, out=ys[i]), 3, warmup, steps)
+    by = score_pass_bytes(n, c, s, 2)
+    out["conv2d_6x11_bf16_2x16x2048x2048"] = {"ms": ms, "algorithmic_bytes": by, "GBps": by / ms / 1e6,
+                                              "frac_hbm_peak": by / ms / 1e6 / HBM_PEAK_GBS}
+    del xs, ys
+    # head-mix alone: (2,32,2048,2048) bf16, groups of 4
+    n, c, s = 2, 32, 2048
+    wm = O.block_diag_head_weight(c, 4, 0.1, g, bf16).to(device)
+    xs = []
+    for _ in range(2):
+        logits = torch.randn(n, c, s, s, generator=g)
+        logits.masked_fill_(torch.triu(torch.ones(s, s, dtype=torch.bool), 1), float("-inf"))
+        xs.append(torch.softmax(logits, -1).to(bf16).to(device))
+        del logits
+    ys = [torch.empty_like(x) for x in xs]
+    by = score_pass_bytes(n, c, s, 2)
+    for label, grp in (("headmix_g4_bf16_2x32x2048x2048", 4), ("headmix_dense_bf16_2x32x2048x2048", None)):
+        ms = time_steps(torch, lambda i: mta.ops.headmix(xs[i], wm, True, 0.0, group_size=grp, out=ys[i]), 2, warmup, steps)
+        out[label] = {"ms": ms, "algorithmic_bytes": by, "GBps": by / ms / 1e6, "frac_hbm_peak": by / ms / 1e6 / HBM_PEAK_GBS}
+    del xs, ys
+    # fused conv-attention: B1 H32 S8192 D128 bf16, 6x11
+    b, h, s, d = 1, 32, 8192, 128
+    sets = [tuple(t.to(device) for t in O.seeded_qkv(b, h, s, d, bf16, seed=200 + i)) for i in range(2)]
+    wc = O.seeded_conv_weight(h, 6, 11, 0.05, bf16).to(device)
+    os_ = [torch.empty_like(sets[0][0]) for _ in range(2)]
+    ms = time_steps(torch, lambda i: mta.ops.conv_attn_fwd(*sets[i], wc, True, None, out=os_[i]), 2, min(warmup, 2),
+                    max(2, steps // 4))
+    mfma_flops = 4 * b * h * tri(s) * d
+    out["conv_attn_fused_bf16_1x32x8192x128"] = {"ms": ms, "mfma_useful_flops": mfma_flops,
+                                                 "TFLOPs": mfma_flops / ms / 1e9,
+                                                 "frac_mfma_peak": mfma_flops / ms / 1e9 / MFMA_BF16_PEAK_TF}
+    return out
+
+
+def cpu_baseline(torch, O, b, h, s, d, budget_s=15.0):
+    """The oracle's torch MTA forward on the host cores, on a bounded sample of the same workload."""
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+    torch.set_num_threads(threads)
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(125)
+    w_pre = O.seeded_conv_weight(h, 6, 11, 0.05, dtype).unsqueeze(1)
+    w_post = O.identity_conv_kernel(h, 3, 3, dtype).unsqueeze(1)
+    wpsm = torch.eye(h, dtype=dtype)
+    wposm = O.block_diag_head_weight(h, 4, 0.1, g, dtype)
+
+    def run(ss):
+        q, k, v = O.seeded_qkv(1, h, ss, d, dtype)
+        t0 = time.perf_counter()
+        with torch.no_grad():
+            O.mta_forward(q, k, v, w_pre, wpsm, w_post, wposm)
+        return time.perf_counter() - t0
+
+    probe_s = 256
+    t_probe = min(run(probe_s), run(probe_s))
+    ss = probe_s
+    while ss * 2 <= s and t_probe * ((ss * 2) / probe_s) ** 2 <= budget_s:
+        ss *= 2
+    t = run(ss) if ss != probe_s else t_probe
+    factor = (b * s * s) / (1 * ss * ss)
+    return {"value": t * 1e3 * factor, "unit": "ms", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle.mta_forward bf16 on B=1,H={h},S={ss},D={d} took {t * 1e3:.1f} ms; "
+                      f"scaled by {factor:.0f} (score-tensor elements) to B={b},S={s}",
+            "cpu_model": _cpu_model()}
+
+
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+
+    import multitokenatention_triton_amd as mta
+    from oracle import mta_oracle as O
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    device = torch.device("cuda:0")
+    b, h, s, d = 2, 16, 4096, 128
+    mod, sets = build_c4(torch, mta, O, device, b, h, s, d)
+
+    with torch.no_grad():
+        ms = time_steps(torch, lambda i: mod(*sets[i], None, None), len(sets), args.warmup, args.steps)
+        stages = stage_breakdown(torch, mod, sets, max(3, min(args.steps, 10)))
+        hip_stages = {k: v for k, v in stages.items() if k not in ("qk", "pv")}
+        dom = max(hip_stages, key=hip_stages.get)
+        dom_bytes = score_pass_bytes(b, h, s, 2)
+        achieved = dom_bytes / hip_stages[dom] / 1e6
+        kernels = {} if args.no_extras else bench_kernels(torch, mta, O, device, args.steps, args.warmup)
+
+    result = {
+        "metric": "MTA fwd latency (ms) + conv/head-mix HBM GB/s, H16 S4096 D128 bf16",
+        "value": ms, "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "full MTA forward B=2 H=16 S=4096 D=128 bf16 causal, conv 6x11 pre-softmax, "
+                               "identity post-softmax conv, head-mix groups of 4 (BASELINE configs[3])",
+                   "global_batch": b, "seq_len": s},
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes": dom_bytes,
+                     "avg_kernel_ms": hip_stages[dom]},
+        "stages_ms": stages,
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(torch, O, b, h, s, d)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
