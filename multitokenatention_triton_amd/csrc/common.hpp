@@ -27,7 +27,8 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f)
 
 template <typename T> __device__ __forceinline__ T from_float(float v);
 template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
-template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return bf16_t{f32_to_bf16_bits(v)}; }
+// gfx950 converts fp32 -> bf16 (round to nearest even) in hardware; the compiler emits it for this cast
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return __builtin_bit_cast(bf16_t, (__bf16)v); }
 template <> __device__ __forceinline__ f16_t from_float<f16_t>(float v) { return f16_t{(_Float16)v}; }
 
 // value of the I/O dtype nearest to v, as fp32 (models an intermediate stored in T)

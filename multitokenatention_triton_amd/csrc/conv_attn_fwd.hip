@@ -22,43 +22,14 @@
 // softmax / PV of a block lag the scores by the right-hand pad so that every tap is
 // already there.  One extra leading key block (mostly out-of-range keys) primes that halo.
 #include "common.hpp"
+#include "mfma.hpp"
 
 namespace {
 using namespace mta;
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
-
 constexpr int NT = 256;  // 4 wavefronts
 constexpr int SR = 128;  // score-tile rows (32 per wavefront)
 constexpr int BK = 64;   // keys per iteration
-
-// 8 contraction slots of one lane: slot t of lane-half h.  A and B fragments use the same
-// slot <-> k assignment, whatever it is in hardware, so only consistency matters here.
-template <typename T> struct alignas(sizeof(T) * 8 > 16 ? 16 : sizeof(T) * 8) frag8 { T v[8]; };
-
-__device__ __forceinline__ void mma32(f32x16 &c, const frag8<bf16_t> &a, const frag8<bf16_t> &b)
-{
-    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-}
-__device__ __forceinline__ void mma32(f32x16 &c, const frag8<f16_t> &a, const frag8<f16_t> &b)
-{
-    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
-}
-__device__ __forceinline__ void mma32(f32x16 &c, const frag8<float> &a, const frag8<float> &b)
-{
-#pragma unroll
-    for (int t = 0; t < 8; ++t) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[t], b.v[t], c, 0, 0, 0);
-}
-
-template <typename T> __device__ __forceinline__ frag8<T> zero_frag()
-{
-    frag8<T> f;
-#pragma unroll
-    for (int t = 0; t < 8; ++t) f.v[t] = from_float<T>(0.0f);
-    return f;
-}
 
 // position of key offset k16 (0..15) inside its 16-key group of the V^T tile: the order in
 // which a lane's accumulator registers enumerate the keys of a 32x32 block (see header).

@@ -1,0 +1,43 @@
+// 32x32 MFMA wrappers shared by the kernels (gfx950).
+//
+// A lane owns 8 contraction slots of an operand fragment: slot t of lane-half h = lane/32,
+// for operand row (A) or column (B) lane%32.  A and B use the same slot <-> k assignment in
+// hardware, so kernels only have to be consistent between the two operands.  The 32x32
+// fp32 accumulator gives lane (n = lane%32, h) the 16 values  D[m][n],
+// m = 8*(v/4) + 4*h + v%4  for v = 0..15.
+#pragma once
+
+#include "common.hpp"
+
+namespace mta {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+
+template <typename T> struct alignas(sizeof(T) * 8 > 16 ? 16 : sizeof(T) * 8) frag8 { T v[8]; };
+
+__device__ __forceinline__ void mma32(f32x16 &c, const frag8<bf16_t> &a, const frag8<bf16_t> &b)
+{
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ void mma32(f32x16 &c, const frag8<f16_t> &a, const frag8<f16_t> &b)
+{
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+}
+// fp32 operands: eight 32x32x2 steps, slot t of both fragments feeding step t
+__device__ __forceinline__ void mma32(f32x16 &c, const frag8<float> &a, const frag8<float> &b)
+{
+#pragma unroll
+    for (int t = 0; t < 8; ++t) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[t], b.v[t], c, 0, 0, 0);
+}
+
+template <typename T> __device__ __forceinline__ frag8<T> zero_frag()
+{
+    frag8<T> f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) f.v[t] = from_float<T>(0.0f);
+    return f;
+}
+
+}  // namespace mta

@@ -42,6 +42,9 @@ CONV_CASES = [
     # N, C, H(=W), R, S
     (1, 2, 1, 3, 3), (1, 1, 7, 1, 1), (2, 3, 37, 3, 5), (1, 2, 64, 6, 11), (1, 2, 130, 6, 11),
     (1, 1, 100, 4, 6), (1, 2, 96, 11, 15), (1, 1, 70, 2, 7), (1, 4, 256, 3, 5), (1, 1, 45, 32, 63),
+    # widths divisible by 8: 16-bit inputs take the MFMA (Toeplitz) kernel
+    (1, 2, 136, 6, 11), (2, 2, 520, 6, 11), (1, 1, 128, 7, 9), (1, 2, 264, 5, 7), (1, 1, 1032, 3, 3),
+    (1, 3, 8, 6, 11), (1, 1, 392, 7, 7), (1, 2, 200, 5, 5),
 ]
 
 
