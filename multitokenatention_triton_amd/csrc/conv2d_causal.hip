@@ -167,29 +167,25 @@ int dispatch_valu(const void *x, const void *w, void *y, int64_t N, int64_t C, i
 // MFMA (Toeplitz) path
 // ------------------------------------------------------------------------------------
 #ifndef MTA_CONV_WAVES_PER_SIMD
-#define MTA_CONV_WAVES_PER_SIMD 2
+#define MTA_CONV_WAVES_PER_SIMD 2  // register budget: 256 VGPRs
+#endif
+#ifndef MTA_CONV_WG_PER_CU
+#define MTA_CONV_WG_PER_CU 6       // LDS budget: two 11.6 KB strip buffers per single-wavefront workgroup
 #endif
 constexpr int M_WT = 64;   // one wavefront per workgroup
-constexpr int M_TM = 32;   // strip rows   (one accumulator column per lane%32)
-constexpr int M_TN = 128;  // strip cols   (4 sub-tiles of 32 keys)
+constexpr int M_TM = 32;   // strip rows: 2 row blocks of 16
+constexpr int M_TN = 128;  // strip cols: 8 column blocks of 16
 
+// 16 outputs + S-1 taps (+ alignment shift) must fit the 32-key contraction of one 16x16x32 MFMA
 template <int R, int S> struct mfma_geom {
     static constexpr int PADW = (S - 1) / 2;
-    static constexpr int HL = (PADW + 7) & ~7;                 // left halo, rounded so 16-byte loads stay aligned
-    static constexpr int SHIFT = HL - PADW;                    // first tap's offset inside a sub-tile's window
-    static constexpr int NCH = (SHIFT + 32 + S - 1 + 15) / 16; // 16-key chunks per 32-output window
-    static constexpr int TW = M_TN - 32 + 16 * NCH;            // staged columns
-    static constexpr int LD = TW + ((24 - TW % 16) % 16);      // row stride = 8 (mod 16) elements: conflict-free b128 reads
+    static constexpr int HL = (PADW + 7) & ~7;             // left halo, rounded so 16-byte loads stay aligned
+    static constexpr int SHIFT = HL - PADW;                // first tap's offset inside a block's 32-key window
+    static constexpr bool fits = SHIFT + 16 + S - 1 <= 32;
+    static constexpr int TW = M_TN - 16 + 32;              // staged columns
+    static constexpr int LD = TW + ((24 - TW % 16) % 16);  // row stride = 8 (mod 16) elements: conflict-free b128 reads
     static constexpr int ROWS = M_TM + R - 1;
 };
-
-// logical output column (0..31) held by accumulator row m.  Accumulator register v of lane-half
-// h is row m = 8*(v/4) + 4*h + v%4; this choice makes it column 16*(v/8) + 8*h + v%8, so one
-// 16-byte store per lane covers 8 consecutive keys and the two halves of a row sit side by side.
-__device__ __forceinline__ int toeplitz_q_of_m(int m)
-{
-    return 16 * (m >> 4) + 8 * ((m >> 2) & 1) + 4 * ((m >> 3) & 1) + (m & 3);
-}
 
 // work item -> (plane, strip row tm (32 rows), strip col tn (128 keys)).
 // `mirror` (causal, square): only strips that touch the lower triangle are enumerated, by 128x128
@@ -226,23 +222,44 @@ __device__ __forceinline__ void zero_fill_strip(T *yp, int H, int W, int p0, int
     }
 }
 
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef const __attribute__((address_space(1))) void glb_void_t;
+
 // Persistent single-wavefront workgroups: each walks a contiguous run of 32x128 strips (so the
 // Toeplitz fragments are rebuilt only when the channel changes).  No workgroup barrier is ever
 // needed; latency is hidden by the other wavefronts resident on the CU, each in its own phase
 // (loading / matrix cores / storing) with its own 11 KB LDS strip.
+//
+// Per 16x16 output block and kernel row i:  out^T[q, p] += T_i^T[q, k] X^T[k, p+i-(R-1)], one
+// v_mfma_f32_16x16x32 whose 32-key contraction window holds the 16 outputs' taps.  A operand =
+// Toeplitz fragment (4 VGPRs per kernel row, kept for the whole kernel), B operand = 16 contiguous
+// bytes of one staged row per lane.  Results go back through the (now free) LDS strip so that the
+// global stores are whole 256-byte row segments.
+//
+// Staging.  A strip whose halo lies wholly inside the tensor and on or below the diagonal (the
+// common case, decided per wavefront) is copied global -> LDS by global_load_lds_dwordx4: no
+// registers, no masks, no LDS store instructions.  The LDS row stride is 19 16-byte slots (18 of
+// data + 1 of padding), so lane L of copy `it` simply owns slot it*64+L.  Edge strips go through
+// registers, where bounds and the causal col<=row rule are applied.
+//
+// SCALED: the result is in_scale * conv(x), the factor being applied to the fp32 accumulator.
 template <typename T, int R, int S, bool SCALED>
 __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     const T *__restrict__ x, const T *__restrict__ w, T *__restrict__ y, int C, int H, int W, int causal, float in_scale,
     int tiles_n, int ipp, int64_t total, int64_t per_xcd, int nw, int mirror)
 {
     using G = mfma_geom<R, S>;
-    constexpr int LD = G::LD, NCH = G::NCH, VEC = 8;
-    constexpr int VPR = G::TW / VEC;                            // 16-byte vectors per staged row
-    constexpr int STAGE_IT = (G::ROWS * VPR + M_WT - 1) / M_WT; // vectors per lane
+    constexpr int LD = G::LD, VEC = 8;
+    constexpr int VPR = G::TW / VEC;                        // data vectors per staged row (18)
+    constexpr int SPR = LD / VEC;                           // 16-byte slots per LDS row (19)
+    constexpr int SLOTS = G::ROWS * SPR;
+    constexpr int STAGE_IT = (SLOTS + M_WT - 1) / M_WT;     // copies per strip
+    static_assert(SPR == VPR + 1, "one padding slot per row");
     // weights of the current channel, each kernel row zero-padded on both sides so that the
     // Toeplitz fragments can be gathered without range checks
-    constexpr int WZ_OFF = G::SHIFT + 32, WZ_LD = WZ_OFF + 16 * NCH + 2;
-    __shared__ __align__(16) T tile[G::ROWS * LD];
+    constexpr int WZ_OFF = G::SHIFT + 16, WZ_LD = WZ_OFF + 32;
+    constexpr int BUF = STAGE_IT * M_WT * VEC;  // elements per LDS strip buffer
+    __shared__ __align__(16) T tiles[2 * BUF];  // double buffer: strip n is computed while strip n+1 lands
     __shared__ T wz[R * WZ_LD];
     using V16 = pack16<T>;
 
@@ -250,40 +267,104 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     // contiguous chunk of the item list (whole planes, mostly), so halo re-reads stay in its L2.
     const int64_t c0 = (int64_t)(blockIdx.x & 7) * per_xcd;
     const int64_t c1 = (c0 + per_xcd < total) ? c0 + per_xcd : total;
-    const int64_t per_wg = (c1 - c0 + nw - 1) / nw;
-    const int64_t first = c0 + (int64_t)(blockIdx.x >> 3) * per_wg;
-    const int64_t last = (first + per_wg < c1) ? first + per_wg : c1;
+    // within the chunk the items are dealt round-robin to the XCD's workgroups, so that at any moment
+    // they sweep the same few hundred rows together (DRAM pages are consumed whole, as by a linear copy)
+    const int64_t first = c0 + (int64_t)(blockIdx.x >> 3);
+    const int64_t last = c1;
+    const int64_t step = nw;
     if (c0 >= total || first >= last) return;
 
-    const int lane = threadIdx.x, ln = lane & 31, hf = lane >> 5;
-    frag8<T> tz[R][NCH];
+    const int lane = threadIdx.x, ln = lane & 15, kg = lane >> 4;
+    frag8<T> tz[R];
     int cur_channel = -1;
 
-    // per-lane staging geometry, fixed for the whole kernel: slot `it` of this lane is row rr, vector vc
-    // of the halo strip; goff/loff are its element offsets from the strip origin in global memory / LDS
-    int goff[STAGE_IT], loff[STAGE_IT];
+    // per-lane geometry of the staging copies, fixed for the whole kernel: slot it*64+lane is row srow,
+    // vector svc of the strip; padding slots and slots past the strip re-read a neighbouring valid vector
+    int goff[STAGE_IT];
 #pragma unroll
     for (int it = 0; it < STAGE_IT; ++it) {
-        const int e = it * M_WT + lane;
-        const bool in = e < G::ROWS * VPR;
-        const int rr = in ? e / VPR : 0, vc = in ? e % VPR : 0;
+        const int slot = it * M_WT + lane;
+        int rr = slot / SPR, vc = slot % SPR;
+        if (rr >= G::ROWS) { rr = 0; vc = 0; }
+        if (vc >= VPR) vc = VPR - 1;
         goff[it] = rr * W + vc * VEC;
-        loff[it] = in ? rr * LD + vc * VEC : -1;
     }
-    const int soff = ln * W + hf * 8;  // this lane's output offset from the strip's first output
 
-    for (int64_t idx = first; idx < last; ++idx) {
-        int64_t plane;
-        int tm, tn;
-        decode_item(idx, ipp, tiles_n, mirror, plane, tm, tn);
+    // a strip is `interior` when its whole halo lies inside the tensor and on or below the diagonal
+    auto is_interior = [&](int p0_, int q0_) {
+        const int h0 = p0_ - (R - 1), k0 = q0_ - G::HL;
+        return h0 >= 0 && p0_ + M_TM <= H && k0 >= 0 && k0 + G::TW <= W && (!causal || k0 + G::TW - 1 <= h0);
+    };
+    // asynchronous copy of an interior strip into LDS buffer `buf`
+    auto prefetch = [&](int64_t plane_, int p0_, int q0_, T *buf) {
+        const T *base = x + plane_ * (int64_t)H * W + (int64_t)(p0_ - (R - 1)) * W + (q0_ - G::HL);
+#pragma unroll
+        for (int it = 0; it < STAGE_IT; ++it)
+            __builtin_amdgcn_global_load_lds((glb_void_t *)(base + goff[it]), (lds_void_t *)(buf + it * M_WT * VEC), 16, 0, 0);
+    };
+
+    int64_t plane;
+    int tm, tn;
+    decode_item(first, ipp, tiles_n, mirror, plane, tm, tn);
+    if (is_interior(tm * M_TM, tn * M_TN)) prefetch(plane, tm * M_TM, tn * M_TN, tiles);
+
+    int parity = 0;
+    for (int64_t idx = first; idx < last; idx += step, parity ^= 1) {
+        T *tile = tiles + parity * BUF;
+        T *other = tiles + (parity ^ 1) * BUF;
         const int p0 = tm * M_TM, q0 = tn * M_TN;
+        const int ctm = tm, ctn = tn;
         const T *xp = x + plane * (int64_t)H * W;
         T *yp = y + plane * (int64_t)H * W;
-        if (causal && q0 > p0 + M_TM - 1) {  // wholly above the diagonal (only reachable when !mirror)
+        const int channel = (int)(plane % C);
+        const bool above = causal && q0 > p0 + M_TM - 1;  // wholly above the diagonal (only reachable when !mirror)
+        const bool interior = is_interior(p0, q0);
+        const int h0 = p0 - (R - 1), k0 = q0 - G::HL;
+
+        // everything issued so far has landed: this strip's copy (if interior) and the previous strip's
+        // stores; LDS reads of `other` by the previous iteration are complete as well
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+
+        // put the next strip's copy in flight (into the buffer the previous iteration has just released)
+        if (idx + step < last) {
+            decode_item(idx + step, ipp, tiles_n, mirror, plane, tm, tn);
+            if (is_interior(tm * M_TM, tn * M_TN)) prefetch(plane, tm * M_TM, tn * M_TN, other);
+        }
+        if (above) {
             zero_fill_strip<T>(yp, H, W, p0, q0, lane);
             continue;
         }
-        const int channel = (int)(plane % C);
+        if (!interior) {
+            // edge strip: through registers.  Loads are unconditional and issued back to back (an invalid
+            // slot re-reads a valid address); what a slot really holds is decided on the way to LDS
+            V16 stage[STAGE_IT];
+#pragma unroll
+            for (int it = 0; it < STAGE_IT; ++it) {
+                const int slot = it * M_WT + lane;
+                const int rr = slot / SPR, vc = slot % SPR;
+                const int h = h0 + rr, col = k0 + vc * VEC;
+                const bool ok = rr < G::ROWS && vc < VPR && h >= 0 && h < H && col >= 0 && col < W && !(causal && col > h);
+                stage[it] = *reinterpret_cast<const V16 *>(xp + (ok ? (int64_t)h * W + col : 0));
+            }
+#pragma unroll
+            for (int it = 0; it < STAGE_IT; ++it) {
+                const int slot = it * M_WT + lane;
+                const int rr = slot / SPR, vc = slot % SPR;
+                const int h = h0 + rr, col = k0 + vc * VEC;
+                const bool ok = rr < G::ROWS && vc < VPR && h >= 0 && h < H && col >= 0 && col < W && !(causal && col > h);
+                V16 v = stage[it];
+                if (!ok) {
+#pragma unroll
+                    for (int u = 0; u < VEC; ++u) v.v[u] = from_float<T>(0.0f);
+                } else if (causal && col + VEC - 1 > h) {  // the one vector of a row that straddles the diagonal
+#pragma unroll
+                    for (int u = 0; u < VEC; ++u)
+                        if (col + u > h) v.v[u] = from_float<T>(0.0f);
+                }
+                *reinterpret_cast<V16 *>(tile + slot * VEC) = v;
+            }
+        }
         if (channel != cur_channel) {
             for (int e = lane; e < R * WZ_LD; e += M_WT) {
                 const int i = e / WZ_LD, j = e % WZ_LD - WZ_OFF;
@@ -292,121 +373,60 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
                 wz[e] = ok ? wv : from_float<T>(0.0f);
             }
         }
-        // interior strip: the whole halo strip is inside the tensor and on or below the diagonal,
-        // so staging and stores need no masks at all (the common case; decided per wavefront)
-        const int h0 = p0 - (R - 1), k0 = q0 - G::HL;
-        const bool interior = h0 >= 0 && p0 + M_TM <= H && k0 >= 0 && k0 + G::TW <= W &&
-                              (!causal || k0 + G::TW - 1 <= h0);
+        __syncthreads();  // LDS stores above are visible (single wavefront: a wait on the LDS counter)
 
-        // ---- stage rows h0.., cols k0.. into LDS.  Loads are unconditional and issued back to back
-        // (an invalid slot re-reads a valid address); masks are applied on the way to LDS.
-        {
-            V16 stage[STAGE_IT];
-            if (interior) {
-                const T *base = xp + (int64_t)h0 * W + k0;
-#pragma unroll
-                for (int it = 0; it < STAGE_IT; ++it) stage[it] = *reinterpret_cast<const V16 *>(base + goff[it]);
-#pragma unroll
-                for (int it = 0; it < STAGE_IT; ++it) {
-                    V16 v = stage[it];
-                    if (SCALED) {
-#pragma unroll
-                        for (int u = 0; u < VEC; ++u) v.v[u] = from_float<T>(to_float(v.v[u]) * in_scale);
-                    }
-                    if (it < STAGE_IT - 1 || loff[it] >= 0) *reinterpret_cast<V16 *>(tile + loff[it]) = v;
-                }
-            } else {
-#pragma unroll
-                for (int it = 0; it < STAGE_IT; ++it) {
-                    const int e = it * M_WT + lane;
-                    const int rr = e / VPR, vc = e % VPR;
-                    const int h = h0 + rr, col = k0 + vc * VEC;
-                    const bool ok = e < G::ROWS * VPR && h >= 0 && h < H && col >= 0 && col < W && !(causal && col > h);
-                    const int64_t off = ok ? (int64_t)h * W + col : 0;
-                    stage[it] = *reinterpret_cast<const V16 *>(xp + off);
-                }
-#pragma unroll
-                for (int it = 0; it < STAGE_IT; ++it) {
-                    const int e = it * M_WT + lane;
-                    const int rr = e / VPR, vc = e % VPR;
-                    const int h = h0 + rr, col = k0 + vc * VEC;
-                    const bool ok = h >= 0 && h < H && col >= 0 && col < W && !(causal && col > h);
-                    V16 v = stage[it];
-                    if (SCALED) {
-#pragma unroll
-                        for (int u = 0; u < VEC; ++u) v.v[u] = from_float<T>(to_float(v.v[u]) * in_scale);
-                    }
-                    if (!ok) {
-#pragma unroll
-                        for (int u = 0; u < VEC; ++u) v.v[u] = from_float<T>(0.0f);
-                    } else if (causal && col + VEC - 1 > h) {  // the one vector of a row that straddles the diagonal
-#pragma unroll
-                        for (int u = 0; u < VEC; ++u)
-                            if (col + u > h) v.v[u] = from_float<T>(0.0f);
-                    }
-                    if (e < G::ROWS * VPR) *reinterpret_cast<V16 *>(tile + rr * LD + vc * VEC) = v;
-                }
-            }
-        }
-        __syncthreads();  // one wavefront: orders the LDS writes above before the reads below
-
-        if (channel != cur_channel) {  // Toeplitz fragments T_i^T of this lane's accumulator row
+        if (channel != cur_channel) {  // Toeplitz fragments T_i^T: row m = ln, slots k = 8*kg + t, tap j = k-SHIFT-m
             cur_channel = channel;
-            const int qm = toeplitz_q_of_m(ln);
 #pragma unroll
-            for (int i = 0; i < R; ++i)
+            for (int i = 0; i < R; ++i) {
+                const T *src = wz + i * WZ_LD + WZ_OFF + kg * 8 - G::SHIFT - ln;
 #pragma unroll
-                for (int ch = 0; ch < NCH; ++ch) {
-                    const T *src = wz + i * WZ_LD + WZ_OFF + ch * 16 + hf * 8 - G::SHIFT - qm;  // tap j = k-SHIFT-q
-#pragma unroll
-                    for (int t = 0; t < 8; ++t) tz[i][ch].v[t] = src[t];
-                    __builtin_amdgcn_sched_barrier(0);  // keep the gathers of one fragment together (register pressure)
-                }
-        }
-
-        // ---- out^T: 32 rows x 4 sub-tiles of 32 keys, one sub-tile at a time (16 accumulators live) ----
-        const int prow = p0 + ln;  // this lane's query row
-        T *ybase = yp + (int64_t)p0 * W + q0;
-#pragma unroll
-        for (int st = 0; st < M_TN / 32; ++st) {
-            f32x16 acc;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
-            if (!(causal && q0 + st * 32 > p0 + M_TM - 1)) {  // else: sub-tile wholly above the diagonal, stays +0
-#pragma unroll
-                for (int i = 0; i < R; ++i) {
-                    const T *rowp = tile + (ln + i) * LD + hf * 8 + st * 32;
-#pragma unroll
-                    for (int ch = 0; ch < NCH; ++ch)
-                        mma32(acc, tz[i][ch], *reinterpret_cast<const frag8<T> *>(rowp + ch * 16));
-                }
-            }
-            // accumulator registers 8a..8a+7 of lane (row, half) are 8 consecutive keys
-            if (interior) {
-#pragma unroll
-                for (int a = 0; a < 2; ++a) {
-                    V16 out;
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) out.v[u] = from_float<T>(acc[a * 8 + u]);
-                    *reinterpret_cast<V16 *>(ybase + soff + st * 32 + a * 16) = out;
-                }
-            } else if (prow < H) {
-#pragma unroll
-                for (int a = 0; a < 2; ++a) {
-                    const int q = q0 + st * 32 + a * 16 + hf * 8;
-                    if (q >= W) continue;
-                    V16 out;
-#pragma unroll
-                    for (int u = 0; u < 8; ++u)
-                        out.v[u] = from_float<T>((causal && q + u > prow) ? 0.0f : acc[a * 8 + u]);
-                    *reinterpret_cast<V16 *>(yp + (int64_t)prow * W + q) = out;
-                }
+                for (int t = 0; t < 8; ++t) tz[i].v[t] = src[t];
             }
         }
-        __syncthreads();  // LDS reads done before the next item's staging overwrites the strip
 
-        if (mirror && tn < (tm >> 2))  // a quarter of the 128x128 block's image above the diagonal
-            zero_fill_strip<T>(yp, H, W, q0 + (tm & 3) * M_TM, (tm >> 2) * M_TN, lane);
+        // ---- 2 row blocks x 8 column blocks of 16x16 outputs; results of a row block go back into its
+        // own (no longer needed) LDS rows: lane (row ln, group kg) holds keys 4*kg..4*kg+3 of each block
+#pragma unroll
+        for (int rb = 0; rb < M_TM / 16; ++rb) {
+            f32x4 acc[M_TN / 16];
+#pragma unroll
+            for (int cb = 0; cb < M_TN / 16; ++cb) {
+                acc[cb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                if (!interior && causal && q0 + cb * 16 > p0 + rb * 16 + 15) continue;  // block wholly above the diagonal: +0
+#pragma unroll
+                for (int i = 0; i < R; ++i)
+                    mma16(acc[cb], tz[i],
+                          *reinterpret_cast<const frag8<T> *>(tile + (rb * 16 + ln + i) * LD + cb * 16 + kg * 8));
+            }
+            const int prow = p0 + rb * 16 + ln;
+#pragma unroll
+            for (int cb = 0; cb < M_TN / 16; ++cb) {
+                struct alignas(8) quad { T v[4]; } out;
+                const int q = q0 + cb * 16 + kg * 4;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float val = SCALED ? acc[cb][v] * in_scale : acc[cb][v];
+                    out.v[v] = from_float<T>((!interior && causal && q + v > prow) ? 0.0f : val);
+                }
+                *reinterpret_cast<quad *>(tile + (rb * 16 + ln) * LD + cb * 16 + kg * 4) = out;
+            }
+        }
+        __syncthreads();
+
+        // ---- coalesced stores: 16 lanes cover one 256-byte output row ----
+        {
+            T *ybase = yp + (int64_t)p0 * W + q0;
+            const int r_l = lane >> 4, cv = (lane & 15) * VEC;
+#pragma unroll
+            for (int it = 0; it < M_TM * (M_TN / VEC) / M_WT; ++it) {
+                const int r = it * 4 + r_l;
+                const V16 v = *reinterpret_cast<const V16 *>(tile + r * LD + cv);
+                if (interior || (p0 + r < H && q0 + cv < W)) *reinterpret_cast<V16 *>(ybase + r * W + cv) = v;
+            }
+        }
+        if (mirror && ctn < (ctm >> 2))  // a quarter of the 128x128 block's image above the diagonal
+            zero_fill_strip<T>(yp, H, W, q0 + (ctm & 3) * M_TM, (ctm >> 2) * M_TN, lane);
     }
 }
 
@@ -436,7 +456,7 @@ int launch_mfma(const void *x, const void *w, void *y, int64_t N, int64_t C, int
     const int ipp = (int)ipp64;
     const int64_t total = N * C * ipp64;
     const int64_t per_xcd = (total + 7) / 8;
-    int nw = device_cu_count() * 4 * MTA_CONV_WAVES_PER_SIMD / 8;  // persistent workgroups per XCD
+    int nw = device_cu_count() * MTA_CONV_WG_PER_CU / 8;  // persistent workgroups per XCD
     if (nw < 1) nw = 1;
     if (per_xcd < nw) nw = (int)per_xcd;
     dim3 grid((unsigned)(nw * 8));
@@ -454,7 +474,8 @@ template <typename T>
 int dispatch_mfma(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H, int64_t W, int R, int S,
                   int causal, float in_scale, int use_scale, hipStream_t st)
 {
-#define MTA_CONV_CASE(r, s) \
+#define MTA_CONV_CASE(r, s)                                       \
+    static_assert(mfma_geom<r, s>::fits, "window exceeds 32 keys"); \
     if (R == r && S == s) return launch_mfma<T, r, s>(x, w, y, N, C, H, W, causal, in_scale, use_scale, st);
     MTA_CONV_CASE(3, 3)
     MTA_CONV_CASE(3, 5)

@@ -32,6 +32,18 @@ __device__ __forceinline__ void mma32(f32x16 &c, const frag8<float> &a, const fr
     for (int t = 0; t < 8; ++t) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[t], b.v[t], c, 0, 0, 0);
 }
 
+// 16x16x32 (16-bit operands only).  Lane (r = lane%16, g = lane/16) owns operand row/column r and
+// the 8 slots of k-group g; the fp32 accumulator gives it D[m][n] with n = r, m = 4*g + v, v = 0..3.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void mma16(f32x4 &c, const frag8<bf16_t> &a, const frag8<bf16_t> &b)
+{
+    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ void mma16(f32x4 &c, const frag8<f16_t> &a, const frag8<f16_t> &b)
+{
+    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+}
+
 template <typename T> __device__ __forceinline__ frag8<T> zero_frag()
 {
     frag8<T> f;
