@@ -111,20 +111,12 @@ __global__ __launch_bounds__(NT) void conv_attn_fwd_kernel(const T *__restrict__
         for (int it = 0; it < KV_IT; ++it) {
             const int idx = it * NT + tid;
             const int row = idx / (D / VEC), vc = idx % (D / VEC);
+            // unconditional loads (an out-of-range key re-reads key 0) so that they are issued back to back;
+            // out-of-range rows are zeroed when they are written to LDS
             const int kr = cb + row;
-            if (kr >= 0 && kr < S) {
-                kreg[it] = *reinterpret_cast<const V16 *>(Kp + (int64_t)kr * D + vc * VEC);
-            } else {
-#pragma unroll
-                for (int u = 0; u < VEC; ++u) kreg[it].v[u] = from_float<T>(0.0f);
-            }
             const int vr = j * BK + row;
-            if (j >= 0 && vr < S) {
-                vreg[it] = *reinterpret_cast<const V16 *>(Vp + (int64_t)vr * D + vc * VEC);
-            } else {
-#pragma unroll
-                for (int u = 0; u < VEC; ++u) vreg[it].v[u] = from_float<T>(0.0f);
-            }
+            kreg[it] = *reinterpret_cast<const V16 *>(Kp + (int64_t)((kr >= 0 && kr < S) ? kr : 0) * D + vc * VEC);
+            vreg[it] = *reinterpret_cast<const V16 *>(Vp + (int64_t)((vr >= 0 && vr < S) ? vr : 0) * D + vc * VEC);
         }
         // ---- retained score columns: read the tail of the previous tile ----------------------
         V16 tailreg[TAIL_IT];
@@ -149,10 +141,17 @@ __global__ __launch_bounds__(NT) void conv_attn_fwd_kernel(const T *__restrict__
         for (int it = 0; it < KV_IT; ++it) {
             const int idx = it * NT + tid;
             const int row = idx / (D / VEC), vc = idx % (D / VEC);
-            *reinterpret_cast<V16 *>(Ks + row * KLD + vc * VEC) = kreg[it];
+            const int kr = cb + row, vr = j * BK + row;
+            const bool k_ok = kr >= 0 && kr < S, v_ok = vr >= 0 && vr < S;
+            V16 kv = kreg[it];
+            if (!k_ok) {
+#pragma unroll
+                for (int u = 0; u < VEC; ++u) kv.v[u] = from_float<T>(0.0f);
+            }
+            *reinterpret_cast<V16 *>(Ks + row * KLD + vc * VEC) = kv;
             const int pos = (row & ~15) + vt_pos16(row & 15);
 #pragma unroll
-            for (int u = 0; u < VEC; ++u) Vt[(vc * VEC + u) * VLD + pos] = vreg[it].v[u];
+            for (int u = 0; u < VEC; ++u) Vt[(vc * VEC + u) * VLD + pos] = v_ok ? vreg[it].v[u] : from_float<T>(0.0f);
         }
         __syncthreads();
 

@@ -36,15 +36,29 @@ __global__ __launch_bounds__(NT) void headmix_fixed(const T *__restrict__ x, con
     const int64_t base = (n * C + (int64_t)g * G) * plane + (int64_t)p * Q + q;
     using V = vecN<T, VEC>;
     const bool chunk_above = causal && (qc * NT * VEC > p);  // uniform per workgroup
-
-    if (!chunk_above) {
-        for (int t = tid; t < G * G; t += NT)
-            wsm[t] = load_any(w, w_dtype, (int64_t)(g * G + t / G) * C + g * G + t % G);
-        __syncthreads();
-    }
-    if (q >= Q) return;
     const T fill_t = from_float<T>(fill);
-    if (causal && q > p) {
+    if (chunk_above) {  // nothing to read: the whole chunk receives the fill value
+        if (q < Q) {
+            V f;
+#pragma unroll
+            for (int u = 0; u < VEC; ++u) f.v[u] = fill_t;
+#pragma unroll
+            for (int o = 0; o < G; ++o) *reinterpret_cast<V *>(y + base + o * plane) = f;
+        }
+        return;
+    }
+    // Issue this lane's loads first (unconditionally: a lane past the row end or above the diagonal
+    // re-reads the row start), then fetch the weights, so that the two latencies overlap.
+    const bool live = q < Q && !(causal && q > p);
+    const int64_t lbase = live ? base : base - q;
+    V xin[G];
+#pragma unroll
+    for (int i = 0; i < G; ++i) xin[i] = *reinterpret_cast<const V *>(x + lbase + i * plane);
+    for (int t = tid; t < G * G; t += NT)
+        wsm[t] = load_any(w, w_dtype, (int64_t)(g * G + t / G) * C + g * G + t % G);
+    __syncthreads();
+    if (q >= Q) return;
+    if (!live) {
         V f;
 #pragma unroll
         for (int u = 0; u < VEC; ++u) f.v[u] = fill_t;
@@ -52,9 +66,6 @@ __global__ __launch_bounds__(NT) void headmix_fixed(const T *__restrict__ x, con
         for (int o = 0; o < G; ++o) *reinterpret_cast<V *>(y + base + o * plane) = f;
         return;
     }
-    V xin[G];
-#pragma unroll
-    for (int i = 0; i < G; ++i) xin[i] = *reinterpret_cast<const V *>(x + base + i * plane);
 #pragma unroll
     for (int o = 0; o < G; ++o) {
         float acc[VEC];

@@ -55,7 +55,7 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, c
 {
     __shared__ float w1s[G * G];
     __shared__ float w2s[G * G];
-    __shared__ float red[NT / 64];
+    __shared__ float red[(NT / 64) * G];
     const int tid = threadIdx.x;
     const int groups = C / G;
     int64_t b = blockIdx.x;
@@ -67,6 +67,16 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, c
     const int last = causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;  // last attended key
     using V = vecN<T, VEC>;
 
+    // All row loads are issued first, unconditionally (a lane beyond the attended keys re-reads the
+    // row start), so that they overlap each other and the weight fetch below.
+    V xin[NV][G];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int q = (k * NT + tid) * VEC;
+        const int qs = (q <= last) ? q : 0;
+#pragma unroll
+        for (int i = 0; i < G; ++i) xin[k][i] = *reinterpret_cast<const V *>(x + base + i * plane + qs);
+    }
     for (int t = tid; t < G * G; t += NT) {
         const int64_t widx = (int64_t)(g * G + t / G) * C + g * G + t % G;
         w1s[t] = w1 ? load_any(w1, w_dtype, widx) : (t / G == t % G ? 1.0f : 0.0f);
@@ -78,58 +88,77 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, c
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
         const int q = (k * NT + tid) * VEC;
-        if (q <= last && q < Q) {
-            V xin[G];
 #pragma unroll
-            for (int i = 0; i < G; ++i) xin[i] = *reinterpret_cast<const V *>(x + base + i * plane + q);
+        for (int o = 0; o < G; ++o) {
 #pragma unroll
-            for (int o = 0; o < G; ++o) {
+            for (int u = 0; u < VEC; ++u) {
+                float acc;
+                if (w1) {
+                    acc = 0.0f;
 #pragma unroll
-                for (int u = 0; u < VEC; ++u) {
-                    float acc;
-                    if (w1) {
-                        acc = 0.0f;
-#pragma unroll
-                        for (int i = 0; i < G; ++i) acc = fmaf(w1s[o * G + i], to_float(xin[i].v[u]), acc);
-                        acc = round_to<T>(acc);
-                    } else {
-                        acc = to_float(xin[o].v[u]);
-                    }
-                    s[o][k][u] = (q + u <= last) ? acc : -INFINITY;
+                    for (int i = 0; i < G; ++i) acc = fmaf(w1s[o * G + i], to_float(xin[k][i].v[u]), acc);
+                    acc = round_to<T>(acc);
+                } else {
+                    acc = to_float(xin[k][o].v[u]);
                 }
+                s[o][k][u] = (q + u <= last) ? acc : -INFINITY;
             }
-        } else {
-#pragma unroll
-            for (int o = 0; o < G; ++o)
-#pragma unroll
-                for (int u = 0; u < VEC; ++u) s[o][k][u] = -INFINITY;
         }
     }
 
+    // row maxima and sums of all G heads are reduced together: two barriers per reduction, not 2*G
+    constexpr int NW = NT / 64;
+    const int wave = tid >> 6, lane = tid & 63;
+    float m[G], inv[G];
 #pragma unroll
     for (int o = 0; o < G; ++o) {
-        float m = -INFINITY;
+        float v = -INFINITY;
 #pragma unroll
         for (int k = 0; k < NV; ++k)
 #pragma unroll
-            for (int u = 0; u < VEC; ++u) m = fmaxf(m, s[o][k][u]);
-        m = block_max<NT>(m, red);
+            for (int u = 0; u < VEC; ++u) v = fmaxf(v, s[o][k][u]);
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+        if (lane == 0) red[wave * G + o] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int o = 0; o < G; ++o) {
+        float v = red[o];
+#pragma unroll
+        for (int i = 1; i < NW; ++i) v = fmaxf(v, red[i * G + o]);
+        m[o] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int o = 0; o < G; ++o) {
         float sum = 0.0f;
 #pragma unroll
         for (int k = 0; k < NV; ++k)
 #pragma unroll
             for (int u = 0; u < VEC; ++u) {
-                const float e = (s[o][k][u] == -INFINITY) ? 0.0f : __expf(s[o][k][u] - m);
+                const float e = (s[o][k][u] == -INFINITY) ? 0.0f : __expf(s[o][k][u] - m[o]);
                 s[o][k][u] = e;
                 sum += e;
             }
-        sum = block_sum<NT>(sum, red);
-        const float inv = 1.0f / sum;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+        if (lane == 0) red[wave * G + o] = sum;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int o = 0; o < G; ++o) {
+        float v = red[o];
+#pragma unroll
+        for (int i = 1; i < NW; ++i) v += red[i * G + o];
+        inv[o] = 1.0f / v;
+    }
+#pragma unroll
+    for (int o = 0; o < G; ++o)
 #pragma unroll
         for (int k = 0; k < NV; ++k)
 #pragma unroll
-            for (int u = 0; u < VEC; ++u) s[o][k][u] = round_to<T>(s[o][k][u] * inv);
-    }
+            for (int u = 0; u < VEC; ++u) s[o][k][u] = round_to<T>(s[o][k][u] * inv[o]);
 
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
