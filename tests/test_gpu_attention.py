@@ -131,6 +131,13 @@ CA_CASES = [
     (1, 2, 500, 128, 11, 15, True, torch.float32),
     (1, 1, 1, 64, 3, 3, True, torch.float32),
     (1, 2, 1000, 128, 6, 11, True, torch.bfloat16),
+    # 16-bit, kernel sizes with an all-MFMA instantiation
+    (2, 2, 300, 64, 3, 3, True, torch.bfloat16),
+    (1, 2, 515, 64, 5, 5, True, torch.float16),
+    (1, 2, 260, 128, 7, 7, False, torch.bfloat16),
+    (1, 2, 777, 128, 6, 11, True, torch.float16),
+    (1, 1, 64, 128, 5, 7, True, torch.bfloat16),
+    (1, 2, 5, 64, 6, 11, True, torch.bfloat16),
 ]
 
 
