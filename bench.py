@@ -184,6 +184,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a plain device copy of 1 GiB five times (scales the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -196,6 +198,14 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     device = torch.device("cuda:0")
+    if args.copy_calibration:
+        src = torch.ones(1 << 29, dtype=torch.bfloat16, device=device)   # 1 GiB read + 1 GiB written per copy
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration_bytes_each_way": src.numel() * 2, "copies": 5}))
+        return
     b, h, s, d = 2, 16, 4096, 128
     mod, sets = build_c4(torch, mta, O, device, b, h, s, d)
 

@@ -14,73 +14,88 @@ namespace {
 using namespace mta;
 
 constexpr int NT = 256;
+#ifndef MTA_HM_ROWS
+#define MTA_HM_ROWS 4
+#endif
 
 template <typename T, int VEC> struct alignas(sizeof(T) * VEC) vecN { T v[VEC]; };
 
-// G heads mixed inside one lane, G known at compile time.
-template <typename T, int G, int VEC>
+// G heads mixed inside one lane, G known at compile time.  A workgroup covers ROWS consecutive
+// query rows of one key chunk, so a lane has ROWS*G independent 16-byte loads in flight.
+template <typename T, int G, int VEC, int ROWS>
 __global__ __launch_bounds__(NT) void headmix_fixed(const T *__restrict__ x, const void *__restrict__ w,
                                                     T *__restrict__ y, int C, int P, int Q, int causal,
-                                                    float fill, int w_dtype, int qchunks)
+                                                    float fill, int w_dtype, int qchunks, int pblocks)
 {
     __shared__ float wsm[G * G];
     const int tid = threadIdx.x;
     const int groups = C / G;
     int64_t b = blockIdx.x;
     const int qc = (int)(b % qchunks); b /= qchunks;
-    const int p = (int)(b % P); b /= P;
+    const int p0 = (int)(b % pblocks) * ROWS; b /= pblocks;
     const int g = (int)(b % groups);
     const int64_t n = b / groups;
     const int q = (qc * NT + tid) * VEC;
     const int64_t plane = (int64_t)P * Q;
-    const int64_t base = (n * C + (int64_t)g * G) * plane + (int64_t)p * Q + q;
+    const int64_t base0 = (n * C + (int64_t)g * G) * plane + q;
     using V = vecN<T, VEC>;
-    const bool chunk_above = causal && (qc * NT * VEC > p);  // uniform per workgroup
     const T fill_t = from_float<T>(fill);
-    if (chunk_above) {  // nothing to read: the whole chunk receives the fill value
+    V fillv;
+#pragma unroll
+    for (int u = 0; u < VEC; ++u) fillv.v[u] = fill_t;
+    const int plast = (p0 + ROWS - 1 < P - 1) ? p0 + ROWS - 1 : P - 1;
+    if (causal && qc * NT * VEC > plast) {  // chunk wholly above the diagonal for all rows: fill only, nothing read
         if (q < Q) {
-            V f;
 #pragma unroll
-            for (int u = 0; u < VEC; ++u) f.v[u] = fill_t;
+            for (int r = 0; r < ROWS; ++r)
+                if (p0 + r < P) {
 #pragma unroll
-            for (int o = 0; o < G; ++o) *reinterpret_cast<V *>(y + base + o * plane) = f;
+                    for (int o = 0; o < G; ++o) *reinterpret_cast<V *>(y + base0 + (int64_t)(p0 + r) * Q + o * plane) = fillv;
+                }
         }
         return;
     }
-    // Issue this lane's loads first (unconditionally: a lane past the row end or above the diagonal
-    // re-reads the row start), then fetch the weights, so that the two latencies overlap.
-    const bool live = q < Q && !(causal && q > p);
-    const int64_t lbase = live ? base : base - q;
-    V xin[G];
+    // Issue all of this lane's loads first (unconditionally: a lane past the row end or above the
+    // diagonal re-reads the row start), then fetch the weights, so that the latencies overlap.
+    V xin[ROWS][G];
 #pragma unroll
-    for (int i = 0; i < G; ++i) xin[i] = *reinterpret_cast<const V *>(x + lbase + i * plane);
+    for (int r = 0; r < ROWS; ++r) {
+        const int p = (p0 + r < P) ? p0 + r : P - 1;
+        const bool live = q < Q && !(causal && q > p);
+        const int64_t lb = base0 + (int64_t)p * Q - (live ? 0 : q);
+#pragma unroll
+        for (int i = 0; i < G; ++i) xin[r][i] = *reinterpret_cast<const V *>(x + lb + i * plane);
+    }
     for (int t = tid; t < G * G; t += NT)
         wsm[t] = load_any(w, w_dtype, (int64_t)(g * G + t / G) * C + g * G + t % G);
     __syncthreads();
     if (q >= Q) return;
-    if (!live) {
-        V f;
 #pragma unroll
-        for (int u = 0; u < VEC; ++u) f.v[u] = fill_t;
+    for (int r = 0; r < ROWS; ++r) {
+        const int p = p0 + r;
+        if (p >= P) break;
+        const int64_t base = base0 + (int64_t)p * Q;
+        if (causal && q > p) {
 #pragma unroll
-        for (int o = 0; o < G; ++o) *reinterpret_cast<V *>(y + base + o * plane) = f;
-        return;
-    }
-#pragma unroll
-    for (int o = 0; o < G; ++o) {
-        float acc[VEC];
-#pragma unroll
-        for (int u = 0; u < VEC; ++u) acc[u] = 0.0f;
-#pragma unroll
-        for (int i = 0; i < G; ++i) {
-            const float wv = wsm[o * G + i];
-#pragma unroll
-            for (int u = 0; u < VEC; ++u) acc[u] = fmaf(wv, to_float(xin[i].v[u]), acc[u]);
+            for (int o = 0; o < G; ++o) *reinterpret_cast<V *>(y + base + o * plane) = fillv;
+            continue;
         }
-        V out;
 #pragma unroll
-        for (int u = 0; u < VEC; ++u) out.v[u] = (causal && q + u > p) ? fill_t : from_float<T>(acc[u]);
-        *reinterpret_cast<V *>(y + base + o * plane) = out;
+        for (int o = 0; o < G; ++o) {
+            float acc[VEC];
+#pragma unroll
+            for (int u = 0; u < VEC; ++u) acc[u] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < G; ++i) {
+                const float wv = wsm[o * G + i];
+#pragma unroll
+                for (int u = 0; u < VEC; ++u) acc[u] = fmaf(wv, to_float(xin[r][i].v[u]), acc[u]);
+            }
+            V out;
+#pragma unroll
+            for (int u = 0; u < VEC; ++u) out.v[u] = (causal && q + u > p) ? fill_t : from_float<T>(acc[u]);
+            *reinterpret_cast<V *>(y + base + o * plane) = out;
+        }
     }
 }
 
@@ -127,24 +142,26 @@ int launch(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t 
            float fill, int w_dtype, hipStream_t st)
 {
     const int qchunks = (int)((Q + (int64_t)NT * VEC - 1) / ((int64_t)NT * VEC));
+#define MTA_HM_CASE(g, rows)                                                                                       \
+    if (G == g) {                                                                                                  \
+        const int pblocks = (int)((P + rows - 1) / rows);                                                          \
+        const int64_t blocks = N * (C / G) * pblocks * qchunks;                                                    \
+        if (blocks > 0x7fffffffLL) return MTA_ERR_SHAPE;                                                           \
+        hipLaunchKernelGGL((headmix_fixed<T, g, VEC, rows>), dim3((unsigned)blocks), dim3(NT), 0, st, (const T *)x, w, \
+                           (T *)y, (int)C, (int)P, (int)Q, causal, fill, w_dtype, qchunks, pblocks);               \
+        return launch_status();                                                                                    \
+    }
+    MTA_HM_CASE(1, MTA_HM_ROWS)
+    MTA_HM_CASE(2, MTA_HM_ROWS)
+    MTA_HM_CASE(4, MTA_HM_ROWS)
+    MTA_HM_CASE(8, 2)
+    MTA_HM_CASE(16, 1)
+    MTA_HM_CASE(32, 1)
+#undef MTA_HM_CASE
     const int64_t blocks = N * (C / G) * P * qchunks;
     if (blocks > 0x7fffffffLL) return MTA_ERR_SHAPE;
-    dim3 grid((unsigned)blocks);
-#define MTA_HM_CASE(g)                                                                                       \
-    if (G == g) {                                                                                            \
-        hipLaunchKernelGGL((headmix_fixed<T, g, VEC>), grid, dim3(NT), 0, st, (const T *)x, w, (T *)y, (int)C, \
-                           (int)P, (int)Q, causal, fill, w_dtype, qchunks);                                  \
-        return launch_status();                                                                              \
-    }
-    MTA_HM_CASE(1)
-    MTA_HM_CASE(2)
-    MTA_HM_CASE(4)
-    MTA_HM_CASE(8)
-    MTA_HM_CASE(16)
-    MTA_HM_CASE(32)
-#undef MTA_HM_CASE
-    hipLaunchKernelGGL((headmix_any<T, VEC>), grid, dim3(NT), 0, st, (const T *)x, w, (T *)y, (int)C, G, (int)P,
-                       (int)Q, causal, fill, w_dtype, qchunks);
+    hipLaunchKernelGGL((headmix_any<T, VEC>), dim3((unsigned)blocks), dim3(NT), 0, st, (const T *)x, w, (T *)y, (int)C, G,
+                       (int)P, (int)Q, causal, fill, w_dtype, qchunks);
     return launch_status();
 }
 }  // namespace

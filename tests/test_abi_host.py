@@ -1,0 +1,171 @@
+"""CPU-only checks of the boundary: the C ABI library loads and exports what include/mta_hip.h declares,
+argument validation returns the documented codes without touching a GPU, and the Python operator
+surface mirrors the reference's names, parameters and error behaviour."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import multitokenatention_triton_amd as mta
+from multitokenatention_triton_amd import _lib, ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mta_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mta_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = declared_functions()
+    assert {"mta_conv2d_fwd", "mta_conv2d_scaled_fwd", "mta_headmix_fwd", "mta_headmix_softmax_fwd",
+            "mta_conv_attn_fwd", "mta_strerror", "mta_abi_version"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/mta_hip.h but not exported"
+    assert sorted(_lib.SIGNATURES) == names, "ctypes signatures out of sync with the header"
+    assert lib.mta_abi_version() == 1
+
+
+def test_no_torch_symbols_in_the_library():
+    out = os.popen(f"nm -D --undefined-only {_lib.LIB_PATH}").read()
+    assert "at::" not in out and "c10" not in out and "torch" not in out
+
+
+def test_error_strings():
+    for code in range(0, -9, -1):
+        s = _lib.strerror(code)
+        assert s and "unknown" not in s
+    assert "unknown" in _lib.strerror(-99)
+
+
+def test_argument_validation_needs_no_gpu():
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.addressof(buf)
+    # null pointers
+    assert lib.mta_conv2d_fwd(None, p, p, 1, 1, 8, 8, 3, 3, 1, 0, 0, None) == -1
+    assert lib.mta_headmix_fwd(p, None, p, 1, 2, 8, 8, 0, 1, 0.0, 0, 0, None) == -1
+    assert lib.mta_conv_attn_fwd(p, p, p, p, None, 1, 1, 8, 64, 3, 3, 1, 0.1, 0, 0, None) == -1
+    # dtype
+    assert lib.mta_conv2d_fwd(p, p, p, 1, 1, 8, 8, 3, 3, 1, 7, 0, None) == -2
+    # shape
+    assert lib.mta_conv2d_fwd(p, p, p, 0, 1, 8, 8, 3, 3, 1, 0, 0, None) == -3
+    assert lib.mta_headmix_fwd(p, p, p, 1, 2, 0, 8, 0, 1, 0.0, 0, 0, None) == -3
+    assert lib.mta_conv_attn_fwd(p, p, p, p, p, 1, 1, 0, 64, 3, 3, 1, 0.1, 0, 0, None) == -3
+    # kernel size
+    assert lib.mta_conv2d_fwd(p, p, p, 1, 1, 8, 8, 33, 3, 1, 0, 0, None) == -4
+    assert lib.mta_conv2d_fwd(p, p, p, 1, 1, 8, 8, 3, 64, 1, 0, 0, None) == -4
+    assert lib.mta_conv_attn_fwd(p, p, p, p, p, 1, 1, 8, 64, 0, 3, 1, 0.1, 0, 0, None) == -4
+    # group
+    assert lib.mta_headmix_fwd(p, p, p, 1, 6, 8, 8, 4, 1, 0.0, 0, 0, None) == -5
+    assert lib.mta_headmix_softmax_fwd(p, p, p, p, 1, 6, 8, 8, 4, 1, 0, 0, None) == -5
+    # alignment (fp32 pointer off by one byte)
+    assert lib.mta_conv2d_fwd(p + 1, p, p, 1, 1, 8, 8, 3, 3, 1, 0, 0, None) == -6
+    # head dim
+    assert lib.mta_conv_attn_fwd(p, p, p, p, p, 1, 1, 8, 48, 3, 3, 1, 0.1, 0, 0, None) == -7
+
+
+def test_check_maps_codes_to_exceptions():
+    with pytest.raises(ValueError, match="kernel size"):
+        _lib.check(-4, "x")
+    with pytest.raises(RuntimeError):
+        _lib.check(1, "x")
+    _lib.check(0, "x")
+
+
+def test_cpu_tensors_are_rejected_loudly():
+    x = torch.zeros(1, 2, 8, 8)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.conv2d_causal(x, torch.zeros(2, 3, 3), True)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.headmix(x, torch.eye(2), True)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        mta.TritonConvAttention(2, 3)(torch.zeros(1, 2, 8, 64), torch.zeros(1, 2, 8, 64), torch.zeros(1, 2, 8, 64), True, 1.0)
+
+
+def test_module_surface_matches_reference_names():
+    cfg = mta.MTAConfig(query_kernel_size=6, key_kernel_size=11)
+    mod = mta.MTAAttentionTriton(n_heads=8, mta=cfg, dropout=0.0, causal=True, use_mask=False)
+    assert list(mod.state_dict()) == ["mta_conv_triton.weight", "wpsm_triton.weight",
+                                      "mta_conv_after_sm_triton.weight", "wposm_triton.weight"]
+    assert mod.mta_conv_triton.weight.shape == (8, 6, 11)
+    assert mod.mta_conv_after_sm_triton.weight.shape == (8, 3, 3)
+    assert mod.wpsm_triton.output_value == float("-inf") and mod.wposm_triton.output_value == 0.0
+    # defaults of the operator modules (convolution_2d_trit.py:393-398, triton_linear_head.py:384)
+    conv = mta.Conv2dTriton(4, (3, 5), causal=True)
+    assert conv.weight[0, 1, 2] == 1 and conv.weight.sum() == 4
+    assert mta.Conv2dTriton(4, 3).kernel_size == (3, 3)
+    assert mta.TritonLinearHead(6).weight.shape == (6, 6)
+    assert "head_dim=6" in repr(mta.TritonLinearHead(6))
+    with pytest.raises(AssertionError, match="chunked"):
+        mod(torch.zeros(1), torch.zeros(1), torch.zeros(1), None, chunk_start_ids=[0])
+
+
+def test_reset_and_copy_parameters():
+    cfg = mta.MTAConfig(query_kernel_size=3, key_kernel_size=5, init_method="identity")
+    mod = mta.MTAAttentionTriton(4, cfg, 0.0, True)
+    mod.reset_mta_parameters()
+    w = mod.mta_conv_triton.weight
+    assert w[0, 2, 2] == 1 and w.sum() == 4            # identity tap at [R-1, S//2]
+    assert torch.equal(mod.wpsm_triton.weight, torch.eye(4)) and torch.equal(mod.wposm_triton.weight, torch.eye(4))
+    assert ops.is_identity_conv_kernel(w) and ops.is_identity_head_weight(mod.wpsm_triton.weight)
+
+    class Src:  # the PyTorch module's parameter layout: conv kernels are (H,1,R,S)
+        mta_kernel = torch.nn.Parameter(torch.randn(4, 1, 3, 5))
+        mta_kernel_after_sm = torch.nn.Parameter(torch.randn(4, 1, 3, 3))
+        wpsm = torch.nn.Linear(4, 4, bias=False)
+        wposm = torch.nn.Linear(4, 4, bias=False)
+    mod.copy_mta_parameters(Src)
+    assert torch.equal(mod.mta_conv_triton.weight, Src.mta_kernel.squeeze(1))
+    assert torch.equal(mod.wposm_triton.weight, Src.wposm.weight)
+    for method in ("uniform", "normal", "diagonal", "const"):
+        cfg.init_method = method
+        m2 = mta.MTAAttentionTriton(4, cfg, 0.0, True)
+        m2.reset_mta_parameters()
+        assert torch.isfinite(m2.mta_conv_triton.weight).all()
+    cfg.init_method = "nope"
+    with pytest.raises(ValueError):
+        mta.MTAAttentionTriton(4, cfg, 0.0, True).reset_mta_parameters()
+
+
+def test_structure_probes():
+    g = torch.Generator().manual_seed(0)
+    w = torch.zeros(8, 8)
+    for b in range(0, 8, 4):
+        w[b:b + 4, b:b + 4] = torch.randn(4, 4, generator=g)
+    assert ops.block_diagonal_group(w) == 4
+    assert ops.block_diagonal_group(torch.eye(8)) == 1
+    assert ops.block_diagonal_group(torch.randn(6, 6, generator=g)) == 6
+    k = torch.zeros(2, 3, 4)
+    k[:, -1, 2] = 1
+    assert not ops.is_identity_conv_kernel(k)          # even key size: the tap is off by one, not a pass-through
+    cfg = mta.MTAConfig()
+    mod = mta.MTAAttentionTriton(4, cfg, 0.0, True)
+    mod.reset_mta_parameters()
+    from multitokenatention_triton_amd.mta_attention_triton import _probe_head
+    assert mod._probe("wposm", mod.wposm_triton.weight, _probe_head) == (True, 1)
+    with torch.no_grad():
+        mod.wposm_triton.weight[0, 3] = 0.5              # in-place under no_grad moves the version counter
+    assert mod._probe("wposm", mod.wposm_triton.weight, _probe_head) == (False, 4)
+    mod.weight_structure = "dense"
+    assert mod._probe("wposm", mod.wposm_triton.weight, _probe_head) == (False, 4)
+
+
+def test_dropin_shims_resolve():
+    import importlib
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "multitokenatention_triton_amd", "dropin"))
+    try:
+        m = importlib.import_module("mta_attention_triton")
+        assert m.MTAAttentionTriton is mta.MTAAttentionTriton
+        assert importlib.import_module("conv_attention_triton").TritonConvAttention is mta.TritonConvAttention
+        assert importlib.import_module("convolution_2d_trit").Conv2dTriton is mta.Conv2dTriton
+        assert importlib.import_module("triton_linear_head").TritonLinearHead is mta.TritonLinearHead
+    finally:
+        sys.path.pop(0)
