@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTA_ABI_VERSION 1
+#define MTA_ABI_VERSION 2
 
 enum mta_dtype { MTA_F32 = 0, MTA_BF16 = 1, MTA_F16 = 2 };
 
@@ -38,7 +38,8 @@ enum mta_error {
     MTA_ERR_GROUP = -5,       /* group_size does not divide the head count */
     MTA_ERR_ALIGN = -6,       /* pointer not aligned to its element size */
     MTA_ERR_HEAD_DIM = -7,    /* head dim unsupported by the fused kernel */
-    MTA_ERR_DEVICE = -8       /* no usable gfx950 device / device query failed */
+    MTA_ERR_DEVICE = -8,      /* no usable gfx950 device / device query failed */
+    MTA_ERR_UNSUPPORTED = -9  /* valid arguments, but this entry point has no kernel for the combination */
 };
 
 /* Largest conv kernel the entry points accept. */
@@ -60,7 +61,7 @@ int mta_conv2d_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, 
 /* Same op with the input multiplied by `in_scale` as it is read (products are formed
  * in fp32 and, for 16-bit I/O, rounded to the I/O dtype before the taps, which is what
  * a separate elementwise scale in that dtype would produce).  Lets the caller fold
- * the 1/sqrt(D) of mta_attention_triton.py:69-71 into the conv's load. */
+ * the 1/sqrt(D) of mta_attention_triton.py:69-71 into the conv's staging pass. */
 int mta_conv2d_scaled_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H,
                           int64_t W, int R, int S, int causal, float in_scale, int io_dtype,
                           int w_dtype, void *stream);
@@ -80,7 +81,9 @@ int mta_headmix_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C,
  *   s[o] = w1 ? sum_i w1[o,i] x[i] : x[o]      (fp32, rounded to the I/O dtype;
  *                                               causal: q>p takes no part)
  *   p[o] = softmax over q of s[o]              (fp32, rounded to the I/O dtype)
- *   y[o] = w2 ? sum_i w2[o,i] p[i] : p[o]      (causal: q>p written as +0.0)
+ *   y[o] = w2 ? sum_i w2[o,i] p[i] : p[o]      (causal: q>p written as +0.0 when fill_upper != 0,
+ *                                               left untouched when fill_upper == 0 -- for a consumer
+ *                                               such as mta_causal_pv_fwd that never reads it)
  * w1 and/or w2 may be NULL (identity); both NULL is a plain causal row softmax.
  * group_size as in mta_headmix_fwd and applies to both weights.
  * Replaces the wpsm_triton -> F.softmax(scores.float()).type_as(xq) -> wposm_triton
@@ -88,7 +91,7 @@ int mta_headmix_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C,
  * conv between them is the identity; otherwise pass w2 = NULL). */
 int mta_headmix_softmax_fwd(const void *x, const void *w1, const void *w2, void *y, int64_t N,
                             int64_t C, int64_t P, int64_t Q, int group_size, int causal,
-                            int io_dtype, int w_dtype, void *stream);
+                            int fill_upper, int io_dtype, int w_dtype, void *stream);
 
 /* Fused conv-attention forward:
  *   O = softmax( mask( conv( mask0(Q K^T) ) ) * scale ) V        per (batch, head)
@@ -100,6 +103,27 @@ int mta_headmix_softmax_fwd(const void *x, const void *w1, const void *w2, void 
 int mta_conv_attn_fwd(const void *q, const void *k, const void *v, const void *w, void *o,
                       int64_t B, int64_t H, int64_t S, int64_t D, int R, int Sk, int causal,
                       float scale, int io_dtype, int w_dtype, void *stream);
+
+/* First half of the fused path, for the MTA pipeline (which must mix heads before its softmax):
+ *   s_out[b,h] = conv( mask0(scale * Q K^T) )           an (S,S) plane per (batch, head)
+ * (Q K^T is rounded to the I/O dtype, scaled and rounded again before the conv, as the unfused
+ * pipeline does)
+ * q,k are (B,H,S,D), w is (H,R,Sk), s_out is (B,H,S,S).  Replaces matmul -> *rsqrt(d) -> conv_fwd_kernel of
+ * mta_attention_triton.py:69-73 without ever writing the raw scores.  When causal only q <= p is
+ * written; fill_upper != 0 also writes +0.0 above the diagonal (needed only if a consumer reads it).
+ * 16-bit I/O with weights of the same dtype, D in {64,128}, S % 8 == 0 and the kernel sizes that have a
+ * matrix-core instantiation; anything else returns MTA_ERR_UNSUPPORTED and the caller takes the
+ * unfused route. */
+int mta_qk_conv_fwd(const void *q, const void *k, const void *w, void *s_out, int64_t B, int64_t H,
+                    int64_t S, int64_t D, int R, int Sk, int causal, float scale, int fill_upper,
+                    int io_dtype, int w_dtype, void *stream);
+
+/* O = P V with P (B,H,S,S), V (B,H,S,D), O (B,H,S,D).  When causal only keys q <= p of P are read
+ * (what lies above the diagonal may be uninitialised).  Replaces torch.matmul(scores, xv) of
+ * mta_attention_triton.py:89 and halves its traffic.  16-bit I/O, D in {64,128}, S % 8 == 0; anything
+ * else returns MTA_ERR_UNSUPPORTED. */
+int mta_causal_pv_fwd(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int64_t D,
+                      int causal, int io_dtype, void *stream);
 
 #ifdef __cplusplus
 }

@@ -25,7 +25,9 @@ SIGNATURES = {
     "mta_conv2d_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _vp]),
     "mta_conv2d_scaled_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _int, _int, _vp]),
     "mta_headmix_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _f32, _int, _int, _vp]),
-    "mta_headmix_softmax_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _vp]),
+    "mta_headmix_softmax_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _vp]),
+    "mta_qk_conv_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _int, _int, _int, _vp]),
+    "mta_causal_pv_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "mta_conv_attn_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _int, _int, _vp]),
 }
 
@@ -55,6 +57,9 @@ def load() -> ctypes.CDLL:
 
 def strerror(code: int) -> str:
     return load().mta_strerror(int(code)).decode()
+
+
+MTA_ERR_UNSUPPORTED = -9
 
 
 def check(code: int, what: str) -> None:

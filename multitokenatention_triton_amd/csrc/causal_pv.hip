@@ -1,0 +1,179 @@
+// O = P V for the MTA pipeline:  P is the (B,H,S,S) post-softmax tensor, V is (B,H,S,D), O is (B,H,S,D).
+//
+// When causal, only keys q <= p of P are read: nothing above the diagonal is touched (it may be
+// uninitialised memory), which halves the traffic of the plain batched GEMM this replaces.
+// HBM-bound: the P triangle is streamed once, V blocks are re-read from L2.
+//
+// 8 wavefronts own 256 query rows; a wavefront owns two blocks of 16 rows.  O^T += V^T P^T on
+// 16x16x32 MFMAs: lane (r = lane%16, g = lane/16) owns query row r of a block and supplies P^T
+// fragments straight from global memory (16 contiguous bytes = 8 keys of its row, loaded one key
+// block ahead), V blocks of 64 keys are copied global -> LDS asynchronously (double buffered,
+// 16-byte chunks XOR-swizzled by key) and V^T fragments come out of them through the LDS transpose
+// read: within 16 lanes, lane c supplies the address of 4 head-dim values of key c/4 and lane i
+// receives head-dim value i of 4 consecutive keys.
+#include "common.hpp"
+#include "mfma.hpp"
+
+namespace {
+using namespace mta;
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef const __attribute__((address_space(1))) void glb_void_t;
+typedef short v4s_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
+
+constexpr int P_NT = 512;  // 8 wavefronts
+constexpr int P_BQ = 256;  // query rows per workgroup
+constexpr int P_BK = 64;   // keys per iteration
+
+template <typename T, int D>
+__global__ __launch_bounds__(P_NT, 2) void causal_pv_kernel(const T *__restrict__ P, const T *__restrict__ V,
+                                                           T *__restrict__ O, int S, int causal, int nqb)
+{
+    constexpr int CPR = D / 8;               // 16-byte chunks per V row
+    constexpr int TILE = P_BK * D;           // elements per V block
+    constexpr int ROUNDS = (TILE / 8 + P_NT - 1) / P_NT;
+    constexpr int DB = D / 16;
+    __shared__ __align__(16) T Vt[2 * TILE];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, ln = lane & 15, kg = lane >> 4;
+    const int qb = nqb - 1 - (int)blockIdx.x;  // longest blocks first
+    const int64_t bh = blockIdx.y;
+    const int q0 = qb * P_BQ;
+    const T *Pp = P + bh * (int64_t)S * S;
+    const T *Vp = V + bh * (int64_t)S * D;
+    T *Op = O + bh * (int64_t)S * D;
+
+    auto issue_v = [&](int j, int buf) {
+#pragma unroll
+        for (int r = 0; r < ROUNDS; ++r) {
+            const int slot = r * P_NT + tid;
+            if (TILE / 8 % P_NT != 0 && slot >= TILE / 8) break;
+            const int row = slot / CPR, c = (slot % CPR) ^ (row & (CPR - 1));
+            int vr = j * P_BK + row;
+            vr = vr >= S ? S - 1 : vr;
+            __builtin_amdgcn_global_load_lds((glb_void_t *)(Vp + (int64_t)vr * D + c * 8),
+                                             (lds_void_t *)(Vt + buf * TILE + (r * P_NT + wave * 64) * 8), 16, 0, 0);
+        }
+    };
+
+    int prow[2];
+    const T *prow_ptr[2];
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+        prow[rb] = q0 + wave * 32 + rb * 16 + ln;
+        const int pc = prow[rb] < S ? prow[rb] : S - 1;
+        prow_ptr[rb] = Pp + (int64_t)pc * S + kg * 8;
+    }
+    // P^T fragments of key block j: slots t = 0..7 of k-step ks are keys j*64 + 32ks + 8kg + t; out-of-range
+    // vectors re-read the row start, the values are masked when used
+    auto load_p = [&](int j, frag8<T> (&pf)[2][2]) {
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const int key = j * P_BK + ks * 32 + kg * 8;
+                const bool ok = key < S && !(causal && key > prow[rb]);
+                pf[rb][ks] = *reinterpret_cast<const frag8<T> *>(prow_ptr[rb] + (ok ? j * P_BK + ks * 32 : -kg * 8));
+            }
+    };
+
+    const int q_last = (q0 + P_BQ - 1 < S - 1) ? q0 + P_BQ - 1 : S - 1;
+    const int j_end = causal ? q_last / P_BK : (S - 1) / P_BK;
+    issue_v(0, 0);
+    frag8<T> pcur[2][2], pnext[2][2];
+    load_p(0, pcur);
+
+    f32x4 oacc[2][DB];
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) oacc[rb][db] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    int buf = 0;
+    for (int j = 0; j <= j_end; ++j, buf ^= 1) {
+        __builtin_amdgcn_s_waitcnt(0);  // V block j (and the P fragments) have arrived
+        __syncthreads();                // for every wavefront; reads of the other buffer are finished
+        if (j < j_end) {
+            issue_v(j + 1, buf ^ 1);
+            load_p(j + 1, pnext);
+        }
+        // mask the fragments of this block: keys beyond the row (causal) or the sequence count as 0
+        frag8<T> pf[2][2];
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const int key0 = j * P_BK + ks * 32 + kg * 8;
+                pf[rb][ks] = pcur[rb][ks];
+                const int lim = causal ? (prow[rb] < S - 1 ? prow[rb] : S - 1) : S - 1;
+                if (key0 + 7 > lim) {
+#pragma unroll
+                    for (int t = 0; t < 8; ++t)
+                        if (key0 + t > lim) pf[rb][ks].v[t] = from_float<T>(0.0f);
+                }
+            }
+        const T *Vb = Vt + buf * TILE;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const int key_a = ks * 32 + kg * 8 + (ln >> 2);  // slots 0..3: keys 8kg+(0..3); slots 4..7: +4
+            const int key_b = key_a + 4;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const int ch = db * 2 + ((ln & 3) >> 1);
+                const int sub = (ln & 1) * 4;
+                const T *pa = Vb + key_a * D + ((ch ^ (key_a & (CPR - 1))) * 8) + sub;
+                const T *pb = Vb + key_b * D + ((ch ^ (key_b & (CPR - 1))) * 8) + sub;
+                const v4s_t va = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)pa);
+                const v4s_t vb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)pb);
+                struct { v4s_t a, b; } both = {va, vb};
+                const frag8<T> vf = __builtin_bit_cast(frag8<T>, both);
+                mma16(oacc[0][db], vf, pf[0][ks]);
+                mma16(oacc[1][db], vf, pf[1][ks]);
+            }
+        }
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) pcur[rb][ks] = pnext[rb][ks];
+    }
+
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+        if (prow[rb] >= S) continue;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            struct alignas(8) quad { T v[4]; } out;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) out.v[v] = from_float<T>(oacc[rb][db][v]);
+            *reinterpret_cast<quad *>(Op + (int64_t)prow[rb] * D + db * 16 + kg * 4) = out;
+        }
+    }
+}
+
+template <typename T, int D>
+int launch(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int causal, hipStream_t st)
+{
+    const int nqb = (int)((S + P_BQ - 1) / P_BQ);
+    dim3 grid((unsigned)nqb, (unsigned)(B * H));
+    hipLaunchKernelGGL((causal_pv_kernel<T, D>), grid, dim3(P_NT), 0, st, (const T *)p, (const T *)v, (T *)o, (int)S, causal,
+                       nqb);
+    return launch_status();
+}
+}  // namespace
+
+extern "C" int mta_causal_pv_fwd(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int64_t D,
+                                 int causal, int io_dtype, void *stream)
+{
+    if (!p || !v || !o) return MTA_ERR_NULL;
+    if (!dtype_size(io_dtype)) return MTA_ERR_DTYPE;
+    if (B <= 0 || H <= 0 || S <= 0 || S > (1 << 24) || B * H > 65535) return MTA_ERR_SHAPE;
+    if (D != 64 && D != 128) return MTA_ERR_HEAD_DIM;
+    if (!aligned_to(p, 16) || !aligned_to(v, 16) || !aligned_to(o, 16)) return MTA_ERR_ALIGN;
+    if (io_dtype == MTA_F32 || S % 8 != 0) return MTA_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    if (io_dtype == MTA_BF16)
+        return D == 64 ? launch<bf16_t, 64>(p, v, o, B, H, S, causal, st) : launch<bf16_t, 128>(p, v, o, B, H, S, causal, st);
+    return D == 64 ? launch<f16_t, 64>(p, v, o, B, H, S, causal, st) : launch<f16_t, 128>(p, v, o, B, H, S, causal, st);
+}

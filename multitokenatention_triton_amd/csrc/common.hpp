@@ -31,6 +31,34 @@ template <> __device__ __forceinline__ float from_float<float>(float v) { return
 template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return __builtin_bit_cast(bf16_t, (__bf16)v); }
 template <> __device__ __forceinline__ f16_t from_float<f16_t>(float v) { return f16_t{(_Float16)v}; }
 
+// two fp32 values rounded to the 16-bit type T and packed into one register (a in the low half): one
+// v_cvt_pk_* instruction on gfx950
+typedef float mta_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 mta_bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 mta_f16x2 __attribute__((ext_vector_type(2)));
+template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b);
+template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float a, float b)
+{
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((mta_f32x2){a, b}, mta_bf16x2));
+}
+template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b)
+{
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((mta_f32x2){a, b}, mta_f16x2));
+}
+// the two halves of such a register, widened back to fp32
+template <typename T> __device__ __forceinline__ void unpack2(uint32_t r, float &a, float &b);
+template <> __device__ __forceinline__ void unpack2<bf16_t>(uint32_t r, float &a, float &b)
+{
+    a = __uint_as_float(r << 16);
+    b = __uint_as_float(r & 0xffff0000u);
+}
+template <> __device__ __forceinline__ void unpack2<f16_t>(uint32_t r, float &a, float &b)
+{
+    const mta_f16x2 h = __builtin_bit_cast(mta_f16x2, r);
+    a = (float)h[0];
+    b = (float)h[1];
+}
+
 // value of the I/O dtype nearest to v, as fp32 (models an intermediate stored in T)
 template <typename T> __device__ __forceinline__ float round_to(float v) { return to_float(from_float<T>(v)); }
 

@@ -242,7 +242,8 @@ typedef const __attribute__((address_space(1))) void glb_void_t;
 // data + 1 of padding), so lane L of copy `it` simply owns slot it*64+L.  Edge strips go through
 // registers, where bounds and the causal col<=row rule are applied.
 //
-// SCALED: the result is in_scale * conv(x), the factor being applied to the fp32 accumulator.
+// SCALED: every strip is staged through registers, where x*in_scale is rounded to the I/O dtype before it
+// reaches LDS (what a separate elementwise scale pass would have produced).
 template <typename T, int R, int S, bool SCALED>
 __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     const T *__restrict__ x, const T *__restrict__ w, T *__restrict__ y, int C, int H, int W, int causal, float in_scale,
@@ -292,6 +293,7 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
 
     // a strip is `interior` when its whole halo lies inside the tensor and on or below the diagonal
     auto is_interior = [&](int p0_, int q0_) {
+        if (SCALED) return false;
         const int h0 = p0_ - (R - 1), k0 = q0_ - G::HL;
         return h0 >= 0 && p0_ + M_TM <= H && k0 >= 0 && k0 + G::TW <= W && (!causal || k0 + G::TW - 1 <= h0);
     };
@@ -354,6 +356,10 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
                 const int h = h0 + rr, col = k0 + vc * VEC;
                 const bool ok = rr < G::ROWS && vc < VPR && h >= 0 && h < H && col >= 0 && col < W && !(causal && col > h);
                 V16 v = stage[it];
+                if (SCALED) {
+#pragma unroll
+                    for (int u = 0; u < VEC; ++u) v.v[u] = from_float<T>(to_float(v.v[u]) * in_scale);
+                }
                 if (!ok) {
 #pragma unroll
                     for (int u = 0; u < VEC; ++u) v.v[u] = from_float<T>(0.0f);
@@ -406,8 +412,7 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
                 const int q = q0 + cb * 16 + kg * 4;
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
-                    const float val = SCALED ? acc[cb][v] * in_scale : acc[cb][v];
-                    out.v[v] = from_float<T>((!interior && causal && q + v > prow) ? 0.0f : val);
+                    out.v[v] = from_float<T>((!interior && causal && q + v > prow) ? 0.0f : acc[cb][v]);
                 }
                 *reinterpret_cast<quad *>(tile + (rb * 16 + ln) * LD + cb * 16 + kg * 4) = out;
             }

@@ -309,11 +309,14 @@ template <int R, int SK> struct fused_geom {
     static constexpr int WZ_OFF = SHIFT + 16, WZ_LD = WZ_OFF + 32;
 };
 
-template <typename T, int D, int R, int SK>
+// SCORES_ONLY: stop after the conv and write  conv(mask0(scale * Q K^T))  as an (S,S) plane per (batch, head)
+// (`O` is then the score tensor, V is unused).  Only q <= p is written when causal, plus +0 above the
+// diagonal when `fill_upper` is set.  The tile is staged through LDS so that stores are 128-byte row segments.
+template <typename T, int D, int R, int SK, bool SCORES_ONLY>
 __global__ __launch_bounds__(F_NT, 2) void conv_attn_fwd_mfma(const T *__restrict__ Q, const T *__restrict__ K,
                                                              const T *__restrict__ V, const T *__restrict__ Wt,
                                                              T *__restrict__ O, int S, int causal, float scale, int H,
-                                                             int nqb)
+                                                             int nqb, int fill_upper)
 {
     using G = fused_geom<R, SK>;
     constexpr int CPR = D / 8;                     // 16-byte chunks per K/V row
@@ -326,8 +329,9 @@ __global__ __launch_bounds__(F_NT, 2) void conv_attn_fwd_mfma(const T *__restric
 
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T *Kt = reinterpret_cast<T *>(smem_raw);       // [2][TILE]
-    T *Vt = Kt + 2 * TILE;                         // [2][TILE]
-    T *Sc = Vt + 2 * TILE;                         // [F_SR][F_SLD]
+    T *Vt = Kt + 2 * TILE;                         // [2][TILE]; SCORES_ONLY: output staging [F_SR][F_BK+8] instead
+    constexpr int VT_ELEMS = SCORES_ONLY ? F_SR * (F_BK + 8) : 2 * TILE;
+    T *Sc = Vt + VT_ELEMS;                         // [F_SR][F_SLD]
     T *wz = Sc + F_SR * F_SLD;                     // [R][WZ_LD] zero-padded kernel rows
 
     const int tid = threadIdx.x;
@@ -338,25 +342,38 @@ __global__ __launch_bounds__(F_NT, 2) void conv_attn_fwd_mfma(const T *__restric
     const int q0 = qb * G::BQ;
     const T *Qp = Q + bh * (int64_t)S * D;
     const T *Kp = K + bh * (int64_t)S * D;
-    const T *Vp = V + bh * (int64_t)S * D;
-    T *Op = O + bh * (int64_t)S * D;
+    const T *Vp = SCORES_ONLY ? Kp : V + bh * (int64_t)S * D;
+    T *Op = O + bh * (int64_t)S * (SCORES_ONLY ? S : D);
 
     // asynchronous copy of key block j into buffer `buf`: K rows cb.., V rows j*BK..; out-of-range keys
     // re-read a valid row (their scores are zeroed / their probabilities are 0 later)
+    // slot r*512+tid of a block is row kv_row[r], 16-byte chunk kv_c of that row (fixed per lane)
+    int kv_off[ROUNDS], kv_row[ROUNDS];
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
+        const int slot = r * F_NT + tid;
+        kv_row[r] = slot / CPR;
+        kv_off[r] = kv_row[r] * D + ((slot % CPR) ^ (kv_row[r] & (CPR - 1))) * 8;
+    }
     auto issue_kv = [&](int j, int buf) {
         const int cb = j * F_BK + G::PWR;
+        const bool inside = cb >= 0 && cb + F_BK <= S && j >= 0 && (j + 1) * F_BK <= S;  // no key needs clamping
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r) {
-            const int slot = r * F_NT + tid;
-            const int row = slot / CPR, c = (slot % CPR) ^ (row & (CPR - 1));
-            int kr = cb + row;
-            kr = kr < 0 ? 0 : (kr >= S ? S - 1 : kr);
-            int vr = j * F_BK + row;
-            vr = vr < 0 ? 0 : (vr >= S ? S - 1 : vr);
-            __builtin_amdgcn_global_load_lds((glb_void_t *)(Kp + (int64_t)kr * D + c * 8),
+            int koff = cb * D + kv_off[r], voff = j * F_BK * D + kv_off[r];
+            if (!inside) {
+                int kr = cb + kv_row[r];
+                kr = kr < 0 ? 0 : (kr >= S ? S - 1 : kr);
+                int vr = j * F_BK + kv_row[r];
+                vr = vr < 0 ? 0 : (vr >= S ? S - 1 : vr);
+                koff = kv_off[r] + (kr - kv_row[r]) * D;
+                voff = kv_off[r] + (vr - kv_row[r]) * D;
+            }
+            __builtin_amdgcn_global_load_lds((glb_void_t *)(Kp + koff),
                                              (lds_void_t *)(Kt + buf * TILE + (r * F_NT + wave * 64) * 8), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((glb_void_t *)(Vp + (int64_t)vr * D + c * 8),
-                                             (lds_void_t *)(Vt + buf * TILE + (r * F_NT + wave * 64) * 8), 16, 0, 0);
+            if (!SCORES_ONLY)
+                __builtin_amdgcn_global_load_lds((glb_void_t *)(Vp + voff),
+                                                 (lds_void_t *)(Vt + buf * TILE + (r * F_NT + wave * 64) * 8), 16, 0, 0);
         }
     };
 
@@ -415,121 +432,232 @@ __global__ __launch_bounds__(F_NT, 2) void conv_attn_fwd_mfma(const T *__restric
     constexpr int TAIL_VECS = F_SR * (G::HC / 8);
     constexpr int TAIL_IT = (TAIL_VECS + F_NT - 1) / F_NT;
 
+    int tail_off[TAIL_IT > 0 ? TAIL_IT : 1];  // element offset of this thread's retained vector(s) in the tile's head
+#pragma unroll
+    for (int it = 0; it < TAIL_IT; ++it) {
+        constexpr int VPRW = G::HC / 8 > 0 ? G::HC / 8 : 1;
+        const int idx = it * F_NT + tid;
+        tail_off[it] = idx < TAIL_VECS ? (idx / VPRW) * F_SLD + (idx % VPRW) * 8 : -1;
+    }
+    // the two 16-row blocks of this wavefront span rows pmin..pmin+31 of the sequence
+    const int pmin = q0 - G::HR + wave * 32;
+
     int buf = 0;
     for (int j = j_start; j <= j_end; ++j, buf ^= 1) {
         const int cbase = j * F_BK + G::PWR;  // first key of the new score block
         pack16<T> tailreg[TAIL_IT > 0 ? TAIL_IT : 1];
 #pragma unroll
-        for (int it = 0; it < TAIL_IT; ++it) {
-            const int idx = it * F_NT + tid;
-            const int row = idx / (G::HC / 8 > 0 ? G::HC / 8 : 1), vc = idx % (G::HC / 8 > 0 ? G::HC / 8 : 1);
-            if (idx < TAIL_VECS) tailreg[it] = *reinterpret_cast<const pack16<T> *>(Sc + row * F_SLD + F_BK + vc * 8);
-        }
+        for (int it = 0; it < TAIL_IT; ++it)
+            if (tail_off[it] >= 0) tailreg[it] = *reinterpret_cast<const pack16<T> *>(Sc + tail_off[it] + F_BK);
         __builtin_amdgcn_s_waitcnt(0);  // this wavefront's part of block j has landed in LDS
         __syncthreads();                // ... and everybody's; all reads of the previous tiles are done
 #pragma unroll
-        for (int it = 0; it < TAIL_IT; ++it) {
-            const int idx = it * F_NT + tid;
-            const int row = idx / (G::HC / 8 > 0 ? G::HC / 8 : 1), vc = idx % (G::HC / 8 > 0 ? G::HC / 8 : 1);
-            if (idx < TAIL_VECS) *reinterpret_cast<pack16<T> *>(Sc + row * F_SLD + vc * 8) = tailreg[it];
-        }
+        for (int it = 0; it < TAIL_IT; ++it)
+            if (tail_off[it] >= 0) *reinterpret_cast<pack16<T> *>(Sc + tail_off[it]) = tailreg[it];
         if (j < j_end) issue_kv(j + 1, buf ^ 1);  // lands while this block is being worked on
 
         // ---- S^T = K Q^T, zero above the diagonal / outside the sequence, to the score tile ----
-        const T *Kb = Kt + buf * TILE;
+        // The K fragments of key block cb+1 are read from LDS while the matrix cores work on block cb.
+        {
+            const T *Kb = Kt + buf * TILE;
+            frag8<T> kf[2][KS];
+            auto load_kf = [&](int cb, frag8<T> (&dst)[KS]) {
+                const int krow = cb * 16 + ln;
 #pragma unroll
-        for (int cb = 0; cb < NCB; ++cb) {
-            f32x4 sacc[2] = {f32x4{0.0f, 0.0f, 0.0f, 0.0f}, f32x4{0.0f, 0.0f, 0.0f, 0.0f}};
-            const int krow = cb * 16 + ln;
+                for (int ks = 0; ks < KS; ++ks)
+                    dst[ks] = *reinterpret_cast<const frag8<T> *>(Kb + krow * D + (((ks * 4 + kg) ^ (krow & (CPR - 1))) * 8));
+            };
+            load_kf(0, kf[0]);
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const int c = (ks * 4 + kg) ^ (krow & (CPR - 1));
-                const frag8<T> kf = *reinterpret_cast<const frag8<T> *>(Kb + krow * D + c * 8);
-                mma16(sacc[0], kf, qf[0][ks]);
-                mma16(sacc[1], kf, qf[1][ks]);
-            }
+            for (int cb = 0; cb < NCB; ++cb) {
+                if (cb + 1 < NCB) load_kf(cb + 1, kf[(cb + 1) & 1]);
+                f32x4 sacc[2] = {f32x4{0.0f, 0.0f, 0.0f, 0.0f}, f32x4{0.0f, 0.0f, 0.0f, 0.0f}};
 #pragma unroll
-            for (int rb = 0; rb < 2; ++rb) {
-                struct alignas(8) quad { T v[4]; } out;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int col = cbase + cb * 16 + kg * 4 + v;
-                    const bool keep = col >= 0 && col < S && !(causal && col > prow[rb]);
-                    out.v[v] = from_float<T>(keep ? sacc[rb][v] : 0.0f);
+                for (int ks = 0; ks < KS; ++ks) {
+                    mma16(sacc[0], kf[cb & 1][ks], qf[0][ks]);
+                    mma16(sacc[1], kf[cb & 1][ks], qf[1][ks]);
                 }
-                *reinterpret_cast<quad *>(Sc + trow[rb] * F_SLD + G::HC + cb * 16 + kg * 4) = out;
+                // key block wholly inside the sequence and on or below the diagonal for all 32 rows: no masks
+                const bool s_plain = cbase + cb * 16 >= 0 && cbase + cb * 16 + 16 <= S && (!causal || cbase + cb * 16 + 15 <= pmin);
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb) {
+                    uint32_t lo = pack2<T>(sacc[rb][0], sacc[rb][1]), hi = pack2<T>(sacc[rb][2], sacc[rb][3]);
+                    if (SCORES_ONLY) {  // MTA scales the scores before the conv, in the I/O dtype: round, scale, round again
+                        float a0, a1, a2, a3;
+                        unpack2<T>(lo, a0, a1);
+                        unpack2<T>(hi, a2, a3);
+                        lo = pack2<T>(a0 * scale, a1 * scale);
+                        hi = pack2<T>(a2 * scale, a3 * scale);
+                    }
+                    if (!s_plain) {
+                        const int col = cbase + cb * 16 + kg * 4;
+                        const int lim = causal ? (prow[rb] < S - 1 ? prow[rb] : S - 1) : S - 1;  // last key kept
+                        if (col < 0 || col > lim) lo &= 0xffff0000u;
+                        if (col + 1 < 0 || col + 1 > lim) lo &= 0x0000ffffu;
+                        if (col + 2 < 0 || col + 2 > lim) hi &= 0xffff0000u;
+                        if (col + 3 < 0 || col + 3 > lim) hi &= 0x0000ffffu;
+                    }
+                    *reinterpret_cast<uint2 *>(Sc + trow[rb] * F_SLD + G::HC + cb * 16 + kg * 4) = make_uint2(lo, hi);
+                }
             }
         }
         __syncthreads();
         if (j < 0) continue;
 
-        // ---- conv (Toeplitz MFMAs over the score tile), scale, mask, online softmax ----
-        frag8<T> pf[2][2];
+        // score fragments of block blk = rb*NCB+cb: rows trow-(R-1)+i, the block's 32-key window
+        auto load_xf = [&](int blk, frag8<T> (&dst)[R]) {
+            const int rb = blk / NCB, cb = blk % NCB;
 #pragma unroll
-        for (int rb = 0; rb < 2; ++rb) {
-            float sv[NCB][4];
-            float mloc = -INFINITY;
+            for (int i = 0; i < R; ++i) {
+                int srow = trow[rb] - (R - 1) + i;
+                srow = srow < 0 ? 0 : srow;  // only halo rows (discarded) can reach above the tile
+                dst[i] = *reinterpret_cast<const frag8<T> *>(Sc + srow * F_SLD + cb * 16 + kg * 8);
+            }
+        };
+
+        if constexpr (SCORES_ONLY) {
+            // ---- conv (Toeplitz MFMAs over the score tile) -> this wavefront's 32 x 64 staging rows -> global ----
+            // The score fragments of block blk+1 are read from LDS while the matrix cores work on block blk.
+            constexpr int OLD = F_BK + 8;  // staging row stride (elements)
+            T *stage = Vt + wave * 32 * OLD;
+            frag8<T> xf[2][R];
+            load_xf(0, xf[0]);
 #pragma unroll
-            for (int cb = 0; cb < NCB; ++cb) {
+            for (int blk = 0; blk < 2 * NCB; ++blk) {
+                const int rb = blk / NCB, cb = blk % NCB;
+                if (blk + 1 < 2 * NCB) load_xf(blk + 1, xf[(blk + 1) & 1]);
                 f32x4 cacc = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int i = 0; i < R; ++i) {
-                    int srow = trow[rb] - (R - 1) + i;
-                    srow = srow < 0 ? 0 : srow;  // only halo rows (discarded) can reach above the tile
-                    mma16(cacc, tz[i], *reinterpret_cast<const frag8<T> *>(Sc + srow * F_SLD + cb * 16 + kg * 8));
+                for (int i = 0; i < R; ++i) mma16(cacc, tz[i], xf[blk & 1][i]);
+                uint32_t lo = pack2<T>(cacc[0], cacc[1]), hi = pack2<T>(cacc[2], cacc[3]);
+                if (causal && j * F_BK + cb * 16 + 15 > pmin) {  // block touches the diagonal for some row
+                    const int col = j * F_BK + cb * 16 + kg * 4;
+                    if (col > prow[rb]) lo &= 0xffff0000u;
+                    if (col + 1 > prow[rb]) lo &= 0x0000ffffu;
+                    if (col + 2 > prow[rb]) hi &= 0xffff0000u;
+                    if (col + 3 > prow[rb]) hi &= 0x0000ffffu;
                 }
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int col = j * F_BK + cb * 16 + kg * 4 + v;
-                    const bool ok = col < S && !(causal && col > prow[rb]);
-                    const float val = round_to<T>(round_to<T>(cacc[v]) * scale);
-                    sv[cb][v] = ok ? val : -INFINITY;
-                    mloc = fmaxf(mloc, sv[cb][v]);
-                }
+                *reinterpret_cast<uint2 *>(stage + (rb * 16 + ln) * OLD + cb * 16 + kg * 4) = make_uint2(lo, hi);
             }
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-            const float m_new = fmaxf(m_i[rb], mloc);
-            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-            const float alpha = __expf(m_i[rb] - m_use);
-            m_i[rb] = m_new;
-            float lsum = 0.0f;
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's staging rows are written
 #pragma unroll
-            for (int cb = 0; cb < NCB; ++cb)
+            for (int it = 0; it < 4; ++it) {
+                const int r = it * 8 + (lane >> 3), cv = (lane & 7) * 8;
+                const int tr_ = wave * 32 + r, p_ = q0 - G::HR + tr_, col = j * F_BK + cv;
+                const pack16<T> v = *reinterpret_cast<const pack16<T> *>(stage + r * OLD + cv);
+                if (tr_ >= G::HR && p_ < S && col < S && (!causal || fill_upper || col <= p_))
+                    *reinterpret_cast<pack16<T> *>(Op + (int64_t)p_ * S + col) = v;
+            }
+            continue;
+        }
+
+        // ---- conv (Toeplitz MFMAs over the score tile), scale, mask, online softmax ----
+        frag8<T> pf[2][2];
+        {
+            frag8<T> xf[2][R];
+            load_xf(0, xf[0]);
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const T et = from_float<T>(__expf(sv[cb][v] - m_use));
-                    lsum += to_float(et);
-                    pf[rb][cb >> 1].v[(cb & 1) * 4 + v] = et;
+            for (int rb = 0; rb < 2; ++rb) {
+                float sv[NCB][4];
+                float mloc = -INFINITY;
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb) {
+                    const int blk = rb * NCB + cb;
+                    if (blk + 1 < 2 * NCB) load_xf(blk + 1, xf[(blk + 1) & 1]);
+                    f32x4 cacc = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int i = 0; i < R; ++i) mma16(cacc, tz[i], xf[blk & 1][i]);
+                    // conv output and scaled logits are rounded to the I/O dtype, as the unfused pipeline stores them
+                    float a[4];
+                    unpack2<T>(pack2<T>(cacc[0], cacc[1]), a[0], a[1]);
+                    unpack2<T>(pack2<T>(cacc[2], cacc[3]), a[2], a[3]);
+                    unpack2<T>(pack2<T>(a[0] * scale, a[1] * scale), a[0], a[1]);
+                    unpack2<T>(pack2<T>(a[2] * scale, a[3] * scale), a[2], a[3]);
+                    const bool c_plain = j * F_BK + cb * 16 + 16 <= S && (!causal || j * F_BK + cb * 16 + 15 <= pmin);
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        float val = a[v];
+                        if (!c_plain) {
+                            const int col = j * F_BK + cb * 16 + kg * 4 + v;
+                            if (!(col < S && !(causal && col > prow[rb]))) val = -INFINITY;
+                        }
+                        sv[cb][v] = val;
+                        mloc = fmaxf(mloc, val);
+                    }
                 }
-            l_i[rb] = l_i[rb] * alpha + lsum;
+                mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
+                mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+                const float m_new = fmaxf(m_i[rb], mloc);
+                const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+                const float alpha = __expf(m_i[rb] - m_use);
+                m_i[rb] = m_new;
+                float lsum = 0.0f;
 #pragma unroll
-            for (int db = 0; db < DB; ++db) oacc[rb][db] *= alpha;
+                for (int cb = 0; cb < NCB; ++cb) {
+                    float e[4];
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) e[v] = __expf(sv[cb][v] - m_use);
+                    const uint32_t lo = pack2<T>(e[0], e[1]), hi = pack2<T>(e[2], e[3]);
+                    float r0, r1, r2, r3;
+                    unpack2<T>(lo, r0, r1);
+                    unpack2<T>(hi, r2, r3);
+                    lsum += (r0 + r1) + (r2 + r3);
+                    uint32_t *dst = reinterpret_cast<uint32_t *>(&pf[rb][cb >> 1]) + (cb & 1) * 2;
+                    dst[0] = lo;
+                    dst[1] = hi;
+                }
+                l_i[rb] = l_i[rb] * alpha + lsum;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) oacc[rb][db] *= alpha;
+            }
         }
 
         // ---- O^T += V^T P^T ; V^T fragments via the LDS transpose read of the row-major V block ----
-        const T *Vb = Vt + buf * TILE;
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
+        {
+            const T *Vb = Vt + buf * TILE;
             // slots 0..3: keys 32ks+4kg+(0..3); slots 4..7: keys 32ks+16+4kg+(0..3) -- the order of pf
-            const int key_a = ks * 32 + kg * 4 + (ln >> 2);
-            const int key_b = key_a + 16;
-#pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                const int ch = db * 2 + ((ln & 3) >> 1);           // 16-byte chunk holding head dims 16db+4(ln%4)..
-                const int sub = (ln & 1) * 4;                      // element offset inside the chunk
+            frag8<T> vf[2];
+            auto load_vf = [&](int blk, frag8<T> &dst) {  // blk = ks * DB + db
+                const int ks = blk / DB, db = blk % DB;
+                const int key_a = ks * 32 + kg * 4 + (ln >> 2), key_b = key_a + 16;
+                const int ch = db * 2 + ((ln & 3) >> 1);  // 16-byte chunk holding head dims 16db+4(ln%4)..
+                const int sub = (ln & 1) * 4;             // element offset inside the chunk
                 const T *pa = Vb + key_a * D + ((ch ^ (key_a & (CPR - 1))) * 8) + sub;
                 const T *pb = Vb + key_b * D + ((ch ^ (key_b & (CPR - 1))) * 8) + sub;
-                const v4s_t va = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)pa);
-                const v4s_t vb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)pb);
-                struct { v4s_t a, b; } both = {va, vb};
-                const frag8<T> vf = __builtin_bit_cast(frag8<T>, both);
-                mma16(oacc[0][db], vf, pf[0][ks]);
-                mma16(oacc[1][db], vf, pf[1][ks]);
+                struct { v4s_t a, b; } both = {__builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)pa),
+                                               __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)pb)};
+                dst = __builtin_bit_cast(frag8<T>, both);
+            };
+            load_vf(0, vf[0]);
+#pragma unroll
+            for (int blk = 0; blk < 2 * DB; ++blk) {
+                const int ks = blk / DB, db = blk % DB;
+                if (blk + 1 < 2 * DB) load_vf(blk + 1, vf[(blk + 1) & 1]);
+                mma16(oacc[0][db], vf[blk & 1], pf[0][ks]);
+                mma16(oacc[1][db], vf[blk & 1], pf[1][ks]);
             }
         }
     }
 
+    if constexpr (SCORES_ONLY) {
+        // +0 for the key blocks to the right of the last one visited (all above the diagonal)
+        if (causal && fill_upper) {
+            pack16<T> z;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) z.v[u] = from_float<T>(0.0f);
+            const int c_first = (j_end + 1) * F_BK;
+            const int vec_per_row = (S - c_first + 7) / 8;
+            for (int r = wave; r < G::BQ; r += F_NT / 64) {
+                const int p_ = q0 + r;
+                if (p_ >= S) break;
+                for (int vc = lane; vc < vec_per_row; vc += 64) {
+                    const int col = c_first + vc * 8;
+                    if (col < S) *reinterpret_cast<pack16<T> *>(Op + (int64_t)p_ * S + col) = z;
+                }
+            }
+        }
+        return;
+    }
     // ---- normalise and store (halo rows are dropped) ----
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb) {
@@ -540,51 +668,49 @@ __global__ __launch_bounds__(F_NT, 2) void conv_attn_fwd_mfma(const T *__restric
             const float inv = 1.0f / l_row;
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-                struct alignas(8) quad { T v[4]; } out;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) out.v[v] = from_float<T>(oacc[rb][db][v] * inv);
-                *reinterpret_cast<quad *>(Op + (int64_t)prow[rb] * D + db * 16 + kg * 4) = out;
+                const uint32_t lo = pack2<T>(oacc[rb][db][0] * inv, oacc[rb][db][1] * inv);
+                const uint32_t hi = pack2<T>(oacc[rb][db][2] * inv, oacc[rb][db][3] * inv);
+                *reinterpret_cast<uint2 *>(Op + (int64_t)prow[rb] * D + db * 16 + kg * 4) = make_uint2(lo, hi);
             }
         }
     }
 }
 
-template <typename T, int D, int R, int SK>
+template <typename T, int D, int R, int SK, bool SCORES_ONLY>
 int launch_mfma(const void *q, const void *k, const void *v, const void *w, void *o, int64_t B, int64_t H, int64_t S,
-                int causal, float scale, hipStream_t st)
+                int causal, float scale, int fill_upper, hipStream_t st)
 {
     using G = fused_geom<R, SK>;
     static_assert(G::fits, "conv window exceeds the 32-key MFMA contraction");
     const int nqb = (int)((S + G::BQ - 1) / G::BQ);
-    const size_t lds = sizeof(T) * ((size_t)4 * F_BK * D + (size_t)F_SR * F_SLD + (size_t)R * G::WZ_LD);
-    auto kern = conv_attn_fwd_mfma<T, D, R, SK>;
+    const size_t vt_elems = SCORES_ONLY ? (size_t)F_SR * (F_BK + 8) : (size_t)2 * F_BK * D;
+    const size_t lds = sizeof(T) * ((size_t)2 * F_BK * D + vt_elems + (size_t)F_SR * F_SLD + (size_t)R * G::WZ_LD);
+    auto kern = conv_attn_fwd_mfma<T, D, R, SK, SCORES_ONLY>;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
     dim3 grid((unsigned)nqb, (unsigned)(B * H));
     hipLaunchKernelGGL(kern, grid, dim3(F_NT), lds, st, (const T *)q, (const T *)k, (const T *)v, (const T *)w, (T *)o,
-                       (int)S, causal, scale, (int)H, nqb);
+                       (int)S, causal, scale, (int)H, nqb, fill_upper);
     return launch_status();
 }
 
 // returns 1 when no instantiation covers the kernel size (the caller then uses the general kernel)
-template <typename T, int D>
+template <typename T, int D, bool SCORES_ONLY>
 int dispatch_mfma(const void *q, const void *k, const void *v, const void *w, void *o, int64_t B, int64_t H, int64_t S,
-                  int R, int Sk, int causal, float scale, hipStream_t st)
+                  int R, int Sk, int causal, float scale, int fill_upper, hipStream_t st)
 {
+    if constexpr (sizeof(T) == 2) {
 #define MTA_FUSED_CASE(r, s) \
-    if (R == r && Sk == s) return launch_mfma<T, D, r, s>(q, k, v, w, o, B, H, S, causal, scale, st);
-    MTA_FUSED_CASE(3, 3)
-    MTA_FUSED_CASE(5, 5)
-    MTA_FUSED_CASE(5, 7)
-    MTA_FUSED_CASE(6, 11)
-    MTA_FUSED_CASE(7, 7)
+    if (R == r && Sk == s) return launch_mfma<T, D, r, s, SCORES_ONLY>(q, k, v, w, o, B, H, S, causal, scale, fill_upper, st);
+        MTA_FUSED_CASE(3, 3)
+        MTA_FUSED_CASE(5, 5)
+        MTA_FUSED_CASE(5, 7)
+        MTA_FUSED_CASE(6, 11)
+        MTA_FUSED_CASE(7, 7)
 #undef MTA_FUSED_CASE
+    }
     return 1;
 }
-template <> int dispatch_mfma<float, 64>(const void *, const void *, const void *, const void *, void *, int64_t, int64_t,
-                                         int64_t, int, int, int, float, hipStream_t) { return 1; }
-template <> int dispatch_mfma<float, 128>(const void *, const void *, const void *, const void *, void *, int64_t, int64_t,
-                                          int64_t, int, int, int, float, hipStream_t) { return 1; }
 
 template <typename T, int D>
 int launch(const void *q, const void *k, const void *v, const void *w, void *o, int64_t B, int64_t H, int64_t S,
@@ -627,12 +753,33 @@ extern "C" int mta_conv_attn_fwd(const void *q, const void *k, const void *v, co
     const bool fast_ok = io_dtype != MTA_F32 && w_dtype == io_dtype && !force_general;
     MTA_DISPATCH_IO(io_dtype, {
         if (fast_ok) {
-            const int rc = D == 64 ? dispatch_mfma<io_t, 64>(q, k, v, w, o, B, H, S, R, Sk, causal, scale, st)
-                                   : dispatch_mfma<io_t, 128>(q, k, v, w, o, B, H, S, R, Sk, causal, scale, st);
+            const int rc = D == 64 ? dispatch_mfma<io_t, 64, false>(q, k, v, w, o, B, H, S, R, Sk, causal, scale, 0, st)
+                                   : dispatch_mfma<io_t, 128, false>(q, k, v, w, o, B, H, S, R, Sk, causal, scale, 0, st);
             if (rc != 1) return rc;
         }
         if (D == 64) return launch<io_t, 64>(q, k, v, w, o, B, H, S, R, Sk, causal, scale, w_dtype, st);
         return launch<io_t, 128>(q, k, v, w, o, B, H, S, R, Sk, causal, scale, w_dtype, st);
     });
     return MTA_ERR_DTYPE;
+}
+
+extern "C" int mta_qk_conv_fwd(const void *q, const void *k, const void *w, void *s_out, int64_t B, int64_t H, int64_t S,
+                               int64_t D, int R, int Sk, int causal, float scale, int fill_upper, int io_dtype,
+                               int w_dtype, void *stream)
+{
+    if (!q || !k || !w || !s_out) return MTA_ERR_NULL;
+    if (!dtype_size(io_dtype) || !dtype_size(w_dtype)) return MTA_ERR_DTYPE;
+    if (B <= 0 || H <= 0 || S <= 0 || S > (1 << 24) || B * H > 65535) return MTA_ERR_SHAPE;
+    if (R < 1 || Sk < 1 || R > MTA_MAX_KERNEL_R || Sk > MTA_MAX_KERNEL_S) return MTA_ERR_KERNEL_SIZE;
+    if (D != 64 && D != 128) return MTA_ERR_HEAD_DIM;
+    if (!aligned_to(q, 16) || !aligned_to(k, 16) || !aligned_to(s_out, 16) || !aligned_to(w, dtype_size(w_dtype)))
+        return MTA_ERR_ALIGN;
+    if (io_dtype == MTA_F32 || w_dtype != io_dtype || S % 8 != 0) return MTA_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    int rc = 1;
+    MTA_DISPATCH_IO(io_dtype, {
+        rc = D == 64 ? dispatch_mfma<io_t, 64, true>(q, k, nullptr, w, s_out, B, H, S, R, Sk, causal, scale, fill_upper, st)
+                     : dispatch_mfma<io_t, 128, true>(q, k, nullptr, w, s_out, B, H, S, R, Sk, causal, scale, fill_upper, st);
+    });
+    return rc == 1 ? MTA_ERR_UNSUPPORTED : rc;
 }

@@ -51,7 +51,7 @@ template <int NT> __device__ __forceinline__ float block_sum(float v, float *red
 template <typename T, int G, int NV, int VEC, int NT>
 __global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, const void *__restrict__ w1,
                                                       const void *__restrict__ w2, T *__restrict__ y, int C,
-                                                      int P, int Q, int causal, int w_dtype)
+                                                      int P, int Q, int causal, int w_dtype, int fill_upper)
 {
     __shared__ float w1s[G * G];
     __shared__ float w2s[G * G];
@@ -163,7 +163,7 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, c
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
         const int q = (k * NT + tid) * VEC;
-        if (q >= Q) continue;
+        if (q >= Q || (!fill_upper && q > last)) continue;  // vectors wholly above the diagonal: +0 only on request
 #pragma unroll
         for (int o = 0; o < G; ++o) {
             V out;
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, c
 template <typename T, int NT>
 __global__ __launch_bounds__(NT) void mix_softmax_mix_any(const T *__restrict__ x, const void *__restrict__ w1,
                                                           const void *__restrict__ w2, T *__restrict__ y, int C,
-                                                          int G, int P, int Q, int causal, int w_dtype)
+                                                          int G, int P, int Q, int causal, int w_dtype, int fill_upper)
 {
     __shared__ float red[NT / 64];
     extern __shared__ float stats[];  // [G] max, [G] 1/sum
@@ -220,7 +220,8 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix_any(const T *__restrict__ 
         if (tid == 0) { stats[o] = m; stats[G + o] = 1.0f / sum; }
     }
     __syncthreads();
-    for (int q = tid; q < Q; q += NT) {
+    const int q_end = fill_upper ? Q : last + 1;
+    for (int q = tid; q < q_end; q += NT) {
         for (int o = 0; o < G; ++o) {
             float acc = 0.0f;
             if (q <= last) {
@@ -240,26 +241,26 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix_any(const T *__restrict__ 
 
 template <typename T, int G, int NV>
 int launch_fixed(const void *x, const void *w1, const void *w2, void *y, int64_t N, int64_t C, int64_t P,
-                 int64_t Q, int causal, int w_dtype, hipStream_t st)
+                 int64_t Q, int causal, int w_dtype, int fill_upper, hipStream_t st)
 {
     constexpr int VEC = vec_of<T>::n;
     constexpr int NT = 256;
     const int64_t blocks = N * (C / G) * P;
     hipLaunchKernelGGL((mix_softmax_mix<T, G, NV, VEC, NT>), dim3((unsigned)blocks), dim3(NT), 0, st, (const T *)x,
-                       w1, w2, (T *)y, (int)C, (int)P, (int)Q, causal, w_dtype);
+                       w1, w2, (T *)y, (int)C, (int)P, (int)Q, causal, w_dtype, fill_upper);
     return launch_status();
 }
 
 template <typename T>
 int dispatch(const void *x, const void *w1, const void *w2, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
-             int G, int causal, int w_dtype, hipStream_t st)
+             int G, int causal, int w_dtype, int fill_upper, hipStream_t st)
 {
     constexpr int VEC = vec_of<T>::n;
     const bool vec_ok = (Q % VEC == 0) && aligned_to(x, 16) && aligned_to(y, 16);
     const int64_t nv = (Q + 256 * VEC - 1) / (256 * VEC);
     if (vec_ok) {
 #define MTA_RS_CASE(g, v)                                                                   \
-    if (G == g && nv <= v) return launch_fixed<T, g, v>(x, w1, w2, y, N, C, P, Q, causal, w_dtype, st);
+    if (G == g && nv <= v) return launch_fixed<T, g, v>(x, w1, w2, y, N, C, P, Q, causal, w_dtype, fill_upper, st);
         MTA_RS_CASE(1, 1) MTA_RS_CASE(1, 2) MTA_RS_CASE(1, 4) MTA_RS_CASE(1, 8)
         MTA_RS_CASE(2, 1) MTA_RS_CASE(2, 2) MTA_RS_CASE(2, 4)
         MTA_RS_CASE(4, 1) MTA_RS_CASE(4, 2) MTA_RS_CASE(4, 4)
@@ -269,14 +270,14 @@ int dispatch(const void *x, const void *w1, const void *w2, void *y, int64_t N, 
     constexpr int NT = 256;
     const int64_t blocks = N * (C / G) * P;
     hipLaunchKernelGGL((mix_softmax_mix_any<T, NT>), dim3((unsigned)blocks), dim3(NT), sizeof(float) * 2 * G, st,
-                       (const T *)x, w1, w2, (T *)y, (int)C, G, (int)P, (int)Q, causal, w_dtype);
+                       (const T *)x, w1, w2, (T *)y, (int)C, G, (int)P, (int)Q, causal, w_dtype, fill_upper);
     return launch_status();
 }
 }  // namespace
 
 extern "C" int mta_headmix_softmax_fwd(const void *x, const void *w1, const void *w2, void *y, int64_t N,
                                        int64_t C, int64_t P, int64_t Q, int group_size, int causal,
-                                       int io_dtype, int w_dtype, void *stream)
+                                       int fill_upper, int io_dtype, int w_dtype, void *stream)
 {
     if (!x || !y) return MTA_ERR_NULL;
     if (!dtype_size(io_dtype) || !dtype_size(w_dtype)) return MTA_ERR_DTYPE;
@@ -289,6 +290,6 @@ extern "C" int mta_headmix_softmax_fwd(const void *x, const void *w1, const void
     if (!w1 && !w2) G = 1;
     if (N * (C / G) * P > 0x7fffffffLL) return MTA_ERR_SHAPE;
     hipStream_t st = (hipStream_t)stream;
-    MTA_DISPATCH_IO(io_dtype, return dispatch<io_t>(x, w1, w2, y, N, C, P, Q, G, causal, w_dtype, st));
+    MTA_DISPATCH_IO(io_dtype, return dispatch<io_t>(x, w1, w2, y, N, C, P, Q, G, causal, w_dtype, fill_upper || !causal, st));
     return MTA_ERR_DTYPE;
 }

@@ -95,31 +95,44 @@ class MTAAttentionTriton(nn.Module):
         head_dim = xq.size(-1)
         # the reference multiplies by rsqrt(tensor(head_dim)), an fp32 scalar (mta_attention_triton.py:69-71)
         scale = float(torch.rsqrt(torch.tensor(float(head_dim))))
-        self._mark("qk")
-        scores = torch.matmul(xq, xk.transpose(2, 3))
-        self._mark("conv_pre")
-        scores = ops.conv2d_causal(scores, self.mta_conv_triton.weight, self.causal, in_scale=scale)
-
         w_pre, w_post = self.wpsm_triton.weight, self.wposm_triton.weight
         pre_eye, g_pre = self._probe("wpsm", w_pre, _probe_head)
         post_eye, g_post = self._probe("wposm", w_post, _probe_head)
         post_conv_identity = self._probe("conv_post", self.mta_conv_after_sm_triton.weight, _probe_conv)
         w1 = None if pre_eye else w_pre
         w2 = None if post_eye else w_post
+        one_pass = post_conv_identity and _lcm(g_pre, g_post) <= _FUSED_MAX_GROUP
+        # the last stage may leave the upper triangle unwritten only if our own P V kernel consumes it
+        own_pv = (xq.size(-2) == xk.size(-2) and xq.dtype == xv.dtype
+                  and ops.causal_pv_supported(xq.dtype, xq.size(-2), xv.size(-1)))
 
-        if post_conv_identity and _lcm(g_pre, g_post) <= _FUSED_MAX_GROUP:
+        # QK^T -> *1/sqrt(d) -> conv: one kernel when it exists for this dtype / size, else GEMM + conv
+        self._mark("qk_conv")
+        scores = None
+        if xq.shape == xk.shape:
+            scores = ops.qk_conv(xq, xk, self.mta_conv_triton.weight, self.causal, scale, fill_upper=False)
+        if scores is None:
+            self._mark("qk")
+            scores = torch.matmul(xq, xk.transpose(2, 3))
+            self._mark("conv_pre")
+            scores = ops.conv2d_causal(scores, self.mta_conv_triton.weight, self.causal, in_scale=scale)
+
+        if one_pass:
             self._mark("mix_softmax_mix")
-            scores = ops.headmix_softmax(scores, w1, w2, self.causal, group_size=_lcm(g_pre, g_post))
+            scores = ops.headmix_softmax(scores, w1, w2, self.causal, group_size=_lcm(g_pre, g_post),
+                                         fill_upper=not own_pv)
         else:
             if g_pre <= _FUSED_MAX_GROUP:
                 self._mark("mix_softmax")
-                scores = ops.headmix_softmax(scores, w1, None, self.causal, group_size=g_pre)
+                scores = ops.headmix_softmax(scores, w1, None, self.causal, group_size=g_pre,
+                                             fill_upper=post_conv_identity and w2 is None and not own_pv)
             else:
                 self._mark("mix_pre")
                 fill = float("-inf") if self.causal else 0.0
                 scores = ops.headmix(scores, w_pre, self.causal, fill, group_size=g_pre)
                 self._mark("softmax")
-                scores = ops.headmix_softmax(scores, None, None, self.causal)
+                scores = ops.headmix_softmax(scores, None, None, self.causal,
+                                             fill_upper=post_conv_identity and w2 is None and not own_pv)
             if not post_conv_identity:
                 self._mark("conv_post")
                 scores = ops.conv2d_causal(scores, self.mta_conv_after_sm_triton.weight, self.causal)
@@ -129,7 +142,9 @@ class MTAAttentionTriton(nn.Module):
 
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         self._mark("pv")
-        output = torch.matmul(scores, xv)
+        output = ops.causal_pv(scores, xv, self.causal) if own_pv else None
+        if output is None:
+            output = torch.matmul(scores, xv)
         self._mark("end")
         return output.transpose(1, 2)
 

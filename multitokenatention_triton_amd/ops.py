@@ -89,8 +89,11 @@ def headmix(x: torch.Tensor, weight: torch.Tensor, causal: bool = True, fill: fl
 
 
 def headmix_softmax(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optional[torch.Tensor], causal: bool = True,
-                    group_size: Optional[int] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """mix(w1) -> causal row softmax -> mix(w2) in one pass; see mta_headmix_softmax_fwd."""
+                    group_size: Optional[int] = None, out: Optional[torch.Tensor] = None,
+                    fill_upper: bool = True) -> torch.Tensor:
+    """mix(w1) -> causal row softmax -> mix(w2) in one pass; see mta_headmix_softmax_fwd.
+
+    ``fill_upper=False`` leaves everything above the diagonal unwritten (for consumers that never read it)."""
     x = _device_tensor(x, "input")
     if x.dim() != 4:
         raise ValueError(f"expected input (N,C,P,Q), got {tuple(x.shape)}")
@@ -110,7 +113,7 @@ def headmix_softmax(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optional[to
         rc = _lib.load().mta_headmix_softmax_fwd(
             x.data_ptr(), ws[0].data_ptr() if ws[0] is not None else None,
             ws[1].data_ptr() if ws[1] is not None else None, y.data_ptr(), n, c, p, q, int(group_size or 0),
-            int(bool(causal)), _code(x, "input"), wcode, _stream(x))
+            int(bool(causal)), int(bool(fill_upper)), _code(x, "input"), wcode, _stream(x))
     _lib.check(rc, "mta_headmix_softmax_fwd")
     return y
 
@@ -138,6 +141,53 @@ def conv_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, weight: tor
                                            float(softmax_scale), _code(q, "Q"), _code(weight, "W"), _stream(q))
     _lib.check(rc, "mta_conv_attn_fwd")
     return o
+
+
+def qk_conv(q: torch.Tensor, k: torch.Tensor, weight: torch.Tensor, causal: bool, scale: float,
+            fill_upper: bool = True) -> Optional[torch.Tensor]:
+    """scale * conv(mask0(Q K^T)) as a (B,H,S,S) tensor without materialising Q K^T; see mta_qk_conv_fwd.
+
+    Returns ``None`` when the library has no kernel for this dtype / size combination (the caller then
+    takes matmul + conv2d_causal).  With ``fill_upper=False`` entries above the diagonal are left unwritten."""
+    q = _device_tensor(q, "Q")
+    k = _device_tensor(k, "K")
+    weight = _device_tensor(weight.detach(), "W")
+    if q.dim() != 4 or q.shape != k.shape or q.dtype != k.dtype:
+        raise ValueError(f"Q and K must share a (B,H,S,D) shape and dtype, got {tuple(q.shape)}, {tuple(k.shape)}")
+    b, h, s, d = q.shape
+    assert weight.dim() == 3 and weight.shape[0] == h, "conv weight must be (H,R,S)"
+    out = torch.empty((b, h, s, s), dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = _lib.load().mta_qk_conv_fwd(q.data_ptr(), k.data_ptr(), weight.data_ptr(), out.data_ptr(), b, h, s, d,
+                                         weight.shape[1], weight.shape[2], int(bool(causal)), float(scale),
+                                         int(bool(fill_upper)), _code(q, "Q"), _code(weight, "W"), _stream(q))
+    if rc in (_lib.MTA_ERR_UNSUPPORTED, -7):
+        return None
+    _lib.check(rc, "mta_qk_conv_fwd")
+    return out
+
+
+def causal_pv(p: torch.Tensor, v: torch.Tensor, causal: bool) -> Optional[torch.Tensor]:
+    """P V for P (B,H,S,S), V (B,H,S,D), reading only the lower triangle of P when causal; see mta_causal_pv_fwd.
+
+    Returns ``None`` when unsupported (the caller then uses torch.matmul on a fully defined P)."""
+    p = _device_tensor(p, "P")
+    v = _device_tensor(v, "V")
+    if p.dim() != 4 or v.dim() != 4 or p.shape[:3] != v.shape[:3] or p.shape[2] != p.shape[3] or p.dtype != v.dtype:
+        return None
+    b, h, s, d = v.shape
+    out = torch.empty_like(v)
+    with torch.cuda.device(p.device):
+        rc = _lib.load().mta_causal_pv_fwd(p.data_ptr(), v.data_ptr(), out.data_ptr(), b, h, s, d, int(bool(causal)),
+                                           _code(p, "P"), _stream(p))
+    if rc in (_lib.MTA_ERR_UNSUPPORTED, -7):
+        return None
+    _lib.check(rc, "mta_causal_pv_fwd")
+    return out
+
+
+def causal_pv_supported(p_dtype: torch.dtype, s: int, d: int) -> bool:
+    return p_dtype in (torch.bfloat16, torch.float16) and d in (64, 128) and s % 8 == 0
 
 
 # ---------------------------------------------------------------------------------------

@@ -25,11 +25,11 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     names = declared_functions()
     assert {"mta_conv2d_fwd", "mta_conv2d_scaled_fwd", "mta_headmix_fwd", "mta_headmix_softmax_fwd",
-            "mta_conv_attn_fwd", "mta_strerror", "mta_abi_version"} <= set(names)
+            "mta_conv_attn_fwd", "mta_qk_conv_fwd", "mta_causal_pv_fwd", "mta_strerror", "mta_abi_version"} <= set(names)
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/mta_hip.h but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes signatures out of sync with the header"
-    assert lib.mta_abi_version() == 1
+    assert lib.mta_abi_version() == 2
 
 
 def test_no_torch_symbols_in_the_library():
@@ -38,7 +38,7 @@ def test_no_torch_symbols_in_the_library():
 
 
 def test_error_strings():
-    for code in range(0, -9, -1):
+    for code in range(0, -10, -1):
         s = _lib.strerror(code)
         assert s and "unknown" not in s
     assert "unknown" in _lib.strerror(-99)
@@ -64,7 +64,11 @@ def test_argument_validation_needs_no_gpu():
     assert lib.mta_conv_attn_fwd(p, p, p, p, p, 1, 1, 8, 64, 0, 3, 1, 0.1, 0, 0, None) == -4
     # group
     assert lib.mta_headmix_fwd(p, p, p, 1, 6, 8, 8, 4, 1, 0.0, 0, 0, None) == -5
-    assert lib.mta_headmix_softmax_fwd(p, p, p, p, 1, 6, 8, 8, 4, 1, 0, 0, None) == -5
+    assert lib.mta_headmix_softmax_fwd(p, p, p, p, 1, 6, 8, 8, 4, 1, 1, 0, 0, None) == -5
+    # combinations without a kernel are reported, not silently served by something else
+    assert lib.mta_qk_conv_fwd(p, p, p, p, 1, 1, 8, 64, 3, 3, 1, 0.1, 1, 0, 0, None) == -9
+    assert lib.mta_causal_pv_fwd(p, p, p, 1, 1, 8, 64, 1, 0, None) == -9
+    assert lib.mta_causal_pv_fwd(p, p, p, 1, 1, 8, 48, 1, 1, None) == -7
     # alignment (fp32 pointer off by one byte)
     assert lib.mta_conv2d_fwd(p + 1, p, p, 1, 1, 8, 8, 3, 3, 1, 0, 0, None) == -6
     # head dim

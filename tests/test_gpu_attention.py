@@ -177,3 +177,87 @@ def test_conv_attention_row_slabs_long_sequence(pkg):
     for r0, r1 in [(0, 128), (2040, 2170), (3968, 4096)]:
         want = O.conv_attention_rows(q, k, v, w, r0, r1, True, None)
         torch.testing.assert_close(got[:, :, r0:r1].float(), want.float(), **tol(dtype))
+
+
+QKC_CASES = [
+    # B, H, S, D, R, Sk, causal, dtype
+    (1, 2, 256, 128, 6, 11, True, torch.bfloat16),
+    (2, 2, 520, 64, 3, 3, True, torch.bfloat16),
+    (1, 2, 248, 128, 6, 11, True, torch.float16),
+    (1, 1, 776, 128, 5, 7, False, torch.bfloat16),
+    (1, 2, 8, 64, 6, 11, True, torch.bfloat16),
+    (1, 1, 1000, 128, 7, 7, True, torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("fill", [True, False])
+@pytest.mark.parametrize("case", QKC_CASES)
+def test_qk_conv_parity(pkg, case, fill):
+    """scale*conv(mask0(QK^T)) vs the oracle's first two stages (mta_attention_pytorch.py:63-67)."""
+    b, h, s, d, r, sk, causal, dtype = case
+    print(f"qk_conv case={case} fill={fill}", flush=True)
+    q, k, _ = O.seeded_qkv(b, h, s, d, dtype, seed=7)
+    w = O.seeded_conv_weight(h, r, sk, 0.05, dtype)
+    scale = float(torch.rsqrt(torch.tensor(float(d))))
+    s0 = torch.matmul(q, k.transpose(2, 3)) * torch.rsqrt(torch.tensor(d))
+    want = O.depthwise_conv(torch.tril(s0) if causal else s0, w, causal)
+    sentinel = 12345.0
+    got = pkg.ops.qk_conv(q.cuda(), k.cuda(), w.cuda(), causal, scale, fill_upper=fill)
+    assert got is not None and got.shape == (b, h, s, s)
+    got = got.cpu()
+    low = torch.tril(torch.ones(s, s, dtype=torch.bool)) if causal else torch.ones(s, s, dtype=torch.bool)
+    # scores of magnitude ~sqrt(d)*|w| pass through two 16-bit roundings: 2 ulp + atol
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    torch.testing.assert_close(got[..., low].float(), want[..., low].float(), rtol=2 * ulp, atol=2e-2)
+    if causal and fill:
+        up = ~low
+        assert (got[..., up] == 0).all() and not torch.signbit(got[..., up]).any()
+    _ = sentinel
+
+
+def test_qk_conv_reports_unsupported(pkg):
+    q = torch.zeros(1, 2, 64, 64, device="cuda")
+    assert pkg.ops.qk_conv(q, q, torch.zeros(2, 3, 3, device="cuda"), True, 0.1) is None          # fp32
+    qb = q.bfloat16()
+    assert pkg.ops.qk_conv(qb, qb, torch.zeros(2, 11, 15, device="cuda").bfloat16(), True, 0.1) is None  # no 11x15 instance
+
+
+PV_CASES = [(1, 2, 256, 128, True, torch.bfloat16), (2, 3, 520, 64, True, torch.float16), (1, 2, 1000, 128, True, torch.bfloat16),
+            (1, 1, 264, 64, False, torch.bfloat16), (1, 2, 8, 128, True, torch.bfloat16)]
+
+
+@pytest.mark.parametrize("case", PV_CASES)
+def test_causal_pv_parity(pkg, case):
+    b, h, s, d, causal, dtype = case
+    print(f"causal_pv case={case}", flush=True)
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn(b, h, s, s, generator=g)
+    if causal:
+        logits.masked_fill_(torch.triu(torch.ones(s, s, dtype=torch.bool), 1), float("-inf"))
+    p = torch.softmax(logits, -1).to(dtype)
+    v = torch.randn(b, h, s, d, generator=g).to(dtype)
+    want = torch.matmul(p, v)
+    p_dev = p.cuda()
+    if causal:  # what lies above the diagonal must never be read: poison it
+        p_dev = p_dev.masked_fill(torch.triu(torch.ones(s, s, dtype=torch.bool, device="cuda"), 1), float("nan"))
+    got = pkg.ops.causal_pv(p_dev, v.cuda(), causal)
+    assert got is not None
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dtype))
+
+
+def test_mta_headline_config_small(pkg):
+    """BASELINE config 4 at reduced S: bf16, 6x11 pre conv, identity post conv, groups of 4 -- the route
+    qk_conv -> mix/softmax/mix -> causal P V, none of which writes or reads above the diagonal."""
+    print("mta headline small", flush=True)
+    dtype = torch.bfloat16
+    q, k, v = O.seeded_qkv(2, 16, 512, 128, dtype)
+    g = torch.Generator().manual_seed(125)
+    params = [O.seeded_conv_weight(16, 6, 11, 0.05, dtype), torch.eye(16, dtype=dtype),
+              O.identity_conv_kernel(16, 3, 3, dtype), O.block_diag_head_weight(16, 4, 0.1, g, dtype)]
+    want = _oracle_mta(q, k, v, params)
+    mod = _mta_module(pkg, 16, 6, 11, 3, 3, *params, dtype)
+    stages = []
+    mod._stage_hook = stages.append
+    got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
+    assert stages == ["qk_conv", "mix_softmax_mix", "pv", "end"]
+    torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
