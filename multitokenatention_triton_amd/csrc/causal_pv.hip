@@ -24,17 +24,26 @@ typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
 
 constexpr int P_NT = 512;  // 8 wavefronts
 constexpr int P_BQ = 256;  // query rows per workgroup
-constexpr int P_BK = 64;   // keys per iteration
+#ifndef MTA_PV_OCC
+#define MTA_PV_OCC 2
+#endif
+#ifndef MTA_PV_BK
+#define MTA_PV_BK 128
+#endif
+constexpr int P_BK = MTA_PV_BK;  // keys per iteration: each lane reads P_BK/4 contiguous bytes of its row per
+                                 // iteration, back to back, so that DRAM pages are used in long runs
+constexpr int P_KS = P_BK / 32;  // 32-key contraction steps per iteration
 
 template <typename T, int D>
-__global__ __launch_bounds__(P_NT, 2) void causal_pv_kernel(const T *__restrict__ P, const T *__restrict__ V,
+__global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__restrict__ P, const T *__restrict__ V,
                                                            T *__restrict__ O, int S, int causal, int nqb)
 {
     constexpr int CPR = D / 8;               // 16-byte chunks per V row
     constexpr int TILE = P_BK * D;           // elements per V block
     constexpr int ROUNDS = (TILE / 8 + P_NT - 1) / P_NT;
     constexpr int DB = D / 16;
-    __shared__ __align__(16) T Vt[2 * TILE];
+    extern __shared__ __align__(16) unsigned char pv_smem[];
+    T *Vt = reinterpret_cast<T *>(pv_smem);  // [2][TILE]
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, ln = lane & 15, kg = lane >> 4;
@@ -68,11 +77,11 @@ __global__ __launch_bounds__(P_NT, 2) void causal_pv_kernel(const T *__restrict_
     }
     // P^T fragments of key block j: slots t = 0..7 of k-step ks are keys j*64 + 32ks + 8kg + t; out-of-range
     // vectors re-read the row start, the values are masked when used
-    auto load_p = [&](int j, frag8<T> (&pf)[2][2]) {
+    auto load_p = [&](int j, frag8<T> (&pf)[2][P_KS]) {
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
+            for (int ks = 0; ks < P_KS; ++ks) {
                 const int key = j * P_BK + ks * 32 + kg * 8;
                 const bool ok = key < S && !(causal && key > prow[rb]);
                 pf[rb][ks] = *reinterpret_cast<const frag8<T> *>(prow_ptr[rb] + (ok ? j * P_BK + ks * 32 : -kg * 8));
@@ -82,7 +91,8 @@ __global__ __launch_bounds__(P_NT, 2) void causal_pv_kernel(const T *__restrict_
     const int q_last = (q0 + P_BQ - 1 < S - 1) ? q0 + P_BQ - 1 : S - 1;
     const int j_end = causal ? q_last / P_BK : (S - 1) / P_BK;
     issue_v(0, 0);
-    frag8<T> pcur[2][2], pnext[2][2];
+    // P fragments are fetched one key block ahead
+    frag8<T> pcur[2][P_KS], pnext[2][P_KS];
     load_p(0, pcur);
 
     f32x4 oacc[2][DB];
@@ -93,18 +103,18 @@ __global__ __launch_bounds__(P_NT, 2) void causal_pv_kernel(const T *__restrict_
 
     int buf = 0;
     for (int j = 0; j <= j_end; ++j, buf ^= 1) {
-        __builtin_amdgcn_s_waitcnt(0);  // V block j (and the P fragments) have arrived
+        __builtin_amdgcn_s_waitcnt(0);  // V block j and the P fragments have arrived
         __syncthreads();                // for every wavefront; reads of the other buffer are finished
         if (j < j_end) {
             issue_v(j + 1, buf ^ 1);
             load_p(j + 1, pnext);
         }
         // mask the fragments of this block: keys beyond the row (causal) or the sequence count as 0
-        frag8<T> pf[2][2];
+        frag8<T> pf[2][P_KS];
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
+            for (int ks = 0; ks < P_KS; ++ks) {
                 const int key0 = j * P_BK + ks * 32 + kg * 8;
                 pf[rb][ks] = pcur[rb][ks];
                 const int lim = causal ? (prow[rb] < S - 1 ? prow[rb] : S - 1) : S - 1;
@@ -116,7 +126,7 @@ __global__ __launch_bounds__(P_NT, 2) void causal_pv_kernel(const T *__restrict_
             }
         const T *Vb = Vt + buf * TILE;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
+        for (int ks = 0; ks < P_KS; ++ks) {
             const int key_a = ks * 32 + kg * 8 + (ln >> 2);  // slots 0..3: keys 8kg+(0..3); slots 4..7: +4
             const int key_b = key_a + 4;
 #pragma unroll
@@ -136,7 +146,7 @@ __global__ __launch_bounds__(P_NT, 2) void causal_pv_kernel(const T *__restrict_
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) pcur[rb][ks] = pnext[rb][ks];
+            for (int ks = 0; ks < P_KS; ++ks) pcur[rb][ks] = pnext[rb][ks];
     }
 
 #pragma unroll
@@ -157,8 +167,13 @@ int launch(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t 
 {
     const int nqb = (int)((S + P_BQ - 1) / P_BQ);
     dim3 grid((unsigned)nqb, (unsigned)(B * H));
-    hipLaunchKernelGGL((causal_pv_kernel<T, D>), grid, dim3(P_NT), 0, st, (const T *)p, (const T *)v, (T *)o, (int)S, causal,
-                       nqb);
+    const size_t lds = sizeof(T) * 2 * (size_t)P_BK * D;
+    auto kern = causal_pv_kernel<T, D>;
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(P_NT), lds, st, (const T *)p, (const T *)v, (T *)o, (int)S, causal, nqb);
     return launch_status();
 }
 }  // namespace

@@ -294,12 +294,14 @@ typedef const __attribute__((address_space(1))) void glb_void_t;
 typedef short v4s_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
 
-constexpr int F_NT = 512;  // 8 wavefronts
-constexpr int F_SR = 256;  // score-tile rows
+// The workgroup has NW wavefronts and owns 32*NW score rows: 8 for the attention kernel (one workgroup per CU,
+// K and V blocks shared by 256 rows), 4 for the scores-only kernel (two workgroups per CU, which overlap each
+// other's barriers and memory latency).
 constexpr int F_BK = 64;   // keys per iteration
 constexpr int F_SLD = 88;  // score-tile row stride (elements): 44 dwords, conflict-free 16-byte reads over 16 rows
 
-template <int R, int SK> struct fused_geom {
+template <int R, int SK, int NW> struct fused_geom {
+    static constexpr int F_SR = 32 * NW;
     static constexpr int HR = (R - 1 + 7) & ~7;    // halo rows above the block (recomputed)
     static constexpr int HC = (SK - 1 + 7) & ~7;   // score columns kept from the previous key block
     static constexpr int BQ = F_SR - HR;           // output rows per workgroup
@@ -312,13 +314,14 @@ template <int R, int SK> struct fused_geom {
 // SCORES_ONLY: stop after the conv and write  conv(mask0(scale * Q K^T))  as an (S,S) plane per (batch, head)
 // (`O` is then the score tensor, V is unused).  Only q <= p is written when causal, plus +0 above the
 // diagonal when `fill_upper` is set.  The tile is staged through LDS so that stores are 128-byte row segments.
-template <typename T, int D, int R, int SK, bool SCORES_ONLY>
-__global__ __launch_bounds__(F_NT, 2) void conv_attn_fwd_mfma(const T *__restrict__ Q, const T *__restrict__ K,
+template <typename T, int D, int R, int SK, bool SCORES_ONLY, int NW>
+__global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__restrict__ Q, const T *__restrict__ K,
                                                              const T *__restrict__ V, const T *__restrict__ Wt,
                                                              T *__restrict__ O, int S, int causal, float scale, int H,
                                                              int nqb, int fill_upper)
 {
-    using G = fused_geom<R, SK>;
+    using G = fused_geom<R, SK, NW>;
+    constexpr int F_NT = 64 * NW, F_SR = 32 * NW;
     constexpr int CPR = D / 8;                     // 16-byte chunks per K/V row
     constexpr int TILE = F_BK * D;                 // elements per K or V block
     constexpr int ROUNDS = TILE / 8 / F_NT;        // copy instructions per block per lane
@@ -680,12 +683,14 @@ template <typename T, int D, int R, int SK, bool SCORES_ONLY>
 int launch_mfma(const void *q, const void *k, const void *v, const void *w, void *o, int64_t B, int64_t H, int64_t S,
                 int causal, float scale, int fill_upper, hipStream_t st)
 {
-    using G = fused_geom<R, SK>;
+    constexpr int NW = SCORES_ONLY ? 4 : 8;
+    constexpr int F_NT = 64 * NW, F_SR = 32 * NW;
+    using G = fused_geom<R, SK, NW>;
     static_assert(G::fits, "conv window exceeds the 32-key MFMA contraction");
     const int nqb = (int)((S + G::BQ - 1) / G::BQ);
     const size_t vt_elems = SCORES_ONLY ? (size_t)F_SR * (F_BK + 8) : (size_t)2 * F_BK * D;
     const size_t lds = sizeof(T) * ((size_t)2 * F_BK * D + vt_elems + (size_t)F_SR * F_SLD + (size_t)R * G::WZ_LD);
-    auto kern = conv_attn_fwd_mfma<T, D, R, SK, SCORES_ONLY>;
+    auto kern = conv_attn_fwd_mfma<T, D, R, SK, SCORES_ONLY, NW>;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
     dim3 grid((unsigned)nqb, (unsigned)(B * H));
