@@ -41,6 +41,34 @@ def score_pass_bytes(b, h, s, esize):
     return b * h * (tri(s) + s * s) * esize
 
 
+def stage_model(name, b, h, s, d, r=6, sk=11, esize=2):
+    """Algorithmic HBM bytes and useful matrix flops of one stage of the forward at (B,H,S,D).
+
+    A stage reads what it needs of the lower triangle and writes what its consumer reads:
+      qk_conv          reads q,k; writes the lower triangle of the scores (QK^T, scale and conv fused)
+      mix_softmax_mix  reads the lower triangle, writes the lower triangle (P V below never reads above it)
+      pv               reads the lower triangle of P and V, writes O
+      conv_pre / mix_* / softmax / conv_post (unfused route) read the triangle and write the full tensor
+      qk, pv_gemm      library GEMMs over the full square
+    """
+    t, full, qkv = b * h * tri(s) * esize, b * h * s * s * esize, b * h * s * d * esize
+    if name == "qk_conv":
+        return 2 * qkv + t, 2 * b * h * tri(s) * d + 2 * r * sk * b * h * tri(s)
+    if name == "mix_softmax_mix":
+        return 2 * t, 0
+    if name == "pv":
+        return t + 2 * qkv, 2 * b * h * tri(s) * d
+    if name in ("qk", "pv_gemm"):
+        return 2 * qkv + full, 2 * b * h * s * s * d
+    return t + full, 0
+
+
+# HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at the benchmark shape
+# (profiles/mta_forward_c4_hbm_traffic.txt); FETCH_SIZE is scaled by 2.0, the factor a plain 1 GiB
+# device copy shows for it on this machine, WRITE_SIZE by 1.0.
+MEASURED_TRAFFIC_BYTES = {}
+
+
 def build_c4(torch, mta, O, device, b=2, h=16, s=4096, d=128, dtype=None, nsets=3):
     dtype = dtype or torch.bfloat16
     g = torch.Generator().manual_seed(125)
@@ -212,10 +240,16 @@ def main():
     with torch.no_grad():
         ms = time_steps(torch, lambda i: mod(*sets[i], None, None), len(sets), args.warmup, args.steps)
         stages = stage_breakdown(torch, mod, sets, max(3, min(args.steps, 10)))
-        hip_stages = {k: v for k, v in stages.items() if k not in ("qk", "pv")}
+        ran_own_pv = "qk" not in stages  # the fused route ends in mta_causal_pv_fwd, the unfused one in a library GEMM
+        hip_stages = {k: v for k, v in stages.items() if k != "qk" and (k != "pv" or ran_own_pv)}
         dom = max(hip_stages, key=hip_stages.get)
-        dom_bytes = score_pass_bytes(b, h, s, 2)
+        dom_bytes, dom_flops = stage_model(dom, b, h, s, d)
         achieved = dom_bytes / hip_stages[dom] / 1e6
+        per_stage = {}
+        for k, v in stages.items():
+            by, fl = stage_model(k if (k != "pv" or ran_own_pv) else "pv_gemm", b, h, s, d)
+            per_stage[k] = {"ms": v, "algorithmic_bytes": by, "GBps": by / v / 1e6, "frac_hbm_peak": by / v / 1e6 / HBM_PEAK_GBS,
+                            "useful_TFLOPs": fl / v / 1e9}
         kernels = {} if args.no_extras else bench_kernels(torch, mta, O, device, args.steps, args.warmup)
 
     result = {
@@ -226,9 +260,11 @@ def main():
                                "identity post-softmax conv, head-mix groups of 4 (BASELINE configs[3])",
                    "global_batch": b, "seq_len": s},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes": dom_bytes,
-                     "avg_kernel_ms": hip_stages[dom]},
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(dom),
+                     "algorithmic_bytes": dom_bytes, "avg_kernel_ms": hip_stages[dom],
+                     "useful_matrix_TFLOPs": dom_flops / hip_stages[dom] / 1e9},
         "stages_ms": stages,
+        "stages": per_stage,
         "kernels": kernels,
     }
     if not args.no_cpu_baseline:

@@ -36,7 +36,8 @@ constexpr int P_KS = P_BK / 32;  // 32-key contraction steps per iteration
 
 template <typename T, int D>
 __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__restrict__ P, const T *__restrict__ V,
-                                                           T *__restrict__ O, int S, int causal, int nqb)
+                                                           T *__restrict__ O, int S, int causal, int nqb, int64_t total_wg,
+                                                           int64_t per_xcd)
 {
     constexpr int CPR = D / 8;               // 16-byte chunks per V row
     constexpr int TILE = P_BK * D;           // elements per V block
@@ -47,8 +48,12 @@ __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, ln = lane & 15, kg = lane >> 4;
-    const int qb = nqb - 1 - (int)blockIdx.x;  // longest blocks first
-    const int64_t bh = blockIdx.y;
+    // XCD-aware order: XCD x (workgroup id % 8) takes the x-th eighth of the (batch*head, query block) list, so
+    // the workgroups that share one head's V run on one L2; within a head the longest query blocks come first
+    const int64_t lid = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (lid >= total_wg) return;
+    const int qb = nqb - 1 - (int)(lid % nqb);
+    const int64_t bh = lid / nqb;
     const int q0 = qb * P_BQ;
     const T *Pp = P + bh * (int64_t)S * S;
     const T *Vp = V + bh * (int64_t)S * D;
@@ -166,14 +171,17 @@ template <typename T, int D>
 int launch(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int causal, hipStream_t st)
 {
     const int nqb = (int)((S + P_BQ - 1) / P_BQ);
-    dim3 grid((unsigned)nqb, (unsigned)(B * H));
+    const int64_t total_wg = B * H * nqb, per_xcd = (total_wg + 7) / 8;
+    if (per_xcd * 8 > 0x7fffffffLL) return MTA_ERR_SHAPE;
+    dim3 grid((unsigned)(per_xcd * 8));
     const size_t lds = sizeof(T) * 2 * (size_t)P_BK * D;
     auto kern = causal_pv_kernel<T, D>;
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
     }
-    hipLaunchKernelGGL(kern, grid, dim3(P_NT), lds, st, (const T *)p, (const T *)v, (T *)o, (int)S, causal, nqb);
+    hipLaunchKernelGGL(kern, grid, dim3(P_NT), lds, st, (const T *)p, (const T *)v, (T *)o, (int)S, causal, nqb, total_wg,
+                       per_xcd);
     return launch_status();
 }
 }  // namespace

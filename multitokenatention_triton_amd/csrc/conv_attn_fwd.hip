@@ -318,7 +318,7 @@ template <typename T, int D, int R, int SK, bool SCORES_ONLY, int NW>
 __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__restrict__ Q, const T *__restrict__ K,
                                                              const T *__restrict__ V, const T *__restrict__ Wt,
                                                              T *__restrict__ O, int S, int causal, float scale, int H,
-                                                             int nqb, int fill_upper)
+                                                             int nqb, int fill_upper, int64_t total_wg, int64_t per_xcd)
 {
     using G = fused_geom<R, SK, NW>;
     constexpr int F_NT = 64 * NW, F_SR = 32 * NW;
@@ -339,8 +339,13 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, ln = lane & 15, kg = lane >> 4;
-    const int qb = nqb - 1 - (int)blockIdx.x;      // longest blocks first
-    const int64_t bh = blockIdx.y;
+    // XCD-aware order: workgroup ids are dealt round-robin to the 8 XCDs, so XCD x takes the x-th eighth of the
+    // (batch*head, query block) list: the workgroups sharing one head's K and V run on one L2.  Within a head
+    // the longest (last) query blocks come first.
+    const int64_t lid = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (lid >= total_wg) return;
+    const int qb = nqb - 1 - (int)(lid % nqb);
+    const int64_t bh = lid / nqb;
     const int head = (int)(bh % H);
     const int q0 = qb * G::BQ;
     const T *Qp = Q + bh * (int64_t)S * D;
@@ -693,9 +698,11 @@ int launch_mfma(const void *q, const void *k, const void *v, const void *w, void
     auto kern = conv_attn_fwd_mfma<T, D, R, SK, SCORES_ONLY, NW>;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
-    dim3 grid((unsigned)nqb, (unsigned)(B * H));
+    const int64_t total_wg = B * H * nqb, per_xcd = (total_wg + 7) / 8;
+    if (per_xcd * 8 > 0x7fffffffLL) return MTA_ERR_SHAPE;
+    dim3 grid((unsigned)(per_xcd * 8));
     hipLaunchKernelGGL(kern, grid, dim3(F_NT), lds, st, (const T *)q, (const T *)k, (const T *)v, (const T *)w, (T *)o,
-                       (int)S, causal, scale, (int)H, nqb, fill_upper);
+                       (int)S, causal, scale, (int)H, nqb, fill_upper, total_wg, per_xcd);
     return launch_status();
 }
 
