@@ -169,6 +169,9 @@ int dispatch_valu(const void *x, const void *w, void *y, int64_t N, int64_t C, i
 #ifndef MTA_CONV_WAVES_PER_SIMD
 #define MTA_CONV_WAVES_PER_SIMD 2  // register budget: 256 VGPRs
 #endif
+#ifndef MTA_CONV_MFMA32
+#define MTA_CONV_MFMA32 1          // 1: 32x32x16 MFMAs (fewer LDS operand bytes per output), 0: 16x16x32
+#endif
 #ifndef MTA_CONV_WG_PER_CU
 #define MTA_CONV_WG_PER_CU 6       // LDS budget: two 11.6 KB strip buffers per single-wavefront workgroup
 #endif
@@ -182,6 +185,7 @@ template <int R, int S> struct mfma_geom {
     static constexpr int HL = (PADW + 7) & ~7;             // left halo, rounded so 16-byte loads stay aligned
     static constexpr int SHIFT = HL - PADW;                // first tap's offset inside a block's 32-key window
     static constexpr bool fits = SHIFT + 16 + S - 1 <= 32;
+    static constexpr bool fits32 = SHIFT + 32 + S - 1 <= 48;  // 3 chunks of 16 keys per 32-output window (32x32x16 MFMA)
     static constexpr int TW = M_TN - 16 + 32;              // staged columns
     static constexpr int LD = TW + ((24 - TW % 16) % 16);  // row stride = 8 (mod 16) elements: conflict-free b128 reads
     static constexpr int ROWS = M_TM + R - 1;
@@ -258,7 +262,9 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     static_assert(SPR == VPR + 1, "one padding slot per row");
     // weights of the current channel, each kernel row zero-padded on both sides so that the
     // Toeplitz fragments can be gathered without range checks
-    constexpr int WZ_OFF = G::SHIFT + 16, WZ_LD = WZ_OFF + 32;
+    constexpr bool M32 = MTA_CONV_MFMA32 && G::fits32;
+    constexpr int NCH = 3;  // 16-key chunks per 32-output window (M32)
+    constexpr int WZ_OFF = G::SHIFT + (M32 ? 32 : 16), WZ_LD = WZ_OFF + (M32 ? 16 * NCH : 32);
     constexpr int BUF = STAGE_IT * M_WT * VEC;  // elements per LDS strip buffer
     __shared__ __align__(16) T tiles[2 * BUF];  // double buffer: strip n is computed while strip n+1 lands
     __shared__ T wz[R * WZ_LD];
@@ -275,8 +281,8 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     const int64_t step = nw;
     if (c0 >= total || first >= last) return;
 
-    const int lane = threadIdx.x, ln = lane & 15, kg = lane >> 4;
-    frag8<T> tz[R];
+    const int lane = threadIdx.x, ln = M32 ? (lane & 31) : (lane & 15), kg = M32 ? (lane >> 5) : (lane >> 4);
+    frag8<T> tz[R][M32 ? NCH : 1];
     int cur_channel = -1;
 
     // per-lane geometry of the staging copies, fixed for the whole kernel: slot it*64+lane is row srow,
@@ -381,16 +387,77 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
         }
         __syncthreads();  // LDS stores above are visible (single wavefront: a wait on the LDS counter)
 
-        if (channel != cur_channel) {  // Toeplitz fragments T_i^T: row m = ln, slots k = 8*kg + t, tap j = k-SHIFT-m
+        if (channel != cur_channel) {  // Toeplitz fragments T_i^T for this lane's accumulator row
             cur_channel = channel;
+            if constexpr (M32) {
+                // accumulator register v of lane-half kg is row m = 8*(v/4) + 4*kg + v%4; giving that row the output
+                // column 16*(v/8) + 8*kg + v%8 makes every 8 registers of a lane 8 consecutive keys
+                const int m = ln, qm = 16 * (m >> 4) + 8 * ((m >> 2) & 1) + 4 * ((m >> 3) & 1) + (m & 3);
 #pragma unroll
-            for (int i = 0; i < R; ++i) {
-                const T *src = wz + i * WZ_LD + WZ_OFF + kg * 8 - G::SHIFT - ln;
+                for (int i = 0; i < R; ++i)
 #pragma unroll
-                for (int t = 0; t < 8; ++t) tz[i].v[t] = src[t];
+                    for (int ch = 0; ch < NCH; ++ch) {
+                        const T *src = wz + i * WZ_LD + WZ_OFF + ch * 16 + kg * 8 - G::SHIFT - qm;  // tap j = k-SHIFT-q
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) tz[i][ch].v[t] = src[t];
+                        __builtin_amdgcn_sched_barrier(0);  // keep the gathers of one fragment together (register pressure)
+                    }
+            } else {
+#pragma unroll
+                for (int i = 0; i < R; ++i) {  // row m = ln, slots k = 8*kg + t, tap j = k-SHIFT-m
+                    const T *src = wz + i * WZ_LD + WZ_OFF + kg * 8 - G::SHIFT - ln;
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) tz[i][0].v[t] = src[t];
+                }
             }
         }
 
+        if constexpr (M32) {
+            // ---- 32 rows x 4 sub-tiles of 32 keys on 32x32x16 MFMAs, two sub-tiles at a time.  Per kernel row
+            // the 5 chunks of this lane's staged row that the pair needs are read once (the windows overlap).
+            const int prow = p0 + ln;
+#pragma unroll
+            for (int pair = 0; pair < M_TN / 64; ++pair) {
+                f32x16 acc[2];
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[s2][v] = 0.0f;
+                if (interior || !causal || q0 + pair * 64 <= p0 + M_TM - 1) {  // else: both wholly above the diagonal
+#pragma unroll
+                    for (int i = 0; i < R; ++i) {
+                        const T *rowp = tile + (ln + i) * LD + pair * 64 + kg * 8;
+                        frag8<T> xf[NCH + 2];
+#pragma unroll
+                        for (int cc = 0; cc < NCH + 2; ++cc) xf[cc] = *reinterpret_cast<const frag8<T> *>(rowp + cc * 16);
+#pragma unroll
+                        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+                            for (int ch = 0; ch < NCH; ++ch) mma32(acc[s2], tz[i][ch], xf[s2 * 2 + ch]);
+                    }
+                }
+                // results back into the strip's own LDS rows: pair 0 overwrites columns 0..63, which pair 1 (reading
+                // columns 64..143) no longer needs
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+                    for (int a = 0; a < 2; ++a) {
+                        const int col = pair * 64 + s2 * 32 + a * 16 + kg * 8;
+                        const int q = q0 + col;
+                        uint32_t pk[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) pk[u] = pack2<T>(acc[s2][a * 8 + 2 * u], acc[s2][a * 8 + 2 * u + 1]);
+                        if (!interior && causal && q + 7 > prow) {
+#pragma unroll
+                            for (int u = 0; u < 4; ++u) {
+                                if (q + 2 * u > prow) pk[u] &= 0xffff0000u;
+                                if (q + 2 * u + 1 > prow) pk[u] &= 0x0000ffffu;
+                            }
+                        }
+                        *reinterpret_cast<uint4 *>(tile + ln * LD + col) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+                    }
+            }
+        } else {
         // ---- 2 row blocks x 8 column blocks of 16x16 outputs; results of a row block go back into its
         // own (no longer needed) LDS rows: lane (row ln, group kg) holds keys 4*kg..4*kg+3 of each block
 #pragma unroll
@@ -402,7 +469,7 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
                 if (!interior && causal && q0 + cb * 16 > p0 + rb * 16 + 15) continue;  // block wholly above the diagonal: +0
 #pragma unroll
                 for (int i = 0; i < R; ++i)
-                    mma16(acc[cb], tz[i],
+                    mma16(acc[cb], tz[i][0],
                           *reinterpret_cast<const frag8<T> *>(tile + (rb * 16 + ln + i) * LD + cb * 16 + kg * 8));
             }
             const int prow = p0 + rb * 16 + ln;
@@ -416,6 +483,7 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
                 }
                 *reinterpret_cast<quad *>(tile + (rb * 16 + ln) * LD + cb * 16 + kg * 4) = out;
             }
+        }
         }
         __syncthreads();
 
