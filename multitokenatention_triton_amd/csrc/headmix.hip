@@ -13,12 +13,47 @@
 namespace {
 using namespace mta;
 
-constexpr int NT = 256;
+#ifndef MTA_HM_THREADS
+#define MTA_HM_THREADS 256
+#endif
+constexpr int NT = MTA_HM_THREADS;
+#ifndef MTA_HM_NT
+#define MTA_HM_NT 1
+#endif
+#ifndef MTA_HM_NTL
+#define MTA_HM_NTL 1
+#endif
+#ifndef MTA_HM_WREG
+#define MTA_HM_WREG 0
+#endif
 #ifndef MTA_HM_ROWS
-#define MTA_HM_ROWS 4
+#define MTA_HM_ROWS 1
 #endif
 
 template <typename T, int VEC> struct alignas(sizeof(T) * VEC) vecN { T v[VEC]; };
+
+// outputs are written once and not read again by this kernel: store them as streaming (non-temporal) data
+template <typename V> __device__ __forceinline__ V load_stream(const V *src)
+{
+#if MTA_HM_NTL
+    if constexpr (sizeof(V) == 16) {
+        typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+        return __builtin_bit_cast(V, __builtin_nontemporal_load(reinterpret_cast<const u4 *>(src)));
+    }
+#endif
+    return *src;
+}
+template <typename V> __device__ __forceinline__ void store_stream(V *dst, const V &v)
+{
+#if MTA_HM_NT
+    if constexpr (sizeof(V) == 16) {
+        typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+        __builtin_nontemporal_store(__builtin_bit_cast(u4, v), reinterpret_cast<u4 *>(dst));
+        return;
+    }
+#endif
+    *dst = v;
+}
 
 // G heads mixed inside one lane, G known at compile time.  A workgroup covers ROWS consecutive
 // query rows of one key chunk, so a lane has ROWS*G independent 16-byte loads in flight.
@@ -27,7 +62,12 @@ __global__ __launch_bounds__(NT) void headmix_fixed(const T *__restrict__ x, con
                                                     T *__restrict__ y, int C, int P, int Q, int causal,
                                                     float fill, int w_dtype, int qchunks, int pblocks)
 {
-    __shared__ float wsm[G * G];
+#if MTA_HM_WREG
+    constexpr bool WREG = G <= 8;
+#else
+    constexpr bool WREG = false;
+#endif
+    __shared__ float wsm[WREG ? 1 : G * G];
     const int tid = threadIdx.x;
     const int groups = C / G;
     int64_t b = blockIdx.x;
@@ -50,7 +90,7 @@ __global__ __launch_bounds__(NT) void headmix_fixed(const T *__restrict__ x, con
             for (int r = 0; r < ROWS; ++r)
                 if (p0 + r < P) {
 #pragma unroll
-                    for (int o = 0; o < G; ++o) *reinterpret_cast<V *>(y + base0 + (int64_t)(p0 + r) * Q + o * plane) = fillv;
+                    for (int o = 0; o < G; ++o) store_stream(reinterpret_cast<V *>(y + base0 + (int64_t)(p0 + r) * Q + o * plane), fillv);
                 }
         }
         return;
@@ -64,11 +104,17 @@ __global__ __launch_bounds__(NT) void headmix_fixed(const T *__restrict__ x, con
         const bool live = q < Q && !(causal && q > p);
         const int64_t lb = base0 + (int64_t)p * Q - (live ? 0 : q);
 #pragma unroll
-        for (int i = 0; i < G; ++i) xin[r][i] = *reinterpret_cast<const V *>(x + lb + i * plane);
+        for (int i = 0; i < G; ++i) xin[r][i] = load_stream(reinterpret_cast<const V *>(x + lb + i * plane));
     }
-    for (int t = tid; t < G * G; t += NT)
-        wsm[t] = load_any(w, w_dtype, (int64_t)(g * G + t / G) * C + g * G + t % G);
-    __syncthreads();
+    float wr[WREG ? G * G : 1];
+    if constexpr (WREG) {  // wave-uniform addresses: the weights arrive through the scalar unit
+#pragma unroll
+        for (int t = 0; t < G * G; ++t) wr[t] = load_any(w, w_dtype, (int64_t)(g * G + t / G) * C + g * G + t % G);
+    } else {
+        for (int t = tid; t < G * G; t += NT)
+            wsm[t] = load_any(w, w_dtype, (int64_t)(g * G + t / G) * C + g * G + t % G);
+        __syncthreads();
+    }
     if (q >= Q) return;
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
@@ -77,7 +123,7 @@ __global__ __launch_bounds__(NT) void headmix_fixed(const T *__restrict__ x, con
         const int64_t base = base0 + (int64_t)p * Q;
         if (causal && q > p) {
 #pragma unroll
-            for (int o = 0; o < G; ++o) *reinterpret_cast<V *>(y + base + o * plane) = fillv;
+            for (int o = 0; o < G; ++o) store_stream(reinterpret_cast<V *>(y + base + o * plane), fillv);
             continue;
         }
 #pragma unroll
@@ -87,14 +133,14 @@ __global__ __launch_bounds__(NT) void headmix_fixed(const T *__restrict__ x, con
             for (int u = 0; u < VEC; ++u) acc[u] = 0.0f;
 #pragma unroll
             for (int i = 0; i < G; ++i) {
-                const float wv = wsm[o * G + i];
+                const float wv = WREG ? wr[o * G + i] : wsm[o * G + i];
 #pragma unroll
                 for (int u = 0; u < VEC; ++u) acc[u] = fmaf(wv, to_float(xin[r][i].v[u]), acc[u]);
             }
             V out;
 #pragma unroll
             for (int u = 0; u < VEC; ++u) out.v[u] = (causal && q + u > p) ? fill_t : from_float<T>(acc[u]);
-            *reinterpret_cast<V *>(y + base + o * plane) = out;
+            store_stream(reinterpret_cast<V *>(y + base + o * plane), out);
         }
     }
 }
@@ -154,7 +200,7 @@ int launch(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t 
     MTA_HM_CASE(1, MTA_HM_ROWS)
     MTA_HM_CASE(2, MTA_HM_ROWS)
     MTA_HM_CASE(4, MTA_HM_ROWS)
-    MTA_HM_CASE(8, 2)
+    MTA_HM_CASE(8, MTA_HM_ROWS)
     MTA_HM_CASE(16, 1)
     MTA_HM_CASE(32, 1)
 #undef MTA_HM_CASE
