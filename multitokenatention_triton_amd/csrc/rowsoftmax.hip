@@ -17,6 +17,47 @@ using namespace mta;
 
 template <typename T, int VEC> struct alignas(sizeof(T) * VEC) vecN { T v[VEC]; };
 
+// a and b rounded to the I/O dtype (one packed convert for the 16-bit types)
+template <typename T> __device__ __forceinline__ void round_pair(float &a, float &b)
+{
+    if constexpr (sizeof(T) == 2) {
+        unpack2<T>(pack2<T>(a, b), a, b);
+    }
+}
+// VEC fp32 values -> a vector of the I/O dtype
+template <typename T, int VEC> __device__ __forceinline__ void pack_vec(const float (&f)[VEC], vecN<T, VEC> &out)
+{
+    if constexpr (sizeof(T) == 2 && VEC % 2 == 0) {
+        uint32_t r[VEC / 2];
+#pragma unroll
+        for (int u = 0; u < VEC / 2; ++u) r[u] = pack2<T>(f[2 * u], f[2 * u + 1]);
+        __builtin_memcpy(&out, r, sizeof(out));
+    } else {
+#pragma unroll
+        for (int u = 0; u < VEC; ++u) out.v[u] = from_float<T>(f[u]);
+    }
+}
+
+// the tensor is streamed: every element is read once and written once
+template <typename V> __device__ __forceinline__ V load_stream(const V *src)
+{
+    if constexpr (sizeof(V) == 16) {
+        typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+        return __builtin_bit_cast(V, __builtin_nontemporal_load(reinterpret_cast<const u4 *>(src)));
+    } else {
+        return *src;
+    }
+}
+template <typename V> __device__ __forceinline__ void store_stream(V *dst, const V &v)
+{
+    if constexpr (sizeof(V) == 16) {
+        typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+        __builtin_nontemporal_store(__builtin_bit_cast(u4, v), reinterpret_cast<u4 *>(dst));
+    } else {
+        *dst = v;
+    }
+}
+
 template <int NT> __device__ __forceinline__ float block_max(float v, float *red)
 {
 #pragma unroll
@@ -55,7 +96,7 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, c
 {
     __shared__ float w1s[G * G];
     __shared__ float w2s[G * G];
-    __shared__ float red[(NT / 64) * G];
+    __shared__ float red[2][(NT / 64) * G];  // [0] maxima, [1] sums: no barrier needed between the two uses
     const int tid = threadIdx.x;
     const int groups = C / G;
     int64_t b = blockIdx.x;
@@ -67,15 +108,20 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, c
     const int last = causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;  // last attended key
     using V = vecN<T, VEC>;
 
-    // All row loads are issued first, unconditionally (a lane beyond the attended keys re-reads the
-    // row start), so that they overlap each other and the weight fetch below.
+    // All row loads are issued first, unconditionally within a wavefront (a lane beyond the attended keys re-reads
+    // the row start), so that they overlap each other and the weight fetch below.  Pass k of wavefront w covers
+    // keys [(k*NT + 64w)*VEC, +64*VEC); a pass wholly beyond the attended keys (a wavefront-uniform condition) is
+    // skipped everywhere below: the arithmetic follows the triangle, not the square.
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    auto dead = [&](int k) { return (k * NT + wave * 64) * VEC > last; };
     V xin[NV][G];
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
+        if (dead(k)) continue;
         const int q = (k * NT + tid) * VEC;
         const int qs = (q <= last) ? q : 0;
 #pragma unroll
-        for (int i = 0; i < G; ++i) xin[k][i] = *reinterpret_cast<const V *>(x + base + i * plane + qs);
+        for (int i = 0; i < G; ++i) xin[k][i] = load_stream(reinterpret_cast<const V *>(x + base + i * plane + qs));
     }
     for (int t = tid; t < G * G; t += NT) {
         const int64_t widx = (int64_t)(g * G + t / G) * C + g * G + t % G;
@@ -87,6 +133,7 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, c
     float s[G][NV][VEC];
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
+        if (dead(k)) continue;
         const int q = (k * NT + tid) * VEC;
 #pragma unroll
         for (int o = 0; o < G; ++o) {
@@ -97,76 +144,116 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, c
                     acc = 0.0f;
 #pragma unroll
                     for (int i = 0; i < G; ++i) acc = fmaf(w1s[o * G + i], to_float(xin[k][i].v[u]), acc);
-                    acc = round_to<T>(acc);
                 } else {
                     acc = to_float(xin[k][o].v[u]);
                 }
-                s[o][k][u] = (q + u <= last) ? acc : -INFINITY;
+                s[o][k][u] = acc;
             }
+            if (w1) {
+                if constexpr (VEC % 2 == 0) {
+#pragma unroll
+                    for (int u = 0; u < VEC; u += 2) round_pair<T>(s[o][k][u], s[o][k][u + 1]);
+                } else {
+#pragma unroll
+                    for (int u = 0; u < VEC; ++u) s[o][k][u] = round_to<T>(s[o][k][u]);
+                }
+            }
+        }
+        if (q + VEC - 1 > last) {  // the vector that straddles the last attended key, and those beyond it
+#pragma unroll
+            for (int o = 0; o < G; ++o)
+#pragma unroll
+                for (int u = 0; u < VEC; ++u)
+                    if (q + u > last) s[o][k][u] = -INFINITY;
         }
     }
 
     // row maxima and sums of all G heads are reduced together: two barriers per reduction, not 2*G
     constexpr int NW = NT / 64;
-    const int wave = tid >> 6, lane = tid & 63;
     float m[G], inv[G];
 #pragma unroll
     for (int o = 0; o < G; ++o) {
         float v = -INFINITY;
 #pragma unroll
-        for (int k = 0; k < NV; ++k)
+        for (int k = 0; k < NV; ++k) {
+            if (dead(k)) continue;
 #pragma unroll
             for (int u = 0; u < VEC; ++u) v = fmaxf(v, s[o][k][u]);
+        }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-        if (lane == 0) red[wave * G + o] = v;
+        if (lane == 0) red[0][wave * G + o] = v;
     }
     __syncthreads();
 #pragma unroll
     for (int o = 0; o < G; ++o) {
-        float v = red[o];
+        float v = red[0][o];
 #pragma unroll
-        for (int i = 1; i < NW; ++i) v = fmaxf(v, red[i * G + o]);
+        for (int i = 1; i < NW; ++i) v = fmaxf(v, red[0][i * G + o]);
         m[o] = v;
     }
-    __syncthreads();
 #pragma unroll
     for (int o = 0; o < G; ++o) {
         float sum = 0.0f;
+        // exp(s - m) = exp2(s*log2(e) - m*log2(e)): one fused multiply-add and one v_exp per element (m is finite:
+        // the row's first key is always attended; s = -inf gives 0)
+        constexpr float LOG2E = 1.4426950408889634f;
+        const float mneg = -m[o] * LOG2E;
 #pragma unroll
-        for (int k = 0; k < NV; ++k)
+        for (int k = 0; k < NV; ++k) {
+            if (dead(k)) continue;
 #pragma unroll
             for (int u = 0; u < VEC; ++u) {
-                const float e = (s[o][k][u] == -INFINITY) ? 0.0f : __expf(s[o][k][u] - m[o]);
+                const float e = __builtin_amdgcn_exp2f(fmaf(s[o][k][u], LOG2E, mneg));
                 s[o][k][u] = e;
                 sum += e;
             }
+        }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
-        if (lane == 0) red[wave * G + o] = sum;
+        if (lane == 0) red[1][wave * G + o] = sum;
     }
     __syncthreads();
 #pragma unroll
     for (int o = 0; o < G; ++o) {
-        float v = red[o];
+        float v = red[1][o];
 #pragma unroll
-        for (int i = 1; i < NW; ++i) v += red[i * G + o];
+        for (int i = 1; i < NW; ++i) v += red[1][i * G + o];
         inv[o] = 1.0f / v;
     }
 #pragma unroll
     for (int o = 0; o < G; ++o)
 #pragma unroll
-        for (int k = 0; k < NV; ++k)
+        for (int k = 0; k < NV; ++k) {
+            if (dead(k)) continue;
 #pragma unroll
-            for (int u = 0; u < VEC; ++u) s[o][k][u] = round_to<T>(s[o][k][u] * inv[o]);
+            for (int u = 0; u < VEC; ++u) s[o][k][u] *= inv[o];
+            if constexpr (VEC % 2 == 0) {
+#pragma unroll
+                for (int u = 0; u < VEC; u += 2) round_pair<T>(s[o][k][u], s[o][k][u + 1]);
+            } else {
+#pragma unroll
+                for (int u = 0; u < VEC; ++u) s[o][k][u] = round_to<T>(s[o][k][u]);
+            }
+        }
 
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
         const int q = (k * NT + tid) * VEC;
+        if (dead(k)) {  // pass wholly above the diagonal: +0 only on request
+            if (fill_upper && q < Q) {
+                V z;
+#pragma unroll
+                for (int u = 0; u < VEC; ++u) z.v[u] = from_float<T>(0.0f);
+#pragma unroll
+                for (int o = 0; o < G; ++o) store_stream(reinterpret_cast<V *>(y + base + o * plane + q), z);
+            }
+            continue;
+        }
         if (q >= Q || (!fill_upper && q > last)) continue;  // vectors wholly above the diagonal: +0 only on request
 #pragma unroll
         for (int o = 0; o < G; ++o) {
-            V out;
+            float of[VEC];
 #pragma unroll
             for (int u = 0; u < VEC; ++u) {
                 float acc;
@@ -177,9 +264,16 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, c
                 } else {
                     acc = s[o][k][u];
                 }
-                out.v[u] = from_float<T>((q + u <= last) ? acc : 0.0f);
+                of[u] = acc;
             }
-            *reinterpret_cast<V *>(y + base + o * plane + q) = out;
+            if (q + VEC - 1 > last) {
+#pragma unroll
+                for (int u = 0; u < VEC; ++u)
+                    if (q + u > last) of[u] = 0.0f;
+            }
+            V out;
+            pack_vec<T, VEC>(of, out);
+            store_stream(reinterpret_cast<V *>(y + base + o * plane + q), out);
         }
     }
 }
@@ -239,12 +333,11 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix_any(const T *__restrict__ 
     }
 }
 
-template <typename T, int G, int NV>
+template <typename T, int G, int NV, int NT = 256>
 int launch_fixed(const void *x, const void *w1, const void *w2, void *y, int64_t N, int64_t C, int64_t P,
                  int64_t Q, int causal, int w_dtype, int fill_upper, hipStream_t st)
 {
     constexpr int VEC = vec_of<T>::n;
-    constexpr int NT = 256;
     const int64_t blocks = N * (C / G) * P;
     hipLaunchKernelGGL((mix_softmax_mix<T, G, NV, VEC, NT>), dim3((unsigned)blocks), dim3(NT), 0, st, (const T *)x,
                        w1, w2, (T *)y, (int)C, (int)P, (int)Q, causal, w_dtype, fill_upper);
