@@ -4,7 +4,7 @@
 // uninitialised memory), which halves the traffic of the plain batched GEMM this replaces.
 // HBM-bound: the P triangle is streamed once, V blocks are re-read from L2.
 //
-// 8 wavefronts own 256 query rows; a wavefront owns two blocks of 16 rows.  O^T += V^T P^T on
+// MTA_PV_WAVES wavefronts own a block of 32 query rows each; a wavefront owns two blocks of 16 rows.  O^T += V^T P^T on
 // 16x16x32 MFMAs: lane (r = lane%16, g = lane/16) owns query row r of a block and supplies P^T
 // fragments straight from global memory (16 contiguous bytes = 8 keys of its row, loaded one key
 // block ahead), V blocks of 64 keys are copied global -> LDS asynchronously (double buffered,
@@ -22,10 +22,16 @@ typedef const __attribute__((address_space(1))) void glb_void_t;
 typedef short v4s_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
 
-constexpr int P_NT = 512;  // 8 wavefronts
-constexpr int P_BQ = 256;  // query rows per workgroup
+#ifndef MTA_PV_WAVES
+#define MTA_PV_WAVES 4
+#endif
+constexpr int P_NT = 64 * MTA_PV_WAVES;
+constexpr int P_BQ = 32 * MTA_PV_WAVES;  // query rows per block: 32 per wavefront
 #ifndef MTA_PV_OCC
 #define MTA_PV_OCC 2
+#endif
+#ifndef MTA_PV_NT_LOAD
+#define MTA_PV_NT_LOAD 1  // P is streamed: every element is read once
 #endif
 #ifndef MTA_PV_BK
 #define MTA_PV_BK 128
@@ -52,12 +58,20 @@ __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__
     // the workgroups that share one head's V run on one L2; within a head the longest query blocks come first
     const int64_t lid = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (lid >= total_wg) return;
-    const int qb = nqb - 1 - (int)(lid % nqb);
-    const int64_t bh = lid / nqb;
-    const int q0 = qb * P_BQ;
+    // A workgroup takes two blocks of query rows of one (batch, head): block nqb-1-pi and block pi.  With causal
+    // rows the first has the most keys and the second the fewest: every workgroup gets the same amount of work
+    // (the whole grid is resident at once, so the longest workgroup would otherwise set the kernel's duration).
+    const int npairs = (nqb + 1) / 2;
+    const int pi = (int)(lid % npairs);
+    const int64_t bh = lid / npairs;
     const T *Pp = P + bh * (int64_t)S * S;
     const T *Vp = V + bh * (int64_t)S * D;
     T *Op = O + bh * (int64_t)S * D;
+  for (int half = 0; half < 2; ++half) {
+    const int qb = half == 0 ? nqb - 1 - pi : pi;
+    if (half == 1 && qb == nqb - 1 - pi) break;  // odd number of blocks: the middle one is alone
+    const int q0 = qb * P_BQ;
+    if (half == 1) __syncthreads();  // the V buffers are reused: everybody has finished reading them
 
     auto issue_v = [&](int j, int buf) {
 #pragma unroll
@@ -89,7 +103,13 @@ __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__
             for (int ks = 0; ks < P_KS; ++ks) {
                 const int key = j * P_BK + ks * 32 + kg * 8;
                 const bool ok = key < S && !(causal && key > prow[rb]);
+#if MTA_PV_NT_LOAD
+                typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+                pf[rb][ks] = __builtin_bit_cast(frag8<T>, __builtin_nontemporal_load(reinterpret_cast<const u4 *>(
+                                                              prow_ptr[rb] + (ok ? j * P_BK + ks * 32 : -kg * 8))));
+#else
                 pf[rb][ks] = *reinterpret_cast<const frag8<T> *>(prow_ptr[rb] + (ok ? j * P_BK + ks * 32 : -kg * 8));
+#endif
             }
     };
 
@@ -165,13 +185,14 @@ __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__
             *reinterpret_cast<quad *>(Op + (int64_t)prow[rb] * D + db * 16 + kg * 4) = out;
         }
     }
+  }
 }
 
 template <typename T, int D>
 int launch(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int causal, hipStream_t st)
 {
     const int nqb = (int)((S + P_BQ - 1) / P_BQ);
-    const int64_t total_wg = B * H * nqb, per_xcd = (total_wg + 7) / 8;
+    const int64_t total_wg = B * H * ((nqb + 1) / 2), per_xcd = (total_wg + 7) / 8;
     if (per_xcd * 8 > 0x7fffffffLL) return MTA_ERR_SHAPE;
     dim3 grid((unsigned)(per_xcd * 8));
     const size_t lds = sizeof(T) * 2 * (size_t)P_BK * D;
