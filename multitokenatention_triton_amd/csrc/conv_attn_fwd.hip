@@ -21,6 +21,8 @@
 // roundup(Sk-1, 8) score columns of the previous block stay in LDS, and the conv /
 // softmax / PV of a block lag the scores by the right-hand pad so that every tap is
 // already there.  One extra leading key block (mostly out-of-range keys) primes that halo.
+#include <algorithm>
+
 #include "common.hpp"
 #include "mfma.hpp"
 
@@ -298,6 +300,9 @@ typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
 // K and V blocks shared by 256 rows), 4 for the scores-only kernel (two workgroups per CU, which overlap each
 // other's barriers and memory latency).
 constexpr int F_BK = 64;   // keys per iteration
+#ifndef MTA_QK_CHUNK
+#define MTA_QK_CHUNK 22    // key blocks per work item of the scores-only kernel
+#endif
 constexpr int F_SLD = 88;  // score-tile row stride (elements): 44 dwords, conflict-free 16-byte reads over 16 rows
 
 template <int R, int SK, int NW> struct fused_geom {
@@ -318,7 +323,8 @@ template <typename T, int D, int R, int SK, bool SCORES_ONLY, int NW>
 __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__restrict__ Q, const T *__restrict__ K,
                                                              const T *__restrict__ V, const T *__restrict__ Wt,
                                                              T *__restrict__ O, int S, int causal, float scale, int H,
-                                                             int nqb, int fill_upper, int64_t total_wg, int64_t per_xcd)
+                                                             int nqb, int fill_upper, int64_t total_wg, int64_t per_xcd,
+                                                             int jc_len, int items_per_bh)
 {
     using G = fused_geom<R, SK, NW>;
     constexpr int F_NT = 64 * NW, F_SR = 32 * NW;
@@ -344,8 +350,19 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
     // the longest (last) query blocks come first.
     const int64_t lid = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (lid >= total_wg) return;
-    const int qb = nqb - 1 - (int)(lid % nqb);
-    const int64_t bh = lid / nqb;
+    // Work item = (batch*head, query block, chunk of jc_len key blocks).  The scores-only kernel splits the key
+    // range of a query block (its output columns are independent; a chunk starts one key block early to rebuild
+    // the retained halo columns), so that items are short and equal and the grid runs in several even rounds;
+    // the attention kernel accumulates over all keys and gets jc_len = all of them.
+    const int64_t bh = lid / items_per_bh;
+    int item = (int)(lid % items_per_bh), qb = nqb - 1, jc = 0;
+    for (; qb > 0; --qb) {  // longest query blocks first
+        const int ql = (qb * G::BQ + G::BQ - 1 < S - 1) ? qb * G::BQ + G::BQ - 1 : S - 1;
+        const int nch = ((causal ? ql / F_BK : (S - 1) / F_BK) + jc_len) / jc_len;
+        if (item < nch) break;
+        item -= nch;
+    }
+    jc = item;
     const int head = (int)(bh % H);
     const int q0 = qb * G::BQ;
     const T *Qp = Q + bh * (int64_t)S * D;
@@ -386,8 +403,11 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
     };
 
     const int q_last = (q0 + G::BQ - 1 < S - 1) ? q0 + G::BQ - 1 : S - 1;
-    const int j_end = causal ? q_last / F_BK : (S - 1) / F_BK;
-    constexpr int j_start = G::PWR > 0 ? -1 : 0;
+    const int j_last = causal ? q_last / F_BK : (S - 1) / F_BK;  // last key block of the query block
+    const int j_lo = jc * jc_len;                                 // first key block whose outputs this item produces
+    const int j_end = (j_lo + jc_len - 1 < j_last) ? j_lo + jc_len - 1 : j_last;
+    // one key block earlier only fills the retained score columns (before the first one: the right pad, if any)
+    const int j_start = j_lo > 0 ? j_lo - 1 : (G::PWR > 0 ? -1 : 0);
     issue_kv(j_start, 0);
 
     // zero the score tile once (columns past HC+BK are read by the last window but never written)
@@ -510,7 +530,7 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
             }
         }
         __syncthreads();
-        if (j < 0) continue;
+        if (j < j_lo) continue;
 
         // score fragments of block blk = rb*NCB+cb: rows trow-(R-1)+i, the block's 32-key window
         auto load_xf = [&](int blk, frag8<T> (&dst)[R]) {
@@ -649,7 +669,7 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
 
     if constexpr (SCORES_ONLY) {
         // +0 for the key blocks to the right of the last one visited (all above the diagonal)
-        if (causal && fill_upper) {
+        if (causal && fill_upper && j_end == j_last) {
             pack16<T> z;
 #pragma unroll
             for (int u = 0; u < 8; ++u) z.v[u] = from_float<T>(0.0f);
@@ -698,11 +718,18 @@ int launch_mfma(const void *q, const void *k, const void *v, const void *w, void
     auto kern = conv_attn_fwd_mfma<T, D, R, SK, SCORES_ONLY, NW>;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
-    const int64_t total_wg = B * H * nqb, per_xcd = (total_wg + 7) / 8;
-    if (per_xcd * 8 > 0x7fffffffLL) return MTA_ERR_SHAPE;
+    // key blocks per work item: all of them for the attention kernel; MTA_QK_CHUNK for the scores-only kernel
+    const int jc_len = SCORES_ONLY ? MTA_QK_CHUNK : (int)((S + F_BK - 1) / F_BK) + 1;
+    int64_t items_per_bh = 0;
+    for (int qb = 0; qb < nqb; ++qb) {
+        const int64_t ql = std::min<int64_t>((int64_t)qb * G::BQ + G::BQ - 1, S - 1);
+        items_per_bh += ((causal ? ql / F_BK : (S - 1) / F_BK) + jc_len) / jc_len;
+    }
+    const int64_t total_wg = B * H * items_per_bh, per_xcd = (total_wg + 7) / 8;
+    if (per_xcd * 8 > 0x7fffffffLL || items_per_bh > 0x7fffffffLL) return MTA_ERR_SHAPE;
     dim3 grid((unsigned)(per_xcd * 8));
     hipLaunchKernelGGL(kern, grid, dim3(F_NT), lds, st, (const T *)q, (const T *)k, (const T *)v, (const T *)w, (T *)o,
-                       (int)S, causal, scale, (int)H, nqb, fill_upper, total_wg, per_xcd);
+                       (int)S, causal, scale, (int)H, nqb, fill_upper, total_wg, per_xcd, jc_len, (int)items_per_bh);
     return launch_status();
 }
 
