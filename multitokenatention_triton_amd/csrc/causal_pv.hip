@@ -34,7 +34,7 @@ constexpr int P_BQ = 32 * MTA_PV_WAVES;  // query rows per block: 32 per wavefro
 #define MTA_PV_NT_LOAD 1  // P is streamed: every element is read once
 #endif
 #ifndef MTA_PV_BK
-#define MTA_PV_BK 128
+#define MTA_PV_BK 64
 #endif
 constexpr int P_BK = MTA_PV_BK;  // keys per iteration: each lane reads P_BK/4 contiguous bytes of its row per
                                  // iteration, back to back, so that DRAM pages are used in long runs
