@@ -49,8 +49,11 @@ __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__
     constexpr int TILE = P_BK * D;           // elements per V block
     constexpr int ROUNDS = (TILE / 8 + P_NT - 1) / P_NT;
     constexpr int DB = D / 16;
-    extern __shared__ __align__(16) unsigned char pv_smem[];
-    T *Vt = reinterpret_cast<T *>(pv_smem);  // [2][TILE]
+    // Double buffer as two separate arrays, and a loop body instantiated once per array: the compiler then sees that
+    // the LDS reads of one block never touch the asynchronous copy in flight into the other.  With one array it
+    // cannot, and waits for the copy (and for every load issued before it) ahead of the first LDS read.
+    __shared__ __align__(16) T v_a[TILE];
+    __shared__ __align__(16) T v_b[TILE];
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, ln = lane & 15, kg = lane >> 4;
@@ -73,7 +76,7 @@ __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__
     const int q0 = qb * P_BQ;
     if (half == 1) __syncthreads();  // the V buffers are reused: everybody has finished reading them
 
-    auto issue_v = [&](int j, int buf) {
+    auto issue_v = [&](int j, T *dst) {
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r) {
             const int slot = r * P_NT + tid;
@@ -82,7 +85,7 @@ __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__
             int vr = j * P_BK + row;
             vr = vr >= S ? S - 1 : vr;
             __builtin_amdgcn_global_load_lds((glb_void_t *)(Vp + (int64_t)vr * D + c * 8),
-                                             (lds_void_t *)(Vt + buf * TILE + (r * P_NT + wave * 64) * 8), 16, 0, 0);
+                                             (lds_void_t *)(dst + (r * P_NT + wave * 64) * 8), 16, 0, 0);
         }
     };
 
@@ -115,10 +118,10 @@ __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__
 
     const int q_last = (q0 + P_BQ - 1 < S - 1) ? q0 + P_BQ - 1 : S - 1;
     const int j_end = causal ? q_last / P_BK : (S - 1) / P_BK;
-    issue_v(0, 0);
-    // P fragments are fetched one key block ahead
-    frag8<T> pcur[2][P_KS], pnext[2][P_KS];
-    load_p(0, pcur);
+    issue_v(0, v_a);
+    // P fragments are fetched one key block ahead, alternately into two register sets
+    frag8<T> p_a[2][P_KS], p_b[2][P_KS];
+    load_p(0, p_a);
 
     f32x4 oacc[2][DB];
 #pragma unroll
@@ -126,12 +129,11 @@ __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__
 #pragma unroll
         for (int db = 0; db < DB; ++db) oacc[rb][db] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    int buf = 0;
-    for (int j = 0; j <= j_end; ++j, buf ^= 1) {
+    auto step = [&](int j, const T *Vb, T *Vn, frag8<T> (&pcur)[2][P_KS], frag8<T> (&pnext)[2][P_KS]) __attribute__((always_inline)) {
         __builtin_amdgcn_s_waitcnt(0);  // V block j and the P fragments have arrived
         __syncthreads();                // for every wavefront; reads of the other buffer are finished
         if (j < j_end) {
-            issue_v(j + 1, buf ^ 1);
+            issue_v(j + 1, Vn);
             load_p(j + 1, pnext);
         }
         // mask the fragments of this block: keys beyond the row (causal) or the sequence count as 0
@@ -149,7 +151,6 @@ __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__
                         if (key0 + t > lim) pf[rb][ks].v[t] = from_float<T>(0.0f);
                 }
             }
-        const T *Vb = Vt + buf * TILE;
 #pragma unroll
         for (int ks = 0; ks < P_KS; ++ks) {
             const int key_a = ks * 32 + kg * 8 + (ln >> 2);  // slots 0..3: keys 8kg+(0..3); slots 4..7: +4
@@ -168,10 +169,12 @@ __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__
                 mma16(oacc[1][db], vf, pf[1][ks]);
             }
         }
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-            for (int ks = 0; ks < P_KS; ++ks) pcur[rb][ks] = pnext[rb][ks];
+    };
+    for (int j = 0;;) {
+        step(j, v_a, v_b, p_a, p_b);
+        if (++j > j_end) break;
+        step(j, v_b, v_a, p_b, p_a);
+        if (++j > j_end) break;
     }
 
 #pragma unroll
@@ -195,13 +198,8 @@ int launch(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t 
     const int64_t total_wg = B * H * ((nqb + 1) / 2), per_xcd = (total_wg + 7) / 8;
     if (per_xcd * 8 > 0x7fffffffLL) return MTA_ERR_SHAPE;
     dim3 grid((unsigned)(per_xcd * 8));
-    const size_t lds = sizeof(T) * 2 * (size_t)P_BK * D;
     auto kern = causal_pv_kernel<T, D>;
-    if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-    }
-    hipLaunchKernelGGL(kern, grid, dim3(P_NT), lds, st, (const T *)p, (const T *)v, (T *)o, (int)S, causal, nqb, total_wg,
+    hipLaunchKernelGGL(kern, grid, dim3(P_NT), 0, st, (const T *)p, (const T *)v, (T *)o, (int)S, causal, nqb, total_wg,
                        per_xcd);
     return launch_status();
 }
