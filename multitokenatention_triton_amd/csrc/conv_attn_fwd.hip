@@ -336,12 +336,16 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
     constexpr int NCB = F_BK / 16;                 // 16-key blocks per iteration
     static_assert(ROUNDS >= 1, "block smaller than one copy round");
 
-    extern __shared__ __align__(16) unsigned char smem_raw[];
-    T *Kt = reinterpret_cast<T *>(smem_raw);       // [2][TILE]
-    T *Vt = Kt + 2 * TILE;                         // [2][TILE]; SCORES_ONLY: output staging [F_SR][F_BK+8] instead
-    constexpr int VT_ELEMS = SCORES_ONLY ? F_SR * (F_BK + 8) : 2 * TILE;
-    T *Sc = Vt + VT_ELEMS;                         // [F_SR][F_SLD]
-    T *wz = Sc + F_SR * F_SLD;                     // [R][WZ_LD] zero-padded kernel rows
+    // Every buffer is an array of its own, and the key-block loop body is instantiated once per K/V buffer: the
+    // compiler then sees that LDS reads never touch the asynchronous copy in flight into the other buffer.  With one
+    // block of dynamic LDS it cannot, and waits for the copy ahead of the first LDS read that follows its issue.
+    __shared__ __align__(16) T Kt0[TILE];
+    __shared__ __align__(16) T Kt1[TILE];
+    __shared__ __align__(16) T Vt0[SCORES_ONLY ? 8 : TILE];
+    __shared__ __align__(16) T Vt1[SCORES_ONLY ? 8 : TILE];
+    __shared__ __align__(16) T stg[SCORES_ONLY ? F_SR * (F_BK + 8) : 8];  // output staging of the scores-only kernel
+    __shared__ __align__(16) T Sc[F_SR * F_SLD];                          // score tile
+    __shared__ __align__(16) T wz[R * G::WZ_LD];                          // zero-padded kernel rows
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, ln = lane & 15, kg = lane >> 4;
@@ -380,7 +384,7 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
         kv_row[r] = slot / CPR;
         kv_off[r] = kv_row[r] * D + ((slot % CPR) ^ (kv_row[r] & (CPR - 1))) * 8;
     }
-    auto issue_kv = [&](int j, int buf) {
+    auto issue_kv = [&](int j, T *Kdst, T *Vdst) {
         const int cb = j * F_BK + G::PWR;
         const bool inside = cb >= 0 && cb + F_BK <= S && j >= 0 && (j + 1) * F_BK <= S;  // no key needs clamping
 #pragma unroll
@@ -395,10 +399,10 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
                 voff = kv_off[r] + (vr - kv_row[r]) * D;
             }
             __builtin_amdgcn_global_load_lds((glb_void_t *)(Kp + koff),
-                                             (lds_void_t *)(Kt + buf * TILE + (r * F_NT + wave * 64) * 8), 16, 0, 0);
+                                             (lds_void_t *)(Kdst + (r * F_NT + wave * 64) * 8), 16, 0, 0);
             if (!SCORES_ONLY)
                 __builtin_amdgcn_global_load_lds((glb_void_t *)(Vp + voff),
-                                                 (lds_void_t *)(Vt + buf * TILE + (r * F_NT + wave * 64) * 8), 16, 0, 0);
+                                                 (lds_void_t *)(Vdst + (r * F_NT + wave * 64) * 8), 16, 0, 0);
         }
     };
 
@@ -408,7 +412,7 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
     const int j_end = (j_lo + jc_len - 1 < j_last) ? j_lo + jc_len - 1 : j_last;
     // one key block earlier only fills the retained score columns (before the first one: the right pad, if any)
     const int j_start = j_lo > 0 ? j_lo - 1 : (G::PWR > 0 ? -1 : 0);
-    issue_kv(j_start, 0);
+    issue_kv(j_start, Kt0, Vt0);
 
     // zero the score tile once (columns past HC+BK are read by the last window but never written)
     for (int e = tid; e < F_SR * F_SLD / 8; e += F_NT) {
@@ -470,8 +474,7 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
     // the two 16-row blocks of this wavefront span rows pmin..pmin+31 of the sequence
     const int pmin = q0 - G::HR + wave * 32;
 
-    int buf = 0;
-    for (int j = j_start; j <= j_end; ++j, buf ^= 1) {
+    auto block = [&](int j, const T *Kb, const T *Vb, T *Kn, T *Vn) __attribute__((always_inline)) {
         const int cbase = j * F_BK + G::PWR;  // first key of the new score block
         pack16<T> tailreg[TAIL_IT > 0 ? TAIL_IT : 1];
 #pragma unroll
@@ -482,12 +485,11 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
 #pragma unroll
         for (int it = 0; it < TAIL_IT; ++it)
             if (tail_off[it] >= 0) *reinterpret_cast<pack16<T> *>(Sc + tail_off[it]) = tailreg[it];
-        if (j < j_end) issue_kv(j + 1, buf ^ 1);  // lands while this block is being worked on
+        if (j < j_end) issue_kv(j + 1, Kn, Vn);  // lands while this block is being worked on
 
         // ---- S^T = K Q^T, zero above the diagonal / outside the sequence, to the score tile ----
         // The K fragments of key block cb+1 are read from LDS while the matrix cores work on block cb.
         {
-            const T *Kb = Kt + buf * TILE;
             frag8<T> kf[2][KS];
             auto load_kf = [&](int cb, frag8<T> (&dst)[KS]) {
                 const int krow = cb * 16 + ln;
@@ -529,8 +531,10 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
                 }
             }
         }
-        __syncthreads();
-        if (j < j_lo) continue;
+        // score tile complete for everybody.  Only the LDS counter is waited for: a fence would also wait for the
+        // copy of the next key block, in flight since the top of the iteration
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (j < j_lo) return;
 
         // score fragments of block blk = rb*NCB+cb: rows trow-(R-1)+i, the block's 32-key window
         auto load_xf = [&](int blk, frag8<T> (&dst)[R]) {
@@ -547,7 +551,7 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
             // ---- conv (Toeplitz MFMAs over the score tile) -> this wavefront's 32 x 64 staging rows -> global ----
             // The score fragments of block blk+1 are read from LDS while the matrix cores work on block blk.
             constexpr int OLD = F_BK + 8;  // staging row stride (elements)
-            T *stage = Vt + wave * 32 * OLD;
+            T *stage = stg + wave * 32 * OLD;
             frag8<T> xf[2][R];
             load_xf(0, xf[0]);
 #pragma unroll
@@ -576,7 +580,7 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
                 if (tr_ >= G::HR && p_ < S && col < S && (!causal || fill_upper || col <= p_))
                     *reinterpret_cast<pack16<T> *>(Op + (int64_t)p_ * S + col) = v;
             }
-            continue;
+            return;
         }
 
         // ---- conv (Toeplitz MFMAs over the score tile), scale, mask, online softmax ----
@@ -642,7 +646,6 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
 
         // ---- O^T += V^T P^T ; V^T fragments via the LDS transpose read of the row-major V block ----
         {
-            const T *Vb = Vt + buf * TILE;
             // slots 0..3: keys 32ks+4kg+(0..3); slots 4..7: keys 32ks+16+4kg+(0..3) -- the order of pf
             frag8<T> vf[2];
             auto load_vf = [&](int blk, frag8<T> &dst) {  // blk = ks * DB + db
@@ -665,6 +668,12 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
                 mma16(oacc[1][db], vf[blk & 1], pf[1][ks]);
             }
         }
+    };
+    for (int j = j_start;;) {
+        block(j, Kt0, Vt0, Kt1, Vt1);
+        if (++j > j_end) break;
+        block(j, Kt1, Vt1, Kt0, Vt0);
+        if (++j > j_end) break;
     }
 
     if constexpr (SCORES_ONLY) {
@@ -709,15 +718,11 @@ int launch_mfma(const void *q, const void *k, const void *v, const void *w, void
                 int causal, float scale, int fill_upper, hipStream_t st)
 {
     constexpr int NW = SCORES_ONLY ? 4 : 8;
-    constexpr int F_NT = 64 * NW, F_SR = 32 * NW;
+    constexpr int F_NT = 64 * NW;
     using G = fused_geom<R, SK, NW>;
     static_assert(G::fits, "conv window exceeds the 32-key MFMA contraction");
     const int nqb = (int)((S + G::BQ - 1) / G::BQ);
-    const size_t vt_elems = SCORES_ONLY ? (size_t)F_SR * (F_BK + 8) : (size_t)2 * F_BK * D;
-    const size_t lds = sizeof(T) * ((size_t)2 * F_BK * D + vt_elems + (size_t)F_SR * F_SLD + (size_t)R * G::WZ_LD);
     auto kern = conv_attn_fwd_mfma<T, D, R, SK, SCORES_ONLY, NW>;
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
     // key blocks per work item: all of them for the attention kernel; MTA_QK_CHUNK for the scores-only kernel
     const int jc_len = SCORES_ONLY ? MTA_QK_CHUNK : (int)((S + F_BK - 1) / F_BK) + 1;
     int64_t items_per_bh = 0;
@@ -728,7 +733,7 @@ int launch_mfma(const void *q, const void *k, const void *v, const void *w, void
     const int64_t total_wg = B * H * items_per_bh, per_xcd = (total_wg + 7) / 8;
     if (per_xcd * 8 > 0x7fffffffLL || items_per_bh > 0x7fffffffLL) return MTA_ERR_SHAPE;
     dim3 grid((unsigned)(per_xcd * 8));
-    hipLaunchKernelGGL(kern, grid, dim3(F_NT), lds, st, (const T *)q, (const T *)k, (const T *)v, (const T *)w, (T *)o,
+    hipLaunchKernelGGL(kern, grid, dim3(F_NT), 0, st, (const T *)q, (const T *)k, (const T *)v, (const T *)w, (T *)o,
                        (int)S, causal, scale, (int)H, nqb, fill_upper, total_wg, per_xcd, jc_len, (int)items_per_bh);
     return launch_status();
 }
