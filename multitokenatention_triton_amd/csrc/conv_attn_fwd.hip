@@ -300,10 +300,14 @@ typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
 // K and V blocks shared by 256 rows), 4 for the scores-only kernel (two workgroups per CU, which overlap each
 // other's barriers and memory latency).
 constexpr int F_BK = 64;   // keys per iteration
+#ifndef MTA_QK_OCC
+#define MTA_QK_OCC 2       // wavefronts per SIMD the scores-only kernel is compiled for (3 spill and measure slower)
+#endif
 #ifndef MTA_QK_CHUNK
 #define MTA_QK_CHUNK 22    // key blocks per work item of the scores-only kernel
 #endif
-constexpr int F_SLD = 88;  // score-tile row stride (elements): 44 dwords, conflict-free 16-byte reads over 16 rows
+constexpr int F_SLD = 80;  // score-tile row stride (elements): exactly the retained columns + one key block (measured
+                           // fastest among 80..120)
 
 template <int R, int SK, int NW> struct fused_geom {
     static constexpr int F_SR = 32 * NW;
@@ -320,7 +324,7 @@ template <int R, int SK, int NW> struct fused_geom {
 // (`O` is then the score tensor, V is unused).  Only q <= p is written when causal, plus +0 above the
 // diagonal when `fill_upper` is set.  The tile is staged through LDS so that stores are 128-byte row segments.
 template <typename T, int D, int R, int SK, bool SCORES_ONLY, int NW>
-__global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__restrict__ Q, const T *__restrict__ K,
+__global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_attn_fwd_mfma(const T *__restrict__ Q, const T *__restrict__ K,
                                                              const T *__restrict__ V, const T *__restrict__ Wt,
                                                              T *__restrict__ O, int S, int causal, float scale, int H,
                                                              int nqb, int fill_upper, int64_t total_wg, int64_t per_xcd,
@@ -343,7 +347,8 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
     __shared__ __align__(16) T Kt1[TILE];
     __shared__ __align__(16) T Vt0[SCORES_ONLY ? 8 : TILE];
     __shared__ __align__(16) T Vt1[SCORES_ONLY ? 8 : TILE];
-    __shared__ __align__(16) T stg[SCORES_ONLY ? F_SR * (F_BK + 8) : 8];  // output staging of the scores-only kernel
+    constexpr bool STG_IN_K = SCORES_ONLY && F_SR * F_BK <= TILE;  // output staging fits a K buffer (D = 128)
+    __shared__ __align__(16) T stg[(SCORES_ONLY && !STG_IN_K) ? F_SR * F_BK : 8];
     __shared__ __align__(16) T Sc[F_SR * F_SLD];                          // score tile
     __shared__ __align__(16) T wz[R * G::WZ_LD];                          // zero-padded kernel rows
 
@@ -550,8 +555,11 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
         if constexpr (SCORES_ONLY) {
             // ---- conv (Toeplitz MFMAs over the score tile) -> this wavefront's 32 x 64 staging rows -> global ----
             // The score fragments of block blk+1 are read from LDS while the matrix cores work on block blk.
-            constexpr int OLD = F_BK + 8;  // staging row stride (elements)
-            T *stage = stg + wave * 32 * OLD;
+            // Staging rows live in the K buffer of this key block when they fit: nobody reads it any more (the
+            // barrier above follows the last K fragment read).  Row stride = one key block, 16-byte chunks
+            // XOR-swizzled by row.
+            constexpr int OLD = F_BK;
+            T *stage = (STG_IN_K ? const_cast<T *>(Kb) : stg) + wave * 32 * OLD;
             frag8<T> xf[2][R];
             load_xf(0, xf[0]);
 #pragma unroll
@@ -569,14 +577,17 @@ __global__ __launch_bounds__(64 * NW, 2) void conv_attn_fwd_mfma(const T *__rest
                     if (col + 2 > prow[rb]) hi &= 0xffff0000u;
                     if (col + 3 > prow[rb]) hi &= 0x0000ffffu;
                 }
-                *reinterpret_cast<uint2 *>(stage + (rb * 16 + ln) * OLD + cb * 16 + kg * 4) = make_uint2(lo, hi);
+                {
+                    const int r_ = rb * 16 + ln, ch_ = (cb * 2 + (kg >> 1)) ^ (r_ & 7);
+                    *reinterpret_cast<uint2 *>(stage + r_ * OLD + ch_ * 8 + (kg & 1) * 4) = make_uint2(lo, hi);
+                }
             }
             __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's staging rows are written
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
                 const int r = it * 8 + (lane >> 3), cv = (lane & 7) * 8;
                 const int tr_ = wave * 32 + r, p_ = q0 - G::HR + tr_, col = j * F_BK + cv;
-                const pack16<T> v = *reinterpret_cast<const pack16<T> *>(stage + r * OLD + cv);
+                const pack16<T> v = *reinterpret_cast<const pack16<T> *>(stage + r * OLD + (((lane & 7) ^ (r & 7)) * 8));
                 if (tr_ >= G::HR && p_ < S && col < S && (!causal || fill_upper || col <= p_))
                     *reinterpret_cast<pack16<T> *>(Op + (int64_t)p_ * S + col) = v;
             }
