@@ -212,22 +212,54 @@ __device__ __forceinline__ void decode_item(int64_t idx, int ipp, int tiles_n, i
     }
 }
 
-template <typename T>
+// Returns its argument, opaquely: what is derived from the result cannot be hoisted out of the (rarely taken) block
+// that computes it, so it does not occupy registers in the main loop.
+__device__ __forceinline__ int opaque(int v)
+{
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
+// FULL: the region lies inside the tensor; the stores are then unconditional (exactly 8 vector-memory instructions)
+template <typename T, bool FULL = false>
 __device__ __forceinline__ void zero_fill_strip(T *yp, int H, int W, int p0, int q0, int lane)
 {
     constexpr int VEC = 8;
     pack16<T> z;
 #pragma unroll
     for (int u = 0; u < VEC; ++u) z.v[u] = from_float<T>(0.0f);
+    lane = opaque(lane);
 #pragma unroll
     for (int e = lane; e < M_TM * (M_TN / VEC); e += M_WT) {
         const int r = e / (M_TN / VEC), col = q0 + (e % (M_TN / VEC)) * VEC;
-        if (p0 + r < H && col < W) *reinterpret_cast<pack16<T> *>(yp + (int64_t)(p0 + r) * W + col) = z;
+        if (FULL || (p0 + r < H && col < W)) *reinterpret_cast<pack16<T> *>(yp + (int64_t)(p0 + r) * W + col) = z;
     }
 }
 
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef const __attribute__((address_space(1))) void glb_void_t;
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// The staged strips are read and written through these, not through C++ accesses: the compiler cannot tell an access
+// to one half of the double buffer from the asynchronous copy in flight into the other half and would wait for the
+// copy first (the copy would then never overlap the matrix products).  LDS operations of a wavefront complete in
+// order; lds_wait() waits for all of them and ties the loaded values to that point.
+__device__ __forceinline__ u32x4 lds_load16(unsigned addr)
+{
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+}
+__device__ __forceinline__ void lds_store16(unsigned addr, u32x4 v)
+{
+    asm volatile("ds_write_b128 %0, %1" : : "v"(addr), "v"(v) : "memory");
+}
+__device__ __forceinline__ void lds_wait() { asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory"); }
+__device__ __forceinline__ void lds_wait(u32x4 &a) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a) : : "memory"); }
+__device__ __forceinline__ void lds_wait(u32x4 (&a)[5])
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]) : : "memory");
+}
 
 // Persistent single-wavefront workgroups: each walks a contiguous run of 32x128 strips (so the
 // Toeplitz fragments are rebuilt only when the channel changes).  No workgroup barrier is ever
@@ -287,14 +319,14 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
 
     // per-lane geometry of the staging copies, fixed for the whole kernel: slot it*64+lane is row srow,
     // vector svc of the strip; padding slots and slots past the strip re-read a neighbouring valid vector
-    int goff[STAGE_IT];
+    unsigned goff[STAGE_IT];  // byte offsets from the strip's first staged element (uniform base + 32-bit lane offset)
 #pragma unroll
     for (int it = 0; it < STAGE_IT; ++it) {
         const int slot = it * M_WT + lane;
         int rr = slot / SPR, vc = slot % SPR;
         if (rr >= G::ROWS) { rr = 0; vc = 0; }
         if (vc >= VPR) vc = VPR - 1;
-        goff[it] = rr * W + vc * VEC;
+        goff[it] = (unsigned)(rr * W + vc * VEC) * (unsigned)sizeof(T);
     }
 
     // a strip is `interior` when its whole halo lies inside the tensor and on or below the diagonal
@@ -305,7 +337,7 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     };
     // asynchronous copy of an interior strip into LDS buffer `buf`
     auto prefetch = [&](int64_t plane_, int p0_, int q0_, T *buf) {
-        const T *base = x + plane_ * (int64_t)H * W + (int64_t)(p0_ - (R - 1)) * W + (q0_ - G::HL);
+        const char *base = reinterpret_cast<const char *>(x + plane_ * (int64_t)H * W + (int64_t)(p0_ - (R - 1)) * W + (q0_ - G::HL));
 #pragma unroll
         for (int it = 0; it < STAGE_IT; ++it)
             __builtin_amdgcn_global_load_lds((glb_void_t *)(base + goff[it]), (lds_void_t *)(buf + it * M_WT * VEC), 16, 0, 0);
@@ -316,6 +348,8 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     decode_item(first, ipp, tiles_n, mirror, plane, tm, tn);
     if (is_interior(tm * M_TM, tn * M_TN)) prefetch(plane, tm * M_TM, tn * M_TN, tiles);
 
+    int younger = -1;                      // stores certainly issued after the copy in flight (-1: unknown)
+    const bool fill_full = H % M_TN == 0;  // mirror images of whole 128x128 blocks lie inside the (square) tensor
     int parity = 0;
     for (int64_t idx = first; idx < last; idx += step, parity ^= 1) {
         T *tile = tiles + parity * BUF;
@@ -328,11 +362,15 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
         const bool above = causal && q0 > p0 + M_TM - 1;  // wholly above the diagonal (only reachable when !mirror)
         const bool interior = is_interior(p0, q0);
         const int h0 = p0 - (R - 1), k0 = q0 - G::HL;
+        const unsigned tile_lds = (unsigned)(uintptr_t)(lds_void_t *)tile;
 
-        // everything issued so far has landed: this strip's copy (if interior) and the previous strip's
-        // stores; LDS reads of `other` by the previous iteration are complete as well
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
+        // This strip's copy (if interior) has landed.  Vector-memory operations complete in issue order, and the only
+        // ones issued after that copy are the previous strip's stores: when their number is known exactly
+        // (`younger`), they may stay in flight.  LDS reads of `other` by the previous iteration are complete.
+        if (younger == 16) asm volatile("s_waitcnt vmcnt(16)" : : : "memory");
+        else if (younger == 8) asm volatile("s_waitcnt vmcnt(8)" : : : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+        younger = 0;
 
         // put the next strip's copy in flight (into the buffer the previous iteration has just released)
         if (idx + step < last) {
@@ -341,15 +379,17 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
         }
         if (above) {
             zero_fill_strip<T>(yp, H, W, p0, q0, lane);
+            younger = -1;
             continue;
         }
         if (!interior) {
             // edge strip: through registers.  Loads are unconditional and issued back to back (an invalid
             // slot re-reads a valid address); what a slot really holds is decided on the way to LDS
             V16 stage[STAGE_IT];
+            const int lane_ = opaque(lane);
 #pragma unroll
             for (int it = 0; it < STAGE_IT; ++it) {
-                const int slot = it * M_WT + lane;
+                const int slot = it * M_WT + lane_;
                 const int rr = slot / SPR, vc = slot % SPR;
                 const int h = h0 + rr, col = k0 + vc * VEC;
                 const bool ok = rr < G::ROWS && vc < VPR && h >= 0 && h < H && col >= 0 && col < W && !(causal && col > h);
@@ -357,7 +397,7 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
             }
 #pragma unroll
             for (int it = 0; it < STAGE_IT; ++it) {
-                const int slot = it * M_WT + lane;
+                const int slot = it * M_WT + lane_;
                 const int rr = slot / SPR, vc = slot % SPR;
                 const int h = h0 + rr, col = k0 + vc * VEC;
                 const bool ok = rr < G::ROWS && vc < VPR && h >= 0 && h < H && col >= 0 && col < W && !(causal && col > h);
@@ -374,7 +414,7 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
                     for (int u = 0; u < VEC; ++u)
                         if (col + u > h) v.v[u] = from_float<T>(0.0f);
                 }
-                *reinterpret_cast<V16 *>(tile + slot * VEC) = v;
+                lds_store16(tile_lds + (unsigned)slot * 16u, __builtin_bit_cast(u32x4, v));
             }
         }
         if (channel != cur_channel) {
@@ -385,7 +425,7 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
                 wz[e] = ok ? wv : from_float<T>(0.0f);
             }
         }
-        __syncthreads();  // LDS stores above are visible (single wavefront: a wait on the LDS counter)
+        lds_wait();  // LDS stores above are complete (single wavefront: no barrier needed)
 
         if (channel != cur_channel) {  // Toeplitz fragments T_i^T for this lane's accumulator row
             cur_channel = channel;
@@ -426,14 +466,17 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
                 if (interior || !causal || q0 + pair * 64 <= p0 + M_TM - 1) {  // else: both wholly above the diagonal
 #pragma unroll
                     for (int i = 0; i < R; ++i) {
-                        const T *rowp = tile + (ln + i) * LD + pair * 64 + kg * 8;
-                        frag8<T> xf[NCH + 2];
+                        const unsigned rowp = tile_lds + (unsigned)((ln + i) * LD + pair * 64 + kg * 8) * sizeof(T);
+                        static_assert(NCH + 2 == 5, "five window chunks per sub-tile pair");
+                        u32x4 xf[NCH + 2];
 #pragma unroll
-                        for (int cc = 0; cc < NCH + 2; ++cc) xf[cc] = *reinterpret_cast<const frag8<T> *>(rowp + cc * 16);
+                        for (int cc = 0; cc < NCH + 2; ++cc) xf[cc] = lds_load16(rowp + (unsigned)(cc * 16) * sizeof(T));
+                        lds_wait(xf);
 #pragma unroll
                         for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-                            for (int ch = 0; ch < NCH; ++ch) mma32(acc[s2], tz[i][ch], xf[s2 * 2 + ch]);
+                            for (int ch = 0; ch < NCH; ++ch)
+                                mma32(acc[s2], tz[i][ch], __builtin_bit_cast(frag8<T>, xf[s2 * 2 + ch]));
                     }
                 }
                 // results back into the strip's own LDS rows: pair 0 overwrites columns 0..63, which pair 1 (reading
@@ -454,52 +497,45 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
                                 if (q + 2 * u + 1 > prow) pk[u] &= 0x0000ffffu;
                             }
                         }
-                        *reinterpret_cast<uint4 *>(tile + ln * LD + col) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+                        lds_store16(tile_lds + (unsigned)(ln * LD + col) * sizeof(T), u32x4{pk[0], pk[1], pk[2], pk[3]});
                     }
             }
-        } else {
-        // ---- 2 row blocks x 8 column blocks of 16x16 outputs; results of a row block go back into its
-        // own (no longer needed) LDS rows: lane (row ln, group kg) holds keys 4*kg..4*kg+3 of each block
-#pragma unroll
-        for (int rb = 0; rb < M_TM / 16; ++rb) {
-            f32x4 acc[M_TN / 16];
-#pragma unroll
-            for (int cb = 0; cb < M_TN / 16; ++cb) {
-                acc[cb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-                if (!interior && causal && q0 + cb * 16 > p0 + rb * 16 + 15) continue;  // block wholly above the diagonal: +0
-#pragma unroll
-                for (int i = 0; i < R; ++i)
-                    mma16(acc[cb], tz[i][0],
-                          *reinterpret_cast<const frag8<T> *>(tile + (rb * 16 + ln + i) * LD + cb * 16 + kg * 8));
-            }
-            const int prow = p0 + rb * 16 + ln;
-#pragma unroll
-            for (int cb = 0; cb < M_TN / 16; ++cb) {
-                struct alignas(8) quad { T v[4]; } out;
-                const int q = q0 + cb * 16 + kg * 4;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    out.v[v] = from_float<T>((!interior && causal && q + v > prow) ? 0.0f : acc[cb][v]);
-                }
-                *reinterpret_cast<quad *>(tile + (rb * 16 + ln) * LD + cb * 16 + kg * 4) = out;
-            }
         }
-        }
-        __syncthreads();
-
-        // ---- coalesced stores: 16 lanes cover one 256-byte output row ----
+        // ---- coalesced stores: 16 lanes cover one 256-byte output row (the LDS writes above precede these reads in
+        // the wavefront's LDS queue) ----
         {
             T *ybase = yp + (int64_t)p0 * W + q0;
             const int r_l = lane >> 4, cv = (lane & 15) * VEC;
+            constexpr int OUT_IT = M_TM * (M_TN / VEC) / M_WT;
 #pragma unroll
-            for (int it = 0; it < M_TM * (M_TN / VEC) / M_WT; ++it) {
-                const int r = it * 4 + r_l;
-                const V16 v = *reinterpret_cast<const V16 *>(tile + r * LD + cv);
-                if (interior || (p0 + r < H && q0 + cv < W)) *reinterpret_cast<V16 *>(ybase + r * W + cv) = v;
+            for (int i0 = 0; i0 < OUT_IT; i0 += 4) {  // four rows' worth in flight per wait
+                u32x4 v[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v[k] = lds_load16(tile_lds + (unsigned)(((i0 + k) * 4 + r_l) * LD + cv) * sizeof(T));
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : : "memory");
+                if (interior) {  // unconditional: exactly OUT_IT vector-memory instructions
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) *reinterpret_cast<u32x4 *>(ybase + ((i0 + k) * 4 + r_l) * W + cv) = v[k];
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const int r = (i0 + k) * 4 + r_l;
+                        if (p0 + r < H && q0 + cv < W) *reinterpret_cast<u32x4 *>(ybase + r * W + cv) = v[k];
+                    }
+                }
+            }
+            static_assert(OUT_IT == 8, "8 stores per strip");
+            younger = interior ? OUT_IT : -1;
+        }
+        if (mirror && ctn < (ctm >> 2)) {  // a quarter of the 128x128 block's image above the diagonal
+            if (fill_full) {
+                zero_fill_strip<T, true>(yp, H, W, q0 + (ctm & 3) * M_TM, (ctm >> 2) * M_TN, lane);
+                if (younger > 0) younger += M_TM * (M_TN / VEC) / M_WT;
+            } else {
+                zero_fill_strip<T>(yp, H, W, q0 + (ctm & 3) * M_TM, (ctm >> 2) * M_TN, lane);
+                younger = -1;
             }
         }
-        if (mirror && ctn < (ctm >> 2))  // a quarter of the 128x128 block's image above the diagonal
-            zero_fill_strip<T>(yp, H, W, q0 + (ctm & 3) * M_TM, (ctm >> 2) * M_TN, lane);
     }
 }
 
