@@ -256,9 +256,9 @@ __device__ __forceinline__ void lds_store16(unsigned addr, u32x4 v)
 }
 __device__ __forceinline__ void lds_wait() { asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory"); }
 __device__ __forceinline__ void lds_wait(u32x4 &a) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a) : : "memory"); }
-__device__ __forceinline__ void lds_wait(u32x4 (&a)[5])
+__device__ __forceinline__ void lds_wait(u32x4 &a, u32x4 &b, u32x4 &c)
 {
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]) : : "memory");
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c) : : "memory");
 }
 
 // Persistent single-wavefront workgroups: each walks a contiguous run of 32x128 strips (so the
@@ -453,52 +453,50 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
         }
 
         if constexpr (M32) {
-            // ---- 32 rows x 4 sub-tiles of 32 keys on 32x32x16 MFMAs, two sub-tiles at a time.  Per kernel row
-            // the 5 chunks of this lane's staged row that the pair needs are read once (the windows overlap).
+            // ---- 32 rows x 4 sub-tiles of 32 keys on 32x32x16 MFMAs, one sub-tile at a time; the three window chunks
+            // of kernel row i+1 are read from LDS while the products of row i run ----
             const int prow = p0 + ln;
 #pragma unroll
-            for (int pair = 0; pair < M_TN / 64; ++pair) {
-                f32x16 acc[2];
+            for (int st = 0; st < M_TN / 32; ++st) {
+                f32x16 acc;
 #pragma unroll
-                for (int s2 = 0; s2 < 2; ++s2)
+                for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+                if (interior || !causal || q0 + st * 32 <= p0 + M_TM - 1) {  // else: wholly above the diagonal
+                    const unsigned xa = tile_lds + (unsigned)(ln * LD + st * 32 + kg * 8) * sizeof(T);
+                    u32x4 xf[2][NCH];
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[s2][v] = 0.0f;
-                if (interior || !causal || q0 + pair * 64 <= p0 + M_TM - 1) {  // else: both wholly above the diagonal
+                    for (int ch = 0; ch < NCH; ++ch) xf[0][ch] = lds_load16(xa + (unsigned)(ch * 16) * sizeof(T));
+                    lds_wait(xf[0][0], xf[0][1], xf[0][2]);
 #pragma unroll
                     for (int i = 0; i < R; ++i) {
-                        const unsigned rowp = tile_lds + (unsigned)((ln + i) * LD + pair * 64 + kg * 8) * sizeof(T);
-                        static_assert(NCH + 2 == 5, "five window chunks per sub-tile pair");
-                        u32x4 xf[NCH + 2];
-#pragma unroll
-                        for (int cc = 0; cc < NCH + 2; ++cc) xf[cc] = lds_load16(rowp + (unsigned)(cc * 16) * sizeof(T));
-                        lds_wait(xf);
-#pragma unroll
-                        for (int s2 = 0; s2 < 2; ++s2)
+                        if (i + 1 < R) {
 #pragma unroll
                             for (int ch = 0; ch < NCH; ++ch)
-                                mma32(acc[s2], tz[i][ch], __builtin_bit_cast(frag8<T>, xf[s2 * 2 + ch]));
+                                xf[(i + 1) & 1][ch] = lds_load16(xa + (unsigned)((i + 1) * LD + ch * 16) * sizeof(T));
+                        }
+#pragma unroll
+                        for (int ch = 0; ch < NCH; ++ch) mma32(acc, tz[i][ch], __builtin_bit_cast(frag8<T>, xf[i & 1][ch]));
+                        if (i + 1 < R) lds_wait(xf[(i + 1) & 1][0], xf[(i + 1) & 1][1], xf[(i + 1) & 1][2]);
                     }
                 }
-                // results back into the strip's own LDS rows: pair 0 overwrites columns 0..63, which pair 1 (reading
-                // columns 64..143) no longer needs
+                // results back into the strip's own LDS rows: sub-tile st overwrites columns 32st..32st+31, which the
+                // later sub-tiles (reading columns >= 32(st+1)) no longer need
 #pragma unroll
-                for (int s2 = 0; s2 < 2; ++s2)
+                for (int a = 0; a < 2; ++a) {
+                    const int col = st * 32 + a * 16 + kg * 8;
+                    const int q = q0 + col;
+                    uint32_t pk[4];
 #pragma unroll
-                    for (int a = 0; a < 2; ++a) {
-                        const int col = pair * 64 + s2 * 32 + a * 16 + kg * 8;
-                        const int q = q0 + col;
-                        uint32_t pk[4];
+                    for (int u = 0; u < 4; ++u) pk[u] = pack2<T>(acc[a * 8 + 2 * u], acc[a * 8 + 2 * u + 1]);
+                    if (!interior && causal && q + 7 > prow) {
 #pragma unroll
-                        for (int u = 0; u < 4; ++u) pk[u] = pack2<T>(acc[s2][a * 8 + 2 * u], acc[s2][a * 8 + 2 * u + 1]);
-                        if (!interior && causal && q + 7 > prow) {
-#pragma unroll
-                            for (int u = 0; u < 4; ++u) {
-                                if (q + 2 * u > prow) pk[u] &= 0xffff0000u;
-                                if (q + 2 * u + 1 > prow) pk[u] &= 0x0000ffffu;
-                            }
+                        for (int u = 0; u < 4; ++u) {
+                            if (q + 2 * u > prow) pk[u] &= 0xffff0000u;
+                            if (q + 2 * u + 1 > prow) pk[u] &= 0x0000ffffu;
                         }
-                        lds_store16(tile_lds + (unsigned)(ln * LD + col) * sizeof(T), u32x4{pk[0], pk[1], pk[2], pk[3]});
                     }
+                    lds_store16(tile_lds + (unsigned)(ln * LD + col) * sizeof(T), u32x4{pk[0], pk[1], pk[2], pk[3]});
+                }
             }
         }
         // ---- coalesced stores: 16 lanes cover one 256-byte output row (the LDS writes above precede these reads in
