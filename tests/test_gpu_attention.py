@@ -187,6 +187,10 @@ QKC_CASES = [
     (1, 1, 776, 128, 5, 7, False, torch.bfloat16),
     (1, 2, 8, 64, 6, 11, True, torch.bfloat16),
     (1, 1, 1000, 128, 7, 7, True, torch.bfloat16),
+    # long enough for the key range of a query block to be split into several work items
+    (1, 1, 2048, 128, 6, 11, True, torch.bfloat16),
+    (1, 2, 1800, 64, 3, 3, True, torch.float16),
+    (1, 1, 1544, 128, 5, 5, False, torch.bfloat16),
 ]
 
 
@@ -256,6 +260,23 @@ def test_mta_headline_config_small(pkg):
               O.identity_conv_kernel(16, 3, 3, dtype), O.block_diag_head_weight(16, 4, 0.1, g, dtype)]
     want = _oracle_mta(q, k, v, params)
     mod = _mta_module(pkg, 16, 6, 11, 3, 3, *params, dtype)
+    stages = []
+    mod._stage_hook = stages.append
+    got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
+    assert stages == ["qk_conv", "mix_softmax_mix", "pv", "end"]
+    torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+
+
+def test_mta_headline_route_long_sequence(pkg):
+    """Same route at S=2048 (several work items per query block in the scores kernel, paired query blocks in P V)."""
+    print("mta headline long", flush=True)
+    dtype = torch.bfloat16
+    q, k, v = O.seeded_qkv(1, 4, 2048, 128, dtype)
+    g = torch.Generator().manual_seed(126)
+    params = [O.seeded_conv_weight(4, 6, 11, 0.05, dtype), torch.eye(4, dtype=dtype),
+              O.identity_conv_kernel(4, 3, 3, dtype), O.block_diag_head_weight(4, 4, 0.1, g, dtype)]
+    want = _oracle_mta(q, k, v, params)
+    mod = _mta_module(pkg, 4, 6, 11, 3, 3, *params, dtype)
     stages = []
     mod._stage_hook = stages.append
     got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
