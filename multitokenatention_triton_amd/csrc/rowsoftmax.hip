@@ -10,7 +10,13 @@
 // Rounding points of the unfused pipeline in a 16-bit dtype are reproduced: the
 // mixed scores and the probabilities are rounded to the I/O dtype before they are
 // used again.
+#include <type_traits>
+
 #include "common.hpp"
+
+#ifndef MTA_RS_OCC
+#define MTA_RS_OCC 5  // wavefronts per SIMD the G*NV = 8 instances (e.g. 4 heads x 4096 keys) are compiled for
+#endif
 
 namespace {
 using namespace mta;
@@ -24,6 +30,18 @@ template <typename T> __device__ __forceinline__ void round_pair(float &a, float
         unpack2<T>(pack2<T>(a, b), a, b);
     }
 }
+// a.lo*b.lo + a.hi*b.hi + c for two packed pairs of the 16-bit type T, accumulated in fp32 (one v_dot2c instruction)
+template <typename T> __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c)
+{
+    if constexpr (sizeof(T) != 2) {
+        return c;
+    } else if constexpr (std::is_same<T, bf16_t>::value) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(mta_bf16x2, a), __builtin_bit_cast(mta_bf16x2, b), c, false);
+    } else {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(mta_f16x2, a), __builtin_bit_cast(mta_f16x2, b), c, false);
+    }
+}
+
 // VEC fp32 values -> a vector of the I/O dtype
 template <typename T, int VEC> __device__ __forceinline__ void pack_vec(const float (&f)[VEC], vecN<T, VEC> &out)
 {
@@ -90,12 +108,13 @@ template <int NT> __device__ __forceinline__ float block_sum(float v, float *red
 
 // Register-resident row: Q <= NT*VEC*NV.
 template <typename T, int G, int NV, int VEC, int NT>
-__global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, const void *__restrict__ w1,
+__global__ __launch_bounds__(NT, (NT == 256 && G * NV == 8) ? MTA_RS_OCC : 1) void mix_softmax_mix(const T *__restrict__ x, const void *__restrict__ w1,
                                                       const void *__restrict__ w2, T *__restrict__ y, int C,
                                                       int P, int Q, int causal, int w_dtype, int fill_upper)
 {
     __shared__ float w1s[G * G];
     __shared__ float w2s[G * G];
+    __shared__ uint32_t w2p[G * (G / 2) + 1];  // w2 as packed pairs of the I/O dtype: (w2[o][2j], w2[o][2j+1])
     __shared__ float red[2][(NT / 64) * G];  // [0] maxima, [1] sums: no barrier needed between the two uses
     const int tid = threadIdx.x;
     const int groups = C / G;
@@ -127,6 +146,20 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, c
         const int64_t widx = (int64_t)(g * G + t / G) * C + g * G + t % G;
         w1s[t] = w1 ? load_any(w1, w_dtype, widx) : (t / G == t % G ? 1.0f : 0.0f);
         w2s[t] = w2 ? load_any(w2, w_dtype, widx) : (t / G == t % G ? 1.0f : 0.0f);
+    }
+    // 16-bit I/O with weights of the same dtype: the second mix runs on packed dot products.  The probabilities are
+    // rounded to the I/O dtype in pairs of heads (the rounding the unfused pipeline applies to them) and each output is
+    // G/2 v_dot2c instructions instead of G fused multiply-adds plus unpacking.
+    constexpr bool DOT_OK = sizeof(T) == 2 && G % 2 == 0;
+    const bool use_dot = DOT_OK && w2 && w_dtype == (std::is_same<T, bf16_t>::value ? MTA_BF16 : MTA_F16);
+    if constexpr (DOT_OK) {
+        if (use_dot) {
+            for (int t = tid; t < G * (G / 2); t += NT) {
+                const int o = t / (G / 2), j = t % (G / 2);
+                const int64_t widx = (int64_t)(g * G + o) * C + g * G + 2 * j;
+                w2p[t] = pack2<T>(load_any(w2, w_dtype, widx), load_any(w2, w_dtype, widx + 1));
+            }
+        }
     }
     __syncthreads();
 
@@ -228,6 +261,7 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, c
             if (dead(k)) continue;
 #pragma unroll
             for (int u = 0; u < VEC; ++u) s[o][k][u] *= inv[o];
+            if (use_dot) continue;  // rounded below, when the heads are packed in pairs
             if constexpr (VEC % 2 == 0) {
 #pragma unroll
                 for (int u = 0; u < VEC; u += 2) round_pair<T>(s[o][k][u], s[o][k][u + 1]);
@@ -251,11 +285,32 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix(const T *__restrict__ x, c
             continue;
         }
         if (q >= Q || (!fill_upper && q > last)) continue;  // vectors wholly above the diagonal: +0 only on request
+        uint32_t pp[DOT_OK ? G / 2 : 1][VEC];  // probabilities of heads (2j, 2j+1), rounded and packed
+        if constexpr (DOT_OK) {
+            if (use_dot) {
+#pragma unroll
+                for (int j = 0; j < G / 2; ++j)
+#pragma unroll
+                    for (int u = 0; u < VEC; ++u) pp[j][u] = pack2<T>(s[2 * j][k][u], s[2 * j + 1][k][u]);
+            }
+        }
 #pragma unroll
         for (int o = 0; o < G; ++o) {
             float of[VEC];
+            if constexpr (DOT_OK) {
+                if (use_dot) {
+#pragma unroll
+                    for (int u = 0; u < VEC; ++u) {
+                        float acc = 0.0f;
+#pragma unroll
+                        for (int j = 0; j < G / 2; ++j) acc = dot2<T>(w2p[o * (G / 2) + j], pp[j][u], acc);
+                        of[u] = acc;
+                    }
+                }
+            }
 #pragma unroll
             for (int u = 0; u < VEC; ++u) {
+                if (use_dot) break;
                 float acc;
                 if (w2) {
                     acc = 0.0f;
