@@ -170,7 +170,11 @@ int dispatch_valu(const void *x, const void *w, void *y, int64_t N, int64_t C, i
 #define MTA_CONV_WAVES_PER_SIMD 2  // register budget: 256 VGPRs
 #endif
 #ifndef MTA_CONV_MFMA32
-#define MTA_CONV_MFMA32 1          // 1: 32x32x16 MFMAs (fewer LDS operand bytes per output), 0: 16x16x32
+#define MTA_CONV_MFMA32 0          // 0: 16x16x32 MFMAs (fewer matrix-core cycles and Toeplitz registers per output;
+                                   // measured faster), 1: 32x32x16 (fewer LDS operand bytes per output)
+#endif
+#ifndef MTA_CONV_DOUBLE_BUF
+#define MTA_CONV_DOUBLE_BUF 1      // 1: the next strip's copy is in flight during the products; 0: one strip buffer
 #endif
 #ifndef MTA_CONV_WG_PER_CU
 #define MTA_CONV_WG_PER_CU 6       // LDS budget: two 11.6 KB strip buffers per single-wavefront workgroup
@@ -254,7 +258,22 @@ __device__ __forceinline__ void lds_store16(unsigned addr, u32x4 v)
 {
     asm volatile("ds_write_b128 %0, %1" : : "v"(addr), "v"(v) : "memory");
 }
+__device__ __forceinline__ void lds_store8(unsigned addr, unsigned lo, unsigned hi)
+{
+    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 v = {lo, hi};
+    asm volatile("ds_write_b64 %0, %1" : : "v"(addr), "v"(v) : "memory");
+}
 __device__ __forceinline__ void lds_wait() { asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory"); }
+template <int N> __device__ __forceinline__ void lds_wait_all(u32x4 (&a)[N])
+{
+    static_assert(N >= 1 && N <= 7, "kernel rows");
+    if constexpr (N == 3) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]) : : "memory");
+    else if constexpr (N == 5) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]) : : "memory");
+    else if constexpr (N == 6) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]) : : "memory");
+    else if constexpr (N == 7) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]) : : "memory");
+    else static_assert(N == 3 || N == 5 || N == 6 || N == 7, "add a case");
+}
 __device__ __forceinline__ void lds_wait(u32x4 &a) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a) : : "memory"); }
 __device__ __forceinline__ void lds_wait(u32x4 &a, u32x4 &b, u32x4 &c)
 {
@@ -298,7 +317,8 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     constexpr int NCH = 3;  // 16-key chunks per 32-output window (M32)
     constexpr int WZ_OFF = G::SHIFT + (M32 ? 32 : 16), WZ_LD = WZ_OFF + (M32 ? 16 * NCH : 32);
     constexpr int BUF = STAGE_IT * M_WT * VEC;  // elements per LDS strip buffer
-    __shared__ __align__(16) T tiles[2 * BUF];  // double buffer: strip n is computed while strip n+1 lands
+    constexpr bool DBUF = MTA_CONV_DOUBLE_BUF != 0;
+    __shared__ __align__(16) T tiles[(DBUF ? 2 : 1) * BUF];  // double buffer: strip n is computed while strip n+1 lands
     __shared__ T wz[R * WZ_LD];
     using V16 = pack16<T>;
 
@@ -346,14 +366,14 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     int64_t plane;
     int tm, tn;
     decode_item(first, ipp, tiles_n, mirror, plane, tm, tn);
-    if (is_interior(tm * M_TM, tn * M_TN)) prefetch(plane, tm * M_TM, tn * M_TN, tiles);
+    if (DBUF && is_interior(tm * M_TM, tn * M_TN)) prefetch(plane, tm * M_TM, tn * M_TN, tiles);
 
     int younger = -1;                      // stores certainly issued after the copy in flight (-1: unknown)
     const bool fill_full = H % M_TN == 0;  // mirror images of whole 128x128 blocks lie inside the (square) tensor
     int parity = 0;
     for (int64_t idx = first; idx < last; idx += step, parity ^= 1) {
-        T *tile = tiles + parity * BUF;
-        T *other = tiles + (parity ^ 1) * BUF;
+        T *tile = tiles + (DBUF ? parity * BUF : 0);
+        T *other = tiles + (DBUF ? (parity ^ 1) * BUF : 0);
         const int p0 = tm * M_TM, q0 = tn * M_TN;
         const int ctm = tm, ctn = tn;
         const T *xp = x + plane * (int64_t)H * W;
@@ -362,20 +382,29 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
         const bool above = causal && q0 > p0 + M_TM - 1;  // wholly above the diagonal (only reachable when !mirror)
         const bool interior = is_interior(p0, q0);
         const int h0 = p0 - (R - 1), k0 = q0 - G::HL;
-        const unsigned tile_lds = (unsigned)(uintptr_t)(lds_void_t *)tile;
+        // (opaque: the addresses derived from it are then formed where they are used instead of being kept, dozens of
+        // them, in registers across the loop)
+        const unsigned tile_lds = (unsigned)opaque((int)(unsigned)(uintptr_t)(lds_void_t *)tile);
 
         // This strip's copy (if interior) has landed.  Vector-memory operations complete in issue order, and the only
         // ones issued after that copy are the previous strip's stores: when their number is known exactly
         // (`younger`), they may stay in flight.  LDS reads of `other` by the previous iteration are complete.
-        if (younger == 16) asm volatile("s_waitcnt vmcnt(16)" : : : "memory");
-        else if (younger == 8) asm volatile("s_waitcnt vmcnt(8)" : : : "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+        if constexpr (DBUF) {
+            if (younger == 16) asm volatile("s_waitcnt vmcnt(16)" : : : "memory");
+            else if (younger == 8) asm volatile("s_waitcnt vmcnt(8)" : : : "memory");
+            else asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+        } else {
+            // one buffer: this strip's copy is issued now and waited for (the other wavefronts of the CU cover the
+            // latency); the previous strip's LDS reads are complete
+            if (interior) prefetch(plane, p0, q0, tile);
+            asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+        }
         younger = 0;
 
         // put the next strip's copy in flight (into the buffer the previous iteration has just released)
         if (idx + step < last) {
             decode_item(idx + step, ipp, tiles_n, mirror, plane, tm, tn);
-            if (is_interior(tm * M_TM, tn * M_TN)) prefetch(plane, tm * M_TM, tn * M_TN, other);
+            if (DBUF && is_interior(tm * M_TM, tn * M_TN)) prefetch(plane, tm * M_TM, tn * M_TN, other);
         }
         if (above) {
             zero_fill_strip<T>(yp, H, W, p0, q0, lane);
@@ -498,12 +527,50 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
                     lds_store16(tile_lds + (unsigned)(ln * LD + col) * sizeof(T), u32x4{pk[0], pk[1], pk[2], pk[3]});
                 }
             }
+        } else {
+            // ---- 2 row blocks x 8 column blocks of 16x16 outputs on 16x16x32 MFMAs (one per kernel row: the 32-key
+            // window holds the 16 outputs' taps).  A third of the Toeplitz registers of the 32x32 form and fewer
+            // matrix-core cycles per output, at more LDS operand bytes.  Results of a row block go back into its own
+            // (no longer needed) LDS rows: lane (row ln, group kg) holds keys 4*kg..4*kg+3 of each block.
+#pragma unroll
+            for (int rb = 0; rb < M_TM / 16; ++rb) {
+                f32x4 acc[M_TN / 16];
+                const unsigned xa = tile_lds + (unsigned)((rb * 16 + ln) * LD + kg * 8) * sizeof(T);
+#pragma unroll
+                for (int cb = 0; cb < M_TN / 16; ++cb) {
+                    acc[cb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                    if (!interior && causal && q0 + cb * 16 > p0 + rb * 16 + 15) continue;  // wholly above the diagonal: +0
+                    u32x4 xf[R];
+#pragma unroll
+                    for (int i = 0; i < R; ++i) xf[i] = lds_load16(xa + (unsigned)(i * LD + cb * 16) * sizeof(T));
+                    lds_wait_all(xf);
+#pragma unroll
+                    for (int i = 0; i < R; ++i) mma16(acc[cb], tz[i][0], __builtin_bit_cast(frag8<T>, xf[i]));
+                }
+                const int prow = p0 + rb * 16 + ln;
+#pragma unroll
+                for (int cb = 0; cb < M_TN / 16; cb += 2) {
+#pragma unroll
+                    for (int c2 = 0; c2 < 2; ++c2) {
+                        const int q = q0 + (cb + c2) * 16 + kg * 4;
+                        uint32_t lo = pack2<T>(acc[cb + c2][0], acc[cb + c2][1]), hi = pack2<T>(acc[cb + c2][2], acc[cb + c2][3]);
+                        if (!interior && causal && q + 3 > prow) {
+                            if (q > prow) lo &= 0xffff0000u;
+                            if (q + 1 > prow) lo &= 0x0000ffffu;
+                            if (q + 2 > prow) hi &= 0xffff0000u;
+                            if (q + 3 > prow) hi &= 0x0000ffffu;
+                        }
+                        lds_store8(tile_lds + (unsigned)((rb * 16 + ln) * LD + (cb + c2) * 16 + kg * 4) * sizeof(T), lo, hi);
+                    }
+                }
+            }
         }
         // ---- coalesced stores: 16 lanes cover one 256-byte output row (the LDS writes above precede these reads in
         // the wavefront's LDS queue) ----
         {
             T *ybase = yp + (int64_t)p0 * W + q0;
-            const int r_l = lane >> 4, cv = (lane & 15) * VEC;
+            const int lane_o = opaque(lane);  // (row offsets formed here, not kept in registers across the loop)
+            const int r_l = lane_o >> 4, cv = (lane_o & 15) * VEC;
             constexpr int OUT_IT = M_TM * (M_TN / VEC) / M_WT;
 #pragma unroll
             for (int i0 = 0; i0 < OUT_IT; i0 += 4) {  // four rows' worth in flight per wait
