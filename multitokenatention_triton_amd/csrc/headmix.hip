@@ -8,7 +8,10 @@
 // and the small GxG contraction happens inside the lane (no cross-lane traffic).
 // Causal: vectors wholly above the diagonal are never read and receive the fill
 // value; the vector that straddles the diagonal is masked per element.
+#include <stdlib.h>
+
 #include "common.hpp"
+#include "mfma.hpp"
 
 namespace {
 using namespace mta;
@@ -55,6 +58,21 @@ template <typename V> __device__ __forceinline__ void store_stream(V *dst, const
     *dst = v;
 }
 
+// Workgroups go to the 8 XCDs round-robin by index.  With the key chunk as the fastest-varying part of the index and
+// a chunk count that divides 8 (or is a multiple of it), an XCD would always see the same chunks - and under the causal
+// mask the chunks near the start of a row carry all the work.  Rotating the chunk by the row spreads every chunk over
+// every XCD.  Returns the chunk of workgroup `id` and leaves the row (id / qchunks) in `id`; a bijection within each row.
+// All index arithmetic is 32-bit and unsigned (the host rejects grids beyond 2^31 workgroups): a workgroup's share is
+// small enough for 64-bit divisions in its prologue to show.
+__device__ __forceinline__ int rotated_chunk(unsigned &id, unsigned qchunks)
+{
+    if (qchunks == 1) return 0;
+    const unsigned row = id / qchunks, qc = id - row * qchunks;
+    const unsigned rot = (qchunks % 8 == 0) ? row : (unsigned)(((uint64_t)row * qchunks) >> 3);
+    id = row;
+    return (int)((qc + rot) % qchunks);
+}
+
 // G heads mixed inside one lane, G known at compile time.  A workgroup covers ROWS consecutive
 // query rows of one key chunk, so a lane has ROWS*G independent 16-byte loads in flight.
 template <typename T, int G, int VEC, int ROWS>
@@ -70,11 +88,11 @@ __global__ __launch_bounds__(NT) void headmix_fixed(const T *__restrict__ x, con
     __shared__ float wsm[WREG ? 1 : G * G];
     const int tid = threadIdx.x;
     const int groups = C / G;
-    int64_t b = blockIdx.x;
-    const int qc = (int)(b % qchunks); b /= qchunks;
-    const int p0 = (int)(b % pblocks) * ROWS; b /= pblocks;
-    const int g = (int)(b % groups);
-    const int64_t n = b / groups;
+    unsigned b = blockIdx.x;
+    const int qc = rotated_chunk(b, qchunks);
+    const int p0 = (int)(b % (unsigned)pblocks) * ROWS; b /= (unsigned)pblocks;
+    const int g = (int)(b % (unsigned)groups);
+    const int64_t n = b / (unsigned)groups;
     const int q = (qc * NT + tid) * VEC;
     const int64_t plane = (int64_t)P * Q;
     const int64_t base0 = (n * C + (int64_t)g * G) * plane + q;
@@ -145,6 +163,101 @@ __global__ __launch_bounds__(NT) void headmix_fixed(const T *__restrict__ x, con
     }
 }
 
+// Dense mixing of 32 heads on the matrix cores (16-bit I/O, weights of the same dtype).
+//
+//   y[o, q] = sum_i w[o, i] * x[i, q]        one v_mfma_f32_16x16x32 per 16 output heads x 16 keys: the contraction
+//                                            covers all 32 input heads at once
+//
+// A wavefront owns 128 keys of one (batch, query row) and needs no LDS.  Lane (ln, kg) fetches keys 8ln .. 8ln+7 of the
+// heads 8kg .. 8kg+7 with eight 16-byte loads (an instruction covers 4 heads x 256 contiguous bytes), transposes that
+// 8 x 8 block inside its own registers (one byte-permute per dword) into the x operands of eight products - product j
+// maps the lane's column to key 8ln + j - and keeps w (output heads 0-15, 16-31) in registers as the other operand.
+// After the eight products the lane holds keys 8ln .. 8ln+7 of output heads 4kg + v: 16-byte stores, again
+// 4 heads x 256 contiguous bytes per instruction.  Columns are independent, so keys beyond the diagonal may carry any
+// data (their lanes re-read the row start); their outputs get the fill.
+#ifndef MTA_HM_DM_WAVES
+#define MTA_HM_DM_WAVES 4
+#endif
+constexpr int DM_WAVES = MTA_HM_DM_WAVES, DM_KEYS = 128;
+
+template <typename T>
+__global__ __launch_bounds__(64 * DM_WAVES, 4) void headmix_dense32(const T *__restrict__ x, const T *__restrict__ w,
+                                                               T *__restrict__ y, int C, int P, int Q, int causal,
+                                                               float fill, int qchunks)
+{
+    constexpr int HG = 32;  // heads mixed together
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, ln = lane & 15, kg = lane >> 4;
+    const int groups = C / HG;
+    unsigned b = blockIdx.x;
+    const int qc = rotated_chunk(b, qchunks);
+    const int p = (int)(b % (unsigned)P); b /= (unsigned)P;
+    const int g = (int)(b % (unsigned)groups);
+    const int64_t n = b / (unsigned)groups;
+    const int q0 = (qc * DM_WAVES + wave) * DM_KEYS;
+    if (q0 >= Q) return;
+    const int64_t plane = (int64_t)P * Q;
+    const int64_t base = (n * C + (int64_t)g * HG) * plane + (int64_t)p * Q;  // head g*32, row p, key 0
+    const int last = causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;              // last key that is mixed
+    const uint32_t fill2 = pack2<T>(fill, fill);
+    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+    const int key = q0 + ln * 8;
+
+    if (q0 > last) {  // wholly beyond the diagonal: fill only
+        const u4 fv = {fill2, fill2, fill2, fill2};
+        if (key < Q) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                __builtin_nontemporal_store(fv, reinterpret_cast<u4 *>(y + base + (kg * 8 + t) * plane + key));
+        }
+        return;
+    }
+
+    const T *xp = x + base + (int64_t)(kg * 8) * plane + (key <= last ? key : 0);
+    u4 xv[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) xv[t] = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(xp + t * plane));
+
+    // w fragments: lane (output head ln of block ob, group kg) holds w[o][8kg .. 8kg+7]
+    frag8<T> wf[2];
+#pragma unroll
+    for (int ob = 0; ob < 2; ++ob)
+        wf[ob] = *reinterpret_cast<const frag8<T> *>(w + (int64_t)(g * HG + ob * 16 + ln) * C + g * HG + kg * 8);
+
+    f32x4 acc[8][2];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        u4 xt;  // heads 8kg .. 8kg+7 of key 8ln + j
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            xt[u] = __builtin_amdgcn_perm(xv[2 * u + 1][j >> 1], xv[2 * u][j >> 1], (j & 1) ? 0x07060302u : 0x05040100u);
+        const frag8<T> xf = __builtin_bit_cast(frag8<T>, xt);
+#pragma unroll
+        for (int ob = 0; ob < 2; ++ob) {
+            acc[j][ob] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            mma16(acc[j][ob], wf[ob], xf);
+        }
+    }
+    if (key >= Q) return;
+    // acc[j][ob][v]: output head 16ob + 4kg + v, key 8ln + j
+#pragma unroll
+    for (int ob = 0; ob < 2; ++ob) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            u4 o;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) o[u] = pack2<T>(acc[2 * u][ob][v], acc[2 * u + 1][ob][v]);
+            if (key + 7 > last) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (key + 2 * u > last) o[u] = (o[u] & 0xffff0000u) | (fill2 & 0x0000ffffu);
+                    if (key + 2 * u + 1 > last) o[u] = (o[u] & 0x0000ffffu) | (fill2 & 0xffff0000u);
+                }
+            }
+            __builtin_nontemporal_store(o, reinterpret_cast<u4 *>(y + base + (int64_t)(ob * 16 + kg * 4 + v) * plane + key));
+        }
+    }
+}
+
 // Any group size: one (output head, vector) per lane-iteration, inputs re-read per output head.
 template <typename T, int VEC>
 __global__ __launch_bounds__(NT) void headmix_any(const T *__restrict__ x, const void *__restrict__ w,
@@ -153,11 +266,11 @@ __global__ __launch_bounds__(NT) void headmix_any(const T *__restrict__ x, const
 {
     const int tid = threadIdx.x;
     const int groups = C / G;
-    int64_t b = blockIdx.x;
-    const int qc = (int)(b % qchunks); b /= qchunks;
-    const int p = (int)(b % P); b /= P;
-    const int g = (int)(b % groups);
-    const int64_t n = b / groups;
+    unsigned b = blockIdx.x;
+    const int qc = rotated_chunk(b, qchunks);
+    const int p = (int)(b % (unsigned)P); b /= (unsigned)P;
+    const int g = (int)(b % (unsigned)groups);
+    const int64_t n = b / (unsigned)groups;
     const int q = (qc * NT + tid) * VEC;
     if (q >= Q) return;
     const int64_t plane = (int64_t)P * Q;
@@ -185,8 +298,21 @@ __global__ __launch_bounds__(NT) void headmix_any(const T *__restrict__ x, const
 
 template <typename T, int VEC>
 int launch(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t P, int64_t Q, int G, int causal,
-           float fill, int w_dtype, hipStream_t st)
+           float fill, int w_dtype, bool w_same_dtype, hipStream_t st)
 {
+    if constexpr (VEC == 8) {
+        // 32 heads mixed densely, 16-bit data and weights of the same dtype: matrix cores (MTA_HEADMIX_NO_MFMA=1 in the
+        // environment keeps the vector-ALU kernel, for comparisons)
+        static const bool no_mfma = [] { const char *e = getenv("MTA_HEADMIX_NO_MFMA"); return e && e[0] == '1'; }();
+        if (G == 32 && !no_mfma && w_same_dtype && aligned_to(w, 16) && C % 8 == 0) {
+            const int qch = (int)((Q + DM_WAVES * DM_KEYS - 1) / (DM_WAVES * DM_KEYS));
+            const int64_t blocks = N * (C / 32) * P * qch;
+            if (blocks > 0x7fffffffLL) return MTA_ERR_SHAPE;
+            hipLaunchKernelGGL((headmix_dense32<T>), dim3((unsigned)blocks), dim3(64 * DM_WAVES), 0, st, (const T *)x,
+                               (const T *)w, (T *)y, (int)C, (int)P, (int)Q, causal, fill, qch);
+            return launch_status();
+        }
+    }
     const int qchunks = (int)((Q + (int64_t)NT * VEC - 1) / ((int64_t)NT * VEC));
 #define MTA_HM_CASE(g, rows)                                                                                       \
     if (G == g) {                                                                                                  \
@@ -228,8 +354,9 @@ extern "C" int mta_headmix_fwd(const void *x, const void *w, void *y, int64_t N,
     MTA_DISPATCH_IO(io_dtype, {
         constexpr int VEC = vec_of<io_t>::n;
         const bool vec_ok = (Q % VEC == 0) && aligned_to(x, 16) && aligned_to(y, 16);
-        return vec_ok ? launch<io_t, VEC>(x, w, y, N, C, P, Q, G, causal, fill, w_dtype, st)
-                      : launch<io_t, 1>(x, w, y, N, C, P, Q, G, causal, fill, w_dtype, st);
+        const bool same = w_dtype == io_dtype;
+        return vec_ok ? launch<io_t, VEC>(x, w, y, N, C, P, Q, G, causal, fill, w_dtype, same, st)
+                      : launch<io_t, 1>(x, w, y, N, C, P, Q, G, causal, fill, w_dtype, same, st);
     });
     return MTA_ERR_DTYPE;
 }

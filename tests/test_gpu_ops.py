@@ -101,6 +101,9 @@ HM_CASES = [
     # N, C, P, Q, group (None = dense)
     (1, 4, 9, 9, None), (2, 4, 64, 64, 2), (1, 8, 40, 40, 4), (1, 6, 33, 33, None), (1, 6, 24, 24, 3),
     (1, 16, 48, 48, None), (1, 32, 16, 16, 4), (1, 32, 24, 24, None), (2, 2, 300, 300, 1), (1, 4, 5, 2056, 2),
+    # 32 heads mixed densely (matrix-core kernel for 16-bit data): several wavefronts and workgroups per row, ragged
+    # last wavefront, rows longer and shorter than the key range, two groups of 32
+    (1, 32, 300, 296, None), (1, 32, 40, 1160, None), (2, 64, 136, 136, 32), (1, 32, 600, 64, None),
 ]
 
 
