@@ -23,6 +23,8 @@
 // already there.  One extra leading key block (mostly out-of-range keys) primes that halo.
 #include <algorithm>
 
+#include <type_traits>
+
 #include "common.hpp"
 #include "mfma.hpp"
 
@@ -294,6 +296,7 @@ __global__ __launch_bounds__(NT) void conv_attn_fwd_kernel(const T *__restrict__
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef const __attribute__((address_space(1))) void glb_void_t;
 typedef short v4s_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
 
 // The workgroup has NW wavefronts and owns 32*NW score rows: 8 for the attention kernel (one workgroup per CU,
@@ -301,10 +304,10 @@ typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
 // other's barriers and memory latency).
 constexpr int F_BK = 64;   // keys per iteration
 #ifndef MTA_QK_OCC
-#define MTA_QK_OCC 2       // wavefronts per SIMD the scores-only kernel is compiled for (3 spill and measure slower)
+#define MTA_QK_OCC 3       // wavefronts per SIMD the scores-only kernel is compiled for (three workgroups per CU)
 #endif
 #ifndef MTA_QK_CHUNK
-#define MTA_QK_CHUNK 22    // key blocks per work item of the scores-only kernel
+#define MTA_QK_CHUNK 32    // key blocks per work item of the scores-only kernel
 #endif
 constexpr int F_SLD = 80;  // score-tile row stride (elements): exactly the retained columns + one key block (measured
                            // fastest among 80..120)
@@ -350,10 +353,15 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
     constexpr bool STG_IN_K = SCORES_ONLY && F_SR * F_BK <= TILE;  // output staging fits a K buffer (D = 128)
     __shared__ __align__(16) T stg[(SCORES_ONLY && !STG_IN_K) ? F_SR * F_BK : 8];
     __shared__ __align__(16) T Sc[F_SR * F_SLD];                          // score tile
-    __shared__ __align__(16) T wz[R * G::WZ_LD];                          // zero-padded kernel rows
+    // zero-padded kernel rows, only needed until the Toeplitz fragments are built: they borrow the second K buffer,
+    // which receives its first copy after that (LDS is granted in 1280-byte units; the array's own 648 bytes were
+    // the difference between two and three workgroups per CU for the scores-only kernel)
+    static_assert(R * G::WZ_LD <= TILE, "kernel rows do not fit the borrowed buffer");
+    T *const wz = Kt1;
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63, ln = lane & 15, kg = lane >> 4;
+    // (the wavefront index through readfirstlane: everything derived from it is then scalar, branches included)
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, ln = lane & 15, kg = lane >> 4;
     // XCD-aware order: workgroup ids are dealt round-robin to the 8 XCDs, so XCD x takes the x-th eighth of the
     // (batch*head, query block) list: the workgroups sharing one head's K and V run on one L2.  Within a head
     // the longest (last) query blocks come first.
@@ -382,26 +390,24 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
     // asynchronous copy of key block j into buffer `buf`: K rows cb.., V rows j*BK..; out-of-range keys
     // re-read a valid row (their scores are zeroed / their probabilities are 0 later)
     // slot r*512+tid of a block is row kv_row[r], 16-byte chunk kv_c of that row (fixed per lane)
-    int kv_off[ROUNDS], kv_row[ROUNDS];
-#pragma unroll
-    for (int r = 0; r < ROUNDS; ++r) {
-        const int slot = r * F_NT + tid;
-        kv_row[r] = slot / CPR;
-        kv_off[r] = kv_row[r] * D + ((slot % CPR) ^ (kv_row[r] & (CPR - 1))) * 8;
-    }
+    // (a round advances the row by F_NT/CPR, a multiple of CPR: the swizzled chunk is the same in every round)
+    static_assert((F_NT / CPR) % CPR == 0 && F_NT % CPR == 0, "copy rounds must keep the swizzle phase");
+    const int kv_row0 = tid / CPR;
+    const int kv_off0 = kv_row0 * D + ((tid % CPR) ^ (kv_row0 & (CPR - 1))) * 8;
     auto issue_kv = [&](int j, T *Kdst, T *Vdst) {
         const int cb = j * F_BK + G::PWR;
         const bool inside = cb >= 0 && cb + F_BK <= S && j >= 0 && (j + 1) * F_BK <= S;  // no key needs clamping
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r) {
-            int koff = cb * D + kv_off[r], voff = j * F_BK * D + kv_off[r];
+            const int kv_row = kv_row0 + r * (F_NT / CPR), kv_off = kv_off0 + r * (F_NT / CPR) * D;
+            int koff = cb * D + kv_off, voff = j * F_BK * D + kv_off;
             if (!inside) {
-                int kr = cb + kv_row[r];
+                int kr = cb + kv_row;
                 kr = kr < 0 ? 0 : (kr >= S ? S - 1 : kr);
-                int vr = j * F_BK + kv_row[r];
+                int vr = j * F_BK + kv_row;
                 vr = vr < 0 ? 0 : (vr >= S ? S - 1 : vr);
-                koff = kv_off[r] + (kr - kv_row[r]) * D;
-                voff = kv_off[r] + (vr - kv_row[r]) * D;
+                koff = kv_off + (kr - kv_row) * D;
+                voff = kv_off + (vr - kv_row) * D;
             }
             __builtin_amdgcn_global_load_lds((glb_void_t *)(Kp + koff),
                                              (lds_void_t *)(Kdst + (r * F_NT + wave * 64) * 8), 16, 0, 0);
@@ -479,17 +485,21 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
     // the two 16-row blocks of this wavefront span rows pmin..pmin+31 of the sequence
     const int pmin = q0 - G::HR + wave * 32;
 
-    auto block = [&](int j, const T *Kb, const T *Vb, T *Kn, T *Vn) __attribute__((always_inline)) {
+    // PLAIN: the key block (its scores and its conv outputs) lies inside the sequence and on or below the diagonal
+    // for all 32 rows of this wavefront: no masks and no per-sub-block tests (most blocks of a long sequence)
+    auto block = [&](auto plain_tag, int j, const T *Kb, const T *Vb, T *Kn, T *Vn) __attribute__((always_inline)) {
+        constexpr bool PLAIN = decltype(plain_tag)::value;
         const int cbase = j * F_BK + G::PWR;  // first key of the new score block
-        pack16<T> tailreg[TAIL_IT > 0 ? TAIL_IT : 1];
+        // (a vector type, read by every lane: a struct read under a lane condition travels through scratch memory)
+        u32x4_t tailreg[TAIL_IT > 0 ? TAIL_IT : 1];
 #pragma unroll
         for (int it = 0; it < TAIL_IT; ++it)
-            if (tail_off[it] >= 0) tailreg[it] = *reinterpret_cast<const pack16<T> *>(Sc + tail_off[it] + F_BK);
+            tailreg[it] = *reinterpret_cast<const u32x4_t *>(Sc + (tail_off[it] >= 0 ? tail_off[it] : 0) + F_BK);
         __builtin_amdgcn_s_waitcnt(0);  // this wavefront's part of block j has landed in LDS
         __syncthreads();                // ... and everybody's; all reads of the previous tiles are done
 #pragma unroll
         for (int it = 0; it < TAIL_IT; ++it)
-            if (tail_off[it] >= 0) *reinterpret_cast<pack16<T> *>(Sc + tail_off[it]) = tailreg[it];
+            if (tail_off[it] >= 0) *reinterpret_cast<u32x4_t *>(Sc + tail_off[it]) = tailreg[it];
         if (j < j_end) issue_kv(j + 1, Kn, Vn);  // lands while this block is being worked on
 
         // ---- S^T = K Q^T, zero above the diagonal / outside the sequence, to the score tile ----
@@ -513,7 +523,7 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
                     mma16(sacc[1], kf[cb & 1][ks], qf[1][ks]);
                 }
                 // key block wholly inside the sequence and on or below the diagonal for all 32 rows: no masks
-                const bool s_plain = cbase + cb * 16 >= 0 && cbase + cb * 16 + 16 <= S && (!causal || cbase + cb * 16 + 15 <= pmin);
+                const bool s_plain = PLAIN || (cbase + cb * 16 >= 0 && cbase + cb * 16 + 16 <= S && (!causal || cbase + cb * 16 + 15 <= pmin));
 #pragma unroll
                 for (int rb = 0; rb < 2; ++rb) {
                     uint32_t lo = pack2<T>(sacc[rb][0], sacc[rb][1]), hi = pack2<T>(sacc[rb][2], sacc[rb][3]);
@@ -570,7 +580,7 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
 #pragma unroll
                 for (int i = 0; i < R; ++i) mma16(cacc, tz[i], xf[blk & 1][i]);
                 uint32_t lo = pack2<T>(cacc[0], cacc[1]), hi = pack2<T>(cacc[2], cacc[3]);
-                if (causal && j * F_BK + cb * 16 + 15 > pmin) {  // block touches the diagonal for some row
+                if (!PLAIN && causal && j * F_BK + cb * 16 + 15 > pmin) {  // block touches the diagonal for some row
                     const int col = j * F_BK + cb * 16 + kg * 4;
                     if (col > prow[rb]) lo &= 0xffff0000u;
                     if (col + 1 > prow[rb]) lo &= 0x0000ffffu;
@@ -588,7 +598,7 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
                 const int r = it * 8 + (lane >> 3), cv = (lane & 7) * 8;
                 const int tr_ = wave * 32 + r, p_ = q0 - G::HR + tr_, col = j * F_BK + cv;
                 const pack16<T> v = *reinterpret_cast<const pack16<T> *>(stage + r * OLD + (((lane & 7) ^ (r & 7)) * 8));
-                if (tr_ >= G::HR && p_ < S && col < S && (!causal || fill_upper || col <= p_))
+                if (tr_ >= G::HR && p_ < S && (PLAIN || (col < S && (!causal || fill_upper || col <= p_))))
                     *reinterpret_cast<pack16<T> *>(Op + (int64_t)p_ * S + col) = v;
             }
             return;
@@ -616,7 +626,7 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
                     unpack2<T>(pack2<T>(cacc[2], cacc[3]), a[2], a[3]);
                     unpack2<T>(pack2<T>(a[0] * scale, a[1] * scale), a[0], a[1]);
                     unpack2<T>(pack2<T>(a[2] * scale, a[3] * scale), a[2], a[3]);
-                    const bool c_plain = j * F_BK + cb * 16 + 16 <= S && (!causal || j * F_BK + cb * 16 + 15 <= pmin);
+                    const bool c_plain = PLAIN || (j * F_BK + cb * 16 + 16 <= S && (!causal || j * F_BK + cb * 16 + 15 <= pmin));
 #pragma unroll
                     for (int v = 0; v < 4; ++v) {
                         float val = a[v];
@@ -680,10 +690,16 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
             }
         }
     };
+    auto plain = [&](int j) {  // (scores-only kernel: the attention kernel has no registers to spare for a second body)
+        const int cbase = j * F_BK + G::PWR;
+        return SCORES_ONLY && j >= 0 && cbase + F_BK <= S && (!causal || cbase + F_BK - 1 <= pmin);
+    };
     for (int j = j_start;;) {
-        block(j, Kt0, Vt0, Kt1, Vt1);
+        if (SCORES_ONLY && plain(j)) block(std::integral_constant<bool, SCORES_ONLY>{}, j, Kt0, Vt0, Kt1, Vt1);
+        else block(std::false_type{}, j, Kt0, Vt0, Kt1, Vt1);
         if (++j > j_end) break;
-        block(j, Kt1, Vt1, Kt0, Vt0);
+        if (SCORES_ONLY && plain(j)) block(std::integral_constant<bool, SCORES_ONLY>{}, j, Kt1, Vt1, Kt0, Vt0);
+        else block(std::false_type{}, j, Kt1, Vt1, Kt0, Vt0);
         if (++j > j_end) break;
     }
 
