@@ -282,3 +282,34 @@ def test_mta_headline_route_long_sequence(pkg):
     got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
     assert stages == ["qk_conv", "mix_softmax_mix", "pv", "end"]
     torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+
+
+def test_mta_headline_full_size(pkg):
+    """BASELINE config 4 at its full size (B2 H16 S4096 D128 bf16, 6x11 pre conv, groups of 4).  The oracle is run on
+    one mixing group of one batch element (the head mixing is block diagonal, so the slice is self-contained, and
+    4 heads x 4096^2 scores is what the CPU finishes in seconds); every other (batch, head) is checked through the
+    closed form of the first query row: one attended key, probability 1 for every head, so
+    out[b,0,h,:] = bf16(sum_i wposm[h,i]) * v[b,h,0,:] (the output is laid out (B,S,H,D))."""
+    print("mta headline full size", flush=True)
+    dtype = torch.bfloat16
+    b, h, s, d, grp = 2, 16, 4096, 128, 4
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=300)
+    g = torch.Generator().manual_seed(127)
+    params = [O.seeded_conv_weight(h, 6, 11, 0.05, dtype), O.block_diag_head_weight(h, grp, 0.1, g, dtype),
+              O.identity_conv_kernel(h, 3, 3, dtype), O.block_diag_head_weight(h, grp, 0.1, g, dtype)]
+    mod = _mta_module(pkg, h, 6, 11, 3, 3, *params, dtype)
+    stages = []
+    mod._stage_hook = stages.append
+    got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
+    assert stages == ["qk_conv", "mix_softmax_mix", "pv", "end"]
+    assert torch.isfinite(got.float()).all()
+    # closed form of query row 0, all batches and heads
+    wsum = params[3].float().sum(dim=1).to(dtype).float()            # (H,) row sums of the post-softmax mix
+    want0 = (wsum[None, :, None] * v[:, :, 0, :].float()).to(dtype)
+    torch.testing.assert_close(got[:, 0, :, :].float(), want0.float(), **tol(dtype))
+    # oracle on batch 1, heads 8..11
+    bi, h0 = 1, 8
+    sl = slice(h0, h0 + grp)
+    sub = [params[0][sl], params[1][sl, sl], params[2][sl], params[3][sl, sl]]
+    want = _oracle_mta(q[bi:bi + 1, sl], k[bi:bi + 1, sl], v[bi:bi + 1, sl], sub)
+    torch.testing.assert_close(got[bi:bi + 1, :, sl].float(), want.float(), **tol(dtype))

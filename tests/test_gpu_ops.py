@@ -190,3 +190,85 @@ def test_error_codes(ops):
         ops.conv2d_causal(x, torch.zeros(3, 3, 3, device="cuda"), True)
     with pytest.raises(RuntimeError, match="no CPU path"):
         ops.conv2d_causal(x.cpu(), torch.zeros(2, 3, 3), True)
+
+
+# ---- the benchmark configurations at their full sizes ---------------------------------------------------------
+# Inputs are drawn on the GPU (a CPU generator needs most of a minute for 2.7e8 values).  Every channel / mixing
+# group is independent of the others, so the oracle is run on a slice (what the CPU finishes in seconds) and the
+# rest of the tensor is covered by properties that hold at any size: the identity kernel / permutation weight
+# reproduces the input bit for bit, the causal fill pattern is exact everywhere, rows of probabilities sum to 1.
+
+def _gpu_randn(shape, seed, dtype, std=1.0):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    return (std * torch.randn(*shape, generator=g, device="cuda")).to(dtype)
+
+
+def test_conv_full_size(ops):
+    """BASELINE config 2: (2,16,2048,2048) bf16, 6x11 causal."""
+    print("conv full size", flush=True)
+    n, c, s, dtype = 2, 16, 2048, torch.bfloat16
+    x = torch.tril(_gpu_randn((n, c, s, s), 20, dtype))
+    w = _randn((c, 6, 11), 21, dtype, 0.2)
+    got = ops.conv2d_causal(x, w.cuda(), True)
+    up = _upper(s, s).cuda()
+    assert (got[..., up] == 0).all() and not torch.signbit(got[..., up]).any()
+    bi, c0 = 1, 5  # oracle on two channels of the second batch element
+    want = O.depthwise_conv(x[bi:bi + 1, c0:c0 + 2].cpu().float(), w[c0:c0 + 2].float(), True).to(dtype)
+    torch.testing.assert_close(got[bi:bi + 1, c0:c0 + 2].cpu().float(), want.float(), **tol(dtype))
+    ident = ops.conv2d_causal(x, O.identity_conv_kernel(c, 6, 11, dtype).cuda(), True)
+    assert torch.equal(ident, x + 0.0)
+
+
+def test_headmix_full_size(ops):
+    """BASELINE config 3: (2,32,2048,2048) bf16, groups of 4, and the dense 32x32 weight on the same tensor."""
+    print("headmix full size", flush=True)
+    n, c, s, dtype = 2, 32, 2048, torch.bfloat16
+    x = _gpu_randn((n, c, s, s), 22, dtype)
+    g = torch.Generator().manual_seed(23)
+    up = _upper(s, s).cuda()
+    low = ~_upper(s, s)
+    for group in (4, None):
+        w = O.block_diag_head_weight(c, 4, 0.1, g, dtype) if group else (
+            torch.eye(c) + 0.1 * torch.randn(c, c, generator=g)).to(dtype)
+        got = ops.headmix(x, w.cuda(), True, 0.0, group_size=group)
+        assert (got[..., up] == 0).all() and not torch.signbit(got[..., up]).any()
+        # oracle on the second batch element: one mixing group, or all 32 heads of the first 256 query rows
+        bi = 1
+        if group:
+            sl, rows = slice(8, 12), slice(0, s)
+            want = O.head_linear(x[bi:bi + 1, sl].cpu().float(), w[sl, sl].float(), True, 0.0).to(dtype)
+        else:
+            sl, rows = slice(0, c), slice(0, 256)
+            want = O.head_linear(x[bi:bi + 1, :, rows].cpu().float(), w.float(), True, 0.0).to(dtype)
+        sub = got[bi:bi + 1, sl, rows].cpu()
+        m = low[rows]
+        torch.testing.assert_close(sub[..., m].float(), want[..., m].float(), **tol(dtype))
+    perm = torch.arange(c).roll(5)
+    wp = torch.zeros(c, c, dtype=dtype)
+    wp[torch.arange(c), perm] = 1.0
+    got = ops.headmix(x, wp.cuda(), True, 0.0)  # dense weight that only permutes the heads: bit exact
+    assert torch.equal(got, torch.tril(x[:, perm]) + 0.0)
+
+
+def test_mix_softmax_mix_full_size(ops):
+    """The score pass of BASELINE config 4: (2,16,4096,4096) bf16, groups of 4, both mixes."""
+    print("mix_softmax_mix full size", flush=True)
+    n, c, s, grp, dtype = 2, 16, 4096, 4, torch.bfloat16
+    x = _gpu_randn((n, c, s, s), 24, dtype, 2.0)
+    g = torch.Generator().manual_seed(25)
+    w1 = O.block_diag_head_weight(c, grp, 0.1, g, dtype)
+    w2 = O.block_diag_head_weight(c, grp, 0.1, g, dtype)
+    got = ops.headmix_softmax(x, w1.cuda(), w2.cuda(), True, group_size=grp)
+    # rows of probabilities sum to 1 before the second mix, so rows of the output sum to the row sums of w2
+    rs = got.float().tril().sum(-1)
+    want_rs = w2.float().sum(1)[None, :, None].cuda().expand_as(rs)
+    torch.testing.assert_close(rs, want_rs, rtol=0.0, atol=3e-2)
+    bi, sl = 1, slice(4, 8)
+    xs = x[bi:bi + 1, sl].cpu()
+    s2 = O.head_linear(xs, w1[sl, sl], True, float("-inf"))
+    p0 = torch.softmax(s2.float(), -1).to(dtype)
+    want = O.head_linear(p0, w2[sl, sl], True, 0.0)
+    sub = got[bi:bi + 1, sl].cpu()
+    up = _upper(s, s)
+    assert (sub[..., up] == 0).all()
+    torch.testing.assert_close(sub.float(), want.float(), rtol=2.0 ** -6, atol=2e-3)
