@@ -10,6 +10,8 @@
 // Rounding points of the unfused pipeline in a 16-bit dtype are reproduced: the
 // mixed scores and the probabilities are rounded to the I/O dtype before they are
 // used again.
+#include <stdlib.h>
+
 #include <type_traits>
 
 #include "common.hpp"
@@ -333,6 +335,268 @@ __global__ __launch_bounds__(NT, (NT == 256 && G * NV == 8) ? MTA_RS_OCC : 1) vo
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// 16-bit data with weights of the same dtype (or none), even group size, rows of at most 256*8*NV keys: the same
+// computation with roughly a fifth fewer vector-ALU instructions - on this kernel the SIMDs' issue slots, not the
+// memory system, are the first limit (about 14 instructions per element in the kernel above).
+//   * both mixes run on packed dot products (v_dot2c: two multiply-adds per instruction).  For the first mix the loaded
+//     vectors (8 keys of one head) are re-paired with byte permutes into (head 2j, head 2j+1) pairs of one key.
+//   * the mixed scores are kept rounded and packed (they are rounded to the I/O dtype anyway); the row maximum is
+//     taken before the rounding, which commutes with it (rounding is monotonic).
+//   * the weights are 2G*G/2 packed pairs read through wavefront-uniform addresses (scalar registers).
+//   * the number of live 2048-key passes of a wavefront (keys at or below the diagonal) selects one of NV+1 straight
+//     instantiations of each phase: no per-pass tests inside.
+//   * wavefront reductions use DPP within rows of 16 lanes.
+typedef unsigned int rs_u4 __attribute__((ext_vector_type(4)));
+
+// max(a, b, c) in one instruction (the compiler only forms it when it can rule out signalling NaNs)
+__device__ __forceinline__ float max3(float a, float b, float c)
+{
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+template <typename Op> __device__ __forceinline__ float wave_reduce(float v, Op op)
+{
+    auto dpp = [](float x, auto ctrl) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value,
+                                                                     0xf, 0xf, true));
+    };
+    v = op(v, dpp(v, std::integral_constant<int, 0xB1>{}));   // quad_perm [1,0,3,2]
+    v = op(v, dpp(v, std::integral_constant<int, 0x4E>{}));   // quad_perm [2,3,0,1]
+    v = op(v, dpp(v, std::integral_constant<int, 0x141>{}));  // row_half_mirror
+    v = op(v, dpp(v, std::integral_constant<int, 0x140>{}));  // row_mirror: every lane of a row of 16 has the row's value
+    v = op(v, __shfl_xor(v, 16));
+    v = op(v, __shfl_xor(v, 32));
+    return v;
+}
+
+template <typename T, int G, int NV, bool HAS1, bool HAS2>
+__global__ __launch_bounds__(256, (G * NV == 8) ? MTA_RS_OCC : 1) void mix_softmax_mix_packed(
+    const T *__restrict__ x, const T *__restrict__ w1, const T *__restrict__ w2, T *__restrict__ y, int C, int P, int Q,
+    int causal, int fill_upper)
+{
+    constexpr int NT = 256, VEC = 8, NW = NT / 64, H2 = G / 2;
+    static_assert(sizeof(T) == 2 && G % 2 == 0, "packed pairs of a 16-bit type");
+    __shared__ float red[2][NW * G];  // [0] maxima, [1] sums
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const unsigned groups = (unsigned)(C / G);
+    unsigned b = blockIdx.x;
+    const int p = (int)(b % (unsigned)P); b /= (unsigned)P;
+    const int g = (int)(b % groups);
+    const int64_t n = b / groups;
+    const int64_t plane = (int64_t)P * Q;
+    const int64_t base = (n * C + (int64_t)g * G) * plane + (int64_t)p * Q;
+    const int last = causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;  // last attended key
+
+    // live passes of this wavefront: pass k covers keys [(k*NT + 64*wave)*VEC, +64*VEC)
+    int nlive = 0;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) nlive += ((k * NT + wave * 64) * VEC <= last) ? 1 : 0;
+
+    // packed weights, (w[o][2j], w[o][2j+1]); identical for all lanes
+    uint32_t w1p[G][H2], w2p[G][H2];
+#pragma unroll
+    for (int o = 0; o < G; ++o)
+#pragma unroll
+        for (int j = 0; j < H2; ++j) {
+            const int64_t widx = (int64_t)(g * G + o) * C + g * G + 2 * j;
+            w1p[o][j] = HAS1 ? *reinterpret_cast<const uint32_t *>(w1 + widx) : 0u;
+            w2p[o][j] = HAS2 ? *reinterpret_cast<const uint32_t *>(w2 + widx) : 0u;
+        }
+
+    // One straight instantiation per (number of live passes L, whether the last of them straddles the last attended
+    // key): masks exist only in the EDGE instantiations and only for pass L-1 (an earlier pass lies wholly below the
+    // diagonal).  The two workgroup barriers sit inside the instantiations - every wavefront passes exactly two.
+    auto run = [&](auto live_tag, auto edge_tag) __attribute__((always_inline)) {
+        constexpr int L = decltype(live_tag)::value;
+        constexpr bool EDGE = decltype(edge_tag)::value;
+        constexpr int LL = L > 0 ? L : 1;
+        uint32_t sp[G][LL][VEC / 2];  // mixed scores, rounded, two keys per register
+        float m[G], inv[G];
+
+        // ---- load, first mix, running maximum, round and pack ----
+        {
+            rs_u4 xin[LL][G];
+#pragma unroll
+            for (int k = 0; k < L; ++k) {
+                const int q = (k * NT + tid) * VEC;
+                const int qs = (!EDGE || k < L - 1 || q <= last) ? q : 0;  // beyond the attended keys: re-read the row start
+#pragma unroll
+                for (int i = 0; i < G; ++i)
+                    xin[k][i] = __builtin_nontemporal_load(reinterpret_cast<const rs_u4 *>(x + base + i * plane + qs));
+            }
+#pragma unroll
+            for (int o = 0; o < G; ++o) m[o] = -INFINITY;
+#pragma unroll
+            for (int k = 0; k < L; ++k) {
+                const int q = (k * NT + tid) * VEC;
+#pragma unroll
+                for (int d = 0; d < VEC / 2; ++d) {
+                    float a[G][2];
+                    if constexpr (HAS1) {
+                        uint32_t lo[H2], hi[H2];  // (head 2j, head 2j+1) of key 2d and of key 2d+1
+#pragma unroll
+                        for (int j = 0; j < H2; ++j) {
+                            lo[j] = __builtin_amdgcn_perm(xin[k][2 * j + 1][d], xin[k][2 * j][d], 0x05040100u);
+                            hi[j] = __builtin_amdgcn_perm(xin[k][2 * j + 1][d], xin[k][2 * j][d], 0x07060302u);
+                        }
+#pragma unroll
+                        for (int o = 0; o < G; ++o) {
+                            a[o][0] = 0.0f;
+                            a[o][1] = 0.0f;
+#pragma unroll
+                            for (int j = 0; j < H2; ++j) {
+                                a[o][0] = dot2<T>(lo[j], w1p[o][j], a[o][0]);
+                                a[o][1] = dot2<T>(hi[j], w1p[o][j], a[o][1]);
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (int o = 0; o < G; ++o) unpack2<T>(xin[k][o][d], a[o][0], a[o][1]);
+                    }
+                    if (EDGE && k == L - 1) {
+#pragma unroll
+                        for (int o = 0; o < G; ++o) {
+                            if (q + 2 * d > last) a[o][0] = -INFINITY;
+                            if (q + 2 * d + 1 > last) a[o][1] = -INFINITY;
+                        }
+                    }
+#pragma unroll
+                    for (int o = 0; o < G; ++o) {
+                        m[o] = max3(m[o], a[o][0], a[o][1]);
+                        sp[o][k][d] = (HAS1 || (EDGE && k == L - 1)) ? pack2<T>(a[o][0], a[o][1]) : xin[k][o][d];
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int o = 0; o < G; ++o) {
+            const float v = wave_reduce(m[o], [](float a_, float b_) { return fmaxf(a_, b_); });
+            if (lane == 0) red[0][wave * G + o] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int o = 0; o < G; ++o) {
+            float v = red[0][o];
+#pragma unroll
+            for (int i = 1; i < NW; ++i) v = fmaxf(v, red[0][i * G + o]);
+            // the maximum of the rounded scores is the rounded maximum (the row's first key is always attended: finite)
+            float dummy = v;
+            if constexpr (HAS1) round_pair<T>(v, dummy);
+            m[o] = v;
+        }
+
+        // ---- exp(s - max) = exp2(s*log2(e) - max*log2(e)), running sum ----
+        float e[G][LL][VEC];
+        constexpr float LOG2E = 1.4426950408889634f;
+#pragma unroll
+        for (int o = 0; o < G; ++o) {
+            const float mneg = -m[o] * LOG2E;
+            float acc = 0.0f;
+#pragma unroll
+            for (int k = 0; k < L; ++k)
+#pragma unroll
+                for (int d = 0; d < VEC / 2; ++d) {
+                    float s0, s1;
+                    unpack2<T>(sp[o][k][d], s0, s1);
+                    e[o][k][2 * d] = __builtin_amdgcn_exp2f(fmaf(s0, LOG2E, mneg));
+                    e[o][k][2 * d + 1] = __builtin_amdgcn_exp2f(fmaf(s1, LOG2E, mneg));
+                    acc += e[o][k][2 * d];
+                    acc += e[o][k][2 * d + 1];
+                }
+            const float v = wave_reduce(acc, [](float a_, float b_) { return a_ + b_; });
+            if (lane == 0) red[1][wave * G + o] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int o = 0; o < G; ++o) {
+            float v = red[1][o];
+#pragma unroll
+            for (int i = 1; i < NW; ++i) v += red[1][i * G + o];
+            inv[o] = 1.0f / v;
+        }
+
+        // ---- normalise, round in pairs of heads, second mix, store ----
+#pragma unroll
+        for (int k = 0; k < L; ++k) {
+            const int q = (k * NT + tid) * VEC;
+            if (EDGE && k == L - 1 && (q >= Q || (!fill_upper && q > last))) continue;  // wholly above: +0 only on request
+            uint32_t out[G][VEC / 2];
+            if constexpr (HAS2) {
+#pragma unroll
+                for (int d = 0; d < VEC / 2; ++d) {
+                    uint32_t pp[H2][2];  // probabilities of heads (2j, 2j+1) at keys 2d and 2d+1, rounded
+#pragma unroll
+                    for (int j = 0; j < H2; ++j)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h)
+                            pp[j][h] = pack2<T>(e[2 * j][k][2 * d + h] * inv[2 * j], e[2 * j + 1][k][2 * d + h] * inv[2 * j + 1]);
+#pragma unroll
+                    for (int o = 0; o < G; ++o) {
+                        float r0 = 0.0f, r1 = 0.0f;
+#pragma unroll
+                        for (int j = 0; j < H2; ++j) {
+                            r0 = dot2<T>(w2p[o][j], pp[j][0], r0);
+                            r1 = dot2<T>(w2p[o][j], pp[j][1], r1);
+                        }
+                        out[o][d] = pack2<T>(r0, r1);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int o = 0; o < G; ++o)
+#pragma unroll
+                    for (int d = 0; d < VEC / 2; ++d)
+                        out[o][d] = pack2<T>(e[o][k][2 * d] * inv[o], e[o][k][2 * d + 1] * inv[o]);
+            }
+            if (EDGE && k == L - 1) {  // +0 beyond the last attended key
+#pragma unroll
+                for (int o = 0; o < G; ++o)
+#pragma unroll
+                    for (int d = 0; d < VEC / 2; ++d) {
+                        if (q + 2 * d > last) out[o][d] &= 0xffff0000u;
+                        if (q + 2 * d + 1 > last) out[o][d] &= 0x0000ffffu;
+                    }
+            }
+#pragma unroll
+            for (int o = 0; o < G; ++o) {
+                const rs_u4 v = {out[o][0], out[o][1], out[o][2], out[o][3]};
+                __builtin_nontemporal_store(v, reinterpret_cast<rs_u4 *>(y + base + o * plane + q));
+            }
+        }
+        if (fill_upper) {  // passes wholly above the diagonal
+#pragma unroll
+            for (int k = L; k < NV; ++k) {
+                const int q = (k * NT + tid) * VEC;
+                if (q >= Q) continue;
+                const rs_u4 z = {0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int o = 0; o < G; ++o) __builtin_nontemporal_store(z, reinterpret_cast<rs_u4 *>(y + base + o * plane + q));
+            }
+        }
+    };
+    // does the last live pass reach beyond the last attended key?
+    const bool edge = nlive > 0 && ((nlive - 1) * NT + wave * 64 + 64) * VEC - 1 > last;
+    static_assert(NV <= 4, "live-pass dispatch");
+    using std::integral_constant;
+    if (nlive == 0) {
+        run(integral_constant<int, 0>{}, std::false_type{});
+    } else if (edge) {
+        if (nlive == 1) run(integral_constant<int, 1>{}, std::true_type{});
+        if constexpr (NV >= 2) { if (nlive == 2) run(integral_constant<int, 2>{}, std::true_type{}); }
+        if constexpr (NV >= 3) { if (nlive == 3) run(integral_constant<int, 3>{}, std::true_type{}); }
+        if constexpr (NV >= 4) { if (nlive == 4) run(integral_constant<int, 4>{}, std::true_type{}); }
+    } else {
+        if (nlive == 1) run(integral_constant<int, 1>{}, std::false_type{});
+        if constexpr (NV >= 2) { if (nlive == 2) run(integral_constant<int, 2>{}, std::false_type{}); }
+        if constexpr (NV >= 3) { if (nlive == 3) run(integral_constant<int, 3>{}, std::false_type{}); }
+        if constexpr (NV >= 4) { if (nlive == 4) run(integral_constant<int, 4>{}, std::false_type{}); }
+    }
+}
+
 // Any row length / any group size: three sweeps over the row, inputs re-read (and re-mixed)
 // in each; scalar accesses.  Correctness fallback for ragged or very long rows.
 template <typename T, int NT>
@@ -406,6 +670,31 @@ int dispatch(const void *x, const void *w1, const void *w2, void *y, int64_t N, 
     constexpr int VEC = vec_of<T>::n;
     const bool vec_ok = (Q % VEC == 0) && aligned_to(x, 16) && aligned_to(y, 16);
     const int64_t nv = (Q + 256 * VEC - 1) / (256 * VEC);
+    if constexpr (sizeof(T) == 2) {
+        // 16-bit data, weights of the same dtype: the packed kernel (MTA_SOFTMAX_NO_PACKED=1 in the environment keeps
+        // the general one, for comparisons)
+        static const bool no_packed = [] { const char *e_ = getenv("MTA_SOFTMAX_NO_PACKED"); return e_ && e_[0] == '1'; }();
+        const int io_code = std::is_same<T, bf16_t>::value ? MTA_BF16 : MTA_F16;
+        if (vec_ok && !no_packed && w_dtype == io_code && (w1 || w2) && (!w1 || aligned_to(w1, 4)) &&
+            (!w2 || aligned_to(w2, 4)) && C % 2 == 0 && Q <= 256 * VEC * 4) {
+#define MTA_RSP_LAUNCH(g, v, h1, h2)                                                                                   \
+    {                                                                                                                  \
+        hipLaunchKernelGGL((mix_softmax_mix_packed<T, g, v, h1, h2>), dim3((unsigned)(N * (C / g) * P)), dim3(256), 0, \
+                           st, (const T *)x, (const T *)w1, (const T *)w2, (T *)y, (int)C, (int)P, (int)Q, causal,     \
+                           fill_upper);                                                                                \
+        return launch_status();                                                                                        \
+    }
+#define MTA_RSP_CASE(g, v)                                                                                             \
+    if (G == g && nv <= v) {                                                                                           \
+        if (w1 && w2) MTA_RSP_LAUNCH(g, v, true, true)                                                                 \
+        if (w1) MTA_RSP_LAUNCH(g, v, true, false)                                                                      \
+        MTA_RSP_LAUNCH(g, v, false, true)                                                                              \
+    }
+            MTA_RSP_CASE(2, 1) MTA_RSP_CASE(2, 2) MTA_RSP_CASE(2, 4) MTA_RSP_CASE(4, 1) MTA_RSP_CASE(4, 2) MTA_RSP_CASE(8, 1)
+#undef MTA_RSP_CASE
+#undef MTA_RSP_LAUNCH
+        }
+    }
     if (vec_ok) {
 #define MTA_RS_CASE(g, v)                                                                   \
     if (G == g && nv <= v) return launch_fixed<T, g, v>(x, w1, w2, y, N, C, P, Q, causal, w_dtype, fill_upper, st);

@@ -153,10 +153,13 @@ MS_CASES = [
     # N, C, P(=Q), group, use_w1, use_w2
     (1, 4, 64, 2, True, True), (2, 4, 100, 4, True, False), (1, 8, 257, 4, False, True), (1, 2, 33, 1, False, False),
     (1, 8, 2048, 4, True, True), (1, 3, 50, 3, True, True), (1, 8, 72, 8, True, True), (1, 4, 4096, 4, True, True),
+    # packed-arithmetic kernel (16-bit data): one weight only, several passes with few heads, rows that end inside
+    # a wavefront's pass / exactly on its boundary (2560 = 5 x 512), rectangular
+    (1, 4, 3000, 4, False, True), (1, 4, 2560, 4, True, False), (1, 2, 6000, 2, True, True), (1, 8, 520, 8, False, True),
 ]
 
 
-@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("case", MS_CASES)
 def test_mix_softmax_mix_parity(ops, case, causal, dt):
