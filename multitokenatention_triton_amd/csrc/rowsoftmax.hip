@@ -349,7 +349,8 @@ __global__ __launch_bounds__(NT, (NT == 256 && G * NV == 8) ? MTA_RS_OCC : 1) vo
 //   * wavefront reductions use DPP within rows of 16 lanes.
 typedef unsigned int rs_u4 __attribute__((ext_vector_type(4)));
 
-// max(a, b, c) in one instruction (the compiler only forms it when it can rule out signalling NaNs)
+// max(a, b, c) in one instruction (the compiler only forms it when it can rule out signalling NaNs).  Only for
+// operands produced by ordinary vector-ALU instructions or loads.
 __device__ __forceinline__ float max3(float a, float b, float c)
 {
     float r;
@@ -357,20 +358,48 @@ __device__ __forceinline__ float max3(float a, float b, float c)
     return r;
 }
 
-template <typename Op> __device__ __forceinline__ float wave_reduce(float v, Op op)
+// max(a, b) without the compiler's canonicalisation of the inputs (no NaNs reach these reductions)
+__device__ __forceinline__ float max_raw(float a, float b)
 {
-    auto dpp = [](float x, auto ctrl) {
-        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value,
-                                                                     0xf, 0xf, true));
-    };
-    v = op(v, dpp(v, std::integral_constant<int, 0xB1>{}));   // quad_perm [1,0,3,2]
-    v = op(v, dpp(v, std::integral_constant<int, 0x4E>{}));   // quad_perm [2,3,0,1]
-    v = op(v, dpp(v, std::integral_constant<int, 0x141>{}));  // row_half_mirror
-    v = op(v, dpp(v, std::integral_constant<int, 0x140>{}));  // row_mirror: every lane of a row of 16 has the row's value
-    v = op(v, __shfl_xor(v, 16));
-    v = op(v, __shfl_xor(v, 32));
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+// Wavefront-wide reduction, result in every lane: four DPP steps inside rows of 16 lanes (the operand permuted on the
+// way into the ALU; the two wait states a DPP read of a just-written register needs are part of the asm), then two
+// exchanges across rows.
+#define MTA_RS_DPP_STEP(op, ctrl) asm("s_nop 1\n\t" op "_dpp %0, %1, %1 " ctrl " row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v)); v = r;
+// The same for operands that dot-product instructions may just have written: a different vector-ALU instruction
+// may read such a register only three wait states later, and the compiler, which inserts those for its own
+// instructions, cannot see into the assembly.
+__device__ __forceinline__ float max3_after_dot(float a, float b, float c)
+{
+    float r;
+    asm("s_nop 2\n\tv_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+template <bool IS_MAX> __device__ __forceinline__ float wave_reduce(float v)
+{
+    float r;
+    if constexpr (IS_MAX) {
+        MTA_RS_DPP_STEP("v_max_f32", "quad_perm:[1,0,3,2]")
+        MTA_RS_DPP_STEP("v_max_f32", "quad_perm:[2,3,0,1]")
+        MTA_RS_DPP_STEP("v_max_f32", "row_half_mirror")
+        MTA_RS_DPP_STEP("v_max_f32", "row_mirror")
+        v = max_raw(v, __shfl_xor(v, 16));
+        v = max_raw(v, __shfl_xor(v, 32));
+    } else {
+        MTA_RS_DPP_STEP("v_add_f32", "quad_perm:[1,0,3,2]")
+        MTA_RS_DPP_STEP("v_add_f32", "quad_perm:[2,3,0,1]")
+        MTA_RS_DPP_STEP("v_add_f32", "row_half_mirror")
+        MTA_RS_DPP_STEP("v_add_f32", "row_mirror")
+        v += __shfl_xor(v, 16);
+        v += __shfl_xor(v, 32);
+    }
     return v;
 }
+#undef MTA_RS_DPP_STEP
 
 template <typename T, int G, int NV, bool HAS1, bool HAS2>
 __global__ __launch_bounds__(256, (G * NV == 8) ? MTA_RS_OCC : 1) void mix_softmax_mix_packed(
@@ -466,7 +495,7 @@ __global__ __launch_bounds__(256, (G * NV == 8) ? MTA_RS_OCC : 1) void mix_softm
                     }
 #pragma unroll
                     for (int o = 0; o < G; ++o) {
-                        m[o] = max3(m[o], a[o][0], a[o][1]);
+                        m[o] = HAS1 ? max3_after_dot(m[o], a[o][0], a[o][1]) : max3(m[o], a[o][0], a[o][1]);
                         sp[o][k][d] = (HAS1 || (EDGE && k == L - 1)) ? pack2<T>(a[o][0], a[o][1]) : xin[k][o][d];
                     }
                 }
@@ -474,7 +503,7 @@ __global__ __launch_bounds__(256, (G * NV == 8) ? MTA_RS_OCC : 1) void mix_softm
         }
 #pragma unroll
         for (int o = 0; o < G; ++o) {
-            const float v = wave_reduce(m[o], [](float a_, float b_) { return fmaxf(a_, b_); });
+            const float v = wave_reduce<true>(m[o]);
             if (lane == 0) red[0][wave * G + o] = v;
         }
         __syncthreads();
@@ -482,7 +511,7 @@ __global__ __launch_bounds__(256, (G * NV == 8) ? MTA_RS_OCC : 1) void mix_softm
         for (int o = 0; o < G; ++o) {
             float v = red[0][o];
 #pragma unroll
-            for (int i = 1; i < NW; ++i) v = fmaxf(v, red[0][i * G + o]);
+            for (int i = 1; i < NW; ++i) v = max_raw(v, red[0][i * G + o]);
             // the maximum of the rounded scores is the rounded maximum (the row's first key is always attended: finite)
             float dummy = v;
             if constexpr (HAS1) round_pair<T>(v, dummy);
@@ -507,7 +536,7 @@ __global__ __launch_bounds__(256, (G * NV == 8) ? MTA_RS_OCC : 1) void mix_softm
                     acc += e[o][k][2 * d];
                     acc += e[o][k][2 * d + 1];
                 }
-            const float v = wave_reduce(acc, [](float a_, float b_) { return a_ + b_; });
+            const float v = wave_reduce<false>(acc);
             if (lane == 0) red[1][wave * G + o] = v;
         }
         __syncthreads();
