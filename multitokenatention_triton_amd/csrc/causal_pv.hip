@@ -40,6 +40,18 @@ constexpr int P_BK = MTA_PV_BK;  // keys per iteration: each lane reads P_BK/4 c
                                  // iteration, back to back, so that DRAM pages are used in long runs
 constexpr int P_KS = P_BK / 32;  // 32-key contraction steps per iteration
 
+// Swizzle of a V block in LDS: row `key` stores its 16-byte chunk c at position c ^ v_swizzle(key).  A transpose read
+// touches, per group of 16 lanes, 32 contiguous bytes (8 banks) of each of 4 consecutive keys, and groups are 8 keys
+// apart: the keys {0..3, 8..11} (+4, +16) that may be served in one cycle must land in 8 different 8-bank regions.
+// D = 128 (a row is all 64 banks): region = chunk pair ^ (key%4 + 4*bit 3 of key).  D = 64 (a row is 32 banks, odd keys
+// take the other half): region = chunk pair ^ (bit 1 + 2*bit 3 of key).  (XOR with the plain key index put keys 2k and
+// 2k+1 into the same region: every transpose read took a two-way bank conflict.)
+template <int D> __device__ __forceinline__ int v_swizzle(int key)
+{
+    if constexpr (D == 128) return 2 * ((key & 3) | ((key >> 1) & 4));
+    else return 2 * (((key >> 1) & 1) | ((key >> 2) & 2));
+}
+
 template <typename T, int D>
 __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__restrict__ P, const T *__restrict__ V,
                                                            T *__restrict__ O, int S, int causal, int nqb, int64_t total_wg,
@@ -81,7 +93,7 @@ __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__
         for (int r = 0; r < ROUNDS; ++r) {
             const int slot = r * P_NT + tid;
             if (TILE / 8 % P_NT != 0 && slot >= TILE / 8) break;
-            const int row = slot / CPR, c = (slot % CPR) ^ (row & (CPR - 1));
+            const int row = slot / CPR, c = (slot % CPR) ^ v_swizzle<D>(row);
             int vr = j * P_BK + row;
             vr = vr >= S ? S - 1 : vr;
             __builtin_amdgcn_global_load_lds((glb_void_t *)(Vp + (int64_t)vr * D + c * 8),
@@ -151,23 +163,30 @@ __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__
                         if (key0 + t > lim) pf[rb][ks].v[t] = from_float<T>(0.0f);
                 }
             }
-#pragma unroll
-        for (int ks = 0; ks < P_KS; ++ks) {
+        // V^T fragments of block blk = ks*DB + db are read from LDS while the matrix cores work on block blk-1 (left to
+        // itself the compiler issues read, wait, product, read, wait, ... : an LDS latency per group of products)
+        auto load_vf = [&](int blk, frag8<T> &dst) {
+            const int ks = blk / DB, db = blk % DB;
             const int key_a = ks * 32 + kg * 8 + (ln >> 2);  // slots 0..3: keys 8kg+(0..3); slots 4..7: +4
             const int key_b = key_a + 4;
+            const int ch = db * 2 + ((ln & 3) >> 1);
+            const int sub = (ln & 1) * 4;
+            const T *pa = Vb + key_a * D + ((ch ^ v_swizzle<D>(key_a)) * 8) + sub;
+            const T *pb = Vb + key_b * D + ((ch ^ v_swizzle<D>(key_b)) * 8) + sub;
+            struct { v4s_t a, b; } both = {__builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)pa),
+                                           __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)pb)};
+            dst = __builtin_bit_cast(frag8<T>, both);
+        };
+        frag8<T> vf[2];
+        load_vf(0, vf[0]);
 #pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                const int ch = db * 2 + ((ln & 3) >> 1);
-                const int sub = (ln & 1) * 4;
-                const T *pa = Vb + key_a * D + ((ch ^ (key_a & (CPR - 1))) * 8) + sub;
-                const T *pb = Vb + key_b * D + ((ch ^ (key_b & (CPR - 1))) * 8) + sub;
-                const v4s_t va = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)pa);
-                const v4s_t vb = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)pb);
-                struct { v4s_t a, b; } both = {va, vb};
-                const frag8<T> vf = __builtin_bit_cast(frag8<T>, both);
-                mma16(oacc[0][db], vf, pf[0][ks]);
-                mma16(oacc[1][db], vf, pf[1][ks]);
-            }
+        for (int blk = 0; blk < P_KS * DB; ++blk) {
+            const int ks = blk / DB, db = blk % DB;
+            if (blk + 1 < P_KS * DB) load_vf(blk + 1, vf[(blk + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);  // (the instruction scheduler would move the reads back behind the products)
+            mma16(oacc[0][db], vf[blk & 1], pf[0][ks]);
+            mma16(oacc[1][db], vf[blk & 1], pf[1][ks]);
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
     for (int j = 0;;) {

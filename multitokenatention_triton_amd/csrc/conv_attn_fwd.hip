@@ -302,6 +302,19 @@ typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
 // The workgroup has NW wavefronts and owns 32*NW score rows: 8 for the attention kernel (one workgroup per CU,
 // K and V blocks shared by 256 rows), 4 for the scores-only kernel (two workgroups per CU, which overlap each
 // other's barriers and memory latency).
+// The kernels read the LDS operands of the next group of matrix products before they issue the current group.  The
+// instruction scheduler largely undoes that (it moves reads down towards their use, which saves registers).  Pinning
+// the source order (matrix products and LDS accesses may not cross the marked points) was measured and is slower -
+// scores-only kernel 0.320 -> 0.340 ms, attention kernel 1.60 -> 1.72 ms at the benchmark shapes, with 12-14 spilled
+// registers - so it stays off: these kernels are not bound by the LDS latency in front of each product.
+#ifndef MTA_FUSED_PIN
+#define MTA_FUSED_PIN 0
+#endif
+#if MTA_FUSED_PIN
+#define MTA_PIN_ORDER() __builtin_amdgcn_sched_barrier(0x6)
+#else
+#define MTA_PIN_ORDER() ((void)0)
+#endif
 constexpr int F_BK = 64;   // keys per iteration
 #ifndef MTA_QK_OCC
 #define MTA_QK_OCC 3       // wavefronts per SIMD the scores-only kernel is compiled for (three workgroups per CU)
@@ -516,12 +529,14 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb) {
                 if (cb + 1 < NCB) load_kf(cb + 1, kf[(cb + 1) & 1]);
+                MTA_PIN_ORDER();
                 f32x4 sacc[2] = {f32x4{0.0f, 0.0f, 0.0f, 0.0f}, f32x4{0.0f, 0.0f, 0.0f, 0.0f}};
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     mma16(sacc[0], kf[cb & 1][ks], qf[0][ks]);
                     mma16(sacc[1], kf[cb & 1][ks], qf[1][ks]);
                 }
+                MTA_PIN_ORDER();
                 // key block wholly inside the sequence and on or below the diagonal for all 32 rows: no masks
                 const bool s_plain = PLAIN || (cbase + cb * 16 >= 0 && cbase + cb * 16 + 16 <= S && (!causal || cbase + cb * 16 + 15 <= pmin));
 #pragma unroll
@@ -576,9 +591,11 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
             for (int blk = 0; blk < 2 * NCB; ++blk) {
                 const int rb = blk / NCB, cb = blk % NCB;
                 if (blk + 1 < 2 * NCB) load_xf(blk + 1, xf[(blk + 1) & 1]);
+                MTA_PIN_ORDER();
                 f32x4 cacc = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int i = 0; i < R; ++i) mma16(cacc, tz[i], xf[blk & 1][i]);
+                MTA_PIN_ORDER();
                 uint32_t lo = pack2<T>(cacc[0], cacc[1]), hi = pack2<T>(cacc[2], cacc[3]);
                 if (!PLAIN && causal && j * F_BK + cb * 16 + 15 > pmin) {  // block touches the diagonal for some row
                     const int col = j * F_BK + cb * 16 + kg * 4;
@@ -617,9 +634,11 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
                 for (int cb = 0; cb < NCB; ++cb) {
                     const int blk = rb * NCB + cb;
                     if (blk + 1 < 2 * NCB) load_xf(blk + 1, xf[(blk + 1) & 1]);
+                    MTA_PIN_ORDER();
                     f32x4 cacc = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                     for (int i = 0; i < R; ++i) mma16(cacc, tz[i], xf[blk & 1][i]);
+                    MTA_PIN_ORDER();
                     // conv output and scaled logits are rounded to the I/O dtype, as the unfused pipeline stores them
                     float a[4];
                     unpack2<T>(pack2<T>(cacc[0], cacc[1]), a[0], a[1]);
@@ -685,8 +704,10 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
             for (int blk = 0; blk < 2 * DB; ++blk) {
                 const int ks = blk / DB, db = blk % DB;
                 if (blk + 1 < 2 * DB) load_vf(blk + 1, vf[(blk + 1) & 1]);
+                MTA_PIN_ORDER();
                 mma16(oacc[0][db], vf[blk & 1], pf[0][ks]);
                 mma16(oacc[1][db], vf[blk & 1], pf[1][ks]);
+                MTA_PIN_ORDER();
             }
         }
     };
