@@ -274,6 +274,19 @@ template <int N> __device__ __forceinline__ void lds_wait_all(u32x4 (&a)[N])
     else if constexpr (N == 7) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]) : : "memory");
     else static_assert(N == 3 || N == 5 || N == 6 || N == 7, "add a case");
 }
+// Wait until at most NEWER LDS operations issued after the 2*N loads of `a` are outstanding (LDS operations complete
+// in order), and tie the loaded values to that point.
+template <int NEWER, int N> __device__ __forceinline__ void lds_wait_pair(u32x4 (&a)[2][N])
+{
+    static_assert(N >= 1 && N <= 7 && NEWER >= 0 && NEWER <= 15, "operand count / counter width");
+#define MTA_TIE2(i) "+v"(a[0][i]), "+v"(a[1][i])
+    if constexpr (N == 3) asm volatile("s_waitcnt lgkmcnt(%6)" : MTA_TIE2(0), MTA_TIE2(1), MTA_TIE2(2) : "n"(NEWER) : "memory");
+    else if constexpr (N == 5) asm volatile("s_waitcnt lgkmcnt(%10)" : MTA_TIE2(0), MTA_TIE2(1), MTA_TIE2(2), MTA_TIE2(3), MTA_TIE2(4) : "n"(NEWER) : "memory");
+    else if constexpr (N == 6) asm volatile("s_waitcnt lgkmcnt(%12)" : MTA_TIE2(0), MTA_TIE2(1), MTA_TIE2(2), MTA_TIE2(3), MTA_TIE2(4), MTA_TIE2(5) : "n"(NEWER) : "memory");
+    else if constexpr (N == 7) asm volatile("s_waitcnt lgkmcnt(%14)" : MTA_TIE2(0), MTA_TIE2(1), MTA_TIE2(2), MTA_TIE2(3), MTA_TIE2(4), MTA_TIE2(5), MTA_TIE2(6) : "n"(NEWER) : "memory");
+    else static_assert(N == 3 || N == 5 || N == 6 || N == 7, "add a case");
+#undef MTA_TIE2
+}
 __device__ __forceinline__ void lds_wait(u32x4 &a) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a) : : "memory"); }
 __device__ __forceinline__ void lds_wait(u32x4 &a, u32x4 &b, u32x4 &c)
 {
@@ -355,7 +368,20 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
         const int h0 = p0_ - (R - 1), k0 = q0_ - G::HL;
         return h0 >= 0 && p0_ + M_TM <= H && k0 >= 0 && k0 + G::TW <= W && (!causal || k0 + G::TW - 1 <= h0);
     };
-    // asynchronous copy of an interior strip into LDS buffer `buf`
+    // A strip is `copyable` when the same copy can be issued for it without faulting: its rows lie inside the plane
+    // and the bytes its slots address (left halo of the first column strip = tail of the previous row, right halo of
+    // the last one = head of the next row) lie inside the tensor.  What such a copy brings in from outside the plane
+    // or from above the diagonal is zeroed in LDS afterwards (diagonal and border strips: a quarter of all strips,
+    // which would otherwise load synchronously through registers).
+    const int64_t total_elems = (int64_t)(total / ipp) * H * W;  // planes * H * W
+    auto is_copyable = [&](int64_t plane_, int p0_, int q0_) {
+        if (SCALED) return false;
+        const int h0 = p0_ - (R - 1), k0 = q0_ - G::HL;
+        if (h0 < 0 || p0_ + M_TM > H) return false;
+        const int64_t e0 = plane_ * (int64_t)H * W + (int64_t)h0 * W + k0;
+        return e0 >= 0 && e0 + (int64_t)(G::ROWS - 1) * W + G::TW <= total_elems;
+    };
+    // asynchronous copy of an interior or copyable strip into LDS buffer `buf`
     auto prefetch = [&](int64_t plane_, int p0_, int q0_, T *buf) {
         const char *base = reinterpret_cast<const char *>(x + plane_ * (int64_t)H * W + (int64_t)(p0_ - (R - 1)) * W + (q0_ - G::HL));
 #pragma unroll
@@ -363,10 +389,30 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
             __builtin_amdgcn_global_load_lds((glb_void_t *)(base + goff[it]), (lds_void_t *)(buf + it * M_WT * VEC), 16, 0, 0);
     };
 
+    // The (zero-padded) kernel rows of a strip's channel are fetched one strip ahead into WPL registers per lane and
+    // written to `wz` at the top of that strip's iteration: the items of a plane are dealt out over all workgroups of
+    // an XCD, so a wavefront changes channel every few strips, and a fetch at the point of use would expose a full
+    // memory latency each time.  The loads are issued from inline assembly, before the strip's copy, and are covered
+    // by the wait for that copy at the top of the next iteration: seen by the compiler, they would make it wait for
+    // every outstanding memory operation - the previous strip's stores included - before the values' first use.
+    constexpr int WPL = (R * WZ_LD + M_WT - 1) / M_WT;
+    static_assert(sizeof(T) == 2, "16-bit loads");
+    unsigned wnext[WPL];
+    auto fetch_weights = [&](int channel_) {
+#pragma unroll
+        for (int it = 0; it < WPL; ++it) {
+            const int e = it * M_WT + lane;
+            const int i = e / WZ_LD, j = e % WZ_LD - WZ_OFF;
+            const bool ok = e < R * WZ_LD && j >= 0 && j < S;
+            const T *src = w + channel_ * R * S + (ok ? i * S + j : 0);
+            asm volatile("global_load_ushort %0, %1, off" : "=v"(wnext[it]) : "v"(src) : "memory");
+        }
+    };
     int64_t plane;
     int tm, tn;
     decode_item(first, ipp, tiles_n, mirror, plane, tm, tn);
-    if (DBUF && is_interior(tm * M_TM, tn * M_TN)) prefetch(plane, tm * M_TM, tn * M_TN, tiles);
+    fetch_weights((int)(plane % C));
+    if (DBUF && is_copyable(plane, tm * M_TM, tn * M_TN)) prefetch(plane, tm * M_TM, tn * M_TN, tiles);
 
     int younger = -1;                      // stores certainly issued after the copy in flight (-1: unknown)
     const bool fill_full = H % M_TN == 0;  // mirror images of whole 128x128 blocks lie inside the (square) tensor
@@ -381,6 +427,7 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
         const int channel = (int)(plane % C);
         const bool above = causal && q0 > p0 + M_TM - 1;  // wholly above the diagonal (only reachable when !mirror)
         const bool interior = is_interior(p0, q0);
+        const bool copyable = interior || is_copyable(plane, p0, q0);
         const int h0 = p0 - (R - 1), k0 = q0 - G::HL;
         // (opaque: the addresses derived from it are then formed where they are used instead of being kept, dozens of
         // them, in registers across the loop)
@@ -396,22 +443,56 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
         } else {
             // one buffer: this strip's copy is issued now and waited for (the other wavefronts of the CU cover the
             // latency); the previous strip's LDS reads are complete
-            if (interior) prefetch(plane, p0, q0, tile);
+            if (copyable) prefetch(plane, p0, q0, tile);
             asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
         }
         younger = 0;
 
+        // this strip's kernel rows, fetched during the previous iteration, go to LDS (every strip: see fetch_weights)
+#pragma unroll
+        for (int it = 0; it < WPL; ++it) {
+            asm volatile("" : "+v"(wnext[it]));  // (the value is defined from the wait above on)
+            const int e = it * M_WT + lane;
+            const int j = e % WZ_LD - WZ_OFF;
+            if (e < R * WZ_LD) wz[e] = (j >= 0 && j < S) ? __builtin_bit_cast(T, (unsigned short)wnext[it]) : from_float<T>(0.0f);
+        }
+
         // put the next strip's copy in flight (into the buffer the previous iteration has just released)
         if (idx + step < last) {
             decode_item(idx + step, ipp, tiles_n, mirror, plane, tm, tn);
-            if (DBUF && is_interior(tm * M_TM, tn * M_TN)) prefetch(plane, tm * M_TM, tn * M_TN, other);
+            fetch_weights((int)(plane % C));  // (before the copy: the loop-top wait counts what is younger than the copy)
+            if (DBUF && is_copyable(plane, tm * M_TM, tn * M_TN)) prefetch(plane, tm * M_TM, tn * M_TN, other);
         }
         if (above) {
             zero_fill_strip<T>(yp, H, W, p0, q0, lane);
             younger = -1;
             continue;
         }
-        if (!interior) {
+        if (copyable && !interior) {
+            // the copy has landed: zero what lies outside the plane or above the diagonal (whole vectors, except the one
+            // vector of a row that straddles the diagonal)
+            const int lane_ = opaque(lane);
+            const u32x4 zero4 = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int it = 0; it < STAGE_IT; ++it) {
+                const int slot = it * M_WT + lane_;
+                const int rr = slot / SPR, vc = slot % SPR;
+                const int h = h0 + rr, col = k0 + vc * VEC;
+                const bool ok = rr < G::ROWS && vc < VPR && col >= 0 && col < W && !(causal && col > h);
+                const unsigned addr = tile_lds + (unsigned)slot * 16u;
+                if (!ok) {
+                    lds_store16(addr, zero4);
+                } else if (causal && col + VEC - 1 > h) {
+                    u32x4 raw = lds_load16(addr);
+                    lds_wait(raw);
+                    V16 v = __builtin_bit_cast(V16, raw);
+#pragma unroll
+                    for (int u = 0; u < VEC; ++u)
+                        if (col + u > h) v.v[u] = from_float<T>(0.0f);
+                    lds_store16(addr, __builtin_bit_cast(u32x4, v));
+                }
+            }
+        } else if (!interior) {
             // edge strip: through registers.  Loads are unconditional and issued back to back (an invalid
             // slot re-reads a valid address); what a slot really holds is decided on the way to LDS
             V16 stage[STAGE_IT];
@@ -444,14 +525,6 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
                         if (col + u > h) v.v[u] = from_float<T>(0.0f);
                 }
                 lds_store16(tile_lds + (unsigned)slot * 16u, __builtin_bit_cast(u32x4, v));
-            }
-        }
-        if (channel != cur_channel) {
-            for (int e = lane; e < R * WZ_LD; e += M_WT) {
-                const int i = e / WZ_LD, j = e % WZ_LD - WZ_OFF;
-                const bool ok = j >= 0 && j < S;
-                const T wv = w[channel * R * S + (ok ? i * S + j : 0)];
-                wz[e] = ok ? wv : from_float<T>(0.0f);
             }
         }
         lds_wait();  // LDS stores above are complete (single wavefront: no barrier needed)
@@ -536,16 +609,38 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
             for (int rb = 0; rb < M_TM / 16; ++rb) {
                 f32x4 acc[M_TN / 16];
                 const unsigned xa = tile_lds + (unsigned)((rb * 16 + ln) * LD + kg * 8) * sizeof(T);
+                // Column blocks in pairs.  A wavefront issues in order, so a run of LDS reads followed by a run of
+                // products leaves the matrix cores idle during the first and the LDS during the second; here one read
+                // of the next pair's operands is issued per product of this pair, and a product waits only for its
+                // own operand, issued 2R reads earlier (LDS operations complete in order: lgkmcnt(2R) at every
+                // step).  Source order is pinned (the scheduler would regroup reads and products).  Blocks above the
+                // diagonal are computed like the others and masked below.
+                constexpr int NPAIR = M_TN / 32, NLD = 2 * R;
+                static_assert(NLD <= 15, "lgkmcnt field");
+                u32x4 xf[2][2][R];
+                auto xaddr = [&](int pr, int c2, int i) { return xa + (unsigned)(i * LD + (pr * 2 + c2) * 16) * sizeof(T); };
 #pragma unroll
-                for (int cb = 0; cb < M_TN / 16; ++cb) {
-                    acc[cb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-                    if (!interior && causal && q0 + cb * 16 > p0 + rb * 16 + 15) continue;  // wholly above the diagonal: +0
-                    u32x4 xf[R];
+                for (int i = 0; i < R; ++i)
 #pragma unroll
-                    for (int i = 0; i < R; ++i) xf[i] = lds_load16(xa + (unsigned)(i * LD + cb * 16) * sizeof(T));
-                    lds_wait_all(xf);
+                    for (int c2 = 0; c2 < 2; ++c2) xf[0][c2][i] = lds_load16(xaddr(0, c2, i));
 #pragma unroll
-                    for (int i = 0; i < R; ++i) mma16(acc[cb], tz[i][0], __builtin_bit_cast(frag8<T>, xf[i]));
+                for (int pr = 0; pr < NPAIR; ++pr) {
+                    acc[2 * pr] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                    acc[2 * pr + 1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int i = 0; i < R; ++i)
+#pragma unroll
+                        for (int c2 = 0; c2 < 2; ++c2) {
+                            u32x4 &cur = xf[pr & 1][c2][i];
+                            if (pr + 1 < NPAIR) {
+                                xf[(pr + 1) & 1][c2][i] = lds_load16(xaddr(pr + 1, c2, i));
+                                asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(cur) : "n"(NLD) : "memory");
+                            } else {  // last pair: only this pair's later reads are newer
+                                asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(cur) : "n"(NLD - 1 - (2 * i + c2)) : "memory");
+                            }
+                            mma16(acc[2 * pr + c2], tz[i][0], __builtin_bit_cast(frag8<T>, cur));
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
                 }
                 const int prow = p0 + rb * 16 + ln;
 #pragma unroll
