@@ -307,8 +307,9 @@ __device__ __forceinline__ void lds_wait(u32x4 &a, u32x4 &b, u32x4 &c)
 // Staging.  A strip whose halo lies wholly inside the tensor and on or below the diagonal (the
 // common case, decided per wavefront) is copied global -> LDS by global_load_lds_dwordx4: no
 // registers, no masks, no LDS store instructions.  The LDS row stride is 19 16-byte slots (18 of
-// data + 1 of padding), so lane L of copy `it` simply owns slot it*64+L.  Edge strips go through
-// registers, where bounds and the causal col<=row rule are applied.
+// data + 1 of padding), so lane L of copy `it` simply owns slot it*64+L.  Diagonal and border strips
+// are copied the same way and fixed up in LDS; the rare strips whose copy could leave the tensor go
+// through registers, where bounds and the causal col<=row rule are applied.
 //
 // SCALED: every strip is staged through registers, where x*in_scale is rounded to the I/O dtype before it
 // reaches LDS (what a separate elementwise scale pass would have produced).
