@@ -95,6 +95,22 @@ def time_steps(torch, fn, nsets, warmup, steps):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
+def time_launches(torch, fn, nsets, warmup, steps):
+    """Average duration of one launch of a single-kernel operator: an event pair around every launch, on the stream
+    the kernel is launched on (what `rocprofv3 --kernel-trace` reports per dispatch, plus the event overhead; the
+    wall clock over a loop of launches also counts the gaps between them)."""
+    for i in range(warmup):
+        fn(i % nsets)
+    torch.cuda.synchronize()
+    pairs = []
+    for i in range(steps):
+        e0 = _record(torch)
+        fn(i % nsets)
+        pairs.append((e0, _record(torch)))
+    torch.cuda.synchronize()
+    return sum(a.elapsed_time(b) for a, b in pairs) / steps
+
+
 def stage_breakdown(torch, mod, sets, steps):
     """Average duration of each stage of forward(), from events on the kernels' own stream."""
     marks = []
@@ -129,7 +145,7 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
     w = O.seeded_conv_weight(c, 6, 11, 0.05, bf16, identity_tap=False).to(device)
     xs = [torch.tril(torch.randn(n, c, s, s, generator=g).to(bf16)).to(device) for _ in range(3)]
     ys = [torch.empty_like(x) for x in xs]
-    ms = time_steps(torch, lambda i: mta.ops.conv2d_causal(xs[i], w, True, out=ys[i]), 3, warmup, steps)
+    ms = time_launches(torch, lambda i: mta.ops.conv2d_causal(xs[i], w, True, out=ys[i]), 3, warmup, steps)
     by = score_pass_bytes(n, c, s, 2)
     out["conv2d_6x11_bf16_2x16x2048x2048"] = {"ms": ms, "algorithmic_bytes": by, "GBps": by / ms / 1e6,
                                               "frac_hbm_peak": by / ms / 1e6 / HBM_PEAK_GBS}
@@ -146,7 +162,7 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
     ys = [torch.empty_like(x) for x in xs]
     by = score_pass_bytes(n, c, s, 2)
     for label, grp in (("headmix_g4_bf16_2x32x2048x2048", 4), ("headmix_dense_bf16_2x32x2048x2048", None)):
-        ms = time_steps(torch, lambda i: mta.ops.headmix(xs[i], wm, True, 0.0, group_size=grp, out=ys[i]), 2, warmup, steps)
+        ms = time_launches(torch, lambda i: mta.ops.headmix(xs[i], wm, True, 0.0, group_size=grp, out=ys[i]), 2, warmup, steps)
         out[label] = {"ms": ms, "algorithmic_bytes": by, "GBps": by / ms / 1e6, "frac_hbm_peak": by / ms / 1e6 / HBM_PEAK_GBS}
     del xs, ys
     # fused conv-attention: B1 H32 S8192 D128 bf16, 6x11
@@ -154,7 +170,7 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
     sets = [tuple(t.to(device) for t in O.seeded_qkv(b, h, s, d, bf16, seed=200 + i)) for i in range(2)]
     wc = O.seeded_conv_weight(h, 6, 11, 0.05, bf16).to(device)
     os_ = [torch.empty_like(sets[0][0]) for _ in range(2)]
-    ms = time_steps(torch, lambda i: mta.ops.conv_attn_fwd(*sets[i], wc, True, None, out=os_[i]), 2, min(warmup, 2),
+    ms = time_launches(torch, lambda i: mta.ops.conv_attn_fwd(*sets[i], wc, True, None, out=os_[i]), 2, min(warmup, 2),
                     max(2, steps // 4))
     mfma_flops = 4 * b * h * tri(s) * d
     out["conv_attn_fused_bf16_1x32x8192x128"] = {"ms": ms, "mfma_useful_flops": mfma_flops,
