@@ -180,8 +180,13 @@ int dispatch_valu(const void *x, const void *w, void *y, int64_t N, int64_t C, i
 #define MTA_CONV_WG_PER_CU 6       // LDS budget: two 11.6 KB strip buffers per single-wavefront workgroup
 #endif
 constexpr int M_WT = 64;   // one wavefront per workgroup
-constexpr int M_TM = 32;   // strip rows: 2 row blocks of 16
+#ifndef MTA_CONV_STRIP_ROWS
+#define MTA_CONV_STRIP_ROWS 32
+#endif
+constexpr int M_TM = MTA_CONV_STRIP_ROWS;  // strip rows: row blocks of 16
 constexpr int M_TN = 128;  // strip cols: 8 column blocks of 16
+constexpr int M_SPB = M_TN / M_TM;  // strips per 128x128 block
+static_assert(M_TM % 16 == 0 && M_TN % M_TM == 0 && (M_SPB & (M_SPB - 1)) == 0, "strip geometry");
 
 // 16 outputs + S-1 taps (+ alignment shift) must fit the 32-key contraction of one 16x16x32 MFMA
 template <int R, int S> struct mfma_geom {
@@ -197,19 +202,19 @@ template <int R, int S> struct mfma_geom {
 
 // work item -> (plane, strip row tm (32 rows), strip col tn (128 keys)).
 // `mirror` (causal, square): only strips that touch the lower triangle are enumerated, by 128x128
-// block in row-major lower-triangular order, 4 strips per block; each strip of an off-diagonal
-// block also zero-fills a quarter of the block's mirror image above the diagonal.
+// block in row-major lower-triangular order, M_SPB strips per block; each strip of an off-diagonal
+// block also zero-fills its share (1/M_SPB) of the block's mirror image above the diagonal.
 __device__ __forceinline__ void decode_item(int64_t idx, int ipp, int tiles_n, int mirror, int64_t &plane, int &tm, int &tn)
 {
     plane = idx / ipp;
     const int t = (int)(idx % ipp);
     if (mirror) {
-        const int blk = t >> 2;
+        const int blk = t / M_SPB;
         int bm = (int)((sqrtf(8.0f * (float)blk + 1.0f) - 1.0f) * 0.5f);
         while ((bm + 1) * (bm + 2) / 2 <= blk) ++bm;
         while (bm * (bm + 1) / 2 > blk) --bm;
         tn = blk - bm * (bm + 1) / 2;
-        tm = bm * 4 + (t & 3);
+        tm = bm * M_SPB + (t % M_SPB);
     } else {
         tm = t / tiles_n;
         tn = t % tiles_n;
@@ -224,7 +229,7 @@ __device__ __forceinline__ int opaque(int v)
     return v;
 }
 
-// FULL: the region lies inside the tensor; the stores are then unconditional (exactly 8 vector-memory instructions)
+// FULL: the region lies inside the tensor; the stores are then unconditional (exactly M_TM/4 vector-memory instructions)
 template <typename T, bool FULL = false>
 __device__ __forceinline__ void zero_fill_strip(T *yp, int H, int W, int p0, int q0, int lane)
 {
@@ -327,7 +332,7 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     static_assert(SPR == VPR + 1, "one padding slot per row");
     // weights of the current channel, each kernel row zero-padded on both sides so that the
     // Toeplitz fragments can be gathered without range checks
-    constexpr bool M32 = MTA_CONV_MFMA32 && G::fits32;
+    constexpr bool M32 = MTA_CONV_MFMA32 && G::fits32 && M_TM == 32;
     constexpr int NCH = 3;  // 16-key chunks per 32-output window (M32)
     constexpr int WZ_OFF = G::SHIFT + (M32 ? 32 : 16), WZ_LD = WZ_OFF + (M32 ? 16 * NCH : 32);
     constexpr int BUF = STAGE_IT * M_WT * VEC;  // elements per LDS strip buffer
@@ -438,8 +443,9 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
         // ones issued after that copy are the previous strip's stores: when their number is known exactly
         // (`younger`), they may stay in flight.  LDS reads of `other` by the previous iteration are complete.
         if constexpr (DBUF) {
-            if (younger == 16) asm volatile("s_waitcnt vmcnt(16)" : : : "memory");
-            else if (younger == 8) asm volatile("s_waitcnt vmcnt(8)" : : : "memory");
+            constexpr int ST = M_TM * (M_TN / VEC) / M_WT;  // stores per strip, and per mirror share
+            if (younger == 2 * ST) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * ST) : "memory");
+            else if (younger == ST) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(ST) : "memory");
             else asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
         } else {
             // one buffer: this strip's copy is issued now and waited for (the other wavefronts of the CU cover the
@@ -685,15 +691,15 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
                     }
                 }
             }
-            static_assert(OUT_IT == 8, "8 stores per strip");
+            static_assert(OUT_IT % 4 == 0, "stores in groups of four");
             younger = interior ? OUT_IT : -1;
         }
-        if (mirror && ctn < (ctm >> 2)) {  // a quarter of the 128x128 block's image above the diagonal
+        if (mirror && ctn < ctm / M_SPB) {  // this strip's share of the 128x128 block's image above the diagonal
             if (fill_full) {
-                zero_fill_strip<T, true>(yp, H, W, q0 + (ctm & 3) * M_TM, (ctm >> 2) * M_TN, lane);
+                zero_fill_strip<T, true>(yp, H, W, q0 + (ctm % M_SPB) * M_TM, (ctm / M_SPB) * M_TN, lane);
                 if (younger > 0) younger += M_TM * (M_TN / VEC) / M_WT;
             } else {
-                zero_fill_strip<T>(yp, H, W, q0 + (ctm & 3) * M_TM, (ctm >> 2) * M_TN, lane);
+                zero_fill_strip<T>(yp, H, W, q0 + (ctm % M_SPB) * M_TM, (ctm / M_SPB) * M_TN, lane);
                 younger = -1;
             }
         }
@@ -721,7 +727,7 @@ int launch_mfma(const void *x, const void *w, void *y, int64_t N, int64_t C, int
     // mirror enumeration needs a square grid of whole 128x128 blocks' worth of strips
     const int blocks = (int)((H + M_TN - 1) / M_TN);
     const int mirror = (causal && H == W) ? 1 : 0;
-    const int64_t ipp64 = mirror ? (int64_t)blocks * (blocks + 1) / 2 * 4 : (int64_t)tiles_m * tiles_n;
+    const int64_t ipp64 = mirror ? (int64_t)blocks * (blocks + 1) / 2 * M_SPB : (int64_t)tiles_m * tiles_n;
     if (ipp64 > (1 << 24)) return MTA_ERR_SHAPE;  // decode_item's float sqrt is exact well beyond this
     const int ipp = (int)ipp64;
     const int64_t total = N * C * ipp64;
