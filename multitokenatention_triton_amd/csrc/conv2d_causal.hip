@@ -166,6 +166,17 @@ int dispatch_valu(const void *x, const void *w, void *y, int64_t N, int64_t C, i
 // ------------------------------------------------------------------------------------
 // MFMA (Toeplitz) path
 // ------------------------------------------------------------------------------------
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+// The output is written once and not read again by this kernel: non-temporal stores keep it from displacing the input
+// rows that neighbouring strips re-read (halos) in the L2.
+#ifndef MTA_CONV_NT_STORE
+#define MTA_CONV_NT_STORE 1
+#endif
+#if MTA_CONV_NT_STORE
+#define MTA_CONV_STORE(ptr, val) __builtin_nontemporal_store((val), (ptr))
+#else
+#define MTA_CONV_STORE(ptr, val) (*(ptr) = (val))
+#endif
 #ifndef MTA_CONV_WAVES_PER_SIMD
 #define MTA_CONV_WAVES_PER_SIMD 2  // register budget: 256 VGPRs
 #endif
@@ -241,13 +252,13 @@ __device__ __forceinline__ void zero_fill_strip(T *yp, int H, int W, int p0, int
 #pragma unroll
     for (int e = lane; e < M_TM * (M_TN / VEC); e += M_WT) {
         const int r = e / (M_TN / VEC), col = q0 + (e % (M_TN / VEC)) * VEC;
-        if (FULL || (p0 + r < H && col < W)) *reinterpret_cast<pack16<T> *>(yp + (int64_t)(p0 + r) * W + col) = z;
+        if (FULL || (p0 + r < H && col < W))
+            MTA_CONV_STORE(reinterpret_cast<u32x4 *>(yp + (int64_t)(p0 + r) * W + col), __builtin_bit_cast(u32x4, z));
     }
 }
 
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef const __attribute__((address_space(1))) void glb_void_t;
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 // The staged strips are read and written through these, not through C++ accesses: the compiler cannot tell an access
 // to one half of the double buffer from the asynchronous copy in flight into the other half and would wait for the
@@ -682,12 +693,12 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
                 asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : : "memory");
                 if (interior) {  // unconditional: exactly OUT_IT vector-memory instructions
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) *reinterpret_cast<u32x4 *>(ybase + ((i0 + k) * 4 + r_l) * W + cv) = v[k];
+                    for (int k = 0; k < 4; ++k) MTA_CONV_STORE(reinterpret_cast<u32x4 *>(ybase + ((i0 + k) * 4 + r_l) * W + cv), v[k]);
                 } else {
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
                         const int r = (i0 + k) * 4 + r_l;
-                        if (p0 + r < H && q0 + cv < W) *reinterpret_cast<u32x4 *>(ybase + r * W + cv) = v[k];
+                        if (p0 + r < H && q0 + cv < W) MTA_CONV_STORE(reinterpret_cast<u32x4 *>(ybase + r * W + cv), v[k]);
                     }
                 }
             }

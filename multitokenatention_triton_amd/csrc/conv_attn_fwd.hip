@@ -325,6 +325,13 @@ constexpr int F_BK = 64;   // keys per iteration
 constexpr int F_SLD = 80;  // score-tile row stride (elements): exactly the retained columns + one key block (measured
                            // fastest among 80..120)
 
+// Returns its argument, opaquely: what is derived from the result cannot be hoisted out of the block that computes it.
+__device__ __forceinline__ int opaque_lane(int v)
+{
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
 template <int R, int SK, int NW> struct fused_geom {
     static constexpr int F_SR = 32 * NW;
     static constexpr int HR = (R - 1 + 7) & ~7;    // halo rows above the block (recomputed)
@@ -510,6 +517,8 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
             tailreg[it] = *reinterpret_cast<const u32x4_t *>(Sc + (tail_off[it] >= 0 ? tail_off[it] : 0) + F_BK);
         __builtin_amdgcn_s_waitcnt(0);  // this wavefront's part of block j has landed in LDS
         __syncthreads();                // ... and everybody's; all reads of the previous tiles are done
+        // (Leaving the previous iteration's result stores in flight here - vmcnt(number of stores) instead of 0 - was
+        // measured: no gain.)
 #pragma unroll
         for (int it = 0; it < TAIL_IT; ++it)
             if (tail_off[it] >= 0) *reinterpret_cast<u32x4_t *>(Sc + tail_off[it]) = tailreg[it];
@@ -610,13 +619,19 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
                 }
             }
             __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's staging rows are written
+            // (row and column from a laundered lane index: the four row addresses are then formed here, 64-bit adds and
+            // all, instead of being kept in registers across the key-block loop - the kernel is at its register limit,
+            // and a spilled value reloaded in this loop makes the compiler wait for every outstanding store)
+            const int lane_o = opaque_lane(lane);
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
-                const int r = it * 8 + (lane >> 3), cv = (lane & 7) * 8;
+                const int r = it * 8 + (lane_o >> 3), cv = (lane_o & 7) * 8;
                 const int tr_ = wave * 32 + r, p_ = q0 - G::HR + tr_, col = j * F_BK + cv;
-                const pack16<T> v = *reinterpret_cast<const pack16<T> *>(stage + r * OLD + (((lane & 7) ^ (r & 7)) * 8));
+                const pack16<T> v = *reinterpret_cast<const pack16<T> *>(stage + r * OLD + (((lane_o & 7) ^ (r & 7)) * 8));
+                // (non-temporal: the scores are written once and next read by another kernel; as ordinary stores they
+                // would push this head's K blocks, which every workgroup of the head re-reads, out of the L2)
                 if (tr_ >= G::HR && p_ < S && (PLAIN || (col < S && (!causal || fill_upper || col <= p_))))
-                    *reinterpret_cast<pack16<T> *>(Op + (int64_t)p_ * S + col) = v;
+                    __builtin_nontemporal_store(__builtin_bit_cast(u32x4_t, v), reinterpret_cast<u32x4_t *>(Op + (int64_t)p_ * S + col));
             }
             return;
         }
