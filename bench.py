@@ -66,7 +66,7 @@ def stage_model(name, b, h, s, d, r=6, sk=11, esize=2):
 # HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at the benchmark shape
 # (profiles/mta_forward_c4_hbm_traffic.txt); FETCH_SIZE is scaled by 2.0, the factor a plain 1 GiB
 # device copy shows for it on this machine, WRITE_SIZE by 1.0.
-MEASURED_TRAFFIC_BYTES = {"qk_conv": 644.7e6, "mix_softmax_mix": 1110.1e6, "pv": 648.8e6}
+MEASURED_TRAFFIC_BYTES = {"qk_conv": 606.7e6, "mix_softmax_mix": 1111.4e6, "pv": 648.7e6}
 
 
 def build_c4(torch, mta, O, device, b=2, h=16, s=4096, d=128, dtype=None, nsets=3):
