@@ -40,18 +40,6 @@ constexpr int P_BK = MTA_PV_BK;  // keys per iteration: each lane reads P_BK/4 c
                                  // iteration, back to back, so that DRAM pages are used in long runs
 constexpr int P_KS = P_BK / 32;  // 32-key contraction steps per iteration
 
-// Swizzle of a V block in LDS: row `key` stores its 16-byte chunk c at position c ^ v_swizzle(key).  A transpose read
-// touches, per group of 16 lanes, 32 contiguous bytes (8 banks) of each of 4 consecutive keys, and groups are 8 keys
-// apart: the keys {0..3, 8..11} (+4, +16) that may be served in one cycle must land in 8 different 8-bank regions.
-// D = 128 (a row is all 64 banks): region = chunk pair ^ (key%4 + 4*bit 3 of key).  D = 64 (a row is 32 banks, odd keys
-// take the other half): region = chunk pair ^ (bit 1 + 2*bit 3 of key).  (XOR with the plain key index put keys 2k and
-// 2k+1 into the same region: every transpose read took a two-way bank conflict.)
-template <int D> __device__ __forceinline__ int v_swizzle(int key)
-{
-    if constexpr (D == 128) return 2 * ((key & 3) | ((key >> 1) & 4));
-    else return 2 * (((key >> 1) & 1) | ((key >> 2) & 2));
-}
-
 template <typename T, int D>
 __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__restrict__ P, const T *__restrict__ V,
                                                            T *__restrict__ O, int S, int causal, int nqb, int64_t total_wg,

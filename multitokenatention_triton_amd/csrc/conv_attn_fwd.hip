@@ -332,6 +332,16 @@ __device__ __forceinline__ int opaque_lane(int v)
     return v;
 }
 
+// Swizzle of a V block for the attention kernel's transpose reads, whose 16-lane groups are 4 keys apart (keys
+// 4kg + 0..3): the 8 consecutive keys that may be served in one cycle must land in 8 different 8-bank regions.
+// D = 128: region = chunk pair ^ key%8.  D = 64 (a row is half the banks, odd keys take the other half):
+// region = chunk pair ^ (key/2)%4.
+template <int D> __device__ __forceinline__ int v_swizzle4(int key)
+{
+    if constexpr (D == 128) return 2 * (key & 7);
+    else return 2 * ((key >> 1) & 3);
+}
+
 template <int R, int SK, int NW> struct fused_geom {
     static constexpr int F_SR = 32 * NW;
     static constexpr int HR = (R - 1 + 7) & ~7;    // halo rows above the block (recomputed)
@@ -414,20 +424,25 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
     static_assert((F_NT / CPR) % CPR == 0 && F_NT % CPR == 0, "copy rounds must keep the swizzle phase");
     const int kv_row0 = tid / CPR;
     const int kv_off0 = kv_row0 * D + ((tid % CPR) ^ (kv_row0 & (CPR - 1))) * 8;
+    // V blocks use the swizzle that keeps the transpose reads free of bank conflicts (it only depends on key bits
+    // below 4, which a copy round does not change either)
+    static_assert((F_NT / CPR) % 16 == 0, "copy rounds must keep the V swizzle phase");
+    const int v_off0 = kv_row0 * D + ((tid % CPR) ^ v_swizzle4<D>(kv_row0)) * 8;
     auto issue_kv = [&](int j, T *Kdst, T *Vdst) {
         const int cb = j * F_BK + G::PWR;
         const bool inside = cb >= 0 && cb + F_BK <= S && j >= 0 && (j + 1) * F_BK <= S;  // no key needs clamping
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r) {
             const int kv_row = kv_row0 + r * (F_NT / CPR), kv_off = kv_off0 + r * (F_NT / CPR) * D;
-            int koff = cb * D + kv_off, voff = j * F_BK * D + kv_off;
+            const int v_off = v_off0 + r * (F_NT / CPR) * D;
+            int koff = cb * D + kv_off, voff = j * F_BK * D + v_off;
             if (!inside) {
                 int kr = cb + kv_row;
                 kr = kr < 0 ? 0 : (kr >= S ? S - 1 : kr);
                 int vr = j * F_BK + kv_row;
                 vr = vr < 0 ? 0 : (vr >= S ? S - 1 : vr);
                 koff = kv_off + (kr - kv_row) * D;
-                voff = kv_off + (vr - kv_row) * D;
+                voff = v_off + (vr - kv_row) * D;
             }
             __builtin_amdgcn_global_load_lds((glb_void_t *)(Kp + koff),
                                              (lds_void_t *)(Kdst + (r * F_NT + wave * 64) * 8), 16, 0, 0);
@@ -708,8 +723,8 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
                 const int key_a = ks * 32 + kg * 4 + (ln >> 2), key_b = key_a + 16;
                 const int ch = db * 2 + ((ln & 3) >> 1);  // 16-byte chunk holding head dims 16db+4(ln%4)..
                 const int sub = (ln & 1) * 4;             // element offset inside the chunk
-                const T *pa = Vb + key_a * D + ((ch ^ (key_a & (CPR - 1))) * 8) + sub;
-                const T *pb = Vb + key_b * D + ((ch ^ (key_b & (CPR - 1))) * 8) + sub;
+                const T *pa = Vb + key_a * D + ((ch ^ v_swizzle4<D>(key_a)) * 8) + sub;
+                const T *pb = Vb + key_b * D + ((ch ^ v_swizzle4<D>(key_b)) * 8) + sub;
                 struct { v4s_t a, b; } both = {__builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)pa),
                                                __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)pb)};
                 dst = __builtin_bit_cast(frag8<T>, both);
