@@ -79,7 +79,9 @@ def build_c4(torch, mta, O, device, b=2, h=16, s=4096, d=128, dtype=None, nsets=
         mod.wpsm_triton.weight.copy_(torch.eye(h))
         mod.mta_conv_after_sm_triton.weight.copy_(O.identity_conv_kernel(h, 3, 3, dtype))
         mod.wposm_triton.weight.copy_(O.block_diag_head_weight(h, 4, 0.1, g, dtype))
-    mod = mod.to(device).eval()
+    mod = mod.to(device).eval().requires_grad_(False)
+    # the configuration states the structure (identity wpsm and post conv, groups of 4): read it off the weights once
+    mod.infer_weight_structure()
     sets = [tuple(t.to(device) for t in O.seeded_qkv(b, h, s, d, dtype, seed=123 + i)) for i in range(nsets)]
     return mod, sets
 

@@ -125,6 +125,18 @@ int mta_qk_conv_fwd(const void *q, const void *k, const void *w, void *s_out, in
 int mta_causal_pv_fwd(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int64_t D,
                       int causal, int io_dtype, void *stream);
 
+/* Structure of the small MTA parameters, evaluated on the device (one workgroup, a few microseconds).  The
+ * reference has no counterpart: its glue (mta_attention_triton.py:69-89) always runs every stage.  The glue
+ * of this build asks these when the caller requests that identity stages be skipped and block-diagonal head
+ * weights be applied block by block.
+ * mta_probe_head_weight: w is (H,H); out[0] = 1 when w is exactly the identity, out[1] = the smallest G
+ * dividing H such that w is zero outside its GxG diagonal blocks (H if none smaller).
+ * mta_probe_conv_kernel: w is (C,R,S); out[0] = 1 when every channel is 1.0 at [R-1, S/2] and 0 elsewhere and
+ * S is odd (the conv then passes its masked input through).
+ * `out` is device memory (2 resp. 1 int32), written on `stream`. */
+int mta_probe_head_weight(const void *w, int64_t H, int w_dtype, int32_t *out, void *stream);
+int mta_probe_conv_kernel(const void *w, int64_t C, int R, int S, int w_dtype, int32_t *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

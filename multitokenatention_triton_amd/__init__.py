@@ -11,8 +11,9 @@ call surface of Gusanidas/multitokenatention_triton:
 from .convolution_2d_trit import Conv2dTriton, Conv2dTritonFunction
 from .triton_linear_head import TritonLinearHead, TritonLinearHeadFunction
 from .conv_attention_triton import TritonAttention, TritonConvAttention
-from .mta_attention_triton import MTAAttentionTriton, MTAConfig
+from .mta_attention_triton import MTAAttentionTriton, MTAConfig, WeightStructure
 from . import ops
 
 __all__ = ["Conv2dTriton", "Conv2dTritonFunction", "TritonLinearHead", "TritonLinearHeadFunction",
-           "TritonAttention", "TritonConvAttention", "MTAAttentionTriton", "MTAConfig", "ops"]
+           "TritonAttention", "TritonConvAttention", "MTAAttentionTriton", "MTAConfig", "WeightStructure",
+           "ops"]

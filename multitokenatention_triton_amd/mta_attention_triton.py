@@ -3,22 +3,37 @@
 Same constructor, attribute names, parameter names and forward signature as
 mta_attention_triton.py:7-201, so state dicts and calling code carry over.  What differs
 is how forward() is executed on the GPU (the values are those of
-mta_attention_pytorch.py:58-83):
+mta_attention_pytorch.py:58-83).
 
-  * the 1/sqrt(D) factor is applied by the pre-softmax conv while it stages its tile
-    (``mta_conv2d_scaled_fwd``) instead of a separate pass over the (B,H,S,S) scores;
+Inference (no input or parameter requires grad, or grad mode is off):
+
+  * QK^T, the 1/sqrt(D) factor and the pre-softmax conv run as one kernel
+    (``mta_qk_conv_fwd``): the raw scores never reach HBM;
   * pre-softmax head mixing, the causal mask, the fp32 softmax and -- when the
     post-softmax conv kernel is the identity tap -- the post-softmax head mixing run
     as one kernel (``mta_headmix_softmax_fwd``): one pass over the score tensor
     instead of four, and no fp32 copy of it;
-  * block-diagonal head-mixing weights are detected and only their blocks are applied.
+  * P V reads only the lower triangle of P (``mta_causal_pv_fwd``).
 
-Weight structure (identity conv tap, identity / block-diagonal head weights) is probed on
-the host and remembered per parameter, keyed by the parameter's autograd version counter
-and storage address.  Optimizer steps, ``load_state_dict``, ``copy_`` under ``no_grad`` and
-this module's own reset/copy methods all move that counter.  A write through ``.data``
-does not: after one, call ``refresh_structure()`` (or construct the module with
-``weight_structure="dense"``, which never assumes any structure).
+Training (something requires grad): the stages run one by one through the autograd
+Functions of convolution_2d_trit / triton_linear_head, as in the reference, so that
+``backward()`` works; torch differentiates the two GEMMs, the softmax and the dropout.
+
+Weight structure.  By default nothing is assumed about the four weights: every stage runs
+with the dense weight it is given.  Skipping identity stages and applying block-diagonal
+head weights block by block is an explicit opt-in, because a parameter can be rewritten
+behind the module's back (``p.data.copy_(...)`` leaves no trace on the host):
+
+  * ``infer_weight_structure()`` looks at the current weights once (on the device, one
+    small read back) and keeps what it found until told otherwise;
+  * ``declare_weight_structure(...)`` states it without looking;
+  * ``weight_structure = "probe"`` looks on every call (one tiny launch and a
+    synchronising 20-byte read per forward; not usable under stream capture);
+  * ``assume_dense_weights()`` returns to the default.
+
+``reset_mta_parameters``, ``copy_mta_parameters`` and ``load_state_dict`` return to the
+default as well.  A declared structure is the caller's promise, like ``group_size`` in the
+C ABI: weights that break it give results for the declared structure.
 """
 from __future__ import annotations
 
@@ -52,6 +67,19 @@ class MTAConfig:
     dim: int = 512
 
 
+@dataclass(frozen=True)
+class WeightStructure:
+    """What the glue may assume about the four weights (all False / None = nothing)."""
+    pre_head_identity: bool = False
+    pre_head_group: Optional[int] = None      # None = dense
+    post_conv_identity: bool = False
+    post_head_identity: bool = False
+    post_head_group: Optional[int] = None
+
+
+_DENSE = WeightStructure()
+
+
 class MTAAttentionTriton(nn.Module):
     def __init__(self, n_heads: int, mta, dropout: float, causal: bool, use_mask: bool = False):
         super().__init__()
@@ -78,9 +106,10 @@ class MTAAttentionTriton(nn.Module):
         self.wposm_triton = TritonLinearHead(n_heads, causal=causal)
         # optional observer: called as hook(stage_name) right before each stage is enqueued
         self._stage_hook = None
-        # "auto": probe weight structure and pick specialised kernels; "dense": assume nothing
-        self.weight_structure = "auto"
-        self._structure = {}
+        # "dense": assume nothing; "declared": use self._declared; "probe": look at the weights on every call
+        self.weight_structure = "dense"
+        self._declared = WeightStructure()
+        self.register_load_state_dict_post_hook(lambda module, incompatible: module.assume_dense_weights())
 
     # ------------------------------------------------------------------ forward
     def _mark(self, name: str) -> None:
@@ -91,16 +120,24 @@ class MTAAttentionTriton(nn.Module):
         assert chunk_start_ids is None, "MTAAttentionTriton does not support chunked attention"
         if self.use_mask:
             return self._forward_with_mask(xq, xk, xv, mask)
+        if torch.is_grad_enabled() and (xq.requires_grad or xk.requires_grad or xv.requires_grad
+                                        or any(p.requires_grad for p in self.parameters())):
+            return self._forward_stagewise(xq, xk, xv)
 
         head_dim = xq.size(-1)
         # the reference multiplies by rsqrt(tensor(head_dim)), an fp32 scalar (mta_attention_triton.py:69-71)
         scale = float(torch.rsqrt(torch.tensor(float(head_dim))))
+        st = self._current_structure()
         w_pre, w_post = self.wpsm_triton.weight, self.wposm_triton.weight
-        pre_eye, g_pre = self._probe("wpsm", w_pre, _probe_head)
-        post_eye, g_post = self._probe("wposm", w_post, _probe_head)
-        post_conv_identity = self._probe("conv_post", self.mta_conv_after_sm_triton.weight, _probe_conv)
-        w1 = None if pre_eye else w_pre
-        w2 = None if post_eye else w_post
+        g_pre = st.pre_head_group or self.n_heads
+        g_post = st.post_head_group or self.n_heads
+        w1 = None if st.pre_head_identity else w_pre
+        w2 = None if st.post_head_identity else w_post
+        if w1 is None:
+            g_pre = 1
+        if w2 is None:
+            g_post = 1
+        post_conv_identity = st.post_conv_identity
         one_pass = post_conv_identity and _lcm(g_pre, g_post) <= _FUSED_MAX_GROUP
         # the last stage may leave the upper triangle unwritten only if our own P V kernel consumes it
         own_pv = (xq.size(-2) == xk.size(-2) and xq.dtype == xv.dtype
@@ -148,19 +185,73 @@ class MTAAttentionTriton(nn.Module):
         self._mark("end")
         return output.transpose(1, 2)
 
-    def _probe(self, name, weight, fn):
-        if self.weight_structure != "auto":
-            return (False, self.n_heads) if fn is _probe_head else False
-        key = (id(weight), weight._version, weight.data_ptr(), weight.dtype)
-        hit = self._structure.get(name)
-        if hit is None or hit[0] != key:
-            hit = (key, fn(weight))
-            self._structure[name] = hit
-        return hit[1]
+    def _forward_stagewise(self, xq, xk, xv):
+        """The reference's own sequence of operators (mta_attention_triton.py:68-92), each differentiable: taken
+        whenever a gradient may be asked for.  No weight structure is assumed here, so every entry of the four
+        weights receives its gradient."""
+        scale = torch.rsqrt(torch.tensor(float(xq.size(-1)), device=xq.device))
+        self._mark("qk")
+        scores = torch.matmul(xq, xk.transpose(2, 3)) * scale
+        self._mark("conv_pre")
+        scores = self.mta_conv_triton(scores)
+        self._mark("mix_pre")
+        scores = self.wpsm_triton(scores)
+        self._mark("softmax")
+        scores = F.softmax(scores.float(), dim=-1).type_as(xq)
+        self._mark("conv_post")
+        scores = self.mta_conv_after_sm_triton(scores)
+        self._mark("mix_post")
+        scores = self.wposm_triton(scores)
+        scores = F.dropout(scores, p=self.dropout, training=self.training)
+        self._mark("pv")
+        output = torch.matmul(scores, xv)
+        self._mark("end")
+        return output.transpose(1, 2)
 
-    def refresh_structure(self):
-        """Forget what was learnt about the weights' structure (needed after writes through ``.data``)."""
-        self._structure.clear()
+    # ------------------------------------------------------------------ weight structure
+    def _current_structure(self) -> "WeightStructure":
+        if self.weight_structure == "dense":
+            return _DENSE
+        if self.weight_structure == "declared":
+            return self._declared
+        if self.weight_structure == "probe":
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError('weight_structure="probe" reads the probe result back on every call and cannot run '
+                                   "under stream capture: call infer_weight_structure() before capturing instead")
+            return self._probe_now()
+        raise ValueError(f"weight_structure must be 'dense', 'declared' or 'probe', got {self.weight_structure!r}")
+
+    def _probe_now(self) -> "WeightStructure":
+        pre_eye, g_pre, post_eye, g_post, conv_eye = ops.probe_mta_weights(
+            self.wpsm_triton.weight, self.wposm_triton.weight, self.mta_conv_after_sm_triton.weight)
+        return WeightStructure(pre_head_identity=pre_eye, pre_head_group=g_pre, post_conv_identity=conv_eye,
+                               post_head_identity=post_eye, post_head_group=g_post)
+
+    def infer_weight_structure(self) -> "WeightStructure":
+        """Look at the current weights once (device-side probe, one small read back) and keep the result for
+        all later calls.  Call again after the weights change; see the module docstring."""
+        self._declared = self._probe_now()
+        self.weight_structure = "declared"
+        return self._declared
+
+    def declare_weight_structure(self, pre_head_identity: bool = False, pre_head_group: Optional[int] = None,
+                                 post_conv_identity: bool = False, post_head_identity: bool = False,
+                                 post_head_group: Optional[int] = None) -> "WeightStructure":
+        """State the structure of the weights without looking at them: ``*_identity`` = that weight is exactly
+        the identity (head weights) / the pass-through tap at [R-1, S//2] (post-softmax conv);
+        ``*_head_group`` = G such that the head weight is zero outside its GxG diagonal blocks."""
+        for g in (pre_head_group, post_head_group):
+            if g is not None and (g <= 0 or self.n_heads % g):
+                raise ValueError(f"head group {g} does not divide n_heads={self.n_heads}")
+        self._declared = WeightStructure(pre_head_identity, pre_head_group, post_conv_identity, post_head_identity,
+                                         post_head_group)
+        self.weight_structure = "declared"
+        return self._declared
+
+    def assume_dense_weights(self) -> None:
+        """Back to the default: nothing is assumed about the weights."""
+        self._declared = WeightStructure()
+        self.weight_structure = "dense"
 
     def _forward_with_mask(self, xq, xk, xv, mask):
         """use_mask=True: an explicit additive mask tensor drives the masking (mta_attention_triton.py:63-64,
@@ -208,6 +299,7 @@ class MTAAttentionTriton(nn.Module):
         with torch.no_grad():
             nn.init.eye_(self.wpsm_triton.weight)
             nn.init.eye_(self.wposm_triton.weight)
+        self.assume_dense_weights()
 
     def _init_conv_kernel(self, kernel, init_std):
         method = self.mta_init_method
@@ -244,17 +336,7 @@ class MTAAttentionTriton(nn.Module):
                 self.wpsm_triton.weight.copy_(mta_attention.wpsm.weight.data)
             if hasattr(mta_attention, "wposm"):
                 self.wposm_triton.weight.copy_(mta_attention.wposm.weight.data)
-
-
-def _probe_head(w):
-    """(is identity, block-diagonal group size)."""
-    if ops.is_identity_head_weight(w):
-        return True, 1
-    return False, ops.block_diagonal_group(w)
-
-
-def _probe_conv(w):
-    return ops.is_identity_conv_kernel(w)
+        self.assume_dense_weights()
 
 
 def _lcm(a: int, b: int) -> int:
@@ -262,5 +344,4 @@ def _lcm(a: int, b: int) -> int:
     return a * b // math.gcd(a, b)
 
 
-__all__ = ["MTAAttentionTriton", "MTAConfig"]
-_ = Optional
+__all__ = ["MTAAttentionTriton", "MTAConfig", "WeightStructure"]

@@ -144,7 +144,7 @@ def conv_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, weight: tor
 
 
 def qk_conv(q: torch.Tensor, k: torch.Tensor, weight: torch.Tensor, causal: bool, scale: float,
-            fill_upper: bool = True) -> Optional[torch.Tensor]:
+            fill_upper: bool = True, out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """scale * conv(mask0(Q K^T)) as a (B,H,S,S) tensor without materialising Q K^T; see mta_qk_conv_fwd.
 
     Returns ``None`` when the library has no kernel for this dtype / size combination (the caller then
@@ -156,7 +156,10 @@ def qk_conv(q: torch.Tensor, k: torch.Tensor, weight: torch.Tensor, causal: bool
         raise ValueError(f"Q and K must share a (B,H,S,D) shape and dtype, got {tuple(q.shape)}, {tuple(k.shape)}")
     b, h, s, d = q.shape
     assert weight.dim() == 3 and weight.shape[0] == h, "conv weight must be (H,R,S)"
-    out = torch.empty((b, h, s, s), dtype=q.dtype, device=q.device)
+    if out is None:
+        out = torch.empty((b, h, s, s), dtype=q.dtype, device=q.device)
+    elif out.shape != (b, h, s, s) or out.dtype != q.dtype or out.device != q.device or not out.is_contiguous():
+        raise ValueError("out must be a contiguous (B,H,S,S) tensor of the inputs' dtype and device")
     with torch.cuda.device(q.device):
         rc = _lib.load().mta_qk_conv_fwd(q.data_ptr(), k.data_ptr(), weight.data_ptr(), out.data_ptr(), b, h, s, d,
                                          weight.shape[1], weight.shape[2], int(bool(causal)), float(scale),
@@ -191,30 +194,46 @@ def causal_pv_supported(p_dtype: torch.dtype, s: int, d: int) -> bool:
 
 
 # ---------------------------------------------------------------------------------------
-# weight structure probes (host side: each call copies the small weight to the host once)
+# weight structure probes (evaluated on the device; the result comes back in one small copy)
 # ---------------------------------------------------------------------------------------
-def block_diagonal_group(weight: torch.Tensor) -> int:
-    """Smallest G dividing H such that the (H,H) weight is zero outside its GxG diagonal blocks."""
-    w = weight.detach().float().cpu()
-    h = w.shape[0]
-    nz = w != 0
-    for g in range(1, h + 1):
-        if h % g:
-            continue
-        idx = torch.arange(h) // g
-        if not bool((nz & (idx[:, None] != idx[None, :])).any()):
-            return g
-    return h
+def _probe_head_into(weight: torch.Tensor, out: torch.Tensor) -> None:
+    w = _device_tensor(weight.detach(), "weight")
+    assert w.dim() == 2 and w.shape[0] == w.shape[1], f"Weight must be square matrix, got {w.shape}"
+    with torch.cuda.device(w.device):
+        rc = _lib.load().mta_probe_head_weight(w.data_ptr(), w.shape[0], _code(w, "weight"), out.data_ptr(), _stream(w))
+    _lib.check(rc, "mta_probe_head_weight")
 
 
-def is_identity_head_weight(weight: torch.Tensor) -> bool:
-    w = weight.detach().float().cpu()
-    return bool(torch.equal(w, torch.eye(w.shape[0])))
+def _probe_conv_into(weight: torch.Tensor, out: torch.Tensor) -> None:
+    w = _device_tensor(weight.detach(), "weight")
+    assert w.dim() == 3, f"conv kernel must be (C,R,S), got {tuple(w.shape)}"
+    with torch.cuda.device(w.device):
+        rc = _lib.load().mta_probe_conv_kernel(w.data_ptr(), w.shape[0], w.shape[1], w.shape[2], _code(w, "weight"),
+                                               out.data_ptr(), _stream(w))
+    _lib.check(rc, "mta_probe_conv_kernel")
 
 
-def is_identity_conv_kernel(weight: torch.Tensor) -> bool:
+def probe_head_weight(weight: torch.Tensor):
+    """(is exactly the identity, smallest G such that the (H,H) weight is zero outside its GxG diagonal blocks)."""
+    out = torch.empty(2, dtype=torch.int32, device=weight.device)
+    _probe_head_into(weight, out)
+    eye, group = out.tolist()
+    return bool(eye), int(group)
+
+
+def probe_conv_kernel(weight: torch.Tensor) -> bool:
     """True when the (C,R,S) kernel is exactly 1.0 at [R-1, S//2] and 0 elsewhere, S odd (a pass-through)."""
-    w = weight.detach().float().cpu()
-    ref = torch.zeros_like(w)
-    ref[:, -1, w.shape[-1] // 2] = 1.0
-    return bool(torch.equal(w, ref)) and (w.shape[-1] % 2 == 1)
+    out = torch.empty(1, dtype=torch.int32, device=weight.device)
+    _probe_conv_into(weight, out)
+    return bool(out.item())
+
+
+def probe_mta_weights(w_pre: torch.Tensor, w_post: torch.Tensor, conv_post: torch.Tensor):
+    """The three probes the MTA glue needs, with a single read back:
+    (pre identity, pre group, post identity, post group, post conv identity)."""
+    out = torch.empty(5, dtype=torch.int32, device=w_pre.device)
+    _probe_head_into(w_pre, out[0:2])
+    _probe_head_into(w_post, out[2:4])
+    _probe_conv_into(conv_post, out[4:5])
+    a, b, c, d, e = out.tolist()
+    return bool(a), int(b), bool(c), int(d), bool(e)

@@ -61,13 +61,17 @@ def headmix(x, w, causal: bool, fill: float):
     return y
 
 
-def mta_forward(q, k, v, w_pre, wpsm, w_post, wposm):
+def mta_forward(q, k, v, w_pre, wpsm, w_post, wposm, mask=None):
+    """``mask``: None = causal, else an additive (B,H,S,S) array of 0 / -inf."""
     q, k, v = _f32(q), _f32(k), _f32(v)
     w_pre, wpsm, w_post, wposm = _f32(w_pre), _f32(wpsm), _f32(w_post), _f32(wposm)
     b, h, s, d = q.shape
     out = np.empty((b, s, h, d), dtype=np.float32)
+    if mask is not None:
+        mask = _f32(mask)
+        assert mask.shape == (b, h, s, s)
     rc = _load().oracle_mta_forward(_p(q), _p(k), _p(v), _p(w_pre), _p(wpsm), _p(w_post), _p(wposm),
-                                    _p(out), _i64(b), _i64(h), _i64(s), _i64(d),
+                                    _p(mask) if mask is not None else None, _p(out), _i64(b), _i64(h), _i64(s), _i64(d),
                                     w_pre.shape[1], w_pre.shape[2], w_post.shape[1], w_post.shape[2])
     assert rc == 0
     return out

@@ -66,7 +66,8 @@ void oracle_headmix(const float *x, const float *wt, float *y, int64_t N, int64_
 
 static void conv_plane_d(const double *x, const float *w, double *y, int64_t S, int R, int Sk)
 {
-    /* causal depthwise conv of one S x S plane held in double; output NOT masked */
+    /* depthwise conv of one S x S plane held in double (blocked entries already zeroed by the
+     * caller); output NOT masked */
     const int pad_h = R - 1, pad_w = (Sk - 1) / 2;
     for (int64_t p = 0; p < S; ++p)
         for (int64_t q = 0; q < S; ++q) {
@@ -76,7 +77,7 @@ static void conv_plane_d(const double *x, const float *w, double *y, int64_t S, 
                 if (h < 0) continue;
                 for (int j = 0; j < Sk; ++j) {
                     int64_t k = q + j - pad_w;
-                    if (k < 0 || k >= S || k > h) continue;
+                    if (k < 0 || k >= S) continue;
                     acc += (double)w[i * Sk + j] * x[h * S + k];
                 }
             }
@@ -84,25 +85,39 @@ static void conv_plane_d(const double *x, const float *w, double *y, int64_t S, 
         }
 }
 
-/* Causal MTA forward (mask=None, pad_key="both", dropout 0), all in double.
+/* MTA forward (pad_key="both", dropout 0), all in double.
  * q,k,v: (B,H,S,D); w_pre: (H,R1,S1); wpsm,wposm: (H,H) row = output head;
- * w_post: (H,R2,S2); out: (B,S,H,D).  Returns 0, or -1 when out of memory. */
+ * w_post: (H,R2,S2); out: (B,S,H,D).
+ * mask: NULL = plain causal, else an additive (B,H,S,S) mask of 0 / -inf entries (what
+ * _update_mask of mta_attention_pytorch.py:114-137 hands to forward): blocked scores are
+ * zeroed before each conv (:89), -inf is added before the softmax (:69), blocked
+ * probabilities are zeroed after the second conv (:74).  A query row with every key
+ * blocked gives NaN, as torch's softmax does.
+ * Returns 0, or -1 when out of memory. */
 int oracle_mta_forward(const float *q, const float *k, const float *v, const float *w_pre,
-                       const float *wpsm, const float *w_post, const float *wposm, float *out,
+                       const float *wpsm, const float *w_post, const float *wposm,
+                       const float *mask, float *out,
                        int64_t B, int64_t H, int64_t S, int64_t D, int R1, int S1, int R2, int S2)
 {
     const int64_t plane = S * S;
     double *a = (double *)malloc(sizeof(double) * H * plane);
     double *b = (double *)malloc(sizeof(double) * H * plane);
-    if (!a || !b) { free(a); free(b); return -1; }
+    unsigned char *blk = (unsigned char *)malloc((size_t)(H * plane));
+    if (!a || !b || !blk) { free(a); free(b); free(blk); return -1; }
     const double scale = 1.0 / sqrt((double)D);
     for (int64_t n = 0; n < B; ++n) {
-        /* s0 = q k^T * scale, zero above the diagonal (the conv's input mask) */
+        for (int64_t h = 0; h < H; ++h)
+            for (int64_t p = 0; p < S; ++p)
+                for (int64_t c = 0; c < S; ++c)
+                    blk[h * plane + p * S + c] =
+                        mask ? (unsigned char)(mask[((n * H + h) * S + p) * S + c] == -INFINITY)
+                             : (unsigned char)(c > p);
+        /* s0 = q k^T * scale, zero where blocked (the conv's input mask) */
         for (int64_t h = 0; h < H; ++h)
             for (int64_t p = 0; p < S; ++p)
                 for (int64_t c = 0; c < S; ++c) {
                     double acc = 0.0;
-                    if (c <= p)
+                    if (!blk[h * plane + p * S + c])
                         for (int64_t d = 0; d < D; ++d)
                             acc += (double)q[((n * H + h) * S + p) * D + d] *
                                    (double)k[((n * H + h) * S + c) * D + d];
@@ -114,8 +129,10 @@ int oracle_mta_forward(const float *q, const float *k, const float *v, const flo
         /* s2 = wpsm . s1 over heads, then + mask, softmax over keys */
         for (int64_t p = 0; p < S; ++p)
             for (int64_t o = 0; o < H; ++o) {
+                const unsigned char *bl = blk + o * plane + p * S;
                 double mx = -INFINITY;
-                for (int64_t c = 0; c <= p; ++c) {
+                for (int64_t c = 0; c < S; ++c) {
+                    if (bl[c]) continue;
                     double acc = 0.0;
                     for (int64_t i = 0; i < H; ++i)
                         acc += (double)wpsm[o * H + i] * b[i * plane + p * S + c];
@@ -123,19 +140,21 @@ int oracle_mta_forward(const float *q, const float *k, const float *v, const flo
                     if (acc > mx) mx = acc;
                 }
                 double den = 0.0;
-                for (int64_t c = 0; c <= p; ++c) {
+                for (int64_t c = 0; c < S; ++c) {
+                    if (bl[c]) continue;
                     double e = exp(a[o * plane + p * S + c] - mx);
                     a[o * plane + p * S + c] = e;
                     den += e;
                 }
                 for (int64_t c = 0; c < S; ++c)
-                    a[o * plane + p * S + c] = (c <= p) ? a[o * plane + p * S + c] / den : 0.0;
+                    a[o * plane + p * S + c] = bl[c] ? 0.0 : a[o * plane + p * S + c] / den;
             }
-        /* p1 = conv_post(p0), zero above the diagonal */
+        /* p1 = conv_post(p0) (p0 is already 0 where blocked), then zero where blocked */
         for (int64_t h = 0; h < H; ++h) {
             conv_plane_d(a + h * plane, w_post + h * R2 * S2, b + h * plane, S, R2, S2);
             for (int64_t p = 0; p < S; ++p)
-                for (int64_t c = p + 1; c < S; ++c) b[h * plane + p * S + c] = 0.0;
+                for (int64_t c = 0; c < S; ++c)
+                    if (blk[h * plane + p * S + c]) b[h * plane + p * S + c] = 0.0;
         }
         /* p2 = wposm . p1 ; out = p2 v, stored (B,S,H,D) */
         for (int64_t o = 0; o < H; ++o)
@@ -156,6 +175,7 @@ int oracle_mta_forward(const float *q, const float *k, const float *v, const flo
     }
     free(a);
     free(b);
+    free(blk);
     return 0;
 }
 

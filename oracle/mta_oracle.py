@@ -13,7 +13,9 @@ follows.  How each one is pinned (see tests/test_oracle.py):
   identity tap == tril(x) bit-exact, linearity.
 * ``head_linear``: einsum against nested C loops, W=I pass-through, permutation W.
 * ``mta_forward``: all-identity weights == causal scaled-dot-product attention,
-  row 0 closed form, stage-by-stage equality with the C restatement.
+  row 0 closed form, stage-by-stage equality with the C restatement; its tensor-mask
+  branch (bool, (1,Sk) key mask, (1,1,S,S) additive) against the C restatement given
+  the same additive mask; ``mta_forward_rows`` (slab form) == full form.
 * ``conv_attention_forward``: identity tap == causal SDPA, C restatement, equality
   with the composition of the pinned stages, slab form == full form.
 
@@ -160,6 +162,39 @@ def mta_forward(xq, xk, xv, mta_kernel, wpsm, mta_kernel_after_sm, wposm, mask=N
     if return_stages:
         return out, {"s0": s0, "s1": s1, "s2": s2, "p0": p0, "p1": p1, "p2": p2}
     return out
+
+
+def mta_forward_rows(xq, xk, xv, mta_kernel, wpsm, mta_kernel_after_sm, wposm, row0: int, row1: int):
+    """Query rows [row0,row1) of the causal ``mta_forward`` (mask=None, pad_key="both", no dropout)
+    without the full S x S tensors; returns (B, row1-row0, H, D).
+
+    A query row of the result depends on the R2-1 probability rows above it (top halo of the
+    second conv), each of which depends on the R1-1 score rows above it (top halo of the
+    first), on all heads at its own positions and on every key and value.  So the same
+    library calls as in ``mta_forward`` are applied to rows [lo,row1) with
+    lo = max(0, row0-(R1-1)-(R2-1)) as if row lo were the first row; rows whose halo was
+    cut off are wrong and are dropped (none when lo = 0).  Equality with the full form is
+    checked in tests/test_oracle.py.
+    """
+    r1, r2 = mta_kernel.shape[-2], mta_kernel_after_sm.shape[-2]
+    sk = xk.size(-2)
+    lo = max(0, row0 - (r1 - 1) - (r2 - 1))
+    rows = torch.arange(lo, row1, device=xq.device)[:, None]
+    cols = torch.arange(sk, device=xq.device)[None, :]
+    mask = torch.zeros(row1 - lo, sk, device=xq.device).masked_fill(cols > rows, NEG_INF).type_as(xq)
+    mask = mask.repeat(xq.size(0), xq.size(1), 1, 1)
+    head_dim = xq.size(-1)
+    scale = torch.rsqrt(torch.tensor(head_dim, requires_grad=False, device=xq.device))
+    s0 = torch.matmul(xq[:, :, lo:row1], xk.transpose(2, 3)) * scale
+    s1 = mta_convolution(s0, mask, mta_kernel, "both")
+    s2 = F.linear(s1.transpose(1, -1), wpsm).transpose(1, -1)
+    s3 = s2 + mask
+    p0 = F.softmax(s3.float(), dim=-1).type_as(xq)
+    p1 = mta_convolution(p0, mask, mta_kernel_after_sm, "both")
+    p1 = torch.where(mask == NEG_INF, 0.0, p1)
+    p2 = F.linear(p1.transpose(1, -1), wposm).transpose(1, -1)
+    out = torch.matmul(p2, xv).transpose(1, 2)
+    return out[:, row0 - lo:]
 
 
 # ---------------------------------------------------------------------------

@@ -25,7 +25,8 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     names = declared_functions()
     assert {"mta_conv2d_fwd", "mta_conv2d_scaled_fwd", "mta_headmix_fwd", "mta_headmix_softmax_fwd",
-            "mta_conv_attn_fwd", "mta_qk_conv_fwd", "mta_causal_pv_fwd", "mta_strerror", "mta_abi_version"} <= set(names)
+            "mta_conv_attn_fwd", "mta_qk_conv_fwd", "mta_causal_pv_fwd", "mta_strerror", "mta_abi_version",
+            "mta_probe_head_weight", "mta_probe_conv_kernel"} <= set(names)
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/mta_hip.h but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes signatures out of sync with the header"
@@ -118,7 +119,6 @@ def test_reset_and_copy_parameters():
     w = mod.mta_conv_triton.weight
     assert w[0, 2, 2] == 1 and w.sum() == 4            # identity tap at [R-1, S//2]
     assert torch.equal(mod.wpsm_triton.weight, torch.eye(4)) and torch.equal(mod.wposm_triton.weight, torch.eye(4))
-    assert ops.is_identity_conv_kernel(w) and ops.is_identity_head_weight(mod.wpsm_triton.weight)
 
     class Src:  # the PyTorch module's parameter layout: conv kernels are (H,1,R,S)
         mta_kernel = torch.nn.Parameter(torch.randn(4, 1, 3, 5))
@@ -138,27 +138,54 @@ def test_reset_and_copy_parameters():
         mta.MTAAttentionTriton(4, cfg, 0.0, True).reset_mta_parameters()
 
 
-def test_structure_probes():
-    g = torch.Generator().manual_seed(0)
-    w = torch.zeros(8, 8)
-    for b in range(0, 8, 4):
-        w[b:b + 4, b:b + 4] = torch.randn(4, 4, generator=g)
-    assert ops.block_diagonal_group(w) == 4
-    assert ops.block_diagonal_group(torch.eye(8)) == 1
-    assert ops.block_diagonal_group(torch.randn(6, 6, generator=g)) == 6
-    k = torch.zeros(2, 3, 4)
-    k[:, -1, 2] = 1
-    assert not ops.is_identity_conv_kernel(k)          # even key size: the tap is off by one, not a pass-through
+def test_weight_structure_is_an_opt_in():
     cfg = mta.MTAConfig()
     mod = mta.MTAAttentionTriton(4, cfg, 0.0, True)
+    assert mod.weight_structure == "dense" and mod._current_structure() == mta.WeightStructure()
+    st = mod.declare_weight_structure(pre_head_identity=True, post_conv_identity=True, post_head_group=2)
+    assert mod.weight_structure == "declared" and mod._current_structure() is st
+    assert st.post_head_group == 2 and st.pre_head_group is None and not st.post_head_identity
+    with pytest.raises(ValueError, match="does not divide"):
+        mod.declare_weight_structure(post_head_group=3)
+    # every way the module itself replaces parameters drops the declaration
     mod.reset_mta_parameters()
-    from multitokenatention_triton_amd.mta_attention_triton import _probe_head
-    assert mod._probe("wposm", mod.wposm_triton.weight, _probe_head) == (True, 1)
-    with torch.no_grad():
-        mod.wposm_triton.weight[0, 3] = 0.5              # in-place under no_grad moves the version counter
-    assert mod._probe("wposm", mod.wposm_triton.weight, _probe_head) == (False, 4)
-    mod.weight_structure = "dense"
-    assert mod._probe("wposm", mod.wposm_triton.weight, _probe_head) == (False, 4)
+    assert mod.weight_structure == "dense"
+    mod.declare_weight_structure(post_head_group=2)
+    mod.load_state_dict(mod.state_dict())
+    assert mod.weight_structure == "dense"
+    mod.declare_weight_structure(post_head_group=2)
+    mod.copy_mta_parameters(object())
+    assert mod.weight_structure == "dense"
+    mod.weight_structure = "sometimes"
+    with pytest.raises(ValueError, match="weight_structure"):
+        mod._current_structure()
+    with pytest.raises(RuntimeError, match="no CPU path"):      # the probes run on the device only
+        mod.infer_weight_structure()
+
+
+def test_forward_route_follows_grad_mode():
+    """With grad enabled and parameters that require grad the module runs operator by operator (so that a graph is
+    recorded); otherwise it takes the fused route.  Neither has a CPU path, so both stop at their first kernel."""
+    mod = mta.MTAAttentionTriton(4, mta.MTAConfig(), 0.0, True)
+    x = torch.zeros(1, 4, 8, 64)
+    seen = []
+    mod._stage_hook = seen.append
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        mod(x, x, x, None, None)
+    assert seen == ["qk", "conv_pre"]
+    seen.clear()
+    with torch.no_grad(), pytest.raises(RuntimeError, match="no CPU path"):
+        mod(x, x, x, None, None)
+    assert seen == ["qk_conv"]
+    seen.clear()
+    mod.requires_grad_(False)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        mod(x, x, x, None, None)
+    assert seen == ["qk_conv"]
+    seen.clear()
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        mod(x.clone().requires_grad_(True), x, x, None, None)
+    assert seen == ["qk", "conv_pre"]
 
 
 def test_dropin_shims_resolve():

@@ -25,16 +25,26 @@ def pkg():
     return m
 
 
-def _mta_module(pkg, h, r1, s1, r2, s2, w_pre, wpsm, w_post, wposm, dtype, causal=True):
+def _mta_module(pkg, h, r1, s1, r2, s2, w_pre, wpsm, w_post, wposm, dtype, causal=True, use_mask=False,
+                structure="infer"):
+    """Inference-mode module on the GPU (parameters do not require grad, so forward takes the fused route).
+    structure: "infer" = look at the weights once, "dense" = assume nothing, "probe" = look on every call."""
     cfg = pkg.MTAConfig(query_kernel_size=r1, key_kernel_size=s1, after_sm_query_kernel_size=r2,
                         after_sm_key_kernel_size=s2)
-    mod = pkg.MTAAttentionTriton(h, cfg, dropout=0.0, causal=causal, use_mask=False)
+    mod = pkg.MTAAttentionTriton(h, cfg, dropout=0.0, causal=causal, use_mask=use_mask)
     with torch.no_grad():
         mod.mta_conv_triton.weight.copy_(w_pre)
         mod.wpsm_triton.weight.copy_(wpsm)
         mod.mta_conv_after_sm_triton.weight.copy_(w_post)
         mod.wposm_triton.weight.copy_(wposm)
-    return mod.to(dtype).cuda().eval()
+    mod = mod.to(dtype).cuda().eval().requires_grad_(False)
+    if structure == "infer":
+        mod.infer_weight_structure()
+    elif structure == "probe":
+        mod.weight_structure = "probe"
+    else:
+        assert structure == "dense" and mod.weight_structure == "dense"
+    return mod
 
 
 def _config_like(h, group, r1, s1, std, dtype, post="identity", seed=123):
@@ -66,14 +76,15 @@ def test_mta_config1_fp32(pkg):
     torch.testing.assert_close(got.cpu(), want, **tol(torch.float32))
 
 
+@pytest.mark.parametrize("structure", ["infer", "dense", "probe"])
 @pytest.mark.parametrize("post", ["identity", "random"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
-def test_mta_general(pkg, dtype, post):
-    print(f"mta general {dtype} post={post}", flush=True)
+def test_mta_general(pkg, dtype, post, structure):
+    print(f"mta general {dtype} post={post} structure={structure}", flush=True)
     q, k, v = O.seeded_qkv(2, 8, 200, 64, dtype)
     params = _config_like(8, 4, 6, 11, 0.05, dtype, post=post)
     want = _oracle_mta(q, k, v, params)
-    mod = _mta_module(pkg, 8, 6, 11, 3, 3, *params, dtype)
+    mod = _mta_module(pkg, 8, 6, 11, 3, 3, *params, dtype, structure=structure)
     got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
     torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
 
@@ -98,9 +109,20 @@ def test_mta_identity_weights_is_sdpa(pkg):
     mod = pkg.MTAAttentionTriton(16, cfg, 0.0, True).cuda().eval()
     mod.reset_mta_parameters()
     q, k, v = O.seeded_qkv(2, 16, 128, 64, torch.float32, seed=123)
-    got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
     want = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2)
-    torch.testing.assert_close(got, want, rtol=1e-3, atol=1e-5)  # the reference script's own bar
+    stages = []
+    mod._stage_hook = stages.append
+    got = mod(q.cuda(), k.cuda(), v.cuda(), None, None)     # parameters require grad: operator by operator
+    assert stages == ["qk", "conv_pre", "mix_pre", "softmax", "conv_post", "mix_post", "pv", "end"]
+    assert got.grad_fn is not None
+    torch.testing.assert_close(got.detach().cpu(), want, rtol=1e-3, atol=1e-5)  # the reference script's own bar
+    torch.testing.assert_close(got.detach().cpu(), want, **tol(torch.float32))
+    with torch.no_grad():                                    # inference: fused route, dense weights assumed
+        got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
+    torch.testing.assert_close(got, want, **tol(torch.float32))
+    assert mod.infer_weight_structure() == pkg.WeightStructure(True, 1, True, True, 1)
+    with torch.no_grad():
+        got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
     torch.testing.assert_close(got, want, **tol(torch.float32))
 
 
@@ -206,8 +228,9 @@ def test_qk_conv_parity(pkg, case, fill):
     s0 = torch.matmul(q, k.transpose(2, 3)) * torch.rsqrt(torch.tensor(d))
     want = O.depthwise_conv(torch.tril(s0) if causal else s0, w, causal)
     sentinel = 12345.0
-    got = pkg.ops.qk_conv(q.cuda(), k.cuda(), w.cuda(), causal, scale, fill_upper=fill)
-    assert got is not None and got.shape == (b, h, s, s)
+    buf = torch.full((b, h, s, s), sentinel, dtype=dtype, device="cuda")
+    got = pkg.ops.qk_conv(q.cuda(), k.cuda(), w.cuda(), causal, scale, fill_upper=fill, out=buf)
+    assert got is buf and got.shape == (b, h, s, s)
     got = got.cpu()
     low = torch.tril(torch.ones(s, s, dtype=torch.bool)) if causal else torch.ones(s, s, dtype=torch.bool)
     # scores of magnitude ~sqrt(d)*|w| pass through two 16-bit roundings: 2 ulp + atol
@@ -216,7 +239,8 @@ def test_qk_conv_parity(pkg, case, fill):
     if causal and fill:
         up = ~low
         assert (got[..., up] == 0).all() and not torch.signbit(got[..., up]).any()
-    _ = sentinel
+    if causal and not fill:     # nothing above the diagonal may have been written
+        assert (got[..., ~low].float() == torch.tensor(sentinel).to(dtype).float()).all()
 
 
 def test_qk_conv_reports_unsupported(pkg):
@@ -346,3 +370,225 @@ def test_mta_forward_graph_capture_replay(pkg):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, want), f"replay {i} differs from the eager forward"
+
+
+# ------------------------------------------------------------------------------------------------------
+# weight structure is an opt-in: a rewritten parameter must never be served from stale assumptions
+# ------------------------------------------------------------------------------------------------------
+def test_mta_data_write_after_forward_is_seen(pkg):
+    """Run with identity / block-diagonal weights, then overwrite the weights through ``.data`` (the reference's own
+    idiom, mta_attention_triton.py:185-201) with dense ones and run again: the second result must follow the new
+    weights, without any call that tells the module about the change."""
+    print("mta .data write", flush=True)
+    dtype = torch.bfloat16
+    h = 8
+    q, k, v = O.seeded_qkv(1, h, 256, 64, dtype, seed=77)
+    g = torch.Generator().manual_seed(78)
+    first = [O.seeded_conv_weight(h, 6, 11, 0.05, dtype), torch.eye(h, dtype=dtype),
+             O.identity_conv_kernel(h, 3, 3, dtype), O.block_diag_head_weight(h, 4, 0.1, g, dtype)]
+    second = [O.seeded_conv_weight(h, 6, 11, 0.05, dtype, seed=5),
+              (torch.eye(h) + 0.1 * torch.randn(h, h, generator=g)).to(dtype),
+              O.seeded_conv_weight(h, 3, 3, 0.05, dtype, seed=6),
+              (torch.eye(h) + 0.1 * torch.randn(h, h, generator=g)).to(dtype)]
+    for structure in ("dense", "probe"):
+        mod = _mta_module(pkg, h, 6, 11, 3, 3, *first, dtype, structure=structure)
+        got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
+        torch.testing.assert_close(got.float(), _oracle_mta(q, k, v, first).float(), **tol(dtype))
+        for dst, src in zip((mod.mta_conv_triton, mod.wpsm_triton, mod.mta_conv_after_sm_triton, mod.wposm_triton),
+                            second):
+            dst.weight.data.copy_(src)
+        got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
+        torch.testing.assert_close(got.float(), _oracle_mta(q, k, v, second).float(), **tol(dtype))
+    # the explicit opt-in is dropped by the module's own ways of replacing parameters
+    mod = _mta_module(pkg, h, 6, 11, 3, 3, *first, dtype, structure="infer")
+    assert mod.weight_structure == "declared" and mod._declared.post_head_group == 4
+    mod.load_state_dict({k_: v_.clone() for k_, v_ in mod.state_dict().items()})
+    assert mod.weight_structure == "dense"
+
+
+def test_weight_probes_on_device(pkg):
+    print("weight probes", flush=True)
+    ops = pkg.ops
+    g = torch.Generator().manual_seed(0)
+    for dtype in (torch.float32, torch.bfloat16, torch.float16):
+        w = torch.zeros(8, 8)
+        for b in range(0, 8, 4):
+            w[b:b + 4, b:b + 4] = torch.randn(4, 4, generator=g)
+        assert ops.probe_head_weight(w.to(dtype).cuda()) == (False, 4)
+        assert ops.probe_head_weight(torch.eye(8, dtype=dtype).cuda()) == (True, 1)
+        assert ops.probe_head_weight((2 * torch.eye(8)).to(dtype).cuda()) == (False, 1)
+        assert ops.probe_head_weight(torch.randn(6, 6, generator=g).to(dtype).cuda()) == (False, 6)
+        w12 = torch.zeros(12, 12)
+        w12[0:3, 0:3] = 1.0
+        w12[3:6, 3:6] = 1.0
+        w12[6:12, 6:12] = torch.randn(6, 6, generator=g)
+        assert ops.probe_head_weight(w12.to(dtype).cuda()) == (False, 6)
+        w12[11, 0] = 1e-3
+        assert ops.probe_head_weight(w12.to(dtype).cuda()) == (False, 12)
+        assert ops.probe_conv_kernel(O.identity_conv_kernel(5, 6, 11, dtype).cuda())
+        assert ops.probe_conv_kernel(O.identity_conv_kernel(3, 1, 1, dtype).cuda())
+        k = O.identity_conv_kernel(5, 6, 11, dtype)
+        k[4, 0, 0] = 1e-3
+        assert not ops.probe_conv_kernel(k.cuda())
+        k = torch.zeros(2, 3, 4, dtype=dtype)
+        k[:, -1, 2] = 1            # even key size: the tap is off by one, not a pass-through
+        assert not ops.probe_conv_kernel(k.cuda())
+        k = torch.zeros(2, 3, 3, dtype=dtype)
+        k[:, 1, 1] = 1             # the module default (geometric centre) is not the pass-through tap
+        assert not ops.probe_conv_kernel(k.cuda())
+    assert ops.probe_head_weight(torch.eye(32).cuda() * float("nan")) == (False, 32)
+
+
+# ------------------------------------------------------------------------------------------------------
+# BASELINE configs at their full size, every head checked
+# ------------------------------------------------------------------------------------------------------
+def test_conv_attention_c5_full_size(pkg):
+    """BASELINE config 5 at its real size: B1 H32 S8192 D128 bf16, 6x11, causal.  All 32 heads are compared with the
+    slab form of the oracle on the first rows, on rows that cross the edge between two of the kernel's 248-row query
+    blocks (248*17 = 4216), and on the last rows; query row 0 has the closed form o[0] = v[0]."""
+    print("conv_attention C5 full size", flush=True)
+    dtype = torch.bfloat16
+    b, h, s, d = 1, 32, 8192, 128
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=500)
+    w = O.seeded_conv_weight(h, 6, 11, 0.05, dtype)
+    got = pkg.ops.conv_attn_fwd(q.cuda(), k.cuda(), v.cuda(), w.cuda(), True, None).cpu()
+    assert torch.isfinite(got.float()).all()
+    torch.testing.assert_close(got[:, :, 0].float(), v[:, :, 0].float(), rtol=0.0, atol=1e-6)
+    for r0, r1 in [(0, 96), (4168, 4264), (8096, 8192)]:
+        print(f"  slab {r0}:{r1}", flush=True)
+        want = O.conv_attention_rows(q, k, v, w, r0, r1, True, None)
+        torch.testing.assert_close(got[:, :, r0:r1].float(), want.float(), **tol(dtype))
+
+
+def test_mta_headline_full_size_all_groups(pkg):
+    """BASELINE config 4 at full size, every (batch, head): three row slabs (first rows; rows crossing the edge
+    between two 248-row query blocks of the scores kernel, 248*8 = 1984; last rows) against the slab form of the
+    oracle, which carries all 16 heads and both batch elements."""
+    print("mta headline full size, all groups", flush=True)
+    dtype = torch.bfloat16
+    b, h, s, d, grp = 2, 16, 4096, 128, 4
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=300)
+    g = torch.Generator().manual_seed(127)
+    params = [O.seeded_conv_weight(h, 6, 11, 0.05, dtype), torch.eye(h, dtype=dtype),
+              O.identity_conv_kernel(h, 3, 3, dtype), O.block_diag_head_weight(h, grp, 0.1, g, dtype)]
+    mod = _mta_module(pkg, h, 6, 11, 3, 3, *params, dtype)
+    stages = []
+    mod._stage_hook = stages.append
+    got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
+    assert stages == ["qk_conv", "mix_softmax_mix", "pv", "end"]
+    assert torch.isfinite(got.float()).all()
+    for r0, r1 in [(0, 64), (1952, 2016), (4032, 4096)]:
+        print(f"  slab {r0}:{r1}", flush=True)
+        want = O.mta_forward_rows(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3], r0, r1)
+        torch.testing.assert_close(got[:, r0:r1].float(), want.float(), **tol(dtype))
+
+
+# ------------------------------------------------------------------------------------------------------
+# use_mask=True with real tensor masks, and the non-causal module
+# ------------------------------------------------------------------------------------------------------
+def _masks(s):
+    g = torch.Generator().manual_seed(31)
+    keep = torch.rand(1, s, generator=g) > 0.3
+    keep[0, 0] = True                       # key 0 stays visible: no query row is fully blocked
+    add = torch.zeros(1, 1, s, s)
+    add.masked_fill_(torch.triu(torch.ones(s, s, dtype=torch.bool), 1), float("-inf"))
+    add[0, 0, 40:, 9:23] = float("-inf")    # a block of keys hidden from the later rows
+    boolean = torch.tril(torch.ones(s, s, dtype=torch.bool))[None, None].clone()
+    boolean[0, 0, 5:, 2] = False
+    return {"key_mask_bool": keep, "key_mask_additive": torch.where(keep, 0.0, float("-inf")),
+            "additive_11SS": add, "bool_11SS": boolean}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("name", ["key_mask_bool", "key_mask_additive", "additive_11SS", "bool_11SS"])
+def test_mta_use_mask_tensor_masks(pkg, name, dtype):
+    """mta_attention_triton.py:63-64, 77-83, 96-127 with a mask tensor, vs the oracle given the same mask."""
+    print(f"mta use_mask {name} {dtype}", flush=True)
+    b, h, s, d = (1, 4, 136, 64)
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=91)
+    params = _config_like(h, 2, 3, 5, 0.1, dtype, post="random")
+    mask = _masks(s)[name]
+    want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3], mask=mask)
+    assert torch.isfinite(want.float()).all()
+    for structure in ("dense", "infer"):
+        mod = _mta_module(pkg, h, 3, 5, 3, 3, *params, dtype, use_mask=True, structure=structure)
+        got = mod(q.cuda(), k.cuda(), v.cuda(), mask.cuda(), None).cpu()
+        torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+
+
+def test_mta_use_mask_key_mask_batched_additive_4d(pkg):
+    """A (B,1,1,Sk)-style key mask cannot be expressed in the reference's 2-D form for B>1 (its repeat() stacks
+    batches along the query axis, mta_attention_pytorch.py:130), so batches with different hidden keys arrive as a
+    full (B,H,S,S) additive mask."""
+    print("mta use_mask (B,H,S,S)", flush=True)
+    dtype = torch.bfloat16
+    b, h, s, d = 2, 4, 96, 64
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=92)
+    params = _config_like(h, 4, 3, 3, 0.1, dtype, post="identity")
+    g = torch.Generator().manual_seed(4)
+    keep = torch.rand(b, s, generator=g) > 0.25
+    keep[:, 0] = True
+    causal = torch.tril(torch.ones(s, s, dtype=torch.bool))
+    visible = (keep[:, None, None, :] & causal[None, None]).expand(b, h, s, s)
+    mask = torch.where(visible, 0.0, float("-inf")).to(dtype).contiguous()
+    want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3], mask=mask)
+    mod = _mta_module(pkg, h, 3, 3, 3, 3, *params, dtype, use_mask=True)
+    got = mod(q.cuda(), k.cuda(), v.cuda(), mask.cuda(), None).cpu()
+    torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_mta_non_causal_module(pkg, dtype):
+    """MTAAttentionTriton(causal=False): no masking anywhere -- the oracle with an all-visible mask."""
+    print(f"mta causal=False {dtype}", flush=True)
+    b, h, s, d = 1, 4, 120, 64
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=93)
+    params = _config_like(h, 2, 3, 5, 0.1, dtype, post="random")
+    mask = torch.zeros(1, 1, s, s)
+    want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3], mask=mask)
+    for structure in ("dense", "infer"):
+        mod = _mta_module(pkg, h, 3, 5, 3, 3, *params, dtype, causal=False, structure=structure)
+        got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
+        torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+    # the same module with use_mask=True and a sliding-window mask (non-causal kernels, mask from the tensor only)
+    band = ((torch.arange(s)[:, None] - torch.arange(s)[None, :]).abs() <= 9)[None, None]
+    want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3], mask=band)
+    mod = _mta_module(pkg, h, 3, 5, 3, 3, *params, dtype, causal=False, use_mask=True)
+    got = mod(q.cuda(), k.cuda(), v.cuda(), band.cuda(), None).cpu()
+    torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+
+
+def test_conv_attention_general_kernel_bf16(pkg):
+    """16-bit inputs with a kernel size that has no matrix-core conv instantiation (11x15) take the general kernel."""
+    print("conv_attention general bf16", flush=True)
+    for dtype in (torch.bfloat16, torch.float16):
+        q, k, v = O.seeded_qkv(1, 2, 333, 128, dtype, seed=42)
+        w = O.seeded_conv_weight(2, 11, 15, 0.05, dtype)
+        want = O.conv_attention_forward(q, k, v, w, True, None)
+        got = pkg.ops.conv_attn_fwd(q.cuda(), k.cuda(), v.cuda(), w.cuda(), True, None).cpu()
+        torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+
+
+def test_mta_unfused_16bit_route_never_reads_above_the_diagonal(pkg):
+    """The stages of the 16-bit route that leave the upper triangle unwritten (scores kernel, mix+softmax with
+    fill_upper=False) feed consumers that must not read it: run them into NaN-filled buffers and pass those on to
+    the conv, the head mixing and P V."""
+    print("mta poisoned upper triangle", flush=True)
+    dtype = torch.bfloat16
+    b, h, s, d = 1, 8, 264, 64
+    ops = pkg.ops
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=95)
+    w_pre, wpsm, w_post, wposm = _config_like(h, 4, 6, 11, 0.05, dtype, post="random")
+    want = _oracle_mta(q, k, v, [w_pre, wpsm, w_post, wposm])
+    nan = lambda: torch.full((b, h, s, s), float("nan"), dtype=dtype, device="cuda")
+    scale = float(torch.rsqrt(torch.tensor(float(d))))
+    s1 = ops.qk_conv(q.cuda(), k.cuda(), w_pre.cuda(), True, scale, fill_upper=False, out=nan())
+    p0 = ops.headmix_softmax(s1, wpsm.cuda(), None, True, group_size=4, out=nan(), fill_upper=False)
+    up = torch.triu(torch.ones(s, s, dtype=torch.bool, device="cuda"), 1)
+    assert torch.isnan(p0[..., up]).all()
+    p1 = ops.conv2d_causal(p0, w_post.cuda(), True)
+    p2 = ops.headmix(p1, wposm.cuda(), True, 0.0, group_size=4)
+    assert torch.isfinite(p2.float()).all() and (p2[..., up] == 0).all()
+    p2 = p2.masked_fill(up, float("nan"))
+    out = ops.causal_pv(p2, v.cuda(), True)
+    torch.testing.assert_close(out.transpose(1, 2).cpu().float(), want.float(), **tol(dtype))

@@ -232,3 +232,56 @@ def test_conv_attention_is_composition_of_pinned_stages():
     want = torch.matmul(torch.softmax(c * 0.25, -1), v)
     got = O.conv_attention_forward(q, k, v, w, True, 0.25)
     torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)
+
+
+def test_mta_slab_form_equals_full_form():
+    q, k, v = O.seeded_qkv(2, 4, 80, 16, torch.float32)
+    g = torch.Generator().manual_seed(21)
+    w_pre = O.seeded_conv_weight(4, 6, 11, 0.05, torch.float32).unsqueeze(1)
+    w_post = O.seeded_conv_weight(4, 3, 3, 0.1, torch.float32, seed=9).unsqueeze(1)
+    wpsm = O.block_diag_head_weight(4, 2, 0.1, g)
+    wposm = O.block_diag_head_weight(4, 4, 0.1, g)
+    full = O.mta_forward(q, k, v, w_pre, wpsm, w_post, wposm)
+    for r0, r1 in [(0, 10), (3, 30), (7, 8), (64, 80)]:
+        slab = O.mta_forward_rows(q, k, v, w_pre, wpsm, w_post, wposm, r0, r1)
+        assert slab.shape == (2, r1 - r0, 4, 16)
+        torch.testing.assert_close(slab, full[:, r0:r1], rtol=1e-5, atol=1e-6)
+
+
+def _mask_cases(s):
+    g = torch.Generator().manual_seed(31)
+    keep = torch.rand(1, s, generator=g) > 0.3
+    keep[0, 0] = True                       # key 0 stays visible: no query row is fully blocked
+    add = torch.zeros(1, 1, s, s)
+    add.masked_fill_(torch.triu(torch.ones(s, s, dtype=torch.bool), 1), float("-inf"))
+    add[0, 0, 10:, 3:7] = float("-inf")     # a block of keys hidden from the later rows
+    boolean = torch.tril(torch.ones(s, s, dtype=torch.bool))[None, None].clone()
+    boolean[0, 0, 5:, 2] = False
+    # non-causal shapes: a sliding window and a fully visible plane
+    band = (torch.arange(s)[:, None] - torch.arange(s)[None, :]).abs() <= 6
+    return {"key_mask_bool": keep, "additive_11SS": add, "bool_11SS": boolean,
+            "band_bool": band[None, None], "all_visible": torch.zeros(1, 1, s, s)}
+
+
+@pytest.mark.parametrize("name", ["key_mask_bool", "additive_11SS", "bool_11SS", "band_bool", "all_visible"])
+def test_mta_tensor_masks_vs_c_restatement(name):
+    """The explicit-mask branch of mta_forward (mta_attention_pytorch.py:58-83, 114-137) against the C loops
+    given the additive mask that update_mask produces."""
+    s = 24
+    q, k, v = O.seeded_qkv(1, 4, s, 8, torch.float32, seed=55)
+    g = torch.Generator().manual_seed(23)
+    w_pre = O.seeded_conv_weight(4, 3, 5, 0.1, torch.float32)
+    w_post = O.seeded_conv_weight(4, 2, 3, 0.1, torch.float32, seed=5)
+    wpsm = O.block_diag_head_weight(4, 2, 0.1, g) + 0.05 * _rand((4, 4), 17)
+    wposm = O.block_diag_head_weight(4, 2, 0.1, g)
+    mask = _mask_cases(s)[name]
+    got = O.mta_forward(q, k, v, w_pre.unsqueeze(1), wpsm, w_post.unsqueeze(1), wposm, mask=mask).numpy()
+    add = O.update_mask(mask, 1, 4, q, s)
+    assert add.shape == (1, 4, s, s) and not torch.isneginf(add).all(-1).any()
+    want = c_oracle.mta_forward(q.numpy(), k.numpy(), v.numpy(), w_pre.numpy(), wpsm.numpy(), w_post.numpy(),
+                                wposm.numpy(), mask=add.numpy())
+    assert np.isfinite(got).all()
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-5)
+    if name == "key_mask_bool":     # hidden keys and the causal rule both took effect
+        hidden = (~mask[0]).nonzero().flatten()
+        assert torch.isneginf(add[0, :, :, hidden]).all() and torch.isneginf(add[0, 0, 3, 4])
