@@ -82,7 +82,8 @@ int mta_headmix_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C,
  *                                               causal: q>p takes no part)
  *   p[o] = softmax over q of s[o]              (fp32, rounded to the I/O dtype)
  *   y[o] = w2 ? sum_i w2[o,i] p[i] : p[o]      (causal: q>p written as +0.0 when fill_upper != 0,
- *                                               left untouched when fill_upper == 0 -- for a consumer
+ *                                               unspecified when fill_upper == 0 (left alone, or zero
+ *                                               where a tile straddles the diagonal) -- for a consumer
  *                                               such as mta_causal_pv_fwd that never reads it)
  * w1 and/or w2 may be NULL (identity); both NULL is a plain causal row softmax.
  * group_size as in mta_headmix_fwd and applies to both weights.
@@ -110,7 +111,8 @@ int mta_conv_attn_fwd(const void *q, const void *k, const void *v, const void *w
  * pipeline does)
  * q,k are (B,H,S,D), w is (H,R,Sk), s_out is (B,H,S,S).  Replaces matmul -> *rsqrt(d) -> conv_fwd_kernel of
  * mta_attention_triton.py:69-73 without ever writing the raw scores.  When causal only q <= p is
- * written; fill_upper != 0 also writes +0.0 above the diagonal (needed only if a consumer reads it).
+ * defined; fill_upper != 0 also writes +0.0 everywhere above the diagonal (needed only if a consumer reads
+ * it), otherwise what lies there is unspecified (left alone, or zero where a tile straddles the diagonal).
  * 16-bit I/O with weights of the same dtype, D in {64,128}, S % 8 == 0 and the kernel sizes that have a
  * matrix-core instantiation; anything else returns MTA_ERR_UNSUPPORTED and the caller takes the
  * unfused route. */

@@ -60,7 +60,11 @@ def test_kernels_reproduce_golden():
         mod.mta_conv_after_sm_triton.weight.copy_(t("mta_w_post"))
         mod.wposm_triton.weight.copy_(t("mta_wposm"))
     mod = mod.to(dev).eval()
-    got = mod(t("mta_q").to(dev), t("mta_k").to(dev), t("mta_v").to(dev), None, None).cpu().numpy()
+    # parameters require grad: the operator-by-operator route; then the fused inference route
+    got = mod(t("mta_q").to(dev), t("mta_k").to(dev), t("mta_v").to(dev), None, None).detach().cpu().numpy()
+    np.testing.assert_allclose(got, GOLD["mta_out"], **TOL)
+    with torch.no_grad():
+        got = mod(t("mta_q").to(dev), t("mta_k").to(dev), t("mta_v").to(dev), None, None).cpu().numpy()
     np.testing.assert_allclose(got, GOLD["mta_out"], **TOL)
     for causal, key in ((True, "ca_out_causal"), (False, "ca_out_full")):
         got = ops.conv_attn_fwd(t("ca_q").to(dev), t("ca_k").to(dev), t("ca_v").to(dev), t("ca_w").to(dev), causal, None)
