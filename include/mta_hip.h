@@ -105,6 +105,14 @@ int mta_conv_attn_fwd(const void *q, const void *k, const void *v, const void *w
                       int64_t B, int64_t H, int64_t S, int64_t D, int R, int Sk, int causal,
                       float scale, int io_dtype, int w_dtype, void *stream);
 
+/* mta_conv_attn_fwd that also writes, when lse != NULL, the row-wise log-sum-exp of the masked, scaled conv scores
+ *   lse[b,h,p] = log sum_q exp( scale * conv(mask0(Q K^T))[p,q] )     (natural log, fp32, (B,H,S))
+ * the per-row statistic a backward pass needs to rebuild the probabilities.  It is the `M` tensor of
+ * TritonAttention.forward (conv_attention_triton.py:352-355, 402-404; m_i + log(l_i)). */
+int mta_conv_attn_fwd_lse(const void *q, const void *k, const void *v, const void *w, void *o, void *lse,
+                          int64_t B, int64_t H, int64_t S, int64_t D, int R, int Sk, int causal, float scale,
+                          int io_dtype, int w_dtype, void *stream);
+
 /* First half of the fused path, for the MTA pipeline (which must mix heads before its softmax):
  *   s_out[b,h] = conv( mask0(scale * Q K^T) )           an (S,S) plane per (batch, head)
  * (Q K^T is rounded to the I/O dtype, scaled and rounded again before the conv, as the unfused

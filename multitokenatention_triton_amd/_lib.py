@@ -28,6 +28,7 @@ SIGNATURES = {
     "mta_headmix_softmax_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _vp]),
     "mta_qk_conv_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _int, _int, _int, _vp]),
     "mta_causal_pv_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
+    "mta_conv_attn_fwd_lse": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _int, _int, _vp]),
     "mta_probe_head_weight": (_int, [_vp, _i64, _int, _vp, _vp]),
     "mta_probe_conv_kernel": (_int, [_vp, _i64, _int, _int, _int, _vp, _vp]),
     "mta_conv_attn_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _int, _int, _vp]),

@@ -23,13 +23,21 @@ class TritonAttention(torch.autograd.Function):
         # shape checks of conv_attention_triton.py:369-370
         assert W.shape[0] == Q.shape[1]
         assert Q.shape[-1] == K.shape[-1] and K.shape[-1] == V.shape[-1]
-        out = ops.conv_attn_fwd(Q, K, V, W, causal, softmax_scale)
+        # the row-wise log-sum-exp is what the reference keeps for a backward pass (its `M`,
+        # conv_attention_triton.py:402-404, 445); it is kept on ctx the same way
+        out, lse = ops.conv_attn_fwd(Q, K, V, W, causal, softmax_scale, return_lse=True)
+        ctx.save_for_backward(Q, K, V, out, lse)
+        ctx.softmax_scale = softmax_scale
+        ctx.causal = causal
         ctx.mark_non_differentiable(out)
         return out, None
 
     @staticmethod
     def backward(ctx, dO, dQK):
-        raise NotImplementedError("the HIP build of TritonAttention is forward-only")
+        # the reference's backward is itself a stub that calls kernels it never defines
+        # (conv_attention_triton.py:455-473)
+        raise NotImplementedError("TritonAttention has no backward (neither has the reference: "
+                                  "conv_attention_triton.py:455-473)")
 
 
 class TritonConvAttention(nn.Module):

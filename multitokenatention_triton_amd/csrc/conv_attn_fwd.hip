@@ -46,8 +46,8 @@ template <typename T> struct lds_pad { static constexpr int n = 16 / sizeof(T); 
 template <typename T, int D>
 __global__ __launch_bounds__(NT) void conv_attn_fwd_kernel(const T *__restrict__ Q, const T *__restrict__ K,
                                                            const T *__restrict__ V, const void *__restrict__ Wt,
-                                                           T *__restrict__ O, int S, int R, int Sk, int causal,
-                                                           float scale, int w_dtype, int H, int nqb)
+                                                           T *__restrict__ O, float *__restrict__ Lse, int S, int R,
+                                                           int Sk, int causal, float scale, int w_dtype, int H, int nqb)
 {
     constexpr int VEC = vec_of<T>::n;           // elements per 16-byte vector
     constexpr int PAD = lds_pad<T>::n;
@@ -265,6 +265,7 @@ __global__ __launch_bounds__(NT) void conv_attn_fwd_kernel(const T *__restrict__
     const float l_row = l_i + __shfl_xor(l_i, 32);
     if (tr >= HR && p < S) {
         const float inv = 1.0f / l_row;
+        if (Lse != nullptr && hf == 0) Lse[bh * (int64_t)S + p] = m_i + __logf(l_row);
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -359,9 +360,9 @@ template <int R, int SK, int NW> struct fused_geom {
 template <typename T, int D, int R, int SK, bool SCORES_ONLY, int NW>
 __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_attn_fwd_mfma(const T *__restrict__ Q, const T *__restrict__ K,
                                                              const T *__restrict__ V, const T *__restrict__ Wt,
-                                                             T *__restrict__ O, int S, int causal, float scale, int H,
-                                                             int nqb, int fill_upper, int64_t total_wg, int64_t per_xcd,
-                                                             int jc_len, int items_per_bh)
+                                                             T *__restrict__ O, float *__restrict__ Lse, int S, int causal,
+                                                             float scale, int H, int nqb, int fill_upper, int64_t total_wg,
+                                                             int64_t per_xcd, int jc_len, int items_per_bh)
 {
     using G = fused_geom<R, SK, NW>;
     constexpr int F_NT = 64 * NW, F_SR = 32 * NW;
@@ -781,6 +782,7 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
         l_row += __shfl_xor(l_row, 32);
         if (trow[rb] >= G::HR && prow[rb] < S) {
             const float inv = 1.0f / l_row;
+            if (Lse != nullptr && kg == 0) Lse[bh * (int64_t)S + prow[rb]] = m_i[rb] + __logf(l_row);
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 const uint32_t lo = pack2<T>(oacc[rb][db][0] * inv, oacc[rb][db][1] * inv);
@@ -792,8 +794,8 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
 }
 
 template <typename T, int D, int R, int SK, bool SCORES_ONLY>
-int launch_mfma(const void *q, const void *k, const void *v, const void *w, void *o, int64_t B, int64_t H, int64_t S,
-                int causal, float scale, int fill_upper, hipStream_t st)
+int launch_mfma(const void *q, const void *k, const void *v, const void *w, void *o, float *lse, int64_t B, int64_t H,
+                int64_t S, int causal, float scale, int fill_upper, hipStream_t st)
 {
     constexpr int NW = SCORES_ONLY ? 4 : 8;
     constexpr int F_NT = 64 * NW;
@@ -812,18 +814,18 @@ int launch_mfma(const void *q, const void *k, const void *v, const void *w, void
     if (per_xcd * 8 > 0x7fffffffLL || items_per_bh > 0x7fffffffLL) return MTA_ERR_SHAPE;
     dim3 grid((unsigned)(per_xcd * 8));
     hipLaunchKernelGGL(kern, grid, dim3(F_NT), 0, st, (const T *)q, (const T *)k, (const T *)v, (const T *)w, (T *)o,
-                       (int)S, causal, scale, (int)H, nqb, fill_upper, total_wg, per_xcd, jc_len, (int)items_per_bh);
+                       lse, (int)S, causal, scale, (int)H, nqb, fill_upper, total_wg, per_xcd, jc_len, (int)items_per_bh);
     return launch_status();
 }
 
 // returns 1 when no instantiation covers the kernel size (the caller then uses the general kernel)
 template <typename T, int D, bool SCORES_ONLY>
-int dispatch_mfma(const void *q, const void *k, const void *v, const void *w, void *o, int64_t B, int64_t H, int64_t S,
-                  int R, int Sk, int causal, float scale, int fill_upper, hipStream_t st)
+int dispatch_mfma(const void *q, const void *k, const void *v, const void *w, void *o, float *lse, int64_t B, int64_t H,
+                  int64_t S, int R, int Sk, int causal, float scale, int fill_upper, hipStream_t st)
 {
     if constexpr (sizeof(T) == 2) {
 #define MTA_FUSED_CASE(r, s) \
-    if (R == r && Sk == s) return launch_mfma<T, D, r, s, SCORES_ONLY>(q, k, v, w, o, B, H, S, causal, scale, fill_upper, st);
+    if (R == r && Sk == s) return launch_mfma<T, D, r, s, SCORES_ONLY>(q, k, v, w, o, lse, B, H, S, causal, scale, fill_upper, st);
         MTA_FUSED_CASE(3, 3)
         MTA_FUSED_CASE(5, 5)
         MTA_FUSED_CASE(5, 7)
@@ -835,8 +837,8 @@ int dispatch_mfma(const void *q, const void *k, const void *v, const void *w, vo
 }
 
 template <typename T, int D>
-int launch(const void *q, const void *k, const void *v, const void *w, void *o, int64_t B, int64_t H, int64_t S,
-           int R, int Sk, int causal, float scale, int w_dtype, hipStream_t st)
+int launch(const void *q, const void *k, const void *v, const void *w, void *o, float *lse, int64_t B, int64_t H,
+           int64_t S, int R, int Sk, int causal, float scale, int w_dtype, hipStream_t st)
 {
     constexpr int PAD = lds_pad<T>::n;
     const int HR = (R - 1 + 7) & ~7, HC = (Sk - 1 + 7) & ~7;
@@ -851,17 +853,19 @@ int launch(const void *q, const void *k, const void *v, const void *w, void *o, 
         if (e != hipSuccess) return (int)e;
     }
     dim3 grid((unsigned)nqb, (unsigned)(B * H));
-    hipLaunchKernelGGL(kern, grid, dim3(NT), lds, st, (const T *)q, (const T *)k, (const T *)v, w, (T *)o, (int)S, R, Sk,
-                       causal, scale, w_dtype, (int)H, nqb);
+    hipLaunchKernelGGL(kern, grid, dim3(NT), lds, st, (const T *)q, (const T *)k, (const T *)v, w, (T *)o, lse, (int)S,
+                       R, Sk, causal, scale, w_dtype, (int)H, nqb);
     return launch_status();
 }
 }  // namespace
 
-extern "C" int mta_conv_attn_fwd(const void *q, const void *k, const void *v, const void *w, void *o, int64_t B,
-                                 int64_t H, int64_t S, int64_t D, int R, int Sk, int causal, float scale,
-                                 int io_dtype, int w_dtype, void *stream)
+extern "C" int mta_conv_attn_fwd_lse(const void *q, const void *k, const void *v, const void *w, void *o, void *lse_out,
+                                     int64_t B, int64_t H, int64_t S, int64_t D, int R, int Sk, int causal, float scale,
+                                     int io_dtype, int w_dtype, void *stream)
 {
     if (!q || !k || !v || !w || !o) return MTA_ERR_NULL;
+    float *lse = (float *)lse_out;
+    if (lse && !aligned_to(lse, 4)) return MTA_ERR_ALIGN;
     if (!dtype_size(io_dtype) || !dtype_size(w_dtype)) return MTA_ERR_DTYPE;
     if (B <= 0 || H <= 0 || S <= 0 || S > (1 << 24) || B * H > 65535) return MTA_ERR_SHAPE;
     if (R < 1 || Sk < 1 || R > MTA_MAX_KERNEL_R || Sk > MTA_MAX_KERNEL_S) return MTA_ERR_KERNEL_SIZE;
@@ -875,14 +879,21 @@ extern "C" int mta_conv_attn_fwd(const void *q, const void *k, const void *v, co
     const bool fast_ok = io_dtype != MTA_F32 && w_dtype == io_dtype && !force_general;
     MTA_DISPATCH_IO(io_dtype, {
         if (fast_ok) {
-            const int rc = D == 64 ? dispatch_mfma<io_t, 64, false>(q, k, v, w, o, B, H, S, R, Sk, causal, scale, 0, st)
-                                   : dispatch_mfma<io_t, 128, false>(q, k, v, w, o, B, H, S, R, Sk, causal, scale, 0, st);
+            const int rc = D == 64 ? dispatch_mfma<io_t, 64, false>(q, k, v, w, o, lse, B, H, S, R, Sk, causal, scale, 0, st)
+                                   : dispatch_mfma<io_t, 128, false>(q, k, v, w, o, lse, B, H, S, R, Sk, causal, scale, 0, st);
             if (rc != 1) return rc;
         }
-        if (D == 64) return launch<io_t, 64>(q, k, v, w, o, B, H, S, R, Sk, causal, scale, w_dtype, st);
-        return launch<io_t, 128>(q, k, v, w, o, B, H, S, R, Sk, causal, scale, w_dtype, st);
+        if (D == 64) return launch<io_t, 64>(q, k, v, w, o, lse, B, H, S, R, Sk, causal, scale, w_dtype, st);
+        return launch<io_t, 128>(q, k, v, w, o, lse, B, H, S, R, Sk, causal, scale, w_dtype, st);
     });
     return MTA_ERR_DTYPE;
+}
+
+extern "C" int mta_conv_attn_fwd(const void *q, const void *k, const void *v, const void *w, void *o, int64_t B,
+                                 int64_t H, int64_t S, int64_t D, int R, int Sk, int causal, float scale,
+                                 int io_dtype, int w_dtype, void *stream)
+{
+    return mta_conv_attn_fwd_lse(q, k, v, w, o, nullptr, B, H, S, D, R, Sk, causal, scale, io_dtype, w_dtype, stream);
 }
 
 extern "C" int mta_qk_conv_fwd(const void *q, const void *k, const void *w, void *s_out, int64_t B, int64_t H, int64_t S,
@@ -900,8 +911,8 @@ extern "C" int mta_qk_conv_fwd(const void *q, const void *k, const void *w, void
     hipStream_t st = (hipStream_t)stream;
     int rc = 1;
     MTA_DISPATCH_IO(io_dtype, {
-        rc = D == 64 ? dispatch_mfma<io_t, 64, true>(q, k, nullptr, w, s_out, B, H, S, R, Sk, causal, scale, fill_upper, st)
-                     : dispatch_mfma<io_t, 128, true>(q, k, nullptr, w, s_out, B, H, S, R, Sk, causal, scale, fill_upper, st);
+        rc = D == 64 ? dispatch_mfma<io_t, 64, true>(q, k, nullptr, w, s_out, nullptr, B, H, S, R, Sk, causal, scale, fill_upper, st)
+                     : dispatch_mfma<io_t, 128, true>(q, k, nullptr, w, s_out, nullptr, B, H, S, R, Sk, causal, scale, fill_upper, st);
     });
     return rc == 1 ? MTA_ERR_UNSUPPORTED : rc;
 }

@@ -119,8 +119,11 @@ def headmix_softmax(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optional[to
 
 
 def conv_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, weight: torch.Tensor, causal: bool,
-                  softmax_scale: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """O = softmax(mask(conv(mask0(QK^T))) * scale) V for (B,H,S,D) inputs; see mta_conv_attn_fwd."""
+                  softmax_scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
+                  return_lse: bool = False):
+    """O = softmax(mask(conv(mask0(QK^T))) * scale) V for (B,H,S,D) inputs; see mta_conv_attn_fwd.
+
+    With ``return_lse`` the result is (O, lse), lse (B,H,S) fp32 = log-sum-exp of each row's scaled conv scores."""
     q = _device_tensor(q, "Q")
     k = _device_tensor(k, "K")
     v = _device_tensor(v, "V")
@@ -135,12 +138,14 @@ def conv_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, weight: tor
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(d)
     o = _out_like(q, out)
+    lse = torch.empty((b, h, s), dtype=torch.float32, device=q.device) if return_lse else None
     with torch.cuda.device(q.device):
-        rc = _lib.load().mta_conv_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), weight.data_ptr(), o.data_ptr(),
-                                           b, h, s, d, weight.shape[1], weight.shape[2], int(bool(causal)),
-                                           float(softmax_scale), _code(q, "Q"), _code(weight, "W"), _stream(q))
+        rc = _lib.load().mta_conv_attn_fwd_lse(q.data_ptr(), k.data_ptr(), v.data_ptr(), weight.data_ptr(), o.data_ptr(),
+                                               lse.data_ptr() if return_lse else None, b, h, s, d, weight.shape[1],
+                                               weight.shape[2], int(bool(causal)), float(softmax_scale), _code(q, "Q"),
+                                               _code(weight, "W"), _stream(q))
     _lib.check(rc, "mta_conv_attn_fwd")
-    return o
+    return (o, lse) if return_lse else o
 
 
 def qk_conv(q: torch.Tensor, k: torch.Tensor, weight: torch.Tensor, causal: bool, scale: float,

@@ -228,6 +228,27 @@ def conv_attention_forward(Q, K, V, conv_weight, causal: bool = True,
     return torch.matmul(attn, V)
 
 
+def conv_attention_scores(Q, K, conv_weight, causal: bool = True, softmax_scale: Optional[float] = None):
+    """The logits ``conv_attention_forward`` feeds its softmax: mask(conv(mask0(Q K^T))) * scale, (B,H,S,S);
+    conv_attention_pytorch.py:44-66.  Its row-wise ``torch.logsumexp`` is the statistic the reference's fused
+    kernel calls M (conv_attention_triton.py:352-355).  Pinned in tests/test_oracle.py by
+    softmax(scores) V == conv_attention_forward and exp(scores - lse) rows summing to 1."""
+    b, h, s, d = Q.shape
+    if softmax_scale is None:
+        softmax_scale = 1.0 / (d ** 0.5)
+    scores = torch.matmul(Q, K.transpose(-2, -1))
+    upper = torch.triu(torch.ones(s, s, device=Q.device), diagonal=1).bool()
+    if causal:
+        scores = scores.masked_fill(upper, 0)
+    r, sk = conv_weight.shape[-2], conv_weight.shape[-1]
+    pad_k = (sk - 1) // 2
+    padded = F.pad(scores, (pad_k, sk - 1 - pad_k, r - 1, 0), value=0.0)
+    conv = F.conv2d(padded, conv_weight.to(Q.dtype).unsqueeze(1), padding=0, groups=h)
+    if causal:
+        conv = conv.masked_fill(upper, NEG_INF)
+    return conv * softmax_scale
+
+
 def conv_attention_rows(Q, K, V, conv_weight, row0: int, row1: int, causal: bool = True,
                         softmax_scale: Optional[float] = None) -> torch.Tensor:
     """Rows [row0,row1) of ``conv_attention_forward`` without the full S x S tensor.

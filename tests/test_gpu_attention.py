@@ -597,3 +597,22 @@ def test_mta_unfused_16bit_route_never_reads_above_the_diagonal(pkg):
     p2 = p2.masked_fill(up, float("nan"))
     out = ops.causal_pv(p2, v.cuda(), True)
     torch.testing.assert_close(out.transpose(1, 2).cpu().float(), want.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("case", [(1, 2, 300, 64, 6, 11, True, torch.float32), (1, 2, 777, 128, 6, 11, True, torch.bfloat16),
+                                  (2, 2, 260, 64, 3, 3, False, torch.float16), (1, 2, 333, 128, 11, 15, True, torch.bfloat16)])
+def test_conv_attention_lse(pkg, case):
+    """The row statistic of the fused kernel (the reference's M, conv_attention_triton.py:352-355, 402-404) against
+    torch.logsumexp of the oracle's masked, scaled conv scores.  16-bit: the kernel rounds the conv output and the scaled
+    logits to the I/O dtype (as the unfused pipeline stores them) and sums probabilities rounded to it, hence atol 2e-2."""
+    b, h, s, d, r, sk, causal, dtype = case
+    print(f"conv_attention lse case={case}", flush=True)
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=42)
+    w = O.seeded_conv_weight(h, r, sk, 0.05, dtype)
+    want = torch.logsumexp(O.conv_attention_scores(q.float(), k.float(), w.float(), causal, None), -1)
+    o, lse = pkg.ops.conv_attn_fwd(q.cuda(), k.cuda(), v.cuda(), w.cuda(), causal, None, return_lse=True)
+    assert lse.shape == (b, h, s) and lse.dtype == torch.float32
+    t = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(rtol=2.0 ** -7, atol=2e-2)
+    torch.testing.assert_close(lse.cpu(), want, **t)
+    o2 = pkg.ops.conv_attn_fwd(q.cuda(), k.cuda(), v.cuda(), w.cuda(), causal, None)
+    assert torch.equal(o, o2)

@@ -285,3 +285,18 @@ def test_mta_tensor_masks_vs_c_restatement(name):
     if name == "key_mask_bool":     # hidden keys and the causal rule both took effect
         hidden = (~mask[0]).nonzero().flatten()
         assert torch.isneginf(add[0, :, :, hidden]).all() and torch.isneginf(add[0, 0, 3, 4])
+
+
+def test_conv_attention_scores_and_lse():
+    q, k, v = O.seeded_qkv(1, 2, 40, 8, torch.float32, seed=3)
+    w = O.seeded_conv_weight(2, 3, 5, 0.1, torch.float32)
+    for causal in (True, False):
+        sc = O.conv_attention_scores(q, k, w, causal, 0.3)
+        lse = torch.logsumexp(sc, -1)
+        p = torch.exp(sc - lse[..., None])
+        torch.testing.assert_close(p.sum(-1), torch.ones(1, 2, 40), rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(torch.matmul(p, v), O.conv_attention_forward(q, k, v, w, causal, 0.3),
+                                   rtol=1e-5, atol=1e-6)
+        if causal:   # row 0 sees one key: lse is that logit, scale * w[R-1, S//2] * (q0 . k0)
+            want = 0.3 * w[:, -1, 2] * (q[0, :, 0] * k[0, :, 0]).sum(-1)
+            torch.testing.assert_close(lse[0, :, 0], want, rtol=1e-5, atol=1e-6)
