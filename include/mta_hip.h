@@ -39,7 +39,8 @@ enum mta_error {
     MTA_ERR_ALIGN = -6,       /* pointer not aligned to its element size */
     MTA_ERR_HEAD_DIM = -7,    /* head dim unsupported by the fused kernel */
     MTA_ERR_DEVICE = -8,      /* no usable gfx950 device / device query failed */
-    MTA_ERR_UNSUPPORTED = -9  /* valid arguments, but this entry point has no kernel for the combination */
+    MTA_ERR_UNSUPPORTED = -9, /* valid arguments, but this entry point has no kernel for the combination */
+    MTA_ERR_WORKSPACE = -10   /* workspace smaller than the matching *_workspace() call reports */
 };
 
 /* Largest conv kernel the entry points accept. */
@@ -134,6 +135,41 @@ int mta_qk_conv_fwd(const void *q, const void *k, const void *w, void *s_out, in
  * else returns MTA_ERR_UNSUPPORTED. */
 int mta_causal_pv_fwd(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int64_t D,
                       int causal, int io_dtype, void *stream);
+
+/* ---- backward of the two standalone operators -------------------------------------------------------------
+ * Gradients flow through the same masks as the forward pass: with `causal`, entries of dy above the diagonal are
+ * never read (the forward wrote a constant there) and gradients with respect to inputs above the diagonal are +0
+ * (the forward never read them).  Weight gradients are written as fp32 whatever the I/O dtype, fully defined
+ * (not accumulated into), and are bit-reproducible from run to run: partial sums are kept in fp32 registers,
+ * written once per workgroup to `workspace` and added in a fixed order by a second kernel (the reference
+ * accumulates in fp64 with atomics).  `workspace` is device memory of at least the size the matching
+ * *_workspace() call returns for the same sizes (0 = sizes rejected); its contents before and after are garbage. */
+
+/* dx[n,c,h,w] = sum_{i,j} w[c,i,j] * dym[n,c, h-i+(R-1), w-j+(S-1)/2], dym = dy with out-of-range and (causal)
+ * q>p entries read as 0.  Replaces conv_bwd_input_kernel + the grad_input half of Conv2dTritonFunction.backward
+ * (convolution_2d_trit.py:143-223, 344-358). */
+int mta_conv2d_bwd_input(const void *dy, const void *w, void *dx, int64_t N, int64_t C, int64_t H, int64_t W,
+                         int R, int S, int causal, int io_dtype, int w_dtype, void *stream);
+
+/* dw[c,i,j] = sum_{n,p,q} xm[n,c, p+i-(R-1), q+j-(S-1)/2] * dym[n,c,p,q]; dw is (C,R,S) fp32.  Replaces
+ * conv_bwd_weight_kernel + the grad_weight half of Conv2dTritonFunction.backward
+ * (convolution_2d_trit.py:225-295, 360-376). */
+int64_t mta_conv2d_bwd_weight_workspace(int64_t N, int64_t C, int64_t H, int64_t W, int R, int S);
+int mta_conv2d_bwd_weight(const void *x, const void *dy, void *dw, void *workspace, int64_t workspace_bytes,
+                          int64_t N, int64_t C, int64_t H, int64_t W, int R, int S, int causal, int io_dtype,
+                          void *stream);
+
+/* dx[n,i,p,q] = sum_o w[o,i] * dy[n,o,p,q].  group_size as in mta_headmix_fwd.  Replaces
+ * linear_head_kernel_backward_input (triton_linear_head.py:144-196, 330-348); the reference leaves dx above the
+ * diagonal uninitialised (torch.empty_like), here it is +0. */
+int mta_headmix_bwd_input(const void *dy, const void *w, void *dx, int64_t N, int64_t C, int64_t P, int64_t Q,
+                          int group_size, int causal, int io_dtype, int w_dtype, void *stream);
+
+/* dw[o,i] = sum_{n,p,q} dy[n,o,p,q] * x[n,i,p,q] (causal: q <= p only); dw is the dense (C,C) matrix in fp32,
+ * C <= 128.  Replaces linear_head_kernel_backward_weight (triton_linear_head.py:199-278, 350-368). */
+int64_t mta_headmix_bwd_weight_workspace(int64_t N, int64_t C, int64_t P, int64_t Q);
+int mta_headmix_bwd_weight(const void *x, const void *dy, void *dw, void *workspace, int64_t workspace_bytes,
+                           int64_t N, int64_t C, int64_t P, int64_t Q, int causal, int io_dtype, void *stream);
 
 /* Structure of the small MTA parameters, evaluated on the device (one workgroup, a few microseconds).  The
  * reference has no counterpart: its glue (mta_attention_triton.py:69-89) always runs every stage.  The glue

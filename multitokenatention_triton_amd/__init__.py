@@ -8,12 +8,12 @@ call surface of Gusanidas/multitokenatention_triton:
     Conv2dTriton            depthwise causal 2-D conv  (convolution_2d_trit.py)
     TritonLinearHead        head mixing                (triton_linear_head.py)
 """
-from .convolution_2d_trit import Conv2dTriton, Conv2dTritonFunction
+from .convolution_2d_trit import Conv2dTriton, Conv2dTritonFunction, PytorchConv, add_causal_mask, pytorch_conv
 from .triton_linear_head import TritonLinearHead, TritonLinearHeadFunction
 from .conv_attention_triton import TritonAttention, TritonConvAttention
 from .mta_attention_triton import MTAAttentionTriton, MTAConfig, WeightStructure
 from . import ops
 
-__all__ = ["Conv2dTriton", "Conv2dTritonFunction", "TritonLinearHead", "TritonLinearHeadFunction",
+__all__ = ["Conv2dTriton", "Conv2dTritonFunction", "PytorchConv", "pytorch_conv", "add_causal_mask", "TritonLinearHead", "TritonLinearHeadFunction",
            "TritonAttention", "TritonConvAttention", "MTAAttentionTriton", "MTAConfig", "WeightStructure",
            "ops"]

@@ -29,6 +29,12 @@ SIGNATURES = {
     "mta_qk_conv_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _int, _int, _int, _vp]),
     "mta_causal_pv_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "mta_conv_attn_fwd_lse": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _int, _int, _vp]),
+    "mta_conv2d_bwd_input": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _vp]),
+    "mta_conv2d_bwd_weight_workspace": (_i64, [_i64, _i64, _i64, _i64, _int, _int]),
+    "mta_conv2d_bwd_weight": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _vp]),
+    "mta_headmix_bwd_input": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _vp]),
+    "mta_headmix_bwd_weight_workspace": (_i64, [_i64, _i64, _i64, _i64]),
+    "mta_headmix_bwd_weight": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "mta_probe_head_weight": (_int, [_vp, _i64, _int, _vp, _vp]),
     "mta_probe_conv_kernel": (_int, [_vp, _i64, _int, _int, _int, _vp, _vp]),
     "mta_conv_attn_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _int, _int, _vp]),

@@ -16,6 +16,7 @@ extern "C" const char *mta_strerror(int code)
     case MTA_ERR_HEAD_DIM: return "head dimension not supported by the fused kernel";
     case MTA_ERR_DEVICE: return "no usable gfx950 device";
     case MTA_ERR_UNSUPPORTED: return "no kernel for this dtype / size combination (use the unfused route)";
+    case MTA_ERR_WORKSPACE: return "workspace smaller than the matching *_workspace() call reports";
     default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);

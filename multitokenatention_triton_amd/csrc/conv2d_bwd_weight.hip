@@ -1,0 +1,294 @@
+// Gradient of the depthwise causal conv with respect to its (C,R,S) kernel:
+//
+//   dw[c,i,j] = sum_{n,p,q} xm[n,c, p+i-(R-1), q+j-(S-1)/2] * dym[n,c,p,q]
+//
+// xm = x with out-of-range taps and (causal) col>row read as 0, dym = dy with (causal) q>p read as 0 -- the masks of
+// the forward pass.  Accumulation is fp32 and hierarchical: a lane keeps its R*S sums in registers over all the
+// tiles it visits, a workgroup reduces them once at the end and writes one partial kernel to a scratch buffer, and a
+// second small kernel adds the partials of each channel in a fixed order (the result does not depend on timing; the
+// reference accumulates in fp64 with atomics, convolution_2d_trit.py:236-295).
+//
+// Work split: the persistent workgroups are divided among the channels; the workgroups of a channel walk that
+// channel's (batch, 32x64 tile) list with a stride.  Tiles wholly above the diagonal are skipped.
+#include "common.hpp"
+
+namespace {
+using namespace mta;
+
+constexpr int NT = 256;
+constexpr int TM = 32;  // tile rows   (thread t: row t/8)
+constexpr int TN = 64;  // tile cols   (thread t: cols 8*(t%8) .. +7)
+
+// sum over the wavefront, result in every lane
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m);
+    return v;
+}
+
+// stage the (TM+R-1) x (TN+S-1) halo tile of x as fp32 with the forward pass's masks applied
+template <typename T>
+__device__ __forceinline__ void stage_x(const T *xp, float *tile, int LD, int H, int W, int p0, int q0, int R, int S,
+                                        int causal, int tid)
+{
+    const int pad_h = R - 1, pad_w = (S - 1) / 2;
+    const int rows = TM + R - 1, cols = TN + S - 1;
+    for (int rr = tid / 64; rr < rows; rr += NT / 64) {
+        const int h = p0 - pad_h + rr;
+        const bool row_ok = h >= 0 && h < H;
+        for (int cc = tid % 64; cc < cols; cc += 64) {
+            const int k = q0 - pad_w + cc;
+            float v = 0.0f;
+            if (row_ok && k >= 0 && k < W && (!causal || k <= h)) v = to_float(xp[(int64_t)h * W + k]);
+            tile[rr * LD + cc] = v;
+        }
+    }
+}
+
+// (channel, first item, item stride) of a workgroup; items of a channel = batch * tiles
+struct split_t { int channel, sub, bpc; };
+__device__ __forceinline__ split_t split_of(int block, int C, int bpc)
+{
+    return split_t{block / bpc, block % bpc, bpc};
+}
+
+// Kernel size known at compile time: all R*S sums of a lane live in registers.
+template <typename T, int R, int S>
+__global__ __launch_bounds__(NT) void conv2d_bwd_weight_fixed(const T *__restrict__ x, const T *__restrict__ dy,
+                                                              float *__restrict__ partial, int N, int C, int H, int W,
+                                                              int causal, int tiles_m, int tiles_n, int bpc, int vec_ok)
+{
+    constexpr int LD = TN + S;  // S-1 halo columns + 1 pad
+    __shared__ float tile[(TM + R - 1) * LD];
+    __shared__ float red[NT / 64][R * S];
+    const int tid = threadIdx.x;
+    const split_t sp = split_of(blockIdx.x, C, bpc);
+    const int c = sp.channel;
+    const int tr = tid >> 3, tc = (tid & 7) * 8;
+
+    float acc[R][S];
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+#pragma unroll
+        for (int j = 0; j < S; ++j) acc[i][j] = 0.0f;
+
+    const int tiles = tiles_m * tiles_n;
+    const int64_t items = (int64_t)N * tiles;
+    for (int64_t it = sp.sub; it < items; it += sp.bpc) {
+        const int n = (int)(it / tiles), t = (int)(it % tiles);
+        const int tm = t / tiles_n, tn = t % tiles_n;
+        const int p0 = tm * TM, q0 = tn * TN;
+        if (causal && q0 > p0 + TM - 1) continue;  // dy is masked to zero on the whole tile (uniform per workgroup)
+        const int64_t plane = ((int64_t)n * C + c) * H * W;
+        __syncthreads();  // the previous tile's readers are done
+        stage_x<T>(x + plane, tile, LD, H, W, p0, q0, R, S, causal, tid);
+        // this lane's 8 gradient values
+        float g[8];
+        const int p = p0 + tr, q = q0 + tc;
+        if (vec_ok && p < H && q + 8 <= W) {  // eight contiguous values, 16-byte aligned
+            const T *src = dy + plane + (int64_t)p * W + q;
+            T raw[8];
+            if constexpr (sizeof(T) == 2) {
+                *reinterpret_cast<pack16<T> *>(raw) = *reinterpret_cast<const pack16<T> *>(src);
+            } else {
+                *reinterpret_cast<pack16<T> *>(raw) = *reinterpret_cast<const pack16<T> *>(src);
+                *reinterpret_cast<pack16<T> *>(raw + 4) = *reinterpret_cast<const pack16<T> *>(src + 4);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) g[u] = (causal && q + u > p) ? 0.0f : to_float(raw[u]);
+        } else {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const bool ok = p < H && q + u < W && !(causal && q + u > p);
+                g[u] = ok ? to_float(dy[plane + (int64_t)p * W + q + u]) : 0.0f;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            float win[S + 7];
+            const float *src = tile + (tr + i) * LD + tc;
+#pragma unroll
+            for (int u = 0; u < S + 7; ++u) win[u] = src[u];
+#pragma unroll
+            for (int j = 0; j < S; ++j) {
+                float a = acc[i][j];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) a = fmaf(g[u], win[u + j], a);
+                acc[i][j] = a;
+            }
+        }
+    }
+    // workgroup reduction, once
+    const int wave = tid >> 6, lane = tid & 63;
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+#pragma unroll
+        for (int j = 0; j < S; ++j) {
+            const float s = wave_sum(acc[i][j]);
+            if (lane == 0) red[wave][i * S + j] = s;
+        }
+    __syncthreads();
+    for (int t = tid; t < R * S; t += NT) {
+        float s = 0.0f;
+#pragma unroll
+        for (int wv = 0; wv < NT / 64; ++wv) s += red[wv][t];
+        partial[((int64_t)c * bpc + sp.sub) * (R * S) + t] = s;
+    }
+}
+
+// Any kernel size: x halo tile and dy tile in LDS, the R*S running sums in LDS too; thread t owns taps t, t+256, ...
+// (nothing is unrolled over the taps: the fixed-size kernel above is the fast path).
+template <typename T>
+__global__ __launch_bounds__(NT) void conv2d_bwd_weight_any(const T *__restrict__ x, const T *__restrict__ dy,
+                                                            float *__restrict__ partial, int N, int C, int H, int W,
+                                                            int R, int S, int causal, int tiles_m, int tiles_n, int bpc)
+{
+    extern __shared__ float smem[];
+    const int LD = TN + S;
+    const int RS = R * S;
+    float *tile = smem;                            // (TM+R-1) x LD
+    float *gt = tile + (TM + R - 1) * LD;          // TM x TN gradient tile
+    float *sums = gt + TM * TN;                    // R*S
+    const int tid = threadIdx.x;
+    const split_t sp = split_of(blockIdx.x, C, bpc);
+    const int c = sp.channel;
+    for (int tap = tid; tap < RS; tap += NT) sums[tap] = 0.0f;
+
+    const int tiles = tiles_m * tiles_n;
+    const int64_t items = (int64_t)N * tiles;
+    for (int64_t it = sp.sub; it < items; it += sp.bpc) {
+        const int n = (int)(it / tiles), t = (int)(it % tiles);
+        const int tm = t / tiles_n, tn = t % tiles_n;
+        const int p0 = tm * TM, q0 = tn * TN;
+        if (causal && q0 > p0 + TM - 1) continue;
+        const int64_t plane = ((int64_t)n * C + c) * H * W;
+        __syncthreads();
+        stage_x<T>(x + plane, tile, LD, H, W, p0, q0, R, S, causal, tid);
+        for (int e = tid; e < TM * TN; e += NT) {
+            const int p = p0 + e / TN, q = q0 + e % TN;
+            const bool ok = p < H && q < W && !(causal && q > p);
+            gt[e] = ok ? to_float(dy[plane + (int64_t)p * W + q]) : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll 1
+        for (int tap = tid; tap < RS; tap += NT) {
+            const int i = tap / S, j = tap % S;
+            float s = 0.0f;
+#pragma unroll 1
+            for (int r = 0; r < TM; ++r) {
+                const float *xr = tile + (r + i) * LD + j;
+                const float *gr = gt + r * TN;
+#pragma unroll 8
+                for (int col = 0; col < TN; ++col) s = fmaf(gr[col], xr[col], s);
+            }
+            sums[tap] += s;  // only the owner thread touches this entry
+        }
+    }
+    for (int tap = tid; tap < RS; tap += NT) partial[((int64_t)c * bpc + sp.sub) * RS + tap] = sums[tap];
+}
+
+// dw[c][t] = sum over the channel's partial kernels, in a fixed order
+__global__ __launch_bounds__(NT) void reduce_partials(const float *__restrict__ partial, float *__restrict__ dw, int total,
+                                                      int RS, int bpc)
+{
+    const int e = blockIdx.x * NT + threadIdx.x;  // (c, tap)
+    if (e >= total) return;
+    const int c = e / RS, t = e % RS;
+    float s = 0.0f;
+    for (int b = 0; b < bpc; ++b) s += partial[((int64_t)c * bpc + b) * RS + t];
+    dw[e] = s;
+}
+
+// workgroups per channel: enough persistent workgroups to fill the device, at most `cap` partial kernels in total
+inline int blocks_per_channel(int64_t N, int64_t C, int64_t H, int64_t W, int64_t cap)
+{
+    const int64_t tiles = ((H + TM - 1) / TM) * ((W + TN - 1) / TN);
+    int64_t bpc = (1024 + C - 1) / C;            // about four workgroups per CU in total
+    if (bpc > N * tiles) bpc = N * tiles;
+    if (bpc * C > cap) bpc = cap / C;
+    return (int)(bpc < 1 ? 1 : bpc);
+}
+
+constexpr int64_t MAX_PARTIALS = 2048;  // partial kernels per launch, over all channels
+
+int check_args(const void *x, const void *dy, const void *dw, int64_t N, int64_t C, int64_t H, int64_t W, int R, int S,
+               int io_dtype)
+{
+    if (!x || !dy || !dw) return MTA_ERR_NULL;
+    if (!dtype_size(io_dtype)) return MTA_ERR_DTYPE;
+    if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || H > (1 << 24) || W > (1 << 24) || N * C > 65535) return MTA_ERR_SHAPE;
+    if (C > MAX_PARTIALS) return MTA_ERR_SHAPE;
+    if (R < 1 || S < 1 || R > MTA_MAX_KERNEL_R || S > MTA_MAX_KERNEL_S) return MTA_ERR_KERNEL_SIZE;
+    if (!aligned_to(x, dtype_size(io_dtype)) || !aligned_to(dy, dtype_size(io_dtype)) || !aligned_to(dw, 4))
+        return MTA_ERR_ALIGN;
+    if (((H + TM - 1) / TM) * ((W + TN - 1) / TN) > 0x7fffffffLL) return MTA_ERR_SHAPE;
+    return MTA_OK;
+}
+
+template <typename T>
+int launch(const void *x, const void *dy, float *dw, float *partial, int bpc, int64_t N, int64_t C, int64_t H, int64_t W,
+           int R, int S, int causal, hipStream_t st)
+{
+    const int tiles_m = (int)((H + TM - 1) / TM), tiles_n = (int)((W + TN - 1) / TN);
+    dim3 grid((unsigned)(C * bpc));
+    const int vec_ok = (W % 8 == 0 && aligned_to(dy, 16)) ? 1 : 0;
+#define MTA_CONV_CASE(r, s)                                                                                          \
+    if (R == r && S == s) {                                                                                          \
+        hipLaunchKernelGGL((conv2d_bwd_weight_fixed<T, r, s>), grid, dim3(NT), 0, st, (const T *)x, (const T *)dy,    \
+                           partial, (int)N, (int)C, (int)H, (int)W, causal, tiles_m, tiles_n, bpc, vec_ok);           \
+        goto reduce;                                                                                                 \
+    }
+    MTA_CONV_CASE(3, 3)
+    MTA_CONV_CASE(3, 5)
+    MTA_CONV_CASE(5, 5)
+    MTA_CONV_CASE(5, 7)
+    MTA_CONV_CASE(6, 11)
+    MTA_CONV_CASE(7, 7)
+    MTA_CONV_CASE(7, 9)
+#undef MTA_CONV_CASE
+    {
+        const size_t lds = sizeof(float) * ((size_t)(TM + R - 1) * (TN + S) + (size_t)TM * TN + (size_t)R * S);
+        auto kern = conv2d_bwd_weight_any<T>;
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return (int)e;
+        }
+        hipLaunchKernelGGL(kern, grid, dim3(NT), lds, st, (const T *)x, (const T *)dy, partial, (int)N, (int)C, (int)H,
+                           (int)W, R, S, causal, tiles_m, tiles_n, bpc);
+    }
+reduce:
+    {
+        const int rc = launch_status();
+        if (rc != MTA_OK) return rc;
+        const int total = (int)(C * R * S);
+        hipLaunchKernelGGL(reduce_partials, dim3((unsigned)((total + NT - 1) / NT)), dim3(NT), 0, st, partial, dw, total,
+                           R * S, bpc);
+        return launch_status();
+    }
+}
+
+}  // namespace
+
+extern "C" int64_t mta_conv2d_bwd_weight_workspace(int64_t N, int64_t C, int64_t H, int64_t W, int R, int S)
+{
+    if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || R < 1 || S < 1 || C > MAX_PARTIALS) return 0;
+    return (int64_t)blocks_per_channel(N, C, H, W, MAX_PARTIALS) * C * R * S * (int64_t)sizeof(float);
+}
+
+extern "C" int mta_conv2d_bwd_weight(const void *x, const void *dy, void *dw, void *workspace, int64_t workspace_bytes,
+                                     int64_t N, int64_t C, int64_t H, int64_t W, int R, int S, int causal, int io_dtype,
+                                     void *stream)
+{
+    const int rc = check_args(x, dy, dw, N, C, H, W, R, S, io_dtype);
+    if (rc != MTA_OK) return rc;
+    if (!workspace) return MTA_ERR_NULL;
+    if (!aligned_to(workspace, 16)) return MTA_ERR_ALIGN;
+    const int bpc = blocks_per_channel(N, C, H, W, MAX_PARTIALS);
+    if (workspace_bytes < (int64_t)bpc * C * R * S * (int64_t)sizeof(float)) return MTA_ERR_WORKSPACE;
+    MTA_DISPATCH_IO(io_dtype, return launch<io_t>(x, dy, (float *)dw, (float *)workspace, bpc, N, C, H, W, R, S, causal,
+                                                  (hipStream_t)stream));
+    return MTA_ERR_DTYPE;
+}
+

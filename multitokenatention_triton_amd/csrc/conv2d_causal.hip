@@ -55,7 +55,11 @@ __device__ __forceinline__ void store_row8(T *yp, int64_t W, int H, int p, int q
     }
 }
 
-template <typename T, int R_T, int S_T>
+// BWD: the gradient with respect to the input,
+//   dx[h,w] = sum_{i,j} w[i,j] * dym[h-i+(R-1), w-j+(S-1)/2]        (dym = dy with q>p read as 0 when causal)
+// which is the same tile computation with the kernel reversed in both axes, the row halo below the tile instead of
+// above it and the key halos swapped; dx is +0 above the diagonal (those inputs were never read).
+template <typename T, int R_T, int S_T, bool BWD>
 __global__ __launch_bounds__(NT) void conv2d_valu(const T *__restrict__ x, const void *__restrict__ w,
                                                   T *__restrict__ y, int C, int H, int W, int R_rt,
                                                   int S_rt, int causal, float in_scale, int use_scale,
@@ -63,7 +67,7 @@ __global__ __launch_bounds__(NT) void conv2d_valu(const T *__restrict__ x, const
 {
     const int R = R_T > 0 ? R_T : R_rt;
     const int S = S_T > 0 ? S_T : S_rt;
-    const int pad_h = R - 1, pad_w = (S - 1) / 2;
+    const int pad_h = BWD ? 0 : R - 1, pad_w = BWD ? S - 1 - (S - 1) / 2 : (S - 1) / 2;
     const int LD = V_TN + S;  // S-1 halo columns + 1 pad
     extern __shared__ float smem[];
     float *wsm = smem;                        // R*S weights of this channel
@@ -87,7 +91,7 @@ __global__ __launch_bounds__(NT) void conv2d_valu(const T *__restrict__ x, const
         return;
     }
 
-    for (int t = tid; t < R * S; t += NT) wsm[t] = load_any(w, w_dtype, (int64_t)c * R * S + t);
+    for (int t = tid; t < R * S; t += NT) wsm[t] = load_any(w, w_dtype, (int64_t)c * R * S + (BWD ? R * S - 1 - t : t));
 
     const int rows = V_TM + R - 1, cols = V_TN + S - 1;
     for (int rr = tid / 64; rr < rows; rr += NT / 64) {
@@ -132,25 +136,25 @@ __global__ __launch_bounds__(NT) void conv2d_valu(const T *__restrict__ x, const
     store_row8<T>(yp, W, H, p0 + tr, q0 + tc, acc, causal != 0);
 }
 
-template <typename T, int R_T, int S_T>
+template <typename T, int R_T, int S_T, bool BWD>
 int launch_valu(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H, int64_t W, int R,
                 int S, int causal, float in_scale, int use_scale, int w_dtype, hipStream_t st)
 {
     const int tiles_m = (int)((H + V_TM - 1) / V_TM), tiles_n = (int)((W + V_TN - 1) / V_TN);
     const size_t lds = sizeof(float) * (((R * S + 3) & ~3) + (size_t)(V_TM + R - 1) * (V_TN + S));
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)(N * C));
-    hipLaunchKernelGGL((conv2d_valu<T, R_T, S_T>), grid, dim3(NT), lds, st, (const T *)x, w, (T *)y, (int)C,
+    hipLaunchKernelGGL((conv2d_valu<T, R_T, S_T, BWD>), grid, dim3(NT), lds, st, (const T *)x, w, (T *)y, (int)C,
                        (int)H, (int)W, R, S, causal, in_scale, use_scale, w_dtype, tiles_n);
     return launch_status();
 }
 
-template <typename T>
+template <typename T, bool BWD>
 int dispatch_valu(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H, int64_t W, int R,
                   int S, int causal, float in_scale, int use_scale, int w_dtype, hipStream_t st)
 {
 #define MTA_CONV_CASE(r, s)                                                                               \
     if (R == r && S == s)                                                                                 \
-        return launch_valu<T, r, s>(x, w, y, N, C, H, W, R, S, causal, in_scale, use_scale, w_dtype, st);
+        return launch_valu<T, r, s, BWD>(x, w, y, N, C, H, W, R, S, causal, in_scale, use_scale, w_dtype, st);
     MTA_CONV_CASE(3, 3)
     MTA_CONV_CASE(3, 5)
     MTA_CONV_CASE(5, 5)
@@ -160,7 +164,7 @@ int dispatch_valu(const void *x, const void *w, void *y, int64_t N, int64_t C, i
     MTA_CONV_CASE(7, 9)
     MTA_CONV_CASE(11, 15)
 #undef MTA_CONV_CASE
-    return launch_valu<T, 0, 0>(x, w, y, N, C, H, W, R, S, causal, in_scale, use_scale, w_dtype, st);
+    return launch_valu<T, 0, 0, BWD>(x, w, y, N, C, H, W, R, S, causal, in_scale, use_scale, w_dtype, st);
 }
 
 // ------------------------------------------------------------------------------------
@@ -329,12 +333,17 @@ __device__ __forceinline__ void lds_wait(u32x4 &a, u32x4 &b, u32x4 &c)
 //
 // SCALED: every strip is staged through registers, where x*in_scale is rounded to the I/O dtype before it
 // reaches LDS (what a separate elementwise scale pass would have produced).
-template <typename T, int R, int S, bool SCALED>
+//
+// BWD: the gradient with respect to the input (see conv2d_valu): kernel rows reversed in both axes, the R-1 halo rows
+// below the strip instead of above it.  Key sizes are odd here, so the key halos are the same on both sides.
+template <typename T, int R, int S, bool SCALED, bool BWD>
 __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     const T *__restrict__ x, const T *__restrict__ w, T *__restrict__ y, int C, int H, int W, int causal, float in_scale,
     int tiles_n, int ipp, int64_t total, int64_t per_xcd, int nw, int mirror)
 {
     using G = mfma_geom<R, S>;
+    static_assert(!BWD || (S % 2 == 1 && !SCALED), "the backward instance assumes symmetric key halos and no scale");
+    constexpr int TOP = BWD ? 0 : R - 1;                    // halo rows above the strip (the others lie below it)
     constexpr int LD = G::LD, VEC = 8;
     constexpr int VPR = G::TW / VEC;                        // data vectors per staged row (18)
     constexpr int SPR = LD / VEC;                           // 16-byte slots per LDS row (19)
@@ -382,8 +391,8 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     // a strip is `interior` when its whole halo lies inside the tensor and on or below the diagonal
     auto is_interior = [&](int p0_, int q0_) {
         if (SCALED) return false;
-        const int h0 = p0_ - (R - 1), k0 = q0_ - G::HL;
-        return h0 >= 0 && p0_ + M_TM <= H && k0 >= 0 && k0 + G::TW <= W && (!causal || k0 + G::TW - 1 <= h0);
+        const int h0 = p0_ - TOP, k0 = q0_ - G::HL;
+        return h0 >= 0 && h0 + G::ROWS <= H && k0 >= 0 && k0 + G::TW <= W && (!causal || k0 + G::TW - 1 <= h0);
     };
     // A strip is `copyable` when the same copy can be issued for it without faulting: its rows lie inside the plane
     // and the bytes its slots address (left halo of the first column strip = tail of the previous row, right halo of
@@ -393,14 +402,14 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     const int64_t total_elems = (int64_t)(total / ipp) * H * W;  // planes * H * W
     auto is_copyable = [&](int64_t plane_, int p0_, int q0_) {
         if (SCALED) return false;
-        const int h0 = p0_ - (R - 1), k0 = q0_ - G::HL;
-        if (h0 < 0 || p0_ + M_TM > H) return false;
+        const int h0 = p0_ - TOP, k0 = q0_ - G::HL;
+        if (h0 < 0 || h0 + G::ROWS > H) return false;
         const int64_t e0 = plane_ * (int64_t)H * W + (int64_t)h0 * W + k0;
         return e0 >= 0 && e0 + (int64_t)(G::ROWS - 1) * W + G::TW <= total_elems;
     };
     // asynchronous copy of an interior or copyable strip into LDS buffer `buf`
     auto prefetch = [&](int64_t plane_, int p0_, int q0_, T *buf) {
-        const char *base = reinterpret_cast<const char *>(x + plane_ * (int64_t)H * W + (int64_t)(p0_ - (R - 1)) * W + (q0_ - G::HL));
+        const char *base = reinterpret_cast<const char *>(x + plane_ * (int64_t)H * W + (int64_t)(p0_ - TOP) * W + (q0_ - G::HL));
 #pragma unroll
         for (int it = 0; it < STAGE_IT; ++it)
             __builtin_amdgcn_global_load_lds((glb_void_t *)(base + goff[it]), (lds_void_t *)(buf + it * M_WT * VEC), 16, 0, 0);
@@ -421,7 +430,7 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
             const int e = it * M_WT + lane;
             const int i = e / WZ_LD, j = e % WZ_LD - WZ_OFF;
             const bool ok = e < R * WZ_LD && j >= 0 && j < S;
-            const T *src = w + channel_ * R * S + (ok ? i * S + j : 0);
+            const T *src = w + channel_ * R * S + (ok ? (BWD ? (R - 1 - i) * S + (S - 1 - j) : i * S + j) : 0);
             asm volatile("global_load_ushort %0, %1, off" : "=v"(wnext[it]) : "v"(src) : "memory");
         }
     };
@@ -445,7 +454,7 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
         const bool above = causal && q0 > p0 + M_TM - 1;  // wholly above the diagonal (only reachable when !mirror)
         const bool interior = is_interior(p0, q0);
         const bool copyable = interior || is_copyable(plane, p0, q0);
-        const int h0 = p0 - (R - 1), k0 = q0 - G::HL;
+        const int h0 = p0 - TOP, k0 = q0 - G::HL;
         // (opaque: the addresses derived from it are then formed where they are used instead of being kept, dozens of
         // them, in registers across the loop)
         const unsigned tile_lds = (unsigned)opaque((int)(unsigned)(uintptr_t)(lds_void_t *)tile);
@@ -730,7 +739,7 @@ inline int device_cu_count()
     return cached[dev];
 }
 
-template <typename T, int R, int S>
+template <typename T, int R, int S, bool BWD>
 int launch_mfma(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H, int64_t W, int causal,
                 float in_scale, int use_scale, hipStream_t st)
 {
@@ -747,23 +756,29 @@ int launch_mfma(const void *x, const void *w, void *y, int64_t N, int64_t C, int
     if (nw < 1) nw = 1;
     if (per_xcd < nw) nw = (int)per_xcd;
     dim3 grid((unsigned)(nw * 8));
-    if (use_scale)
-        hipLaunchKernelGGL((conv2d_mfma<T, R, S, true>), grid, dim3(M_WT), 0, st, (const T *)x, (const T *)w, (T *)y, (int)C,
-                           (int)H, (int)W, causal, in_scale, tiles_n, ipp, total, per_xcd, nw, mirror);
-    else
-        hipLaunchKernelGGL((conv2d_mfma<T, R, S, false>), grid, dim3(M_WT), 0, st, (const T *)x, (const T *)w, (T *)y, (int)C,
-                           (int)H, (int)W, causal, in_scale, tiles_n, ipp, total, per_xcd, nw, mirror);
+    if constexpr (BWD) {
+        hipLaunchKernelGGL((conv2d_mfma<T, R, S, false, true>), grid, dim3(M_WT), 0, st, (const T *)x, (const T *)w, (T *)y,
+                           (int)C, (int)H, (int)W, causal, in_scale, tiles_n, ipp, total, per_xcd, nw, mirror);
+    } else if (use_scale) {
+        hipLaunchKernelGGL((conv2d_mfma<T, R, S, true, false>), grid, dim3(M_WT), 0, st, (const T *)x, (const T *)w, (T *)y,
+                           (int)C, (int)H, (int)W, causal, in_scale, tiles_n, ipp, total, per_xcd, nw, mirror);
+    } else {
+        hipLaunchKernelGGL((conv2d_mfma<T, R, S, false, false>), grid, dim3(M_WT), 0, st, (const T *)x, (const T *)w, (T *)y,
+                           (int)C, (int)H, (int)W, causal, in_scale, tiles_n, ipp, total, per_xcd, nw, mirror);
+    }
     return launch_status();
 }
 
 // returns 1 when no MFMA instantiation covers (R,S) -- the caller then takes the VALU path
-template <typename T>
+template <typename T, bool BWD>
 int dispatch_mfma(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H, int64_t W, int R, int S,
                   int causal, float in_scale, int use_scale, hipStream_t st)
 {
+    if constexpr (sizeof(T) != 2) return 1;
+    else {
 #define MTA_CONV_CASE(r, s)                                       \
     static_assert(mfma_geom<r, s>::fits, "window exceeds 32 keys"); \
-    if (R == r && S == s) return launch_mfma<T, r, s>(x, w, y, N, C, H, W, causal, in_scale, use_scale, st);
+    if (R == r && S == s) return launch_mfma<T, r, s, BWD>(x, w, y, N, C, H, W, causal, in_scale, use_scale, st);
     MTA_CONV_CASE(3, 3)
     MTA_CONV_CASE(3, 5)
     MTA_CONV_CASE(5, 5)
@@ -773,14 +788,10 @@ int dispatch_mfma(const void *x, const void *w, void *y, int64_t N, int64_t C, i
     MTA_CONV_CASE(7, 9)
 #undef MTA_CONV_CASE
     return 1;
-}
-template <>
-int dispatch_mfma<float>(const void *, const void *, void *, int64_t, int64_t, int64_t, int64_t, int, int, int, float,
-                         int, hipStream_t)
-{
-    return 1;
+    }
 }
 
+template <bool BWD>
 int conv2d_entry(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H, int64_t W, int R,
                  int S, int causal, float in_scale, int use_scale, int io_dtype, int w_dtype, void *stream)
 {
@@ -801,10 +812,10 @@ int conv2d_entry(const void *x, const void *w, void *y, int64_t N, int64_t C, in
                          aligned_to(y, 16) && !force_valu;
     MTA_DISPATCH_IO(io_dtype, {
         if (mfma_ok) {
-            const int rc = dispatch_mfma<io_t>(x, w, y, N, C, H, W, R, S, causal, in_scale, use_scale, st);
+            const int rc = dispatch_mfma<io_t, BWD>(x, w, y, N, C, H, W, R, S, causal, in_scale, use_scale, st);
             if (rc != 1) return rc;
         }
-        return dispatch_valu<io_t>(x, w, y, N, C, H, W, R, S, causal, in_scale, use_scale, w_dtype, st);
+        return dispatch_valu<io_t, BWD>(x, w, y, N, C, H, W, R, S, causal, in_scale, use_scale, w_dtype, st);
     });
     return MTA_ERR_DTYPE;
 }
@@ -813,12 +824,18 @@ int conv2d_entry(const void *x, const void *w, void *y, int64_t N, int64_t C, in
 extern "C" int mta_conv2d_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H,
                               int64_t W, int R, int S, int causal, int io_dtype, int w_dtype, void *stream)
 {
-    return conv2d_entry(x, w, y, N, C, H, W, R, S, causal, 1.0f, 0, io_dtype, w_dtype, stream);
+    return conv2d_entry<false>(x, w, y, N, C, H, W, R, S, causal, 1.0f, 0, io_dtype, w_dtype, stream);
+}
+
+extern "C" int mta_conv2d_bwd_input(const void *dy, const void *w, void *dx, int64_t N, int64_t C, int64_t H,
+                                    int64_t W, int R, int S, int causal, int io_dtype, int w_dtype, void *stream)
+{
+    return conv2d_entry<true>(dy, w, dx, N, C, H, W, R, S, causal, 1.0f, 0, io_dtype, w_dtype, stream);
 }
 
 extern "C" int mta_conv2d_scaled_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H,
                                      int64_t W, int R, int S, int causal, float in_scale, int io_dtype,
                                      int w_dtype, void *stream)
 {
-    return conv2d_entry(x, w, y, N, C, H, W, R, S, causal, in_scale, 1, io_dtype, w_dtype, stream);
+    return conv2d_entry<false>(x, w, y, N, C, H, W, R, S, causal, in_scale, 1, io_dtype, w_dtype, stream);
 }

@@ -16,47 +16,32 @@
 namespace {
 using namespace mta;
 
-#ifndef MTA_HM_THREADS
-#define MTA_HM_THREADS 256
-#endif
-constexpr int NT = MTA_HM_THREADS;
-#ifndef MTA_HM_NT
-#define MTA_HM_NT 1
-#endif
-#ifndef MTA_HM_NTL
-#define MTA_HM_NTL 1
-#endif
-#ifndef MTA_HM_WREG
-#define MTA_HM_WREG 0
-#endif
-#ifndef MTA_HM_ROWS
-#define MTA_HM_ROWS 1
-#endif
+constexpr int NT = 256;
 
 template <typename T, int VEC> struct alignas(sizeof(T) * VEC) vecN { T v[VEC]; };
 
-// outputs are written once and not read again by this kernel: store them as streaming (non-temporal) data
+// inputs are read once and outputs written once by this kernel: move them as streaming (non-temporal) data
 template <typename V> __device__ __forceinline__ V load_stream(const V *src)
 {
-#if MTA_HM_NTL
     if constexpr (sizeof(V) == 16) {
         typedef unsigned int u4 __attribute__((ext_vector_type(4)));
         return __builtin_bit_cast(V, __builtin_nontemporal_load(reinterpret_cast<const u4 *>(src)));
     }
-#endif
     return *src;
 }
 template <typename V> __device__ __forceinline__ void store_stream(V *dst, const V &v)
 {
-#if MTA_HM_NT
     if constexpr (sizeof(V) == 16) {
         typedef unsigned int u4 __attribute__((ext_vector_type(4)));
         __builtin_nontemporal_store(__builtin_bit_cast(u4, v), reinterpret_cast<u4 *>(dst));
         return;
     }
-#endif
     *dst = v;
 }
+
+// element (o, i) of the mixing matrix the kernels apply: w[o][i], or w[i][o] when `wt` (the transposed matrix is what
+// the gradient with respect to the input is mixed with)
+__device__ __forceinline__ int64_t w_index(int o, int i, int C, int wt) { return wt ? (int64_t)i * C + o : (int64_t)o * C + i; }
 
 // Workgroups go to the 8 XCDs round-robin by index.  With the key chunk as the fastest-varying part of the index and
 // a chunk count that divides 8 (or is a multiple of it), an XCD would always see the same chunks - and under the causal
@@ -73,93 +58,68 @@ __device__ __forceinline__ int rotated_chunk(unsigned &id, unsigned qchunks)
     return (int)((qc + rot) % qchunks);
 }
 
-// G heads mixed inside one lane, G known at compile time.  A workgroup covers ROWS consecutive
-// query rows of one key chunk, so a lane has ROWS*G independent 16-byte loads in flight.
-template <typename T, int G, int VEC, int ROWS>
+// G heads mixed inside one lane, G known at compile time.  A workgroup covers one query row of one key chunk: on this
+// part the fewer independent streams a wavefront holds, the higher the delivered bandwidth.
+template <typename T, int G, int VEC>
 __global__ __launch_bounds__(NT) void headmix_fixed(const T *__restrict__ x, const void *__restrict__ w,
                                                     T *__restrict__ y, int C, int P, int Q, int causal,
-                                                    float fill, int w_dtype, int qchunks, int pblocks)
+                                                    float fill, int w_dtype, int wt, int qchunks)
 {
-#if MTA_HM_WREG
-    constexpr bool WREG = G <= 8;
-#else
-    constexpr bool WREG = false;
-#endif
-    __shared__ float wsm[WREG ? 1 : G * G];
+    __shared__ float wsm[G * G];
     const int tid = threadIdx.x;
     const int groups = C / G;
     unsigned b = blockIdx.x;
     const int qc = rotated_chunk(b, qchunks);
-    const int p0 = (int)(b % (unsigned)pblocks) * ROWS; b /= (unsigned)pblocks;
+    const int p = (int)(b % (unsigned)P); b /= (unsigned)P;
     const int g = (int)(b % (unsigned)groups);
     const int64_t n = b / (unsigned)groups;
     const int q = (qc * NT + tid) * VEC;
     const int64_t plane = (int64_t)P * Q;
-    const int64_t base0 = (n * C + (int64_t)g * G) * plane + q;
+    const int64_t base = (n * C + (int64_t)g * G) * plane + (int64_t)p * Q + q;
     using V = vecN<T, VEC>;
     const T fill_t = from_float<T>(fill);
     V fillv;
 #pragma unroll
     for (int u = 0; u < VEC; ++u) fillv.v[u] = fill_t;
-    const int plast = (p0 + ROWS - 1 < P - 1) ? p0 + ROWS - 1 : P - 1;
-    if (causal && qc * NT * VEC > plast) {  // chunk wholly above the diagonal for all rows: fill only, nothing read
+    if (causal && qc * NT * VEC > p) {  // chunk wholly above the diagonal: fill only, nothing read
         if (q < Q) {
 #pragma unroll
-            for (int r = 0; r < ROWS; ++r)
-                if (p0 + r < P) {
-#pragma unroll
-                    for (int o = 0; o < G; ++o) store_stream(reinterpret_cast<V *>(y + base0 + (int64_t)(p0 + r) * Q + o * plane), fillv);
-                }
+            for (int o = 0; o < G; ++o) store_stream(reinterpret_cast<V *>(y + base + o * plane), fillv);
         }
         return;
     }
     // Issue all of this lane's loads first (unconditionally: a lane past the row end or above the
     // diagonal re-reads the row start), then fetch the weights, so that the latencies overlap.
-    V xin[ROWS][G];
-#pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-        const int p = (p0 + r < P) ? p0 + r : P - 1;
+    V xin[G];
+    {
         const bool live = q < Q && !(causal && q > p);
-        const int64_t lb = base0 + (int64_t)p * Q - (live ? 0 : q);
+        const int64_t lb = base - (live ? 0 : q);
 #pragma unroll
-        for (int i = 0; i < G; ++i) xin[r][i] = load_stream(reinterpret_cast<const V *>(x + lb + i * plane));
+        for (int i = 0; i < G; ++i) xin[i] = load_stream(reinterpret_cast<const V *>(x + lb + i * plane));
     }
-    float wr[WREG ? G * G : 1];
-    if constexpr (WREG) {  // wave-uniform addresses: the weights arrive through the scalar unit
-#pragma unroll
-        for (int t = 0; t < G * G; ++t) wr[t] = load_any(w, w_dtype, (int64_t)(g * G + t / G) * C + g * G + t % G);
-    } else {
-        for (int t = tid; t < G * G; t += NT)
-            wsm[t] = load_any(w, w_dtype, (int64_t)(g * G + t / G) * C + g * G + t % G);
-        __syncthreads();
-    }
+    for (int t = tid; t < G * G; t += NT) wsm[t] = load_any(w, w_dtype, w_index(g * G + t / G, g * G + t % G, C, wt));
+    __syncthreads();
     if (q >= Q) return;
+    if (causal && q > p) {
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-        const int p = p0 + r;
-        if (p >= P) break;
-        const int64_t base = base0 + (int64_t)p * Q;
-        if (causal && q > p) {
+        for (int o = 0; o < G; ++o) store_stream(reinterpret_cast<V *>(y + base + o * plane), fillv);
+        return;
+    }
 #pragma unroll
-            for (int o = 0; o < G; ++o) store_stream(reinterpret_cast<V *>(y + base + o * plane), fillv);
-            continue;
+    for (int o = 0; o < G; ++o) {
+        float acc[VEC];
+#pragma unroll
+        for (int u = 0; u < VEC; ++u) acc[u] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < G; ++i) {
+            const float wv = wsm[o * G + i];
+#pragma unroll
+            for (int u = 0; u < VEC; ++u) acc[u] = fmaf(wv, to_float(xin[i].v[u]), acc[u]);
         }
+        V out;
 #pragma unroll
-        for (int o = 0; o < G; ++o) {
-            float acc[VEC];
-#pragma unroll
-            for (int u = 0; u < VEC; ++u) acc[u] = 0.0f;
-#pragma unroll
-            for (int i = 0; i < G; ++i) {
-                const float wv = WREG ? wr[o * G + i] : wsm[o * G + i];
-#pragma unroll
-                for (int u = 0; u < VEC; ++u) acc[u] = fmaf(wv, to_float(xin[r][i].v[u]), acc[u]);
-            }
-            V out;
-#pragma unroll
-            for (int u = 0; u < VEC; ++u) out.v[u] = (causal && q + u > p) ? fill_t : from_float<T>(acc[u]);
-            store_stream(reinterpret_cast<V *>(y + base + o * plane), out);
-        }
+        for (int u = 0; u < VEC; ++u) out.v[u] = (causal && q + u > p) ? fill_t : from_float<T>(acc[u]);
+        store_stream(reinterpret_cast<V *>(y + base + o * plane), out);
     }
 }
 
@@ -175,15 +135,12 @@ __global__ __launch_bounds__(NT) void headmix_fixed(const T *__restrict__ x, con
 // After the eight products the lane holds keys 8ln .. 8ln+7 of output heads 4kg + v: 16-byte stores, again
 // 4 heads x 256 contiguous bytes per instruction.  Columns are independent, so keys beyond the diagonal may carry any
 // data (their lanes re-read the row start); their outputs get the fill.
-#ifndef MTA_HM_DM_WAVES
-#define MTA_HM_DM_WAVES 4
-#endif
-constexpr int DM_WAVES = MTA_HM_DM_WAVES, DM_KEYS = 128;
+constexpr int DM_WAVES = 4, DM_KEYS = 128;
 
 template <typename T>
 __global__ __launch_bounds__(64 * DM_WAVES, 4) void headmix_dense32(const T *__restrict__ x, const T *__restrict__ w,
                                                                T *__restrict__ y, int C, int P, int Q, int causal,
-                                                               float fill, int qchunks)
+                                                               float fill, int wt, int qchunks)
 {
     constexpr int HG = 32;  // heads mixed together
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, ln = lane & 15, kg = lane >> 4;
@@ -220,8 +177,14 @@ __global__ __launch_bounds__(64 * DM_WAVES, 4) void headmix_dense32(const T *__r
     // w fragments: lane (output head ln of block ob, group kg) holds w[o][8kg .. 8kg+7]
     frag8<T> wf[2];
 #pragma unroll
-    for (int ob = 0; ob < 2; ++ob)
-        wf[ob] = *reinterpret_cast<const frag8<T> *>(w + (int64_t)(g * HG + ob * 16 + ln) * C + g * HG + kg * 8);
+    for (int ob = 0; ob < 2; ++ob) {
+        if (!wt) {
+            wf[ob] = *reinterpret_cast<const frag8<T> *>(w + (int64_t)(g * HG + ob * 16 + ln) * C + g * HG + kg * 8);
+        } else {  // the transposed matrix: a column of w, gathered element by element (once per wavefront)
+#pragma unroll
+            for (int t = 0; t < 8; ++t) wf[ob].v[t] = w[(int64_t)(g * HG + kg * 8 + t) * C + g * HG + ob * 16 + ln];
+        }
+    }
 
     f32x4 acc[8][2];
 #pragma unroll
@@ -262,7 +225,7 @@ __global__ __launch_bounds__(64 * DM_WAVES, 4) void headmix_dense32(const T *__r
 template <typename T, int VEC>
 __global__ __launch_bounds__(NT) void headmix_any(const T *__restrict__ x, const void *__restrict__ w,
                                                   T *__restrict__ y, int C, int G, int P, int Q, int causal,
-                                                  float fill, int w_dtype, int qchunks)
+                                                  float fill, int w_dtype, int wt, int qchunks)
 {
     const int tid = threadIdx.x;
     const int groups = C / G;
@@ -283,7 +246,7 @@ __global__ __launch_bounds__(NT) void headmix_any(const T *__restrict__ x, const
         for (int u = 0; u < VEC; ++u) acc[u] = 0.0f;
         if (!(causal && q > p)) {
             for (int i = 0; i < G; ++i) {
-                const float wv = load_any(w, w_dtype, (int64_t)(g * G + o) * C + g * G + i);
+                const float wv = load_any(w, w_dtype, w_index(g * G + o, g * G + i, C, wt));
                 const V xv = *reinterpret_cast<const V *>(x + base + i * plane);
 #pragma unroll
                 for (int u = 0; u < VEC; ++u) acc[u] = fmaf(wv, to_float(xv.v[u]), acc[u]);
@@ -298,7 +261,7 @@ __global__ __launch_bounds__(NT) void headmix_any(const T *__restrict__ x, const
 
 template <typename T, int VEC>
 int launch(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t P, int64_t Q, int G, int causal,
-           float fill, int w_dtype, bool w_same_dtype, hipStream_t st)
+           float fill, int w_dtype, int wt, bool w_same_dtype, hipStream_t st)
 {
     if constexpr (VEC == 8) {
         // 32 heads mixed densely, 16-bit data and weights of the same dtype: matrix cores (MTA_HEADMIX_NO_MFMA=1 in the
@@ -309,38 +272,35 @@ int launch(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t 
             const int64_t blocks = N * (C / 32) * P * qch;
             if (blocks > 0x7fffffffLL) return MTA_ERR_SHAPE;
             hipLaunchKernelGGL((headmix_dense32<T>), dim3((unsigned)blocks), dim3(64 * DM_WAVES), 0, st, (const T *)x,
-                               (const T *)w, (T *)y, (int)C, (int)P, (int)Q, causal, fill, qch);
+                               (const T *)w, (T *)y, (int)C, (int)P, (int)Q, causal, fill, wt, qch);
             return launch_status();
         }
     }
     const int qchunks = (int)((Q + (int64_t)NT * VEC - 1) / ((int64_t)NT * VEC));
-#define MTA_HM_CASE(g, rows)                                                                                       \
-    if (G == g) {                                                                                                  \
-        const int pblocks = (int)((P + rows - 1) / rows);                                                          \
-        const int64_t blocks = N * (C / G) * pblocks * qchunks;                                                    \
-        if (blocks > 0x7fffffffLL) return MTA_ERR_SHAPE;                                                           \
-        hipLaunchKernelGGL((headmix_fixed<T, g, VEC, rows>), dim3((unsigned)blocks), dim3(NT), 0, st, (const T *)x, w, \
-                           (T *)y, (int)C, (int)P, (int)Q, causal, fill, w_dtype, qchunks, pblocks);               \
-        return launch_status();                                                                                    \
+#define MTA_HM_CASE(g)                                                                                         \
+    if (G == g) {                                                                                              \
+        const int64_t blocks = N * (C / G) * P * qchunks;                                                      \
+        if (blocks > 0x7fffffffLL) return MTA_ERR_SHAPE;                                                       \
+        hipLaunchKernelGGL((headmix_fixed<T, g, VEC>), dim3((unsigned)blocks), dim3(NT), 0, st, (const T *)x, w, \
+                           (T *)y, (int)C, (int)P, (int)Q, causal, fill, w_dtype, wt, qchunks);                 \
+        return launch_status();                                                                                \
     }
-    MTA_HM_CASE(1, MTA_HM_ROWS)
-    MTA_HM_CASE(2, MTA_HM_ROWS)
-    MTA_HM_CASE(4, MTA_HM_ROWS)
-    MTA_HM_CASE(8, MTA_HM_ROWS)
-    MTA_HM_CASE(16, 1)
-    MTA_HM_CASE(32, 1)
+    MTA_HM_CASE(1)
+    MTA_HM_CASE(2)
+    MTA_HM_CASE(4)
+    MTA_HM_CASE(8)
+    MTA_HM_CASE(16)
+    MTA_HM_CASE(32)
 #undef MTA_HM_CASE
     const int64_t blocks = N * (C / G) * P * qchunks;
     if (blocks > 0x7fffffffLL) return MTA_ERR_SHAPE;
     hipLaunchKernelGGL((headmix_any<T, VEC>), dim3((unsigned)blocks), dim3(NT), 0, st, (const T *)x, w, (T *)y, (int)C, G,
-                       (int)P, (int)Q, causal, fill, w_dtype, qchunks);
+                       (int)P, (int)Q, causal, fill, w_dtype, wt, qchunks);
     return launch_status();
 }
-}  // namespace
 
-extern "C" int mta_headmix_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t P,
-                               int64_t Q, int group_size, int causal, float fill, int io_dtype, int w_dtype,
-                               void *stream)
+int headmix_entry(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t P, int64_t Q, int group_size,
+                  int causal, float fill, int io_dtype, int w_dtype, int wt, void *stream)
 {
     if (!x || !w || !y) return MTA_ERR_NULL;
     if (!dtype_size(io_dtype) || !dtype_size(w_dtype)) return MTA_ERR_DTYPE;
@@ -355,8 +315,24 @@ extern "C" int mta_headmix_fwd(const void *x, const void *w, void *y, int64_t N,
         constexpr int VEC = vec_of<io_t>::n;
         const bool vec_ok = (Q % VEC == 0) && aligned_to(x, 16) && aligned_to(y, 16);
         const bool same = w_dtype == io_dtype;
-        return vec_ok ? launch<io_t, VEC>(x, w, y, N, C, P, Q, G, causal, fill, w_dtype, same, st)
-                      : launch<io_t, 1>(x, w, y, N, C, P, Q, G, causal, fill, w_dtype, same, st);
+        return vec_ok ? launch<io_t, VEC>(x, w, y, N, C, P, Q, G, causal, fill, w_dtype, wt, same, st)
+                      : launch<io_t, 1>(x, w, y, N, C, P, Q, G, causal, fill, w_dtype, wt, same, st);
     });
     return MTA_ERR_DTYPE;
+}
+}  // namespace
+
+extern "C" int mta_headmix_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t P,
+                               int64_t Q, int group_size, int causal, float fill, int io_dtype, int w_dtype,
+                               void *stream)
+{
+    return headmix_entry(x, w, y, N, C, P, Q, group_size, causal, fill, io_dtype, w_dtype, 0, stream);
+}
+
+// dx[n,i,p,q] = sum_o w[o,i] dy[n,o,p,q]: the forward kernels with the transposed matrix; above the diagonal the
+// gradient is +0 (those inputs were never read)
+extern "C" int mta_headmix_bwd_input(const void *dy, const void *w, void *dx, int64_t N, int64_t C, int64_t P,
+                                     int64_t Q, int group_size, int causal, int io_dtype, int w_dtype, void *stream)
+{
+    return headmix_entry(dy, w, dx, N, C, P, Q, group_size, causal, 0.0f, io_dtype, w_dtype, 1, stream);
 }

@@ -88,6 +88,81 @@ def headmix(x: torch.Tensor, weight: torch.Tensor, causal: bool = True, fill: fl
     return y
 
 
+def _workspace(nbytes: int, device) -> torch.Tensor:
+    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
+
+
+def conv2d_bwd_input(dy: torch.Tensor, weight: torch.Tensor, causal: bool) -> torch.Tensor:
+    """Gradient of ``conv2d_causal`` with respect to its input; see mta_conv2d_bwd_input."""
+    dy = _device_tensor(dy, "grad_output")
+    weight = _device_tensor(weight.detach(), "weight")
+    n, c, h, w = dy.shape
+    c_out, r, s = weight.shape
+    assert c == c_out, "This implementation assumes depthwise convolution (C_in == C_out)"
+    dx = torch.empty_like(dy, memory_format=torch.contiguous_format)
+    with torch.cuda.device(dy.device):
+        rc = _lib.load().mta_conv2d_bwd_input(dy.data_ptr(), weight.data_ptr(), dx.data_ptr(), n, c, h, w, r, s,
+                                              int(bool(causal)), _code(dy, "grad_output"), _code(weight, "weight"),
+                                              _stream(dy))
+    _lib.check(rc, "mta_conv2d_bwd_input")
+    return dx
+
+
+def conv2d_bwd_weight(x: torch.Tensor, dy: torch.Tensor, kernel_size, causal: bool) -> torch.Tensor:
+    """Gradient of ``conv2d_causal`` with respect to its (C,R,S) kernel, in fp32; see mta_conv2d_bwd_weight."""
+    x = _device_tensor(x, "input")
+    dy = _device_tensor(dy, "grad_output")
+    if x.shape != dy.shape or x.dtype != dy.dtype:
+        raise ValueError("input and grad_output must share shape and dtype")
+    n, c, h, w = x.shape
+    r, s = kernel_size
+    lib = _lib.load()
+    dw = torch.empty((c, r, s), dtype=torch.float32, device=x.device)
+    nbytes = lib.mta_conv2d_bwd_weight_workspace(n, c, h, w, r, s)
+    ws = _workspace(nbytes, x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.mta_conv2d_bwd_weight(x.data_ptr(), dy.data_ptr(), dw.data_ptr(), ws.data_ptr(), ws.numel(), n, c, h, w,
+                                       r, s, int(bool(causal)), _code(x, "input"), _stream(x))
+    _lib.check(rc, "mta_conv2d_bwd_weight")
+    return dw
+
+
+def headmix_bwd_input(dy: torch.Tensor, weight: torch.Tensor, causal: bool = True,
+                      group_size: Optional[int] = None) -> torch.Tensor:
+    """Gradient of ``headmix`` with respect to its input (+0 above the diagonal); see mta_headmix_bwd_input."""
+    dy = _device_tensor(dy, "grad_output")
+    weight = _device_tensor(weight.detach(), "weight")
+    n, c, p, q = dy.shape
+    assert tuple(weight.shape) == (c, c), f"Weight must be ({c},{c}), got {tuple(weight.shape)}"
+    dx = torch.empty_like(dy, memory_format=torch.contiguous_format)
+    with torch.cuda.device(dy.device):
+        rc = _lib.load().mta_headmix_bwd_input(dy.data_ptr(), weight.data_ptr(), dx.data_ptr(), n, c, p, q,
+                                               int(group_size or 0), int(bool(causal)), _code(dy, "grad_output"),
+                                               _code(weight, "weight"), _stream(dy))
+    _lib.check(rc, "mta_headmix_bwd_input")
+    return dx
+
+
+def headmix_bwd_weight(x: torch.Tensor, dy: torch.Tensor, causal: bool = True) -> torch.Tensor:
+    """Gradient of ``headmix`` with respect to its (C,C) weight, dense, in fp32; see mta_headmix_bwd_weight."""
+    x = _device_tensor(x, "input")
+    dy = _device_tensor(dy, "grad_output")
+    if x.shape != dy.shape or x.dtype != dy.dtype:
+        raise ValueError("input and grad_output must share shape and dtype")
+    n, c, p, q = x.shape
+    lib = _lib.load()
+    dw = torch.empty((c, c), dtype=torch.float32, device=x.device)
+    nbytes = lib.mta_headmix_bwd_weight_workspace(n, c, p, q)
+    if nbytes <= 0:
+        raise ValueError(f"mta_headmix_bwd_weight: no kernel for {c} heads (at most 128)")
+    ws = _workspace(nbytes, x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.mta_headmix_bwd_weight(x.data_ptr(), dy.data_ptr(), dw.data_ptr(), ws.data_ptr(), ws.numel(), n, c, p, q,
+                                        int(bool(causal)), _code(x, "input"), _stream(x))
+    _lib.check(rc, "mta_headmix_bwd_weight")
+    return dw
+
+
 def headmix_softmax(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optional[torch.Tensor], causal: bool = True,
                     group_size: Optional[int] = None, out: Optional[torch.Tensor] = None,
                     fill_upper: bool = True) -> torch.Tensor:

@@ -1,10 +1,12 @@
 """Head-axis linear ("head mixing") operator (HIP-backed).
 
 Mirrors TritonLinearHead (triton_linear_head.py:373-401) and TritonLinearHeadFunction
-(:281-319) of the reference; the Triton launch is replaced by ``mta_headmix_fwd``.
-Forward only.  One addition: an optional ``group_size`` hint.  The reference weight is
-always a dense (H,H) matrix; when it is block diagonal, passing the block size lets the
-kernel skip the zero blocks (the result is identical).
+(:281-370) of the reference; the Triton launches are replaced by ``mta_headmix_fwd``,
+``mta_headmix_bwd_input`` and ``mta_headmix_bwd_weight``.  One addition: an optional
+``group_size`` hint.  The reference weight is always a dense (H,H) matrix; when it is
+block diagonal, passing the block size lets the kernels skip the zero blocks (the result
+is identical); the weight gradient is then confined to the blocks as well, so that an
+optimizer step keeps the structure the caller promised.
 """
 from __future__ import annotations
 
@@ -19,11 +21,26 @@ class TritonLinearHeadFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, weight, causal=True, output_value=0.0, group_size=None):
+        ctx.save_for_backward(input, weight)
+        ctx.causal = causal
+        ctx.group_size = group_size
         return ops.headmix(input, weight, causal, output_value, group_size)
 
     @staticmethod
     def backward(ctx, grad_output):
-        raise NotImplementedError("the HIP build of TritonLinearHeadFunction is forward-only")
+        """triton_linear_head.py:322-370.  Above the diagonal the input gradient is 0 (the reference leaves
+        ``torch.empty_like`` memory there); the weight gradient is accumulated in fp32 and cast."""
+        input, weight = ctx.saved_tensors
+        grad_input = grad_weight = None
+        if ctx.needs_input_grad[0]:
+            grad_input = ops.headmix_bwd_input(grad_output, weight, ctx.causal, ctx.group_size)
+        if ctx.needs_input_grad[1]:
+            grad_weight = ops.headmix_bwd_weight(input, grad_output.to(input.dtype), ctx.causal)
+            if ctx.group_size:
+                blk = torch.arange(weight.shape[0], device=weight.device) // ctx.group_size
+                grad_weight = grad_weight * (blk[:, None] == blk[None, :])
+            grad_weight = grad_weight.to(weight.dtype)
+        return grad_input, grad_weight, None, None, None
 
 
 class TritonLinearHead(nn.Module):

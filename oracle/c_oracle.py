@@ -85,3 +85,23 @@ def conv_attention(q, k, v, w, causal: bool, scale: float):
                                        _i64(d), w.shape[1], w.shape[2], int(causal), ctypes.c_float(scale))
     assert rc == 0
     return o
+
+
+def conv2d_bwd(x, w, dy, causal: bool):
+    """(dx float32, dw float64) from the C restatement of the reference's backward kernels."""
+    x, w, dy = _f32(x), _f32(w), _f32(dy)
+    n, c, h, wd = x.shape
+    _, r, s = w.shape
+    dx = np.empty_like(x)
+    dw = np.empty((c, r, s), dtype=np.float64)
+    _load().oracle_conv2d_bwd(_p(x), _p(w), _p(dy), _p(dx), _p(dw), _i64(n), _i64(c), _i64(h), _i64(wd), r, s, int(causal))
+    return dx, dw
+
+
+def headmix_bwd(x, w, dy, causal: bool):
+    x, w, dy = _f32(x), _f32(w), _f32(dy)
+    n, c, p, q = x.shape
+    dx = np.empty_like(x)
+    dw = np.empty((c, c), dtype=np.float64)
+    _load().oracle_headmix_bwd(_p(x), _p(w), _p(dy), _p(dx), _p(dw), _i64(n), _i64(c), _i64(p), _i64(q), int(causal))
+    return dx, dw

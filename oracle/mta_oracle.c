@@ -12,6 +12,7 @@
  *   head mixing     mta_attention_pytorch.py:68,76, triton_linear_head.py:89-95,111-113,135-139,294-297
  *   MTA forward     mta_attention_pytorch.py:58-83
  *   conv attention  conv_attention_pytorch.py:33-92
+ *   backward        convolution_2d_trit.py:143-295, triton_linear_head.py:144-278
  */
 #include <math.h>
 #include <stdint.h>
@@ -62,6 +63,80 @@ void oracle_headmix(const float *x, const float *wt, float *y, int64_t N, int64_
                         acc += (double)wt[o * C + i] * (double)x[((n * C + i) * P + p) * Q + q];
                     *dst = (float)acc;
                 }
+}
+
+/* Backward of the conv, restated from the reference's own backward kernels (not derived from the forward above):
+ * conv_bwd_input_kernel (convolution_2d_trit.py:143-223):
+ *   dx[h,w] = sum_{i,j} w[i,j] * dy[h-i+pad_h, w-j+pad_w], dy read as 0 out of range and (causal) where col>row;
+ *   (causal) dx stays 0 where w>h.
+ * conv_bwd_weight_kernel (convolution_2d_trit.py:225-295):
+ *   dw[i,j] = sum_{n,p,q} x[p+i-pad_h, q+j-pad_w] * dy[p,q], both read as 0 out of range and (causal) where col>row. */
+void oracle_conv2d_bwd(const float *x, const float *w, const float *dy, float *dx, double *dw, int64_t N,
+                       int64_t C, int64_t H, int64_t W, int R, int S, int causal)
+{
+    const int pad_h = R - 1, pad_w = (S - 1) / 2;
+    for (int64_t c = 0; c < C; ++c)
+        for (int t = 0; t < R * S; ++t) dw[c * R * S + t] = 0.0;
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t c = 0; c < C; ++c) {
+            const float *xp = x + (n * C + c) * H * W, *gp = dy + (n * C + c) * H * W;
+            float *dxp = dx + (n * C + c) * H * W;
+            const float *wp = w + c * R * S;
+            for (int64_t h = 0; h < H; ++h)
+                for (int64_t k = 0; k < W; ++k) {
+                    double acc = 0.0;
+                    if (!(causal && k > h))
+                        for (int i = 0; i < R; ++i) {
+                            int64_t oh = h - i + pad_h;
+                            if (oh < 0 || oh >= H) continue;
+                            for (int j = 0; j < S; ++j) {
+                                int64_t ow = k - j + pad_w;
+                                if (ow < 0 || ow >= W) continue;
+                                if (causal && ow > oh) continue;
+                                acc += (double)wp[i * S + j] * (double)gp[oh * W + ow];
+                            }
+                        }
+                    dxp[h * W + k] = (float)acc;
+                }
+            for (int i = 0; i < R; ++i)
+                for (int j = 0; j < S; ++j) {
+                    double acc = 0.0;
+                    for (int64_t p = 0; p < H; ++p)
+                        for (int64_t q = 0; q < W; ++q) {
+                            if (causal && q > p) continue;
+                            int64_t ih = p + i - pad_h, iw = q + j - pad_w;
+                            if (ih < 0 || ih >= H || iw < 0 || iw >= W) continue;
+                            if (causal && iw > ih) continue;
+                            acc += (double)xp[ih * W + iw] * (double)gp[p * W + q];
+                        }
+                    dw[c * R * S + i * S + j] += acc;
+                }
+        }
+}
+
+/* Backward of the head mixing, restated from linear_head_kernel_backward_input / _weight
+ * (triton_linear_head.py:144-278): dx[n,i,p,q] = sum_o dy[n,o,p,q] w[o,i]; dw[o,i] = sum_{n,p,q} dy[n,o,p,q] x[n,i,p,q];
+ * with causal only q <= p take part (dx is left untouched above the diagonal there; 0 here). */
+void oracle_headmix_bwd(const float *x, const float *wt, const float *dy, float *dx, double *dw, int64_t N, int64_t C,
+                        int64_t P, int64_t Q, int causal)
+{
+    for (int64_t e = 0; e < C * C; ++e) dw[e] = 0.0;
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t p = 0; p < P; ++p)
+            for (int64_t q = 0; q < Q; ++q) {
+                const int live = !(causal && q > p);
+                for (int64_t i = 0; i < C; ++i) {
+                    double acc = 0.0;
+                    if (live)
+                        for (int64_t o = 0; o < C; ++o)
+                            acc += (double)dy[((n * C + o) * P + p) * Q + q] * (double)wt[o * C + i];
+                    dx[((n * C + i) * P + p) * Q + q] = (float)acc;
+                }
+                if (live)
+                    for (int64_t o = 0; o < C; ++o)
+                        for (int64_t i = 0; i < C; ++i)
+                            dw[o * C + i] += (double)dy[((n * C + o) * P + p) * Q + q] * (double)x[((n * C + i) * P + p) * Q + q];
+            }
 }
 
 static void conv_plane_d(const double *x, const float *w, double *y, int64_t S, int R, int Sk)

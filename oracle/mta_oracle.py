@@ -16,6 +16,9 @@ follows.  How each one is pinned (see tests/test_oracle.py):
   row 0 closed form, stage-by-stage equality with the C restatement; its tensor-mask
   branch (bool, (1,Sk) key mask, (1,1,S,S) additive) against the C restatement given
   the same additive mask; ``mta_forward_rows`` (slab form) == full form.
+* ``depthwise_conv_grads`` / ``head_linear_grads`` (autograd through the two operators):
+  gradcheck in fp64, the C restatement of the reference's backward kernels, adjoint
+  identities.
 * ``conv_attention_forward``: identity tap == causal SDPA, C restatement, equality
   with the composition of the pinned stages, slab form == full form.
 
@@ -130,6 +133,33 @@ def head_linear(x: torch.Tensor, weight: torch.Tensor, causal: bool = True,
         upper = torch.triu(torch.ones(p, q, dtype=torch.bool, device=x.device), diagonal=1)
         y = y.masked_fill(upper, output_value)
     return y
+
+
+# ---------------------------------------------------------------------------
+# backward of the two operators: torch.autograd through the forward restatements above
+# ---------------------------------------------------------------------------
+def depthwise_conv_grads(x, weight, causal, dy):
+    """(dx, dw) of ``depthwise_conv`` for the output gradient ``dy``, by torch.autograd.
+
+    What Conv2dTritonFunction.backward computes (convolution_2d_trit.py:336-378).  Pinned in
+    tests/test_oracle.py by torch.autograd.gradcheck in fp64 (finite differences), by the C
+    restatement of the reference's two backward kernels, and by the adjoint identities
+    <conv(x), dy> = <x, dx> = <w, dw>."""
+    x = x.detach().clone().requires_grad_(True)
+    w = weight.detach().clone().requires_grad_(True)
+    y = depthwise_conv(x, w, causal)
+    dx, dw = torch.autograd.grad(y, (x, w), dy)
+    return dx, dw
+
+
+def head_linear_grads(x, weight, causal, output_value, dy):
+    """(dx, dw) of ``head_linear``, by torch.autograd; what TritonLinearHeadFunction.backward computes
+    (triton_linear_head.py:322-370).  Pinned like ``depthwise_conv_grads``."""
+    x = x.detach().clone().requires_grad_(True)
+    w = weight.detach().clone().requires_grad_(True)
+    y = head_linear(x, w, causal, output_value)
+    dx, dw = torch.autograd.grad(y, (x, w), dy)
+    return dx, dw
 
 
 # ---------------------------------------------------------------------------

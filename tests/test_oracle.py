@@ -300,3 +300,45 @@ def test_conv_attention_scores_and_lse():
         if causal:   # row 0 sees one key: lse is that logit, scale * w[R-1, S//2] * (q0 . k0)
             want = 0.3 * w[:, -1, 2] * (q[0, :, 0] * k[0, :, 0]).sum(-1)
             torch.testing.assert_close(lse[0, :, 0], want, rtol=1e-5, atol=1e-6)
+
+
+# ---------------------------------------------------------------------------------------
+# backward of the two operators
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("rs", [(3, 3), (2, 5), (4, 4)])
+def test_conv_grads_pinned(causal, rs):
+    r, s = rs
+    x, w, dy = _rand((2, 3, 9, 9), 41), _rand((3, r, s), 42), _rand((2, 3, 9, 9), 43)
+    dx, dw = O.depthwise_conv_grads(x, w, causal, dy)
+    # the reference's own backward kernels, as nested loops
+    cdx, cdw = c_oracle.conv2d_bwd(x.numpy(), w.numpy(), dy.numpy(), causal)
+    np.testing.assert_allclose(dx.numpy(), cdx, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(dw.numpy(), cdw, rtol=1e-5, atol=1e-5)
+    # adjoint identities of an operator that is linear in x and in w
+    y = O.depthwise_conv(x, w, causal)
+    torch.testing.assert_close((y * dy).sum(), (x * dx).sum(), rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close((y * dy).sum(), (w * dw).sum(), rtol=1e-4, atol=1e-4)
+    if causal:
+        assert (dx.triu(1) == 0).all()
+    # finite differences
+    xd = x[:1, :, :6, :6].double().requires_grad_(True)
+    wd = w.double().requires_grad_(True)
+    assert torch.autograd.gradcheck(lambda a, b: O.depthwise_conv(a, b, causal), (xd, wd), eps=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("causal,fill", [(True, 0.0), (True, float("-inf")), (False, 0.0)])
+def test_headmix_grads_pinned(causal, fill):
+    x, w, dy = _rand((2, 5, 7, 7), 51), _rand((5, 5), 52), _rand((2, 5, 7, 7), 53)
+    dx, dw = O.head_linear_grads(x, w, causal, fill, dy)
+    cdx, cdw = c_oracle.headmix_bwd(x.numpy(), w.numpy(), dy.numpy(), causal)
+    np.testing.assert_allclose(dx.numpy(), cdx, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(dw.numpy(), cdw, rtol=1e-5, atol=1e-5)
+    if causal:
+        assert (dx.triu(1) == 0).all()
+    if fill == 0.0:
+        y = O.head_linear(x, w, causal, fill)
+        live = torch.tril(torch.ones(7, 7)) if causal else torch.ones(7, 7)
+        torch.testing.assert_close((y * dy * live).sum(), (w * dw).sum(), rtol=1e-4, atol=1e-4)
+        xd, wd = x[:1].double().requires_grad_(True), w.double().requires_grad_(True)
+        assert torch.autograd.gradcheck(lambda a, b: O.head_linear(a, b, causal, 0.0), (xd, wd), eps=1e-6, atol=1e-6)
