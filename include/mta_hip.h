@@ -159,6 +159,15 @@ int mta_conv2d_bwd_weight(const void *x, const void *dy, void *dw, void *workspa
                           int64_t N, int64_t C, int64_t H, int64_t W, int R, int S, int causal, int io_dtype,
                           void *stream);
 
+/* mta_conv2d_bwd_weight for callers that cannot allocate device memory or pass a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same kernels
+ * and same result; the partial sums live in a 1 MiB array that the library holds statically on each device it runs
+ * on.  Needs C*R*S*4 bytes <= 1 MiB (else MTA_ERR_WORKSPACE, nothing launched); with fewer partial kernels than
+ * mta_conv2d_bwd_weight would use (large kernels) the sums are added in a different order.  Calls that overlap on
+ * one device share that array and race: serialise them (one stream). */
+int mta_conv2d_bwd_weight_noalloc(const void *x, const void *dy, void *dw, int64_t N, int64_t C, int64_t H, int64_t W,
+                                  int R, int S, int causal, int io_dtype, void *stream);
+
 /* dx[n,i,p,q] = sum_o w[o,i] * dy[n,o,p,q].  group_size as in mta_headmix_fwd.  Replaces
  * linear_head_kernel_backward_input (triton_linear_head.py:144-196, 330-348); the reference leaves dx above the
  * diagonal uninitialised (torch.empty_like), here it is +0. */

@@ -32,6 +32,7 @@ SIGNATURES = {
     "mta_conv2d_bwd_input": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _vp]),
     "mta_conv2d_bwd_weight_workspace": (_i64, [_i64, _i64, _i64, _i64, _int, _int]),
     "mta_conv2d_bwd_weight": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _vp]),
+    "mta_conv2d_bwd_weight_noalloc": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _vp]),
     "mta_headmix_bwd_input": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _vp]),
     "mta_headmix_bwd_weight_workspace": (_i64, [_i64, _i64, _i64, _i64]),
     "mta_headmix_bwd_weight": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _int, _vp]),

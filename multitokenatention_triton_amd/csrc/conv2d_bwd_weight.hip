@@ -269,6 +269,30 @@ reduce:
     }
 }
 
+// ---- scratch buffer of the entry point that allocates nothing -----------------------------------------------------
+// One array per device, alive until the process ends.  In host code the array's name is only a handle: the address the
+// kernels get is the one hipGetSymbolAddress returns for the current device, looked up once per device and kept.  Every
+// call on a device shares that device's array: calls that overlap on one device (two streams, two threads) race.  The
+// kernels write every partial sum they later read, so nothing has to be cleared between calls.
+constexpr int64_t STATIC_FLOATS = 256 * 1024;  // 1 MiB: e.g. 2048 partial kernels of up to 128 taps
+static __device__ __align__(256) float scratch[STATIC_FLOATS];
+
+float *static_scratch(int *err)
+{
+    static float *ptr[64] = {nullptr};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { *err = (int)e; return nullptr; }
+    if (dev < 0 || dev >= 64) { *err = MTA_ERR_DEVICE; return nullptr; }
+    if (!ptr[dev]) {
+        float *p = nullptr;
+        e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) { *err = (int)e; return nullptr; }
+        ptr[dev] = p;
+    }
+    *err = MTA_OK;
+    return ptr[dev];
+}
 }  // namespace
 
 extern "C" int64_t mta_conv2d_bwd_weight_workspace(int64_t N, int64_t C, int64_t H, int64_t W, int R, int S)
@@ -292,3 +316,19 @@ extern "C" int mta_conv2d_bwd_weight(const void *x, const void *dy, void *dw, vo
     return MTA_ERR_DTYPE;
 }
 
+
+extern "C" int mta_conv2d_bwd_weight_noalloc(const void *x, const void *dy, void *dw, int64_t N, int64_t C, int64_t H,
+                                             int64_t W, int R, int S, int causal, int io_dtype, void *stream)
+{
+    int rc = check_args(x, dy, dw, N, C, H, W, R, S, io_dtype);
+    if (rc != MTA_OK) return rc;
+    // as many partial kernels as the fixed array holds
+    const int64_t cap = STATIC_FLOATS / ((int64_t)R * S);
+    if (cap < C) return MTA_ERR_WORKSPACE;  // C*R*S floats do not fit: one partial kernel per channel is the minimum
+    const int bpc = blocks_per_channel(N, C, H, W, cap < MAX_PARTIALS ? cap : MAX_PARTIALS);
+    float *ws = static_scratch(&rc);
+    if (!ws) return rc;
+    MTA_DISPATCH_IO(io_dtype, return launch<io_t>(x, dy, (float *)dw, ws, bpc, N, C, H, W, R, S, causal,
+                                                  (hipStream_t)stream));
+    return MTA_ERR_DTYPE;
+}
