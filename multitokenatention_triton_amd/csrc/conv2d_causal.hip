@@ -173,35 +173,15 @@ int dispatch_valu(const void *x, const void *w, void *y, int64_t N, int64_t C, i
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // The output is written once and not read again by this kernel: non-temporal stores keep it from displacing the input
 // rows that neighbouring strips re-read (halos) in the L2.
-#ifndef MTA_CONV_NT_STORE
-#define MTA_CONV_NT_STORE 1
-#endif
-#if MTA_CONV_NT_STORE
 #define MTA_CONV_STORE(ptr, val) __builtin_nontemporal_store((val), (ptr))
-#else
-#define MTA_CONV_STORE(ptr, val) (*(ptr) = (val))
-#endif
-#ifndef MTA_CONV_WAVES_PER_SIMD
-#define MTA_CONV_WAVES_PER_SIMD 2  // register budget: 256 VGPRs
-#endif
-#ifndef MTA_CONV_MFMA32
-#define MTA_CONV_MFMA32 0          // 0: 16x16x32 MFMAs (fewer matrix-core cycles and Toeplitz registers per output;
-                                   // measured faster), 1: 32x32x16 (fewer LDS operand bytes per output)
-#endif
-#ifndef MTA_CONV_DOUBLE_BUF
-#define MTA_CONV_DOUBLE_BUF 1      // 1: the next strip's copy is in flight during the products; 0: one strip buffer
-#endif
-#ifndef MTA_CONV_WG_PER_CU
-#define MTA_CONV_WG_PER_CU 6       // LDS budget: two 11.6 KB strip buffers per single-wavefront workgroup
-#endif
-constexpr int M_WT = 64;   // one wavefront per workgroup
-#ifndef MTA_CONV_STRIP_ROWS
-#define MTA_CONV_STRIP_ROWS 32
-#endif
-constexpr int M_TM = MTA_CONV_STRIP_ROWS;  // strip rows: row blocks of 16
-constexpr int M_TN = 128;  // strip cols: 8 column blocks of 16
+
+constexpr int M_NW = 2;            // wavefronts per workgroup; each owns one 16-row block of the workgroup's strip
+constexpr int M_WT = 64 * M_NW;    // threads per workgroup
+constexpr int M_TM = 16 * M_NW;    // strip rows
+constexpr int M_TN = 128;          // strip cols: 8 column blocks of 16
 constexpr int M_SPB = M_TN / M_TM;  // strips per 128x128 block
-static_assert(M_TM % 16 == 0 && M_TN % M_TM == 0 && (M_SPB & (M_SPB - 1)) == 0, "strip geometry");
+constexpr int M_WG_PER_CU = 4;     // persistent workgroups per CU (two 12 KB strip buffers each); 3, 5 and 6 measured slower
+static_assert(M_TN % M_TM == 0 && (M_SPB & (M_SPB - 1)) == 0, "strip geometry");
 
 // 16 outputs + S-1 taps (+ alignment shift) must fit the 32-key contraction of one 16x16x32 MFMA
 template <int R, int S> struct mfma_geom {
@@ -209,20 +189,17 @@ template <int R, int S> struct mfma_geom {
     static constexpr int HL = (PADW + 7) & ~7;             // left halo, rounded so 16-byte loads stay aligned
     static constexpr int SHIFT = HL - PADW;                // first tap's offset inside a block's 32-key window
     static constexpr bool fits = SHIFT + 16 + S - 1 <= 32;
-    static constexpr bool fits32 = SHIFT + 32 + S - 1 <= 48;  // 3 chunks of 16 keys per 32-output window (32x32x16 MFMA)
     static constexpr int TW = M_TN - 16 + 32;              // staged columns
     static constexpr int LD = TW + ((24 - TW % 16) % 16);  // row stride = 8 (mod 16) elements: conflict-free b128 reads
     static constexpr int ROWS = M_TM + R - 1;
 };
 
-// work item -> (plane, strip row tm (32 rows), strip col tn (128 keys)).
+// position t of a work item inside its plane -> (strip row tm (M_TM rows), strip col tn (128 keys)).
 // `mirror` (causal, square): only strips that touch the lower triangle are enumerated, by 128x128
 // block in row-major lower-triangular order, M_SPB strips per block; each strip of an off-diagonal
 // block also zero-fills its share (1/M_SPB) of the block's mirror image above the diagonal.
-__device__ __forceinline__ void decode_item(int64_t idx, int ipp, int tiles_n, int mirror, int64_t &plane, int &tm, int &tn)
+__device__ __forceinline__ void decode_item(int t, int tiles_n, int mirror, int &tm, int &tn)
 {
-    plane = idx / ipp;
-    const int t = (int)(idx % ipp);
     if (mirror) {
         const int blk = t / M_SPB;
         int bm = (int)((sqrtf(8.0f * (float)blk + 1.0f) - 1.0f) * 0.5f);
@@ -244,20 +221,26 @@ __device__ __forceinline__ int opaque(int v)
     return v;
 }
 
-// FULL: the region lies inside the tensor; the stores are then unconditional (exactly M_TM/4 vector-memory instructions)
+// +0 over an M_TM x M_TN region, all threads of the workgroup.  FULL: the region lies inside the tensor; the stores are
+// then unconditional (exactly M_TM*M_TN/8/M_WT vector-memory instructions per lane)
 template <typename T, bool FULL = false>
-__device__ __forceinline__ void zero_fill_strip(T *yp, int H, int W, int p0, int q0, int lane)
+__device__ __forceinline__ void zero_fill_strip(T *yp, int H, int W, int p0, int q0, int tid)
 {
     constexpr int VEC = 8;
     pack16<T> z;
 #pragma unroll
     for (int u = 0; u < VEC; ++u) z.v[u] = from_float<T>(0.0f);
-    lane = opaque(lane);
+    tid = opaque(tid);
+    // thread t covers rows t/16 + 8k, vector t%16: a uniform base, one 32-bit per-lane byte offset, uniform row steps
+    static_assert(M_WT == 128 && M_TN / VEC == 16, "region rows per pass");
+    char *base = reinterpret_cast<char *>(yp + (int64_t)p0 * W + q0);
+    const int r0 = tid >> 4, cv = (tid & 15) * VEC;
+    const unsigned off = (unsigned)(r0 * W + cv) * (unsigned)sizeof(T);
+    const int64_t rstep = (int64_t)(M_WT / 16) * W * (int64_t)sizeof(T);
 #pragma unroll
-    for (int e = lane; e < M_TM * (M_TN / VEC); e += M_WT) {
-        const int r = e / (M_TN / VEC), col = q0 + (e % (M_TN / VEC)) * VEC;
-        if (FULL || (p0 + r < H && col < W))
-            MTA_CONV_STORE(reinterpret_cast<u32x4 *>(yp + (int64_t)(p0 + r) * W + col), __builtin_bit_cast(u32x4, z));
+    for (int k = 0; k < M_TM / (M_WT / 16); ++k) {
+        if (FULL || (p0 + r0 + k * (M_WT / 16) < H && q0 + cv < W))
+            MTA_CONV_STORE(reinterpret_cast<u32x4 *>(base + k * rstep + off), __builtin_bit_cast(u32x4, z));
     }
 }
 
@@ -274,6 +257,20 @@ __device__ __forceinline__ u32x4 lds_load16(unsigned addr)
     asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
     return v;
 }
+// the same with a compile-time byte offset in the instruction (no address arithmetic per access)
+// (`off` must fold to a constant below 65536: it goes into the instruction's offset field)
+__device__ __forceinline__ u32x4 lds_load16_at(unsigned addr, int off)
+{
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(off) : "memory");
+    return v;
+}
+__device__ __forceinline__ void lds_store8_at(unsigned addr, int off, unsigned lo, unsigned hi)
+{
+    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 v = {lo, hi};
+    asm volatile("ds_write_b64 %0, %1 offset:%2" : : "v"(addr), "v"(v), "n"(off) : "memory");
+}
 __device__ __forceinline__ void lds_store16(unsigned addr, u32x4 v)
 {
     asm volatile("ds_write_b128 %0, %1" : : "v"(addr), "v"(v) : "memory");
@@ -285,49 +282,29 @@ __device__ __forceinline__ void lds_store8(unsigned addr, unsigned lo, unsigned 
     asm volatile("ds_write_b64 %0, %1" : : "v"(addr), "v"(v) : "memory");
 }
 __device__ __forceinline__ void lds_wait() { asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory"); }
-template <int N> __device__ __forceinline__ void lds_wait_all(u32x4 (&a)[N])
-{
-    static_assert(N >= 1 && N <= 7, "kernel rows");
-    if constexpr (N == 3) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]) : : "memory");
-    else if constexpr (N == 5) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]) : : "memory");
-    else if constexpr (N == 6) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]) : : "memory");
-    else if constexpr (N == 7) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]) : : "memory");
-    else static_assert(N == 3 || N == 5 || N == 6 || N == 7, "add a case");
-}
-// Wait until at most NEWER LDS operations issued after the 2*N loads of `a` are outstanding (LDS operations complete
-// in order), and tie the loaded values to that point.
-template <int NEWER, int N> __device__ __forceinline__ void lds_wait_pair(u32x4 (&a)[2][N])
-{
-    static_assert(N >= 1 && N <= 7 && NEWER >= 0 && NEWER <= 15, "operand count / counter width");
-#define MTA_TIE2(i) "+v"(a[0][i]), "+v"(a[1][i])
-    if constexpr (N == 3) asm volatile("s_waitcnt lgkmcnt(%6)" : MTA_TIE2(0), MTA_TIE2(1), MTA_TIE2(2) : "n"(NEWER) : "memory");
-    else if constexpr (N == 5) asm volatile("s_waitcnt lgkmcnt(%10)" : MTA_TIE2(0), MTA_TIE2(1), MTA_TIE2(2), MTA_TIE2(3), MTA_TIE2(4) : "n"(NEWER) : "memory");
-    else if constexpr (N == 6) asm volatile("s_waitcnt lgkmcnt(%12)" : MTA_TIE2(0), MTA_TIE2(1), MTA_TIE2(2), MTA_TIE2(3), MTA_TIE2(4), MTA_TIE2(5) : "n"(NEWER) : "memory");
-    else if constexpr (N == 7) asm volatile("s_waitcnt lgkmcnt(%14)" : MTA_TIE2(0), MTA_TIE2(1), MTA_TIE2(2), MTA_TIE2(3), MTA_TIE2(4), MTA_TIE2(5), MTA_TIE2(6) : "n"(NEWER) : "memory");
-    else static_assert(N == 3 || N == 5 || N == 6 || N == 7, "add a case");
-#undef MTA_TIE2
-}
 __device__ __forceinline__ void lds_wait(u32x4 &a) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a) : : "memory"); }
-__device__ __forceinline__ void lds_wait(u32x4 &a, u32x4 &b, u32x4 &c)
-{
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c) : : "memory");
-}
+// workgroup barrier without the memory fence __syncthreads() carries (which would wait for the copy in flight)
+__device__ __forceinline__ void wg_barrier() { asm volatile("s_barrier" : : : "memory"); }
 
-// Persistent single-wavefront workgroups: each walks a contiguous run of 32x128 strips (so the
-// Toeplitz fragments are rebuilt only when the channel changes).  No workgroup barrier is ever
-// needed; latency is hidden by the other wavefronts resident on the CU, each in its own phase
-// (loading / matrix cores / storing) with its own 11 KB LDS strip.
+// Persistent two-wavefront workgroups: each walks a run of M_TM x 128 strips dealt round-robin within its XCD's share
+// of the item list.  Wavefront w owns row block w (16 rows) of the strip: it issues half of the staging copies, computes
+// its row block and stores it.  The wavefronts meet at one barrier per strip (the strip has landed; the previous
+// strip's buffer may be overwritten); latency is hidden by the other workgroups resident on the CU, each in its own
+// phase (loading / matrix cores / storing) with its own two 11.6 KB LDS strip buffers.
 //
 // Per 16x16 output block and kernel row i:  out^T[q, p] += T_i^T[q, k] X^T[k, p+i-(R-1)], one
 // v_mfma_f32_16x16x32 whose 32-key contraction window holds the 16 outputs' taps.  A operand =
-// Toeplitz fragment (4 VGPRs per kernel row, kept for the whole kernel), B operand = 16 contiguous
-// bytes of one staged row per lane.  Results go back through the (now free) LDS strip so that the
-// global stores are whole 256-byte row segments.
+// Toeplitz fragment (4 VGPRs per kernel row, kept while the channel is unchanged), B operand = 16 contiguous
+// bytes of one staged row per lane.  A wavefront sustains about one such 1 KB LDS operand per 35 cycles whatever the
+// addresses, against 16 cycles for the product: the products of a strip are therefore split over two wavefronts (on
+// two SIMDs).  Results go back through LDS rows that only the owning wavefront reads (row block 0: the strip's first
+// 16 staged rows; row block w > 0: the last 16 staged rows of its window) so that the global stores are whole
+// 256-byte row segments.
 //
 // Staging.  A strip whose halo lies wholly inside the tensor and on or below the diagonal (the
-// common case, decided per wavefront) is copied global -> LDS by global_load_lds_dwordx4: no
+// common case, decided per workgroup) is copied global -> LDS by global_load_lds_dwordx4: no
 // registers, no masks, no LDS store instructions.  The LDS row stride is 19 16-byte slots (18 of
-// data + 1 of padding), so lane L of copy `it` simply owns slot it*64+L.  Diagonal and border strips
+// data + 1 of padding), so thread t of copy `it` simply owns slot it*128+t.  Diagonal and border strips
 // are copied the same way and fixed up in LDS; the rare strips whose copy could leave the tensor go
 // through registers, where bounds and the causal col<=row rule are applied.
 //
@@ -337,7 +314,7 @@ __device__ __forceinline__ void lds_wait(u32x4 &a, u32x4 &b, u32x4 &c)
 // BWD: the gradient with respect to the input (see conv2d_valu): kernel rows reversed in both axes, the R-1 halo rows
 // below the strip instead of above it.  Key sizes are odd here, so the key halos are the same on both sides.
 template <typename T, int R, int S, bool SCALED, bool BWD>
-__global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
+__global__ __launch_bounds__(M_WT, 2) void conv2d_mfma(
     const T *__restrict__ x, const T *__restrict__ w, T *__restrict__ y, int C, int H, int W, int causal, float in_scale,
     int tiles_n, int ipp, int64_t total, int64_t per_xcd, int nw, int mirror)
 {
@@ -348,17 +325,14 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     constexpr int VPR = G::TW / VEC;                        // data vectors per staged row (18)
     constexpr int SPR = LD / VEC;                           // 16-byte slots per LDS row (19)
     constexpr int SLOTS = G::ROWS * SPR;
-    constexpr int STAGE_IT = (SLOTS + M_WT - 1) / M_WT;     // copies per strip
+    constexpr int STAGE_IT = (SLOTS + M_WT - 1) / M_WT;     // copies per strip and lane
     static_assert(SPR == VPR + 1, "one padding slot per row");
     // weights of the current channel, each kernel row zero-padded on both sides so that the
     // Toeplitz fragments can be gathered without range checks
-    constexpr bool M32 = MTA_CONV_MFMA32 && G::fits32 && M_TM == 32;
-    constexpr int NCH = 3;  // 16-key chunks per 32-output window (M32)
-    constexpr int WZ_OFF = G::SHIFT + (M32 ? 32 : 16), WZ_LD = WZ_OFF + (M32 ? 16 * NCH : 32);
-    constexpr int BUF = STAGE_IT * M_WT * VEC;  // elements per LDS strip buffer
-    constexpr bool DBUF = MTA_CONV_DOUBLE_BUF != 0;
-    __shared__ __align__(16) T tiles[(DBUF ? 2 : 1) * BUF];  // double buffer: strip n is computed while strip n+1 lands
-    __shared__ T wz[R * WZ_LD];
+    constexpr int WZ_OFF = G::SHIFT + 16, WZ_LD = WZ_OFF + 32;
+    constexpr int BUF = STAGE_IT * M_WT * VEC;               // elements per LDS strip buffer
+    __shared__ __align__(16) T tiles[2 * BUF];               // double buffer: strip n is computed while strip n+1 lands
+    __shared__ T wz[2][R * WZ_LD];                           // by strip parity: a wavefront may run one strip ahead
     using V16 = pack16<T>;
 
     // XCD-aware split: workgroup ids are dealt round-robin to the 8 XCDs; each XCD gets one
@@ -369,19 +343,23 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     // they sweep the same few hundred rows together (DRAM pages are consumed whole, as by a linear copy)
     const int64_t first = c0 + (int64_t)(blockIdx.x >> 3);
     const int64_t last = c1;
-    const int64_t step = nw;
+    const int step = nw;
     if (c0 >= total || first >= last) return;
+    const int n_items = (int)((last - first + step - 1) / step);
+    const int64_t HW = (int64_t)H * W;
 
-    const int lane = threadIdx.x, ln = M32 ? (lane & 31) : (lane & 15), kg = M32 ? (lane >> 5) : (lane >> 4);
-    frag8<T> tz[R][M32 ? NCH : 1];
+    const int tid = threadIdx.x, lane = tid & 63, ln = lane & 15, kg = lane >> 4;
+    // (the wavefront index through readfirstlane: everything derived from it is then scalar)
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    frag8<T> tz[R];
     int cur_channel = -1;
 
-    // per-lane geometry of the staging copies, fixed for the whole kernel: slot it*64+lane is row srow,
+    // per-thread geometry of the staging copies, fixed for the whole kernel: slot it*M_WT+tid is row srow,
     // vector svc of the strip; padding slots and slots past the strip re-read a neighbouring valid vector
     unsigned goff[STAGE_IT];  // byte offsets from the strip's first staged element (uniform base + 32-bit lane offset)
 #pragma unroll
     for (int it = 0; it < STAGE_IT; ++it) {
-        const int slot = it * M_WT + lane;
+        const int slot = it * M_WT + tid;
         int rr = slot / SPR, vc = slot % SPR;
         if (rr >= G::ROWS) { rr = 0; vc = 0; }
         if (vc >= VPR) vc = VPR - 1;
@@ -399,79 +377,95 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
     // the last one = head of the next row) lie inside the tensor.  What such a copy brings in from outside the plane
     // or from above the diagonal is zeroed in LDS afterwards (diagonal and border strips: a quarter of all strips,
     // which would otherwise load synchronously through registers).
-    const int64_t total_elems = (int64_t)(total / ipp) * H * W;  // planes * H * W
-    auto is_copyable = [&](int64_t plane_, int p0_, int q0_) {
+    // (a plane is named by the offset of its first element, `pbase`: kept up to date by additions, no 64-bit divisions)
+    const int64_t total_elems = (int64_t)(total / ipp) * HW;  // planes * H * W
+    auto is_copyable = [&](int64_t pbase_, int p0_, int q0_) {
         if (SCALED) return false;
         const int h0 = p0_ - TOP, k0 = q0_ - G::HL;
         if (h0 < 0 || h0 + G::ROWS > H) return false;
-        const int64_t e0 = plane_ * (int64_t)H * W + (int64_t)h0 * W + k0;
+        const int64_t e0 = pbase_ + (int64_t)h0 * W + k0;
         return e0 >= 0 && e0 + (int64_t)(G::ROWS - 1) * W + G::TW <= total_elems;
     };
-    // asynchronous copy of an interior or copyable strip into LDS buffer `buf`
-    auto prefetch = [&](int64_t plane_, int p0_, int q0_, T *buf) {
-        const char *base = reinterpret_cast<const char *>(x + plane_ * (int64_t)H * W + (int64_t)(p0_ - TOP) * W + (q0_ - G::HL));
+    // asynchronous copy of an interior or copyable strip into LDS buffer `buf` (this wavefront's half of the slots)
+    auto prefetch = [&](int64_t pbase_, int p0_, int q0_, T *buf) {
+        const char *base = reinterpret_cast<const char *>(x + pbase_ + (int64_t)(p0_ - TOP) * W + (q0_ - G::HL));
 #pragma unroll
         for (int it = 0; it < STAGE_IT; ++it)
-            __builtin_amdgcn_global_load_lds((glb_void_t *)(base + goff[it]), (lds_void_t *)(buf + it * M_WT * VEC), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((glb_void_t *)(base + goff[it]),
+                                             (lds_void_t *)(buf + (it * M_WT + wave * 64) * VEC), 16, 0, 0);
     };
 
     // The (zero-padded) kernel rows of a strip's channel are fetched one strip ahead into WPL registers per lane and
     // written to `wz` at the top of that strip's iteration: the items of a plane are dealt out over all workgroups of
-    // an XCD, so a wavefront changes channel every few strips, and a fetch at the point of use would expose a full
+    // an XCD, so a workgroup changes channel every few strips, and a fetch at the point of use would expose a full
     // memory latency each time.  The loads are issued from inline assembly, before the strip's copy, and are covered
     // by the wait for that copy at the top of the next iteration: seen by the compiler, they would make it wait for
     // every outstanding memory operation - the previous strip's stores included - before the values' first use.
+    // (The build fails if this kernel spills registers: a spill between the load and that wait would save a value
+    // that has not arrived yet.)
     constexpr int WPL = (R * WZ_LD + M_WT - 1) / M_WT;
     static_assert(sizeof(T) == 2, "16-bit loads");
     unsigned wnext[WPL];
-    auto fetch_weights = [&](int channel_) {
+    unsigned woff[WPL];   // byte offset of this lane's tap inside a channel's kernel (0 where the slot is padding)
+    unsigned wvalid = 0;  // bit it: slot it*M_WT+tid of the padded kernel rows holds a tap
 #pragma unroll
-        for (int it = 0; it < WPL; ++it) {
-            const int e = it * M_WT + lane;
-            const int i = e / WZ_LD, j = e % WZ_LD - WZ_OFF;
-            const bool ok = e < R * WZ_LD && j >= 0 && j < S;
-            const T *src = w + channel_ * R * S + (ok ? (BWD ? (R - 1 - i) * S + (S - 1 - j) : i * S + j) : 0);
-            asm volatile("global_load_ushort %0, %1, off" : "=v"(wnext[it]) : "v"(src) : "memory");
-        }
+    for (int it = 0; it < WPL; ++it) {
+        const int e = it * M_WT + tid;
+        const int i = e / WZ_LD, j = e % WZ_LD - WZ_OFF;
+        const bool ok = e < R * WZ_LD && j >= 0 && j < S;
+        woff[it] = ok ? (unsigned)(BWD ? (R - 1 - i) * S + (S - 1 - j) : i * S + j) * (unsigned)sizeof(T) : 0u;
+        wvalid |= ok ? (1u << it) : 0u;
+    }
+    auto fetch_weights = [&](int channel_) {
+        const char *wc = reinterpret_cast<const char *>(w + channel_ * R * S);
+#pragma unroll
+        for (int it = 0; it < WPL; ++it)
+            asm volatile("global_load_ushort %0, %1, %2" : "=v"(wnext[it]) : "v"(woff[it]), "s"(wc) : "memory");
     };
-    int64_t plane;
+    // current and next work item: position inside the plane, plane (as element offset) and channel
+    int t_nx;
+    int64_t pbase_nx;
+    int chan_nx;
+    {
+        const int64_t plane0 = first / ipp;
+        t_nx = (int)(first - plane0 * ipp);
+        pbase_nx = plane0 * HW;
+        chan_nx = (int)(plane0 % C);
+    }
     int tm, tn;
-    decode_item(first, ipp, tiles_n, mirror, plane, tm, tn);
-    fetch_weights((int)(plane % C));
-    if (DBUF && is_copyable(plane, tm * M_TM, tn * M_TN)) prefetch(plane, tm * M_TM, tn * M_TN, tiles);
+    decode_item(t_nx, tiles_n, mirror, tm, tn);
+    fetch_weights(chan_nx);
+    if (is_copyable(pbase_nx, tm * M_TM, tn * M_TN)) prefetch(pbase_nx, tm * M_TM, tn * M_TN, tiles);
 
     int younger = -1;                      // stores certainly issued after the copy in flight (-1: unknown)
     const bool fill_full = H % M_TN == 0;  // mirror images of whole 128x128 blocks lie inside the (square) tensor
     int parity = 0;
-    for (int64_t idx = first; idx < last; idx += step, parity ^= 1) {
-        T *tile = tiles + (DBUF ? parity * BUF : 0);
-        T *other = tiles + (DBUF ? (parity ^ 1) * BUF : 0);
+    for (int item = 0; item < n_items; ++item, parity ^= 1) {
+        T *tile = tiles + parity * BUF;
+        T *other = tiles + (parity ^ 1) * BUF;
+        T *wzp = wz[parity];
         const int p0 = tm * M_TM, q0 = tn * M_TN;
         const int ctm = tm, ctn = tn;
-        const T *xp = x + plane * (int64_t)H * W;
-        T *yp = y + plane * (int64_t)H * W;
-        const int channel = (int)(plane % C);
+        const int64_t pbase = pbase_nx;
+        const T *xp = x + pbase;
+        T *yp = y + pbase;
+        const int channel = chan_nx;
         const bool above = causal && q0 > p0 + M_TM - 1;  // wholly above the diagonal (only reachable when !mirror)
         const bool interior = is_interior(p0, q0);
-        const bool copyable = interior || is_copyable(plane, p0, q0);
+        const bool copyable = interior || is_copyable(pbase, p0, q0);
         const int h0 = p0 - TOP, k0 = q0 - G::HL;
         // (opaque: the addresses derived from it are then formed where they are used instead of being kept, dozens of
         // them, in registers across the loop)
         const unsigned tile_lds = (unsigned)opaque((int)(unsigned)(uintptr_t)(lds_void_t *)tile);
 
-        // This strip's copy (if interior) has landed.  Vector-memory operations complete in issue order, and the only
-        // ones issued after that copy are the previous strip's stores: when their number is known exactly
-        // (`younger`), they may stay in flight.  LDS reads of `other` by the previous iteration are complete.
-        if constexpr (DBUF) {
-            constexpr int ST = M_TM * (M_TN / VEC) / M_WT;  // stores per strip, and per mirror share
+        // This wavefront's half of the strip's copy (if any) has landed.  Vector-memory operations complete in issue
+        // order, and the only ones this wavefront issued after that copy are the previous strip's stores: when their
+        // number is known exactly (`younger`), they may stay in flight.
+        {
+            constexpr int ST = M_TM * (M_TN / VEC) / M_WT;  // stores per strip and lane, and per mirror share
             if (younger == 2 * ST) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * ST) : "memory");
             else if (younger == ST) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(ST) : "memory");
             else asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
-        } else {
-            // one buffer: this strip's copy is issued now and waited for (the other wavefronts of the CU cover the
-            // latency); the previous strip's LDS reads are complete
-            if (copyable) prefetch(plane, p0, q0, tile);
-            asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
         }
         younger = 0;
 
@@ -479,30 +473,18 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
 #pragma unroll
         for (int it = 0; it < WPL; ++it) {
             asm volatile("" : "+v"(wnext[it]));  // (the value is defined from the wait above on)
-            const int e = it * M_WT + lane;
-            const int j = e % WZ_LD - WZ_OFF;
-            if (e < R * WZ_LD) wz[e] = (j >= 0 && j < S) ? __builtin_bit_cast(T, (unsigned short)wnext[it]) : from_float<T>(0.0f);
+            const int e = it * M_WT + tid;
+            if (e < R * WZ_LD) wzp[e] = ((wvalid >> it) & 1u) ? __builtin_bit_cast(T, (unsigned short)wnext[it]) : from_float<T>(0.0f);
         }
 
-        // put the next strip's copy in flight (into the buffer the previous iteration has just released)
-        if (idx + step < last) {
-            decode_item(idx + step, ipp, tiles_n, mirror, plane, tm, tn);
-            fetch_weights((int)(plane % C));  // (before the copy: the loop-top wait counts what is younger than the copy)
-            if (DBUF && is_copyable(plane, tm * M_TM, tn * M_TN)) prefetch(plane, tm * M_TM, tn * M_TN, other);
-        }
-        if (above) {
-            zero_fill_strip<T>(yp, H, W, p0, q0, lane);
-            younger = -1;
-            continue;
-        }
-        if (copyable && !interior) {
+        if (!above && copyable && !interior) {
             // the copy has landed: zero what lies outside the plane or above the diagonal (whole vectors, except the one
             // vector of a row that straddles the diagonal)
-            const int lane_ = opaque(lane);
+            const int tid_ = opaque(tid);
             const u32x4 zero4 = {0u, 0u, 0u, 0u};
 #pragma unroll
             for (int it = 0; it < STAGE_IT; ++it) {
-                const int slot = it * M_WT + lane_;
+                const int slot = it * M_WT + tid_;
                 const int rr = slot / SPR, vc = slot % SPR;
                 const int h = h0 + rr, col = k0 + vc * VEC;
                 const bool ok = rr < G::ROWS && vc < VPR && col >= 0 && col < W && !(causal && col > h);
@@ -519,14 +501,14 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
                     lds_store16(addr, __builtin_bit_cast(u32x4, v));
                 }
             }
-        } else if (!interior) {
+        } else if (!above && !interior) {
             // edge strip: through registers.  Loads are unconditional and issued back to back (an invalid
             // slot re-reads a valid address); what a slot really holds is decided on the way to LDS
             V16 stage[STAGE_IT];
-            const int lane_ = opaque(lane);
+            const int tid_ = opaque(tid);
 #pragma unroll
             for (int it = 0; it < STAGE_IT; ++it) {
-                const int slot = it * M_WT + lane_;
+                const int slot = it * M_WT + tid_;
                 const int rr = slot / SPR, vc = slot % SPR;
                 const int h = h0 + rr, col = k0 + vc * VEC;
                 const bool ok = rr < G::ROWS && vc < VPR && h >= 0 && h < H && col >= 0 && col < W && !(causal && col > h);
@@ -534,7 +516,7 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
             }
 #pragma unroll
             for (int it = 0; it < STAGE_IT; ++it) {
-                const int slot = it * M_WT + lane_;
+                const int slot = it * M_WT + tid_;
                 const int rr = slot / SPR, vc = slot % SPR;
                 const int h = h0 + rr, col = k0 + vc * VEC;
                 const bool ok = rr < G::ROWS && vc < VPR && h >= 0 && h < H && col >= 0 && col < W && !(causal && col > h);
@@ -554,172 +536,127 @@ __global__ __launch_bounds__(M_WT, MTA_CONV_WAVES_PER_SIMD) void conv2d_mfma(
                 lds_store16(tile_lds + (unsigned)slot * 16u, __builtin_bit_cast(u32x4, v));
             }
         }
-        lds_wait();  // LDS stores above are complete (single wavefront: no barrier needed)
+        lds_wait();    // this wavefront's LDS stores above are complete
+        wg_barrier();  // the strip and its kernel rows are in LDS; every wavefront is done with the previous strip
+
+        // put the next strip's copy in flight (into the buffer the previous iteration has just released)
+        if (item + 1 < n_items) {
+            t_nx += step;
+            while (t_nx >= ipp) {  // (at most once, unless a plane holds fewer items than there are workgroups)
+                t_nx -= ipp;
+                pbase_nx += HW;
+                chan_nx = chan_nx + 1 == C ? 0 : chan_nx + 1;
+            }
+            decode_item(t_nx, tiles_n, mirror, tm, tn);
+            fetch_weights(chan_nx);  // (before the copy: the loop-top wait counts what is younger than the copy)
+            if (is_copyable(pbase_nx, tm * M_TM, tn * M_TN)) prefetch(pbase_nx, tm * M_TM, tn * M_TN, other);
+        }
+        if (above) {
+            zero_fill_strip<T>(yp, H, W, p0, q0, tid);
+            younger = -1;
+            continue;
+        }
 
         if (channel != cur_channel) {  // Toeplitz fragments T_i^T for this lane's accumulator row
             cur_channel = channel;
-            if constexpr (M32) {
-                // accumulator register v of lane-half kg is row m = 8*(v/4) + 4*kg + v%4; giving that row the output
-                // column 16*(v/8) + 8*kg + v%8 makes every 8 registers of a lane 8 consecutive keys
-                const int m = ln, qm = 16 * (m >> 4) + 8 * ((m >> 2) & 1) + 4 * ((m >> 3) & 1) + (m & 3);
 #pragma unroll
-                for (int i = 0; i < R; ++i)
+            for (int i = 0; i < R; ++i) {  // row m = ln, slots k = 8*kg + t, tap j = k-SHIFT-m
+                const T *src = wzp + i * WZ_LD + WZ_OFF + kg * 8 - G::SHIFT - ln;
 #pragma unroll
-                    for (int ch = 0; ch < NCH; ++ch) {
-                        const T *src = wz + i * WZ_LD + WZ_OFF + ch * 16 + kg * 8 - G::SHIFT - qm;  // tap j = k-SHIFT-q
-#pragma unroll
-                        for (int t = 0; t < 8; ++t) tz[i][ch].v[t] = src[t];
-                        __builtin_amdgcn_sched_barrier(0);  // keep the gathers of one fragment together (register pressure)
-                    }
-            } else {
-#pragma unroll
-                for (int i = 0; i < R; ++i) {  // row m = ln, slots k = 8*kg + t, tap j = k-SHIFT-m
-                    const T *src = wz + i * WZ_LD + WZ_OFF + kg * 8 - G::SHIFT - ln;
-#pragma unroll
-                    for (int t = 0; t < 8; ++t) tz[i][0].v[t] = src[t];
-                }
+                for (int t = 0; t < 8; ++t) tz[i].v[t] = src[t];
             }
         }
 
-        if constexpr (M32) {
-            // ---- 32 rows x 4 sub-tiles of 32 keys on 32x32x16 MFMAs, one sub-tile at a time; the three window chunks
-            // of kernel row i+1 are read from LDS while the products of row i run ----
-            const int prow = p0 + ln;
+        // ---- this wavefront's row block: 8 column blocks of 16x16 outputs on 16x16x32 MFMAs (one per kernel row: the
+        // 32-key window holds the 16 outputs' taps).  Lane (row ln, group kg) holds keys 4*kg..4*kg+3 of each block.
+        const int rb0 = wave * 16;                                   // first strip row of the block
+        const int res0 = wave == 0 ? 0 : wave * 16 + R - 1;          // staged rows that receive the results
+        {
+            f32x4 acc[M_TN / 16];
+            const unsigned xa = tile_lds + (unsigned)((rb0 + ln) * LD + kg * 8) * sizeof(T);
+            // Column blocks in pairs.  A wavefront issues in order, so a run of LDS reads followed by a run of
+            // products leaves the matrix cores idle during the first and the LDS idle during the second; here one read
+            // of the next pair's operands is issued per product of this pair, and a product waits only for its
+            // own operand, issued 2R reads earlier (LDS operations complete in order: lgkmcnt(2R) at every
+            // step).  Source order is pinned (the scheduler would regroup reads and products).  Blocks above the
+            // diagonal are computed like the others and masked below.
+            constexpr int NPAIR = M_TN / 32, NLD = 2 * R;
+            static_assert(NLD <= 15, "lgkmcnt field");
+            u32x4 xf[2][2][R];
+            auto xoff = [&](int pr, int c2, int i) { return (int)((i * LD + (pr * 2 + c2) * 16) * sizeof(T)); };
 #pragma unroll
-            for (int st = 0; st < M_TN / 32; ++st) {
-                f32x16 acc;
+            for (int i = 0; i < R; ++i)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
-                if (interior || !causal || q0 + st * 32 <= p0 + M_TM - 1) {  // else: wholly above the diagonal
-                    const unsigned xa = tile_lds + (unsigned)(ln * LD + st * 32 + kg * 8) * sizeof(T);
-                    u32x4 xf[2][NCH];
+                for (int c2 = 0; c2 < 2; ++c2) xf[0][c2][i] = lds_load16_at(xa, xoff(0, c2, i));
 #pragma unroll
-                    for (int ch = 0; ch < NCH; ++ch) xf[0][ch] = lds_load16(xa + (unsigned)(ch * 16) * sizeof(T));
-                    lds_wait(xf[0][0], xf[0][1], xf[0][2]);
-#pragma unroll
-                    for (int i = 0; i < R; ++i) {
-                        if (i + 1 < R) {
-#pragma unroll
-                            for (int ch = 0; ch < NCH; ++ch)
-                                xf[(i + 1) & 1][ch] = lds_load16(xa + (unsigned)((i + 1) * LD + ch * 16) * sizeof(T));
-                        }
-#pragma unroll
-                        for (int ch = 0; ch < NCH; ++ch) mma32(acc, tz[i][ch], __builtin_bit_cast(frag8<T>, xf[i & 1][ch]));
-                        if (i + 1 < R) lds_wait(xf[(i + 1) & 1][0], xf[(i + 1) & 1][1], xf[(i + 1) & 1][2]);
-                    }
-                }
-                // results back into the strip's own LDS rows: sub-tile st overwrites columns 32st..32st+31, which the
-                // later sub-tiles (reading columns >= 32(st+1)) no longer need
-#pragma unroll
-                for (int a = 0; a < 2; ++a) {
-                    const int col = st * 32 + a * 16 + kg * 8;
-                    const int q = q0 + col;
-                    uint32_t pk[4];
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) pk[u] = pack2<T>(acc[a * 8 + 2 * u], acc[a * 8 + 2 * u + 1]);
-                    if (!interior && causal && q + 7 > prow) {
-#pragma unroll
-                        for (int u = 0; u < 4; ++u) {
-                            if (q + 2 * u > prow) pk[u] &= 0xffff0000u;
-                            if (q + 2 * u + 1 > prow) pk[u] &= 0x0000ffffu;
-                        }
-                    }
-                    lds_store16(tile_lds + (unsigned)(ln * LD + col) * sizeof(T), u32x4{pk[0], pk[1], pk[2], pk[3]});
-                }
-            }
-        } else {
-            // ---- 2 row blocks x 8 column blocks of 16x16 outputs on 16x16x32 MFMAs (one per kernel row: the 32-key
-            // window holds the 16 outputs' taps).  A third of the Toeplitz registers of the 32x32 form and fewer
-            // matrix-core cycles per output, at more LDS operand bytes.  Results of a row block go back into its own
-            // (no longer needed) LDS rows: lane (row ln, group kg) holds keys 4*kg..4*kg+3 of each block.
-#pragma unroll
-            for (int rb = 0; rb < M_TM / 16; ++rb) {
-                f32x4 acc[M_TN / 16];
-                const unsigned xa = tile_lds + (unsigned)((rb * 16 + ln) * LD + kg * 8) * sizeof(T);
-                // Column blocks in pairs.  A wavefront issues in order, so a run of LDS reads followed by a run of
-                // products leaves the matrix cores idle during the first and the LDS during the second; here one read
-                // of the next pair's operands is issued per product of this pair, and a product waits only for its
-                // own operand, issued 2R reads earlier (LDS operations complete in order: lgkmcnt(2R) at every
-                // step).  Source order is pinned (the scheduler would regroup reads and products).  Blocks above the
-                // diagonal are computed like the others and masked below.
-                constexpr int NPAIR = M_TN / 32, NLD = 2 * R;
-                static_assert(NLD <= 15, "lgkmcnt field");
-                u32x4 xf[2][2][R];
-                auto xaddr = [&](int pr, int c2, int i) { return xa + (unsigned)(i * LD + (pr * 2 + c2) * 16) * sizeof(T); };
+            for (int pr = 0; pr < NPAIR; ++pr) {
+                acc[2 * pr] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                acc[2 * pr + 1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int i = 0; i < R; ++i)
 #pragma unroll
-                    for (int c2 = 0; c2 < 2; ++c2) xf[0][c2][i] = lds_load16(xaddr(0, c2, i));
-#pragma unroll
-                for (int pr = 0; pr < NPAIR; ++pr) {
-                    acc[2 * pr] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-                    acc[2 * pr + 1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-                    for (int i = 0; i < R; ++i)
-#pragma unroll
-                        for (int c2 = 0; c2 < 2; ++c2) {
-                            u32x4 &cur = xf[pr & 1][c2][i];
-                            if (pr + 1 < NPAIR) {
-                                xf[(pr + 1) & 1][c2][i] = lds_load16(xaddr(pr + 1, c2, i));
-                                asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(cur) : "n"(NLD) : "memory");
-                            } else {  // last pair: only this pair's later reads are newer
-                                asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(cur) : "n"(NLD - 1 - (2 * i + c2)) : "memory");
-                            }
-                            mma16(acc[2 * pr + c2], tz[i][0], __builtin_bit_cast(frag8<T>, cur));
-                            __builtin_amdgcn_sched_barrier(0);
-                        }
-                }
-                const int prow = p0 + rb * 16 + ln;
-#pragma unroll
-                for (int cb = 0; cb < M_TN / 16; cb += 2) {
-#pragma unroll
                     for (int c2 = 0; c2 < 2; ++c2) {
-                        const int q = q0 + (cb + c2) * 16 + kg * 4;
-                        uint32_t lo = pack2<T>(acc[cb + c2][0], acc[cb + c2][1]), hi = pack2<T>(acc[cb + c2][2], acc[cb + c2][3]);
-                        if (!interior && causal && q + 3 > prow) {
-                            if (q > prow) lo &= 0xffff0000u;
-                            if (q + 1 > prow) lo &= 0x0000ffffu;
-                            if (q + 2 > prow) hi &= 0xffff0000u;
-                            if (q + 3 > prow) hi &= 0x0000ffffu;
+                        u32x4 &cur = xf[pr & 1][c2][i];
+                        if (pr + 1 < NPAIR) {
+                            xf[(pr + 1) & 1][c2][i] = lds_load16_at(xa, xoff(pr + 1, c2, i));
+                            asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(cur) : "n"(NLD) : "memory");
+                        } else {  // last pair: only this pair's later reads are newer
+                            asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(cur) : "n"(NLD - 1 - (2 * i + c2)) : "memory");
                         }
-                        lds_store8(tile_lds + (unsigned)((rb * 16 + ln) * LD + (cb + c2) * 16 + kg * 4) * sizeof(T), lo, hi);
+                        mma16(acc[2 * pr + c2], tz[i], __builtin_bit_cast(frag8<T>, cur));
+                        __builtin_amdgcn_sched_barrier(0);
                     }
+            }
+            // results into the staged rows res0.. (read by this wavefront only, and no longer needed by it)
+            const int prow = p0 + rb0 + ln;
+            const unsigned ra = tile_lds + (unsigned)((res0 + ln) * LD + kg * 4) * sizeof(T);
+#pragma unroll
+            for (int cb = 0; cb < M_TN / 16; ++cb) {
+                const int q = q0 + cb * 16 + kg * 4;
+                uint32_t lo = pack2<T>(acc[cb][0], acc[cb][1]), hi = pack2<T>(acc[cb][2], acc[cb][3]);
+                if (!interior && causal && q + 3 > prow) {
+                    if (q > prow) lo &= 0xffff0000u;
+                    if (q + 1 > prow) lo &= 0x0000ffffu;
+                    if (q + 2 > prow) hi &= 0xffff0000u;
+                    if (q + 3 > prow) hi &= 0x0000ffffu;
                 }
+                lds_store8_at(ra, (int)(cb * 16 * sizeof(T)), lo, hi);
             }
         }
-        // ---- coalesced stores: 16 lanes cover one 256-byte output row (the LDS writes above precede these reads in
-        // the wavefront's LDS queue) ----
+        // ---- coalesced stores of this wavefront's 16 rows: 16 lanes cover one 256-byte output row (the LDS writes
+        // above precede these reads in the wavefront's LDS queue) ----
         {
-            T *ybase = yp + (int64_t)p0 * W + q0;
+            // (uniform row base + one 32-bit per-lane byte offset: no 64-bit address arithmetic per store)
+            char *ybase = reinterpret_cast<char *>(yp + (int64_t)(p0 + rb0) * W + q0);
             const int lane_o = opaque(lane);  // (row offsets formed here, not kept in registers across the loop)
             const int r_l = lane_o >> 4, cv = (lane_o & 15) * VEC;
-            constexpr int OUT_IT = M_TM * (M_TN / VEC) / M_WT;
+            const unsigned yoff = (unsigned)(r_l * W + cv) * (unsigned)sizeof(T);
+            const int64_t ystep = (int64_t)4 * W * (int64_t)sizeof(T);
+            constexpr int OUT_IT = 16 * (M_TN / VEC) / 64;
+            static_assert(OUT_IT == 4, "four row groups per wavefront");
+            u32x4 v[4];
+            const unsigned va = tile_lds + (unsigned)((res0 + r_l) * LD + cv) * sizeof(T);
 #pragma unroll
-            for (int i0 = 0; i0 < OUT_IT; i0 += 4) {  // four rows' worth in flight per wait
-                u32x4 v[4];
+            for (int k = 0; k < 4; ++k) v[k] = lds_load16_at(va, (int)(k * 4 * LD * sizeof(T)));
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : : "memory");
+            if (interior) {  // unconditional: exactly OUT_IT vector-memory instructions
 #pragma unroll
-                for (int k = 0; k < 4; ++k) v[k] = lds_load16(tile_lds + (unsigned)(((i0 + k) * 4 + r_l) * LD + cv) * sizeof(T));
-                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : : "memory");
-                if (interior) {  // unconditional: exactly OUT_IT vector-memory instructions
+                for (int k = 0; k < 4; ++k) MTA_CONV_STORE(reinterpret_cast<u32x4 *>(ybase + k * ystep + yoff), v[k]);
+            } else {
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) MTA_CONV_STORE(reinterpret_cast<u32x4 *>(ybase + ((i0 + k) * 4 + r_l) * W + cv), v[k]);
-                } else {
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        const int r = (i0 + k) * 4 + r_l;
-                        if (p0 + r < H && q0 + cv < W) MTA_CONV_STORE(reinterpret_cast<u32x4 *>(ybase + r * W + cv), v[k]);
-                    }
+                for (int k = 0; k < 4; ++k) {
+                    const int r = k * 4 + r_l;
+                    if (p0 + rb0 + r < H && q0 + cv < W) MTA_CONV_STORE(reinterpret_cast<u32x4 *>(ybase + k * ystep + yoff), v[k]);
                 }
             }
-            static_assert(OUT_IT % 4 == 0, "stores in groups of four");
             younger = interior ? OUT_IT : -1;
         }
         if (mirror && ctn < ctm / M_SPB) {  // this strip's share of the 128x128 block's image above the diagonal
             if (fill_full) {
-                zero_fill_strip<T, true>(yp, H, W, q0 + (ctm % M_SPB) * M_TM, (ctm / M_SPB) * M_TN, lane);
+                zero_fill_strip<T, true>(yp, H, W, q0 + (ctm % M_SPB) * M_TM, (ctm / M_SPB) * M_TN, tid);
                 if (younger > 0) younger += M_TM * (M_TN / VEC) / M_WT;
             } else {
-                zero_fill_strip<T>(yp, H, W, q0 + (ctm % M_SPB) * M_TM, (ctm / M_SPB) * M_TN, lane);
+                zero_fill_strip<T>(yp, H, W, q0 + (ctm % M_SPB) * M_TM, (ctm / M_SPB) * M_TN, tid);
                 younger = -1;
             }
         }
@@ -752,7 +689,7 @@ int launch_mfma(const void *x, const void *w, void *y, int64_t N, int64_t C, int
     const int ipp = (int)ipp64;
     const int64_t total = N * C * ipp64;
     const int64_t per_xcd = (total + 7) / 8;
-    int nw = device_cu_count() * MTA_CONV_WG_PER_CU / 8;  // persistent workgroups per XCD
+    int nw = device_cu_count() * M_WG_PER_CU / 8;  // persistent workgroups per XCD
     if (nw < 1) nw = 1;
     if (per_xcd < nw) nw = (int)per_xcd;
     dim3 grid((unsigned)(nw * 8));

@@ -97,6 +97,55 @@ def test_conv_delta_is_shift(ops):
         assert torch.equal(got, O.depthwise_conv(x, w, True))
 
 
+MFMA_KERNEL_SIZES = [(3, 3), (3, 5), (5, 5), (5, 7), (6, 11), (7, 7), (7, 9)]
+
+
+@pytest.mark.parametrize("rs", MFMA_KERNEL_SIZES)
+def test_conv_channel_changes_on_every_strip(ops, rs):
+    """Every kernel size with a matrix-core instance, forward and input gradient, on planes that hold a single strip
+    (32 rows x 128 keys) each: consecutive work items of a workgroup then always belong to different channels, so the
+    kernel rows fetched one strip ahead are consumed on every iteration.  Channels get very different weights so that
+    a kernel row applied to the wrong strip cannot pass."""
+    r, s = rs
+    print(f"conv channel change rs={rs}", flush=True)
+    dtype = torch.bfloat16
+    n, c, h, wd = 3, 24, 32, 128
+    x = _randn((n, c, h, wd), 31, dtype)
+    w = (_randn((c, r, s), 32, torch.float32, 0.2) * (1.0 + torch.arange(c)[:, None, None])).to(dtype)
+    for causal in (False, True):
+        want = O.depthwise_conv(x.float(), w.float(), causal).to(dtype)
+        got = ops.conv2d_causal(x.cuda(), w.cuda(), causal).cpu()
+        torch.testing.assert_close(got.float(), want.float(), rtol=2.0 ** -7, atol=2e-2 * c)
+        dy = _randn((n, c, h, wd), 33, dtype)
+        want_dx, _ = O.depthwise_conv_grads(x.float(), w.float(), causal, dy.float())
+        got_dx = ops.conv2d_bwd_input(dy.cuda(), w.cuda(), causal).cpu()
+        torch.testing.assert_close(got_dx.float(), want_dx.to(dtype).float(), rtol=2.0 ** -7, atol=2e-2 * c)
+
+
+def test_conv_non_finite_input_stays_local(ops):
+    """The matrix-core kernel multiplies a 32-key window by a zero-padded tap matrix, so one inf at an attended
+    position turns every output of its 16-key block (and of the neighbouring block whose window holds it), in the R
+    rows below it, into NaN -- a wider footprint than the R x S taps of the fp32-FMA kernel.  Outputs further away
+    must be what they are without the inf, and the true footprint must be non-finite in both kernels."""
+    print("conv inf input", flush=True)
+    r, s = 6, 11
+    w = _randn((1, r, s), 41, torch.float32, 0.2).abs() + 0.05      # no zero taps: the true footprint is all non-finite
+    x = torch.tril(_randn((1, 1, 256, 256), 42, torch.float32))
+    clean16 = ops.conv2d_causal(x.bfloat16().cuda(), w.bfloat16().cuda(), True).cpu().float()
+    clean32 = ops.conv2d_causal(x.cuda(), w.cuda(), True).cpu()
+    p0, q0 = 100, 40
+    x[0, 0, p0, q0] = float("inf")
+    got16 = ops.conv2d_causal(x.bfloat16().cuda(), w.bfloat16().cuda(), True).cpu().float()   # matrix cores
+    got32 = ops.conv2d_causal(x.cuda(), w.cuda(), True).cpu()                                 # fp32 FMAs
+    foot = torch.zeros(256, 256, dtype=torch.bool)
+    foot[p0:p0 + r, q0 - (s - 1) // 2:q0 + (s - 1) // 2 + 1] = True
+    assert not torch.isfinite(got32[0, 0][foot]).any() and not torch.isfinite(got16[0, 0][foot]).any()
+    assert torch.equal(got32[0, 0][~foot], clean32[0, 0][~foot])
+    wide = torch.zeros(256, 256, dtype=torch.bool)
+    wide[p0:p0 + r, q0 - 32:q0 + 32] = True
+    assert torch.equal(got16[0, 0][~wide], clean16[0, 0][~wide])
+
+
 HM_CASES = [
     # N, C, P, Q, group (None = dense)
     (1, 4, 9, 9, None), (2, 4, 64, 64, 2), (1, 8, 40, 40, 4), (1, 6, 33, 33, None), (1, 6, 24, 24, 3),
