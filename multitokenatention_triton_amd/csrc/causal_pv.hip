@@ -4,7 +4,7 @@
 // uninitialised memory), which halves the traffic of the plain batched GEMM this replaces.
 // HBM-bound: the P triangle is streamed once, V blocks are re-read from L2.
 //
-// MTA_PV_WAVES wavefronts own a block of 32 query rows each; a wavefront owns two blocks of 16 rows.  O^T += V^T P^T on
+// P_WAVES wavefronts own a block of 32 query rows each; a wavefront owns two blocks of 16 rows.  O^T += V^T P^T on
 // 16x16x32 MFMAs: lane (r = lane%16, g = lane/16) owns query row r of a block and supplies P^T
 // fragments straight from global memory (16 contiguous bytes = 8 keys of its row, loaded one key
 // block ahead), V blocks of 64 keys are copied global -> LDS asynchronously (double buffered,
@@ -22,26 +22,16 @@ typedef const __attribute__((address_space(1))) void glb_void_t;
 typedef short v4s_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
 
-#ifndef MTA_PV_WAVES
-#define MTA_PV_WAVES 4
-#endif
-constexpr int P_NT = 64 * MTA_PV_WAVES;
-constexpr int P_BQ = 32 * MTA_PV_WAVES;  // query rows per block: 32 per wavefront
-#ifndef MTA_PV_OCC
-#define MTA_PV_OCC 2
-#endif
-#ifndef MTA_PV_NT_LOAD
-#define MTA_PV_NT_LOAD 1  // P is streamed: every element is read once
-#endif
-#ifndef MTA_PV_BK
-#define MTA_PV_BK 64
-#endif
-constexpr int P_BK = MTA_PV_BK;  // keys per iteration: each lane reads P_BK/4 contiguous bytes of its row per
+constexpr int P_WAVES = 4;          // wavefronts per workgroup (8, i.e. half the V re-reads, measured no faster)
+constexpr int P_NT = 64 * P_WAVES;
+constexpr int P_BQ = 32 * P_WAVES;  // query rows per block: 32 per wavefront
+constexpr int P_OCC = 2;            // workgroups per CU the kernel is compiled for
+constexpr int P_BK = 64;  // keys per iteration (128 measured no faster): each lane reads P_BK/4 contiguous bytes of its row per
                                  // iteration, back to back, so that DRAM pages are used in long runs
 constexpr int P_KS = P_BK / 32;  // 32-key contraction steps per iteration
 
 template <typename T, int D>
-__global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__restrict__ P, const T *__restrict__ V,
+__global__ __launch_bounds__(P_NT, P_OCC) void causal_pv_kernel(const T *__restrict__ P, const T *__restrict__ V,
                                                            T *__restrict__ O, int S, int causal, int nqb, int64_t total_wg,
                                                            int64_t per_xcd)
 {
@@ -106,13 +96,10 @@ __global__ __launch_bounds__(P_NT, MTA_PV_OCC) void causal_pv_kernel(const T *__
             for (int ks = 0; ks < P_KS; ++ks) {
                 const int key = j * P_BK + ks * 32 + kg * 8;
                 const bool ok = key < S && !(causal && key > prow[rb]);
-#if MTA_PV_NT_LOAD
+                // (non-temporal: P is streamed, every element is read once)
                 typedef unsigned int u4 __attribute__((ext_vector_type(4)));
                 pf[rb][ks] = __builtin_bit_cast(frag8<T>, __builtin_nontemporal_load(reinterpret_cast<const u4 *>(
                                                               prow_ptr[rb] + (ok ? j * P_BK + ks * 32 : -kg * 8))));
-#else
-                pf[rb][ks] = *reinterpret_cast<const frag8<T> *>(prow_ptr[rb] + (ok ? j * P_BK + ks * 32 : -kg * 8));
-#endif
             }
     };
 

@@ -24,6 +24,7 @@
 #include <algorithm>
 
 #include <type_traits>
+#include <utility>
 
 #include "common.hpp"
 #include "mfma.hpp"
@@ -298,34 +299,55 @@ typedef __attribute__((address_space(3))) void lds_void_t;
 typedef const __attribute__((address_space(1))) void glb_void_t;
 typedef short v4s_t __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
 
 // The workgroup has NW wavefronts and owns 32*NW score rows: 8 for the attention kernel (one workgroup per CU,
-// K and V blocks shared by 256 rows), 4 for the scores-only kernel (two workgroups per CU, which overlap each
+// K and V blocks shared by 256 rows), 4 for the scores-only kernel (three workgroups per CU, which overlap each
 // other's barriers and memory latency).
-// The kernels read the LDS operands of the next group of matrix products before they issue the current group.  The
-// instruction scheduler largely undoes that (it moves reads down towards their use, which saves registers).  Pinning
-// the source order (matrix products and LDS accesses may not cross the marked points) was measured and is slower -
-// scores-only kernel 0.320 -> 0.340 ms, attention kernel 1.60 -> 1.72 ms at the benchmark shapes, with 12-14 spilled
-// registers - so it stays off: these kernels are not bound by the LDS latency in front of each product.
-#ifndef MTA_FUSED_PIN
-#define MTA_FUSED_PIN 0
-#endif
-#if MTA_FUSED_PIN
-#define MTA_PIN_ORDER() __builtin_amdgcn_sched_barrier(0x6)
-#else
-#define MTA_PIN_ORDER() ((void)0)
-#endif
+// The attention kernel reads the LDS operands of the next group of matrix products before it issues the current group;
+// the instruction scheduler largely undoes that (it moves reads down towards their use, which saves registers).  Pinning
+// the source order there was measured and is slower (1.60 -> 1.72 ms at the benchmark shape, 12-14 spilled registers).
+// The scores-only kernel pins its conv phase by hand instead (reads issued from assembly, see below).
 constexpr int F_BK = 64;   // keys per iteration
-#ifndef MTA_QK_OCC
-#define MTA_QK_OCC 3       // wavefronts per SIMD the scores-only kernel is compiled for (three workgroups per CU)
-#endif
-#ifndef MTA_QK_CHUNK
-#define MTA_QK_CHUNK 32    // key blocks per work item of the scores-only kernel
-#endif
-constexpr int F_SLD = 80;  // score-tile row stride (elements): exactly the retained columns + one key block (measured
-                           // fastest among 80..120)
+constexpr int QK_OCC = 3;     // wavefronts per SIMD the scores-only kernel is compiled for (three workgroups per CU)
+constexpr int QK_CHUNK = 32;  // key blocks per work item of the scores-only kernel
+constexpr int F_SLD = 80;  // score-tile row stride (elements): exactly the retained columns + one key block.  A wider
+                           // row costs the scores-only kernel its third workgroup per CU, and with this one a fragment
+                           // read (16 consecutive rows x 64 bytes) is free of bank conflicts as it is: the LDS serves
+                           // lanes 0-7 together with lanes 24-31 (8-15 with 16-23, ...), and rows 160 bytes apart put
+                           // those on the even and the odd 16-byte positions (measured; 144 or 176 bytes halve the rate)
 
+// LDS accesses issued from assembly: the compiler neither reorders them nor waits for the asynchronous copy in flight
+// ahead of them (it cannot tell a read of the score tile from the copy's target), and the wait points are placed by
+// hand.  LDS operations of a wavefront complete in order, so "at most n operations outstanding" names the oldest ones
+// as complete; a loaded value is tied to the wait that covers it through an in/out operand.
+__device__ __forceinline__ unsigned lds_addr(const void *p) { return (unsigned)(uintptr_t)(lds_void_t *)p; }
+__device__ __forceinline__ u32x4_t lds_read16_at(unsigned addr, int off)
+{
+    u32x4_t v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(off) : "memory");
+    return v;
+}
+__device__ __forceinline__ void lds_write8_at(unsigned addr, int off, uint32_t lo, uint32_t hi)
+{
+    const u32x2_t v = {lo, hi};
+    asm volatile("ds_write_b64 %0, %1 offset:%2" : : "v"(addr), "v"(v), "n"(off) : "memory");
+}
+template <int N> __device__ __forceinline__ void lds_wait_upto(u32x4_t &v)
+{
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(N) : "memory");
+}
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), in order
+template <int... I, typename F> __device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F &&f)
+{
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F> __device__ __forceinline__ void static_for(F &&f)
+{
+    static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
 // Returns its argument, opaquely: what is derived from the result cannot be hoisted out of the block that computes it.
 __device__ __forceinline__ int opaque_lane(int v)
 {
@@ -356,13 +378,13 @@ template <int R, int SK, int NW> struct fused_geom {
 
 // SCORES_ONLY: stop after the conv and write  conv(mask0(scale * Q K^T))  as an (S,S) plane per (batch, head)
 // (`O` is then the score tensor, V is unused).  Only q <= p is written when causal, plus +0 above the
-// diagonal when `fill_upper` is set.  The tile is staged through LDS so that stores are 128-byte row segments.
+// diagonal when `fill_upper` is set.
 template <typename T, int D, int R, int SK, bool SCORES_ONLY, int NW>
-__global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_attn_fwd_mfma(const T *__restrict__ Q, const T *__restrict__ K,
+__global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_fwd_mfma(const T *__restrict__ Q, const T *__restrict__ K,
                                                              const T *__restrict__ V, const T *__restrict__ Wt,
                                                              T *__restrict__ O, float *__restrict__ Lse, int S, int causal,
                                                              float scale, int H, int nqb, int fill_upper, int64_t total_wg,
-                                                             int64_t per_xcd, int jc_len, int items_per_bh)
+                                                             int64_t per_xcd, int jc_len, int items_per_bh, int hpx)
 {
     using G = fused_geom<R, SK, NW>;
     constexpr int F_NT = 64 * NW, F_SR = 32 * NW;
@@ -381,8 +403,6 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
     __shared__ __align__(16) T Kt1[TILE];
     __shared__ __align__(16) T Vt0[SCORES_ONLY ? 8 : TILE];
     __shared__ __align__(16) T Vt1[SCORES_ONLY ? 8 : TILE];
-    constexpr bool STG_IN_K = SCORES_ONLY && F_SR * F_BK <= TILE;  // output staging fits a K buffer (D = 128)
-    __shared__ __align__(16) T stg[(SCORES_ONLY && !STG_IN_K) ? F_SR * F_BK : 8];
     __shared__ __align__(16) T Sc[F_SR * F_SLD];                          // score tile
     // zero-padded kernel rows, only needed until the Toeplitz fragments are built: they borrow the second K buffer,
     // which receives its first copy after that (LDS is granted in 1280-byte units; the array's own 648 bytes were
@@ -396,8 +416,15 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
     // XCD-aware order: workgroup ids are dealt round-robin to the 8 XCDs, so XCD x takes the x-th eighth of the
     // (batch*head, query block) list: the workgroups sharing one head's K and V run on one L2.  Within a head
     // the longest (last) query blocks come first.
-    const int64_t lid = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    // When the (batch, head) pairs divide evenly over the XCDs (hpx > 0 of them each), the items of an XCD's heads are
+    // taken rank by rank - the longest item of each head, then the second longest of each, ... - so that the long items
+    // all start early and the short ones fill the end of the grid (workgroups start in index order as slots free up).
+    int64_t lid = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (lid >= total_wg) return;
+    if (hpx > 0) {
+        const int64_t pos = blockIdx.x >> 3;
+        lid = ((int64_t)(blockIdx.x & 7) * hpx + pos % hpx) * items_per_bh + pos / hpx;
+    }
     // Work item = (batch*head, query block, chunk of jc_len key blocks).  The scores-only kernel splits the key
     // range of a query block (its output columns are independent; a chunk starts one key block early to rebuild
     // the retained halo columns), so that items are short and equal and the grid runs in several even rounds;
@@ -551,17 +578,17 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
                     dst[ks] = *reinterpret_cast<const frag8<T> *>(Kb + krow * D + (((ks * 4 + kg) ^ (krow & (CPR - 1))) * 8));
             };
             load_kf(0, kf[0]);
+            uint32_t held[2][2];
+            static_assert(NCB % 2 == 0, "score blocks are written in pairs");
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb) {
                 if (cb + 1 < NCB) load_kf(cb + 1, kf[(cb + 1) & 1]);
-                MTA_PIN_ORDER();
                 f32x4 sacc[2] = {f32x4{0.0f, 0.0f, 0.0f, 0.0f}, f32x4{0.0f, 0.0f, 0.0f, 0.0f}};
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     mma16(sacc[0], kf[cb & 1][ks], qf[0][ks]);
                     mma16(sacc[1], kf[cb & 1][ks], qf[1][ks]);
                 }
-                MTA_PIN_ORDER();
                 // key block wholly inside the sequence and on or below the diagonal for all 32 rows: no masks
                 const bool s_plain = PLAIN || (cbase + cb * 16 >= 0 && cbase + cb * 16 + 16 <= S && (!causal || cbase + cb * 16 + 15 <= pmin));
 #pragma unroll
@@ -582,7 +609,19 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
                         if (col + 2 < 0 || col + 2 > lim) hi &= 0xffff0000u;
                         if (col + 3 < 0 || col + 3 > lim) hi &= 0x0000ffffu;
                     }
-                    *reinterpret_cast<uint2 *>(Sc + trow[rb] * F_SLD + G::HC + cb * 16 + kg * 4) = make_uint2(lo, hi);
+                    // Two 16-key blocks go to the tile together.  A lane holds keys 4kg..4kg+3 of each; after the
+                    // exchange between neighbouring lane groups (even groups give their second block's part and take
+                    // the neighbour's first block's part) it holds 8 consecutive keys of one block: one 16-byte write
+                    // per lane and block pair instead of two 8-byte ones, which conflicted four ways in the banks.
+                    if ((cb & 1) == 0) {
+                        held[rb][0] = lo;
+                        held[rb][1] = hi;
+                    } else {
+                        const u32x2_t s0 = __builtin_amdgcn_permlane16_swap(held[rb][0], lo, false, false);
+                        const u32x2_t s1 = __builtin_amdgcn_permlane16_swap(held[rb][1], hi, false, false);
+                        *reinterpret_cast<u32x4_t *>(Sc + trow[rb] * F_SLD + G::HC + (cb - 1 + (kg & 1)) * 16 + (kg >> 1) * 8) =
+                            u32x4_t{s0[0], s1[0], s0[1], s1[1]};
+                    }
                 }
             }
         }
@@ -603,52 +642,81 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
         };
 
         if constexpr (SCORES_ONLY) {
-            // ---- conv (Toeplitz MFMAs over the score tile) -> this wavefront's 32 x 64 staging rows -> global ----
-            // The score fragments of block blk+1 are read from LDS while the matrix cores work on block blk.
-            // Staging rows live in the K buffer of this key block when they fit: nobody reads it any more (the
-            // barrier above follows the last K fragment read).  Row stride = one key block, 16-byte chunks
-            // XOR-swizzled by row.
-            constexpr int OLD = F_BK;
-            T *stage = (STG_IN_K ? const_cast<T *>(Kb) : stg) + wave * 32 * OLD;
-            frag8<T> xf[2][R];
-            load_xf(0, xf[0]);
-#pragma unroll
-            for (int blk = 0; blk < 2 * NCB; ++blk) {
-                const int rb = blk / NCB, cb = blk % NCB;
-                if (blk + 1 < 2 * NCB) load_xf(blk + 1, xf[(blk + 1) & 1]);
-                MTA_PIN_ORDER();
-                f32x4 cacc = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-                for (int i = 0; i < R; ++i) mma16(cacc, tz[i], xf[blk & 1][i]);
-                MTA_PIN_ORDER();
-                uint32_t lo = pack2<T>(cacc[0], cacc[1]), hi = pack2<T>(cacc[2], cacc[3]);
+            // ---- conv (Toeplitz MFMAs over the score tile) -> global ----
+            // One product needs one fresh 1 KB score fragment from LDS, and a wavefront that waits for each fragment
+            // where it is used spends four times the products' own time here.  The reads are therefore issued NLD
+            // products ahead, from assembly (see lds_read16_at), into a ring of registers; every product is preceded by
+            // a wait that leaves exactly the younger operations outstanding.  The result of an output block is packed
+            // LAG products into the next block, when it is long complete.
+            constexpr int NB = 2 * NCB, NREAD = NB * R;
+            constexpr int NLD = 8;  // score fragments in flight (8 and 12 measure the same; 15 spills)
+            constexpr int NSLOT = NLD + 1;
+            constexpr int LAG = 2;
+            static_assert(NREAD > NLD && R >= LAG && NLD <= 15, "pipeline deeper than the work or than the counter");
+            // Rows of the conv.  The first wavefront's rows are taken R-1 further down than the rows it computed scores
+            // for: its windows then start at tile row 0 instead of above the tile, every address below is the same
+            // affine function of (row block, kernel row), and what it leaves out are halo rows nobody stores.  Its last
+            // R-1 rows belong to the second wavefront too and are not stored from here.
+            const int cshift = wave == 0 ? R - 1 : 0;
+            const unsigned xa = lds_addr(Sc) + (unsigned)(((trow[0] + cshift - (R - 1)) * F_SLD + kg * 8) * (int)sizeof(T));
+            u32x4_t ring[NSLOT];
+            f32x4 cacc[2];
+            uint32_t held[2];
+            auto issue = [&](auto ic) __attribute__((always_inline)) {
+                constexpr int n = decltype(ic)::value;
+                constexpr int blk = n / R, i = n % R;
+                ring[n % NSLOT] = lds_read16_at(xa, (((blk / NCB) * 16 + i) * F_SLD + (blk % NCB) * 16) * (int)sizeof(T));
+            };
+            // Pack and mask output block b.  Blocks leave in pairs, like the scores above: after the exchange a lane
+            // holds 8 consecutive keys of one of the two blocks and stores them itself, 16 rows x 64 bytes per
+            // instruction; no staging through LDS.
+            // (non-temporal: the scores are written once and next read by another kernel; as ordinary stores they
+            // would push this head's K blocks, which every workgroup of the head re-reads, out of the L2)
+            auto finish = [&](auto bc) __attribute__((always_inline)) {
+                constexpr int b = decltype(bc)::value;
+                constexpr int rb = b / NCB, cb = b % NCB;
+                const f32x4 a = cacc[b & 1];
+                uint32_t lo = pack2<T>(a[0], a[1]), hi = pack2<T>(a[2], a[3]);
+                const int tr_ = trow[rb] + cshift, p_ = prow[rb] + cshift;
                 if (!PLAIN && causal && j * F_BK + cb * 16 + 15 > pmin) {  // block touches the diagonal for some row
                     const int col = j * F_BK + cb * 16 + kg * 4;
-                    if (col > prow[rb]) lo &= 0xffff0000u;
-                    if (col + 1 > prow[rb]) lo &= 0x0000ffffu;
-                    if (col + 2 > prow[rb]) hi &= 0xffff0000u;
-                    if (col + 3 > prow[rb]) hi &= 0x0000ffffu;
+                    if (col > p_) lo &= 0xffff0000u;
+                    if (col + 1 > p_) lo &= 0x0000ffffu;
+                    if (col + 2 > p_) hi &= 0xffff0000u;
+                    if (col + 3 > p_) hi &= 0x0000ffffu;
                 }
-                {
-                    const int r_ = rb * 16 + ln, ch_ = (cb * 2 + (kg >> 1)) ^ (r_ & 7);
-                    *reinterpret_cast<uint2 *>(stage + r_ * OLD + ch_ * 8 + (kg & 1) * 4) = make_uint2(lo, hi);
+                if constexpr ((cb & 1) == 0) {
+                    held[0] = lo;
+                    held[1] = hi;
+                } else {
+                    const u32x2_t s0 = __builtin_amdgcn_permlane16_swap(held[0], lo, false, false);
+                    const u32x2_t s1 = __builtin_amdgcn_permlane16_swap(held[1], hi, false, false);
+                    // (column from a laundered lane index: the address is then formed here, 64-bit adds and all, instead
+                    // of being kept in registers across the key-block loop - the kernel is at its register limit)
+                    const int kg_o = opaque_lane(kg);
+                    const int col = j * F_BK + (cb - 1 + (kg_o & 1)) * 16 + (kg_o >> 1) * 8;
+                    if (tr_ >= G::HR && tr_ < wave * 32 + 32 && p_ < S && (PLAIN || (col < S && (!causal || fill_upper || col <= p_))))
+                        __builtin_nontemporal_store(u32x4_t{s0[0], s1[0], s0[1], s1[1]},
+                                                    reinterpret_cast<u32x4_t *>(Op + (int64_t)p_ * S + col));
                 }
-            }
-            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's staging rows are written
-            // (row and column from a laundered lane index: the four row addresses are then formed here, 64-bit adds and
-            // all, instead of being kept in registers across the key-block loop - the kernel is at its register limit,
-            // and a spilled value reloaded in this loop makes the compiler wait for every outstanding store)
-            const int lane_o = opaque_lane(lane);
-#pragma unroll
-            for (int it = 0; it < 4; ++it) {
-                const int r = it * 8 + (lane_o >> 3), cv = (lane_o & 7) * 8;
-                const int tr_ = wave * 32 + r, p_ = q0 - G::HR + tr_, col = j * F_BK + cv;
-                const pack16<T> v = *reinterpret_cast<const pack16<T> *>(stage + r * OLD + (((lane_o & 7) ^ (r & 7)) * 8));
-                // (non-temporal: the scores are written once and next read by another kernel; as ordinary stores they
-                // would push this head's K blocks, which every workgroup of the head re-reads, out of the L2)
-                if (tr_ >= G::HR && p_ < S && (PLAIN || (col < S && (!causal || fill_upper || col <= p_))))
-                    __builtin_nontemporal_store(__builtin_bit_cast(u32x4_t, v), reinterpret_cast<u32x4_t *>(Op + (int64_t)p_ * S + col));
-            }
+            };
+            static_for<NLD>(issue);
+            static_for<NREAD>([&](auto ic) __attribute__((always_inline)) {
+                constexpr int n = decltype(ic)::value;
+                constexpr int blk = n / R, i = n % R;
+                if constexpr (n + NLD < NREAD) issue(std::integral_constant<int, n + NLD>{});
+                // LDS operations younger than read n: exactly the reads issued after it
+                constexpr int younger = (n + NLD < NREAD ? n + NLD : NREAD - 1) - n;
+                lds_wait_upto<younger>(ring[n % NSLOT]);
+                if constexpr (i == 0) cacc[blk & 1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                mma16(cacc[blk & 1], tz[i], __builtin_bit_cast(frag8<T>, ring[n % NSLOT]));
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (blk >= 1 && i == LAG - 1) {
+                    finish(std::integral_constant<int, blk - 1>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            });
+            finish(std::integral_constant<int, NB - 1>{});
             return;
         }
 
@@ -665,12 +733,10 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
                 for (int cb = 0; cb < NCB; ++cb) {
                     const int blk = rb * NCB + cb;
                     if (blk + 1 < 2 * NCB) load_xf(blk + 1, xf[(blk + 1) & 1]);
-                    MTA_PIN_ORDER();
-                    f32x4 cacc = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                        f32x4 cacc = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                     for (int i = 0; i < R; ++i) mma16(cacc, tz[i], xf[blk & 1][i]);
-                    MTA_PIN_ORDER();
-                    // conv output and scaled logits are rounded to the I/O dtype, as the unfused pipeline stores them
+                        // conv output and scaled logits are rounded to the I/O dtype, as the unfused pipeline stores them
                     float a[4];
                     unpack2<T>(pack2<T>(cacc[0], cacc[1]), a[0], a[1]);
                     unpack2<T>(pack2<T>(cacc[2], cacc[3]), a[2], a[3]);
@@ -735,10 +801,8 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? MTA_QK_OCC : 2) void conv_at
             for (int blk = 0; blk < 2 * DB; ++blk) {
                 const int ks = blk / DB, db = blk % DB;
                 if (blk + 1 < 2 * DB) load_vf(blk + 1, vf[(blk + 1) & 1]);
-                MTA_PIN_ORDER();
                 mma16(oacc[0][db], vf[blk & 1], pf[0][ks]);
                 mma16(oacc[1][db], vf[blk & 1], pf[1][ks]);
-                MTA_PIN_ORDER();
             }
         }
     };
@@ -803,8 +867,8 @@ int launch_mfma(const void *q, const void *k, const void *v, const void *w, void
     static_assert(G::fits, "conv window exceeds the 32-key MFMA contraction");
     const int nqb = (int)((S + G::BQ - 1) / G::BQ);
     auto kern = conv_attn_fwd_mfma<T, D, R, SK, SCORES_ONLY, NW>;
-    // key blocks per work item: all of them for the attention kernel; MTA_QK_CHUNK for the scores-only kernel
-    const int jc_len = SCORES_ONLY ? MTA_QK_CHUNK : (int)((S + F_BK - 1) / F_BK) + 1;
+    // key blocks per work item: all of them for the attention kernel; QK_CHUNK for the scores-only kernel
+    const int jc_len = SCORES_ONLY ? QK_CHUNK : (int)((S + F_BK - 1) / F_BK) + 1;
     int64_t items_per_bh = 0;
     for (int qb = 0; qb < nqb; ++qb) {
         const int64_t ql = std::min<int64_t>((int64_t)qb * G::BQ + G::BQ - 1, S - 1);
@@ -814,7 +878,8 @@ int launch_mfma(const void *q, const void *k, const void *v, const void *w, void
     if (per_xcd * 8 > 0x7fffffffLL || items_per_bh > 0x7fffffffLL) return MTA_ERR_SHAPE;
     dim3 grid((unsigned)(per_xcd * 8));
     hipLaunchKernelGGL(kern, grid, dim3(F_NT), 0, st, (const T *)q, (const T *)k, (const T *)v, (const T *)w, (T *)o,
-                       lse, (int)S, causal, scale, (int)H, nqb, fill_upper, total_wg, per_xcd, jc_len, (int)items_per_bh);
+                       lse, (int)S, causal, scale, (int)H, nqb, fill_upper, total_wg, per_xcd, jc_len, (int)items_per_bh,
+                       (B * H) % 8 == 0 ? (int)(B * H / 8) : 0);
     return launch_status();
 }
 

@@ -16,9 +16,7 @@
 
 #include "common.hpp"
 
-#ifndef MTA_RS_OCC
-#define MTA_RS_OCC 5  // wavefronts per SIMD the G*NV = 8 instances (e.g. 4 heads x 4096 keys) are compiled for
-#endif
+constexpr int RS_OCC = 5;  // wavefronts per SIMD the G*NV = 8 instances (e.g. 4 heads x 4096 keys) are compiled for
 
 namespace {
 using namespace mta;
@@ -110,7 +108,7 @@ template <int NT> __device__ __forceinline__ float block_sum(float v, float *red
 
 // Register-resident row: Q <= NT*VEC*NV.
 template <typename T, int G, int NV, int VEC, int NT>
-__global__ __launch_bounds__(NT, (NT == 256 && G * NV == 8) ? MTA_RS_OCC : 1) void mix_softmax_mix(const T *__restrict__ x, const void *__restrict__ w1,
+__global__ __launch_bounds__(NT, (NT == 256 && G * NV == 8) ? RS_OCC : 1) void mix_softmax_mix(const T *__restrict__ x, const void *__restrict__ w1,
                                                       const void *__restrict__ w2, T *__restrict__ y, int C,
                                                       int P, int Q, int causal, int w_dtype, int fill_upper)
 {
@@ -402,7 +400,7 @@ template <bool IS_MAX> __device__ __forceinline__ float wave_reduce(float v)
 #undef MTA_RS_DPP_STEP
 
 template <typename T, int G, int NV, bool HAS1, bool HAS2>
-__global__ __launch_bounds__(256, (G * NV == 8) ? MTA_RS_OCC : 1) void mix_softmax_mix_packed(
+__global__ __launch_bounds__(256, (G * NV == 8) ? RS_OCC : 1) void mix_softmax_mix_packed(
     const T *__restrict__ x, const T *__restrict__ w1, const T *__restrict__ w2, T *__restrict__ y, int C, int P, int Q,
     int causal, int fill_upper)
 {
