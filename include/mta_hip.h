@@ -95,6 +95,16 @@ int mta_headmix_softmax_fwd(const void *x, const void *w1, const void *w2, void 
                             int64_t C, int64_t P, int64_t Q, int group_size, int causal,
                             int fill_upper, int io_dtype, int w_dtype, void *stream);
 
+/* The same with an additive bias per (batch entry, key) on the mixed scores, ahead of the softmax:
+ *   s[o] = round(s[o] + key_bias[n, q])        key_bias is fp32, (N,Q), 0 = keep, -inf = key hidden, or any
+ *                                              finite value; NULL = none (identical to the entry point above).
+ * This is the `scores = scores + mask` of mta_attention_triton.py:77-78 for the masks the reference builds from a
+ * 2-D key mask (mta_attention_triton.py:118-122): causal rule plus one value per key, without the (B,H,S,S) mask
+ * tensor.  A row whose attended keys are all hidden comes out as NaN, as the softmax of a row of -inf does. */
+int mta_headmix_softmax_bias_fwd(const void *x, const void *w1, const void *w2, const void *key_bias, void *y,
+                                 int64_t N, int64_t C, int64_t P, int64_t Q, int group_size, int causal,
+                                 int fill_upper, int io_dtype, int w_dtype, void *stream);
+
 /* Fused conv-attention forward:
  *   O = softmax( mask( conv( mask0(Q K^T) ) ) * scale ) V        per (batch, head)
  * q,k,v,o are (B,H,S,D); w is (H,R,Sk).  mask0 zeroes col>row before the conv, mask

@@ -118,12 +118,17 @@ class MTAAttentionTriton(nn.Module):
 
     def forward(self, xq, xk, xv, mask, chunk_start_ids):
         assert chunk_start_ids is None, "MTAAttentionTriton does not support chunked attention"
+        wants_grad = torch.is_grad_enabled() and (xq.requires_grad or xk.requires_grad or xv.requires_grad
+                                                  or any(p.requires_grad for p in self.parameters()))
         if self.use_mask:
-            return self._forward_with_mask(xq, xk, xv, mask)
-        if torch.is_grad_enabled() and (xq.requires_grad or xk.requires_grad or xv.requires_grad
-                                        or any(p.requires_grad for p in self.parameters())):
+            return self._forward_with_mask(xq, xk, xv, mask, wants_grad)
+        if wants_grad:
             return self._forward_stagewise(xq, xk, xv)
+        return self._forward_fused(xq, xk, xv)
 
+    def _forward_fused(self, xq, xk, xv, key_bias=None):
+        """Inference route (module docstring).  ``key_bias``: fp32 (B,Sk), added to the mixed scores ahead of the
+        softmax -- the caller has zeroed the K and V rows of the keys it hides."""
         head_dim = xq.size(-1)
         # the reference multiplies by rsqrt(tensor(head_dim)), an fp32 scalar (mta_attention_triton.py:69-71)
         scale = float(torch.rsqrt(torch.tensor(float(head_dim))))
@@ -157,18 +162,18 @@ class MTAAttentionTriton(nn.Module):
         if one_pass:
             self._mark("mix_softmax_mix")
             scores = ops.headmix_softmax(scores, w1, w2, self.causal, group_size=_lcm(g_pre, g_post),
-                                         fill_upper=not own_pv)
+                                         fill_upper=not own_pv, key_bias=key_bias)
         else:
             if g_pre <= _FUSED_MAX_GROUP:
                 self._mark("mix_softmax")
-                scores = ops.headmix_softmax(scores, w1, None, self.causal, group_size=g_pre,
+                scores = ops.headmix_softmax(scores, w1, None, self.causal, group_size=g_pre, key_bias=key_bias,
                                              fill_upper=post_conv_identity and w2 is None and not own_pv)
             else:
                 self._mark("mix_pre")
                 fill = float("-inf") if self.causal else 0.0
                 scores = ops.headmix(scores, w_pre, self.causal, fill, group_size=g_pre)
                 self._mark("softmax")
-                scores = ops.headmix_softmax(scores, None, None, self.causal,
+                scores = ops.headmix_softmax(scores, None, None, self.causal, key_bias=key_bias,
                                              fill_upper=post_conv_identity and w2 is None and not own_pv)
             if not post_conv_identity:
                 self._mark("conv_post")
@@ -253,9 +258,28 @@ class MTAAttentionTriton(nn.Module):
         self._declared = WeightStructure()
         self.weight_structure = "dense"
 
-    def _forward_with_mask(self, xq, xk, xv, mask):
+    def _forward_with_mask(self, xq, xk, xv, mask, wants_grad=True):
         """use_mask=True: an explicit additive mask tensor drives the masking (mta_attention_triton.py:63-64,
-        77-83, 96-98); the kernels still apply their own causal rule when ``causal`` is set."""
+        77-83, 96-98); the kernels still apply their own causal rule when ``causal`` is set.
+
+        Two kinds of mask never become a (B,H,S,S) tensor here (inference, causal module): no mask at all, which the
+        reference turns into the causal rule the kernels apply anyway, and a 2-D key mask, which the reference turns
+        into "causal rule + one value per key" (mta_attention_triton.py:118-122).  A hidden key's scores enter the
+        pre-softmax conv as 0 -- which is what a zero K row produces -- its mixed score gets -inf ahead of the softmax
+        (the kernel's per-key bias), its probability is 0, and whatever the post-softmax conv writes into its column,
+        which the reference zeroes, meets a zero V row."""
+        if self.causal and not wants_grad and xq.size(-2) == xk.size(-2):
+            if not isinstance(mask, torch.Tensor):
+                return self._forward_fused(xq, xk, xv)
+            if mask.dim() == 2 and xq.size(0) == 1:
+                assert mask.size(0) == xq.size(0)
+                if mask.dtype == torch.bool:
+                    bias = torch.where(mask, 0.0, float("-inf")).to(torch.float32)
+                else:
+                    bias = mask.type(xq.dtype).to(torch.float32)   # the reference adds it in the I/O dtype
+                hidden = (bias == float("-inf"))[:, None, :, None]
+                return self._forward_fused(xq, xk.masked_fill(hidden, 0), xv.masked_fill(hidden, 0),
+                                           key_bias=bias.contiguous())
         mask = self._update_mask(mask=mask, bsz=xq.size(0), xq=xq, xk_size=xk.size(-2))
         scale = torch.rsqrt(torch.tensor(float(xq.size(-1)), device=xq.device))
         scores = torch.matmul(xq, xk.transpose(2, 3)) * scale

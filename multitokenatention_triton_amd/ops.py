@@ -165,10 +165,12 @@ def headmix_bwd_weight(x: torch.Tensor, dy: torch.Tensor, causal: bool = True) -
 
 def headmix_softmax(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optional[torch.Tensor], causal: bool = True,
                     group_size: Optional[int] = None, out: Optional[torch.Tensor] = None,
-                    fill_upper: bool = True) -> torch.Tensor:
+                    fill_upper: bool = True, key_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """mix(w1) -> causal row softmax -> mix(w2) in one pass; see mta_headmix_softmax_fwd.
 
-    ``fill_upper=False`` leaves everything above the diagonal unwritten (for consumers that never read it)."""
+    ``fill_upper=False`` leaves everything above the diagonal unwritten (for consumers that never read it).
+    ``key_bias``: fp32 (N,Q), added to the mixed scores ahead of the softmax (0 = keep, -inf = key hidden); see
+    mta_headmix_softmax_bias_fwd."""
     x = _device_tensor(x, "input")
     if x.dim() != 4:
         raise ValueError(f"expected input (N,C,P,Q), got {tuple(x.shape)}")
@@ -183,13 +185,18 @@ def headmix_softmax(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optional[to
     if len(present) == 2 and present[0].dtype != present[1].dtype:
         raise TypeError("w1 and w2 must share a dtype")
     wcode = _code(present[0], "weight") if present else _lib.MTA_F32
+    if key_bias is not None:
+        key_bias = _device_tensor(key_bias, "key_bias")
+        if key_bias.dtype != torch.float32 or tuple(key_bias.shape) != (n, q):
+            raise ValueError(f"key_bias must be fp32 of shape ({n},{q}), got {key_bias.dtype} {tuple(key_bias.shape)}")
     y = _out_like(x, out)
     with torch.cuda.device(x.device):
-        rc = _lib.load().mta_headmix_softmax_fwd(
+        rc = _lib.load().mta_headmix_softmax_bias_fwd(
             x.data_ptr(), ws[0].data_ptr() if ws[0] is not None else None,
-            ws[1].data_ptr() if ws[1] is not None else None, y.data_ptr(), n, c, p, q, int(group_size or 0),
-            int(bool(causal)), int(bool(fill_upper)), _code(x, "input"), wcode, _stream(x))
-    _lib.check(rc, "mta_headmix_softmax_fwd")
+            ws[1].data_ptr() if ws[1] is not None else None, key_bias.data_ptr() if key_bias is not None else None,
+            y.data_ptr(), n, c, p, q, int(group_size or 0), int(bool(causal)), int(bool(fill_upper)), _code(x, "input"),
+            wcode, _stream(x))
+    _lib.check(rc, "mta_headmix_softmax_bias_fwd")
     return y
 
 

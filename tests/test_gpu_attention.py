@@ -515,7 +515,34 @@ def test_mta_use_mask_tensor_masks(pkg, name, dtype):
     assert torch.isfinite(want.float()).all()
     for structure in ("dense", "infer"):
         mod = _mta_module(pkg, h, 3, 5, 3, 3, *params, dtype, use_mask=True, structure=structure)
+        stages = []
+        mod._stage_hook = stages.append
         got = mod(q.cuda(), k.cuda(), v.cuda(), mask.cuda(), None).cpu()
+        torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+        # a 2-D key mask runs through the kernels (per-key bias in the softmax stage, zeroed K and V rows); only a
+        # full mask tensor takes the elementwise route, which calls no stage hook
+        assert (("qk_conv" in stages or "conv_pre" in stages) and "pv" in stages) == name.startswith("key_mask")
+
+
+@pytest.mark.parametrize("post", ["identity", "random"])
+def test_mta_use_mask_key_mask_long_rows(pkg, post):
+    """Key mask at a size where the 16-bit kernels run several passes per row (one-pass mix/softmax/mix and the
+    stage-by-stage route), and use_mask=True without a mask tensor (the causal rule alone)."""
+    print(f"mta use_mask key mask S=2304 post={post}", flush=True)
+    dtype = torch.bfloat16
+    b, h, s, d = 1, 4, 2304, 64
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=95)
+    params = _config_like(h, 2, 6, 11, 0.05, dtype, post=post)
+    g = torch.Generator().manual_seed(5)
+    keep = torch.rand(1, s, generator=g) > 0.2
+    keep[0, 0] = True
+    for mask in (keep, None):
+        want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3], mask=mask)
+        mod = _mta_module(pkg, h, 6, 11, 3, 3, *params, dtype, use_mask=True, structure="infer")
+        stages = []
+        mod._stage_hook = stages.append
+        got = mod(q.cuda(), k.cuda(), v.cuda(), None if mask is None else mask.cuda(), None).cpu()
+        assert "qk_conv" in stages and "pv" in stages
         torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
 
 

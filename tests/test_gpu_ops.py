@@ -232,6 +232,40 @@ def test_mix_softmax_mix_parity(ops, case, causal, dt):
     torch.testing.assert_close(got.float(), want.float(), rtol=t["rtol"] * 2, atol=2e-3 if dtype != torch.float32 else 1e-6)
 
 
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("case", [(1, 4, 64, 2, True, True), (2, 4, 100, 4, True, False), (1, 8, 257, 4, False, True),
+                                  (2, 8, 2048, 4, True, True), (1, 8, 72, 8, True, True), (1, 2, 33, 1, False, False),
+                                  (1, 4, 4096, 4, False, True)])
+def test_mix_softmax_mix_key_bias(ops, case, dt):
+    """`scores = scores + mask` of mta_attention_triton.py:77-78 for a mask that is the causal rule plus one value per
+    key: hidden keys (-inf) get probability 0, finite values are added in the I/O dtype."""
+    n, c, s, group, use1, use2 = case
+    dtype = DT[dt]
+    print(f"mix_softmax_mix key bias case={case} dt={dt}", flush=True)
+    x = _randn((n, c, s, s), 12, dtype, 2.0)
+    g = torch.Generator().manual_seed(13)
+    w1 = O.block_diag_head_weight(c, group, 0.1, g, dtype) if use1 else None
+    w2 = O.block_diag_head_weight(c, group, 0.1, g, dtype) if use2 else None
+    bias = torch.randn(n, s, generator=g).to(dtype).float()        # finite part, representable in the I/O dtype
+    bias[torch.rand(n, s, generator=g) < 0.3] = float("-inf")
+    bias[:, 0] = 0.0                                                # key 0 stays visible: no row is fully hidden
+    s2 = O.head_linear(x, w1, True, float("-inf")) if use1 else x.masked_fill(_upper(s, s), float("-inf"))
+    s3 = s2 + bias[:, None, None, :].to(dtype)                       # the reference's add, in the I/O dtype
+    p0 = torch.softmax(s3.float(), -1).to(dtype)
+    want = O.head_linear(p0, w2, True, 0.0) if use2 else p0
+    got = ops.headmix_softmax(x.cuda(), w1.cuda() if use1 else None, w2.cuda() if use2 else None, True,
+                              group_size=group, key_bias=bias.cuda()).cpu()
+    up = _upper(s, s)
+    assert (got[..., up] == 0).all() and not torch.signbit(got[..., up]).any()
+    if not use2:
+        hidden = torch.isinf(bias)[:, None, None, :].expand_as(got)
+        assert (got[hidden] == 0).all()
+    t = tol(dtype)
+    torch.testing.assert_close(got.float(), want.float(), rtol=t["rtol"] * 2, atol=2e-3 if dtype != torch.float32 else 1e-6)
+    with pytest.raises(ValueError):
+        ops.headmix_softmax(x.cuda(), None, None, True, key_bias=bias.cuda().half())
+
+
 def test_error_codes(ops):
     x = torch.zeros(1, 2, 8, 8, device="cuda")
     with pytest.raises(ValueError, match="kernel size"):
