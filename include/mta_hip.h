@@ -105,6 +105,19 @@ int mta_headmix_softmax_bias_fwd(const void *x, const void *w1, const void *w2, 
                                  int64_t N, int64_t C, int64_t P, int64_t Q, int group_size, int causal,
                                  int fill_upper, int io_dtype, int w_dtype, void *stream);
 
+/* Depthwise causal conv followed by head mixing, the conv result never written:
+ *   t[h] = round(conv2d(x[h], w_conv[h]))                     as mta_conv2d_fwd
+ *   y[o] = round(sum_h w_mix[o,h] t[h])                        as mta_headmix_fwd with fill 0
+ * x, y are (N,C,H,W); w_conv is (C,R,S); w_mix is (C,C) row = output head; group_size as in mta_headmix_fwd
+ * (supported mixing groups: 1, 2, 4, 8, 16 heads; others return MTA_ERR_UNSUPPORTED and the two separate entry
+ * points apply).  causal: q>p is written as +0.0 when fill_upper != 0 and left unspecified otherwise.
+ * Replaces mta_conv_after_sm_triton -> wposm_triton of mta_attention_triton.py:81-85 (conv_fwd_kernel,
+ * convolution_2d_trit.py:52-135, then linear_head_kernel_forward, triton_linear_head.py:76-139): one read and one
+ * write of the probabilities instead of two of each. */
+int mta_conv2d_headmix_fwd(const void *x, const void *w_conv, const void *w_mix, void *y, int64_t N, int64_t C,
+                           int64_t H, int64_t W, int R, int S, int group_size, int causal, int fill_upper,
+                           int io_dtype, int wconv_dtype, int wmix_dtype, void *stream);
+
 /* Fused conv-attention forward:
  *   O = softmax( mask( conv( mask0(Q K^T) ) ) * scale ) V        per (batch, head)
  * q,k,v,o are (B,H,S,D); w is (H,R,Sk).  mask0 zeroes col>row before the conv, mask

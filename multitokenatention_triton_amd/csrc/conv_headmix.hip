@@ -1,0 +1,281 @@
+// Depthwise causal conv followed by head mixing, in one pass over an (N,C,H,W) tensor:
+//
+//     t[h]   = round( conv2d(x[h], w_conv[h]) )            causal: taps with col > row read as 0, outputs q > p are +0
+//     y[o]   = round( sum_h w_mix[o,h] * t[h] )            over the heads of o's mixing group
+//
+// which is what mta_conv_after_sm_triton -> wposm_triton compute on the probabilities
+// (mta_attention_triton.py:81-85; conv_fwd_kernel, convolution_2d_trit.py:52-135; linear_head_kernel_forward,
+// triton_linear_head.py:76-139) with the conv result never leaving the chip: one read and one write of the tensor
+// instead of two of each.
+//
+// A workgroup owns a 32 x 64 tile of positions for all G heads of one mixing group.  It walks the group's heads:
+// stage the head's (32+R-1) x (64+S-1) input window in LDS as fp32 (the causal input rule and the borders are
+// applied on the way in), convolve - a lane owns 8 consecutive keys of one row, as in the stand-alone conv - round
+// to the I/O dtype, and add the head's contribution to the G x 8 output accumulators of the lane.  For 16-bit data
+// with mix weights of the same dtype the heads are taken in pairs and the mixing runs on packed dot products (two
+// multiply-adds per instruction; the pair is packed from the rounded conv results, which is the rounding the
+// unfused pipeline applies to them).
+#include <type_traits>
+
+#include "common.hpp"
+
+namespace {
+using namespace mta;
+
+constexpr int CH_NT = 256;
+constexpr int CH_TM = 32;  // tile rows
+constexpr int CH_TN = 64;  // tile keys
+
+template <typename T> __device__ __forceinline__ float dot2_io(uint32_t a, uint32_t b, float c)
+{
+    if constexpr (std::is_same<T, bf16_t>::value) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(mta_bf16x2, a), __builtin_bit_cast(mta_bf16x2, b), c, false);
+    } else if constexpr (std::is_same<T, f16_t>::value) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(mta_f16x2, a), __builtin_bit_cast(mta_f16x2, b), c, false);
+    } else {
+        return c;
+    }
+}
+
+// DOT: mix on packed dot products (16-bit data, mix weights of the same dtype, even group size)
+template <typename T, int G, int R_T, int S_T, bool DOT>
+__global__ __launch_bounds__(CH_NT) void conv_headmix_kernel(const T *__restrict__ x, const void *__restrict__ wc,
+                                                            const void *__restrict__ wm, T *__restrict__ y, int C, int H,
+                                                            int W, int R_rt, int S_rt, int causal, int fill_upper,
+                                                            int wc_dtype, int wm_dtype, int tiles_n)
+{
+    const int R = R_T > 0 ? R_T : R_rt;
+    const int S = S_T > 0 ? S_T : S_rt;
+    const int pad_h = R - 1, pad_w = (S - 1) / 2;
+    const int LD = CH_TN + S;  // S-1 halo columns + 1 pad
+    extern __shared__ float smem[];
+    float *wms = smem;                              // G*G mix weights of this group, [o][h]
+    float *wcs = wms + G * G;                       // G*R*S conv weights of the group's heads
+    float *tile = wcs + ((G * R * S + 3) & ~3);     // (CH_TM+R-1) x LD
+    // mix weights as packed pairs of the I/O dtype, (w[o][2j], w[o][2j+1])
+    static_assert(!DOT || (sizeof(T) == 2 && G % 2 == 0), "packed pairs of a 16-bit type");
+    __shared__ uint32_t wmp[DOT ? G * (G / 2) : 1];
+
+    const int tid = threadIdx.x;
+    const int groups = C / G;
+    const int64_t n = blockIdx.y / groups;
+    const int g = (int)(blockIdx.y % groups);
+    const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
+    const int p0 = tm * CH_TM, q0 = tn * CH_TN;
+    const int64_t plane = (int64_t)H * W;
+    const T *xg = x + (n * C + (int64_t)g * G) * plane;
+    T *yg = y + (n * C + (int64_t)g * G) * plane;
+    const int tr = tid >> 3, tc = (tid & 7) * 8;
+    const int p = p0 + tr, q = q0 + tc;
+    const bool vec_ok = (W % 8 == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
+
+    auto store8 = [&](int o, const float (&v)[8]) {
+        if (p >= H || q >= W) return;
+        T *dst = yg + o * plane + (int64_t)p * W + q;
+        if (vec_ok) {
+            pack16<T> out;
+            if constexpr (sizeof(T) == 2) {
+                uint32_t r[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) r[u] = pack2<T>(v[2 * u], v[2 * u + 1]);
+                __builtin_memcpy(&out, r, 16);
+                typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+                __builtin_nontemporal_store(__builtin_bit_cast(u4, out), reinterpret_cast<u4 *>(dst));
+            } else {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) out.v[u] = from_float<T>(v[u]);
+                *reinterpret_cast<pack16<T> *>(dst) = out;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) out.v[u] = from_float<T>(v[4 + u]);
+                *reinterpret_cast<pack16<T> *>(dst + 4) = out;
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (q + u < W) dst[u] = from_float<T>(v[u]);
+        }
+    };
+
+    if (causal && q0 > p0 + CH_TM - 1) {  // wholly above the diagonal: +0 on request, nothing else
+        if (fill_upper) {
+            const float z[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int o = 0; o < G; ++o) store8(o, z);
+        }
+        return;
+    }
+
+    for (int t = tid; t < G * G; t += CH_NT)
+        wms[t] = load_any(wm, wm_dtype, (int64_t)(g * G + t / G) * C + g * G + t % G);
+    for (int t = tid; t < G * R * S; t += CH_NT) wcs[t] = load_any(wc, wc_dtype, (int64_t)g * G * R * S + t);
+    if constexpr (DOT) {
+        for (int t = tid; t < G * (G / 2); t += CH_NT) {
+            const int o = t / (G / 2), j = t % (G / 2);
+            const int64_t widx = (int64_t)(g * G + o) * C + g * G + 2 * j;
+            wmp[t] = pack2<T>(load_any(wm, wm_dtype, widx), load_any(wm, wm_dtype, widx + 1));
+        }
+    }
+
+    float out[G][8];
+#pragma unroll
+    for (int o = 0; o < G; ++o)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) out[o][u] = 0.0f;
+
+    const int rows = CH_TM + R - 1, cols = CH_TN + S - 1;
+    // rounded conv result of head h for this lane's 8 positions
+    auto conv_head = [&](int h, float (&acc)[8]) __attribute__((always_inline)) {
+        const T *xp = xg + h * plane;
+        __syncthreads();  // everybody is done with the previous head's window
+        for (int rr = tid / 64; rr < rows; rr += CH_NT / 64) {
+            const int hh = p0 - pad_h + rr;
+            const bool row_ok = hh >= 0 && hh < H;
+            for (int cc = tid % 64; cc < cols; cc += 64) {
+                const int k = q0 - pad_w + cc;
+                float v = 0.0f;
+                if (row_ok && k >= 0 && k < W && (!causal || k <= hh)) v = to_float(xp[(int64_t)hh * W + k]);
+                tile[rr * LD + cc] = v;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc[u] = 0.0f;
+        const float *wch = wcs + h * R * S;
+        if constexpr (R_T > 0 && S_T > 0) {
+#pragma unroll
+            for (int i = 0; i < R_T; ++i) {
+                float win[S_T + 7];
+                const float *src = tile + (tr + i) * LD + tc;
+#pragma unroll
+                for (int u = 0; u < S_T + 7; ++u) win[u] = src[u];
+#pragma unroll
+                for (int j = 0; j < S_T; ++j) {
+                    const float wv = wch[i * S_T + j];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) acc[u] = fmaf(wv, win[u + j], acc[u]);
+                }
+            }
+        } else {
+            for (int i = 0; i < R; ++i) {
+                const float *src = tile + (tr + i) * LD + tc;
+                for (int j = 0; j < S; ++j) {
+                    const float wv = wch[i * S + j];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) acc[u] = fmaf(wv, src[u + j], acc[u]);
+                }
+            }
+        }
+        // the conv's causal output rule, then its rounding to the I/O dtype
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc[u] = (causal && q + u > p) ? 0.0f : round_to<T>(acc[u]);
+    };
+    if constexpr (DOT) {
+        for (int h = 0; h < G; h += 2) {
+            float a0[8], a1[8];
+            conv_head(h, a0);
+            uint32_t pp[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) pp[u] = pack2<T>(a0[u], 0.0f) & 0xffffu;  // (exact: already rounded)
+            conv_head(h + 1, a1);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) pp[u] |= pack2<T>(0.0f, a1[u]) & 0xffff0000u;
+#pragma unroll
+            for (int o = 0; o < G; ++o) {
+                const uint32_t wv = wmp[o * (G / 2) + (h >> 1)];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) out[o][u] = dot2_io<T>(wv, pp[u], out[o][u]);
+            }
+        }
+    } else {
+        for (int h = 0; h < G; ++h) {
+            float acc[8];
+            conv_head(h, acc);
+#pragma unroll
+            for (int o = 0; o < G; ++o) {
+                const float wv = wms[o * G + h];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) out[o][u] = fmaf(wv, acc[u], out[o][u]);
+            }
+        }
+    }
+#pragma unroll
+    for (int o = 0; o < G; ++o) {
+        if (causal) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (q + u > p) out[o][u] = 0.0f;
+        }
+        if (!causal || fill_upper || q <= p) store8(o, out[o]);
+    }
+}
+
+template <typename T, int G, int R_T, int S_T>
+int launch(const void *x, const void *wc, const void *wm, void *y, int64_t N, int64_t C, int64_t H, int64_t W, int R,
+           int S, int causal, int fill_upper, int wc_dtype, int wm_dtype, hipStream_t st)
+{
+    const int tiles_m = (int)((H + CH_TM - 1) / CH_TM), tiles_n = (int)((W + CH_TN - 1) / CH_TN);
+    const size_t lds = sizeof(float) * ((size_t)G * G + ((G * R * S + 3) & ~3) + (size_t)(CH_TM + R - 1) * (CH_TN + S));
+    if (lds > 60 * 1024) return MTA_ERR_KERNEL_SIZE;
+    dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)(N * (C / G)));
+    constexpr bool DOT_OK = sizeof(T) == 2 && G % 2 == 0;
+    const bool use_dot = DOT_OK && wm_dtype == (std::is_same<T, bf16_t>::value ? MTA_BF16 : MTA_F16);
+    if constexpr (DOT_OK) {
+        if (use_dot) {
+            hipLaunchKernelGGL((conv_headmix_kernel<T, G, R_T, S_T, true>), grid, dim3(CH_NT), lds, st, (const T *)x, wc, wm,
+                               (T *)y, (int)C, (int)H, (int)W, R, S, causal, fill_upper, wc_dtype, wm_dtype, tiles_n);
+            return launch_status();
+        }
+    }
+    hipLaunchKernelGGL((conv_headmix_kernel<T, G, R_T, S_T, false>), grid, dim3(CH_NT), lds, st, (const T *)x, wc, wm,
+                       (T *)y, (int)C, (int)H, (int)W, R, S, causal, fill_upper, wc_dtype, wm_dtype, tiles_n);
+    return launch_status();
+}
+
+template <typename T, int G>
+int dispatch_size(const void *x, const void *wc, const void *wm, void *y, int64_t N, int64_t C, int64_t H, int64_t W,
+                  int R, int S, int causal, int fill_upper, int wc_dtype, int wm_dtype, hipStream_t st)
+{
+#define MTA_CH_CASE(r, s) \
+    if (R == r && S == s) return launch<T, G, r, s>(x, wc, wm, y, N, C, H, W, R, S, causal, fill_upper, wc_dtype, wm_dtype, st);
+    MTA_CH_CASE(3, 3)
+    MTA_CH_CASE(7, 7)
+#undef MTA_CH_CASE
+    return launch<T, G, 0, 0>(x, wc, wm, y, N, C, H, W, R, S, causal, fill_upper, wc_dtype, wm_dtype, st);
+}
+
+template <typename T>
+int dispatch(const void *x, const void *wc, const void *wm, void *y, int64_t N, int64_t C, int64_t H, int64_t W, int R,
+             int S, int G, int causal, int fill_upper, int wc_dtype, int wm_dtype, hipStream_t st)
+{
+#define MTA_CH_GROUP(g) \
+    if (G == g) return dispatch_size<T, g>(x, wc, wm, y, N, C, H, W, R, S, causal, fill_upper, wc_dtype, wm_dtype, st);
+    MTA_CH_GROUP(1)
+    MTA_CH_GROUP(2)
+    MTA_CH_GROUP(4)
+    MTA_CH_GROUP(8)
+    MTA_CH_GROUP(16)
+#undef MTA_CH_GROUP
+    return MTA_ERR_UNSUPPORTED;
+}
+}  // namespace
+
+extern "C" int mta_conv2d_headmix_fwd(const void *x, const void *w_conv, const void *w_mix, void *y, int64_t N, int64_t C,
+                                      int64_t H, int64_t W, int R, int S, int group_size, int causal, int fill_upper,
+                                      int io_dtype, int wconv_dtype, int wmix_dtype, void *stream)
+{
+    if (!x || !w_conv || !w_mix || !y) return MTA_ERR_NULL;
+    if (!dtype_size(io_dtype) || !dtype_size(wconv_dtype) || !dtype_size(wmix_dtype)) return MTA_ERR_DTYPE;
+    if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || H > (1 << 24) || W > (1 << 24) || C > 4096) return MTA_ERR_SHAPE;
+    if (R < 1 || S < 1 || R > MTA_MAX_KERNEL_R || S > MTA_MAX_KERNEL_S) return MTA_ERR_KERNEL_SIZE;
+    if (group_size < 0 || (group_size > 0 && C % group_size != 0)) return MTA_ERR_GROUP;
+    if (!aligned_to(x, dtype_size(io_dtype)) || !aligned_to(y, dtype_size(io_dtype)) ||
+        !aligned_to(w_conv, dtype_size(wconv_dtype)) || !aligned_to(w_mix, dtype_size(wmix_dtype)))
+        return MTA_ERR_ALIGN;
+    const int G = group_size > 0 ? group_size : (int)C;
+    const int64_t tiles = ((H + CH_TM - 1) / CH_TM) * ((W + CH_TN - 1) / CH_TN);
+    if (tiles > 0x7fffffffLL || N * (C / G) > 65535) return MTA_ERR_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    MTA_DISPATCH_IO(io_dtype, return dispatch<io_t>(x, w_conv, w_mix, y, N, C, H, W, R, S, G, causal, causal ? fill_upper : 1,
+                                                    wconv_dtype, wmix_dtype, st));
+    return MTA_ERR_DTYPE;
+}

@@ -13,6 +13,8 @@ Inference (no input or parameter requires grad, or grad mode is off):
     post-softmax conv kernel is the identity tap -- the post-softmax head mixing run
     as one kernel (``mta_headmix_softmax_fwd``): one pass over the score tensor
     instead of four, and no fp32 copy of it;
+  * otherwise the post-softmax conv and head mixing run as one kernel
+    (``mta_conv2d_headmix_fwd``): the conv result never reaches HBM;
   * P V reads only the lower triangle of P (``mta_causal_pv_fwd``).
 
 Training (something requires grad): the stages run one by one through the autograd
@@ -175,12 +177,20 @@ class MTAAttentionTriton(nn.Module):
                 self._mark("softmax")
                 scores = ops.headmix_softmax(scores, None, None, self.causal, key_bias=key_bias,
                                              fill_upper=post_conv_identity and w2 is None and not own_pv)
-            if not post_conv_identity:
-                self._mark("conv_post")
-                scores = ops.conv2d_causal(scores, self.mta_conv_after_sm_triton.weight, self.causal)
-            if w2 is not None:
-                self._mark("mix_post")
-                scores = ops.headmix(scores, w_post, self.causal, 0.0, group_size=g_post)
+            done = None
+            if not post_conv_identity and w2 is not None:   # conv and mix in one pass, the conv result never written
+                self._mark("conv_mix_post")
+                done = ops.conv2d_headmix(scores, self.mta_conv_after_sm_triton.weight, w_post, self.causal,
+                                          group_size=g_post, fill_upper=not own_pv)
+            if done is not None:
+                scores = done
+            else:
+                if not post_conv_identity:
+                    self._mark("conv_post")
+                    scores = ops.conv2d_causal(scores, self.mta_conv_after_sm_triton.weight, self.causal)
+                if w2 is not None:
+                    self._mark("mix_post")
+                    scores = ops.headmix(scores, w_post, self.causal, 0.0, group_size=g_post)
 
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         self._mark("pv")

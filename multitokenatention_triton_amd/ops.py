@@ -200,6 +200,31 @@ def headmix_softmax(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optional[to
     return y
 
 
+def conv2d_headmix(x: torch.Tensor, w_conv: torch.Tensor, w_mix: torch.Tensor, causal: bool = True,
+                   group_size: Optional[int] = None, out: Optional[torch.Tensor] = None,
+                   fill_upper: bool = True) -> Optional[torch.Tensor]:
+    """Depthwise causal conv, then head mixing, in one pass; see mta_conv2d_headmix_fwd.  Returns None when the
+    library has no kernel for the mixing-group size (the caller then runs the two operators one after the other)."""
+    x = _device_tensor(x, "input")
+    if x.dim() != 4:
+        raise ValueError(f"expected input (N,C,H,W), got {tuple(x.shape)}")
+    n, c, h, w = x.shape
+    w_conv = _device_tensor(w_conv.detach(), "conv weight")
+    w_mix = _device_tensor(w_mix.detach(), "mix weight")
+    assert w_conv.dim() == 3 and w_conv.size(0) == c, "Input and weight channels must match"
+    assert tuple(w_mix.shape) == (c, c), f"Weight must be ({c},{c}), got {tuple(w_mix.shape)}"
+    y = _out_like(x, out)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().mta_conv2d_headmix_fwd(
+            x.data_ptr(), w_conv.data_ptr(), w_mix.data_ptr(), y.data_ptr(), n, c, h, w, w_conv.size(1), w_conv.size(2),
+            int(group_size or 0), int(bool(causal)), int(bool(fill_upper)), _code(x, "input"), _code(w_conv, "weight"),
+            _code(w_mix, "weight"), _stream(x))
+    if rc == _lib.MTA_ERR_UNSUPPORTED:
+        return None
+    _lib.check(rc, "mta_conv2d_headmix_fwd")
+    return y
+
+
 def conv_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, weight: torch.Tensor, causal: bool,
                   softmax_scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
                   return_lse: bool = False):

@@ -524,6 +524,28 @@ def test_mta_use_mask_tensor_masks(pkg, name, dtype):
         assert (("qk_conv" in stages or "conv_pre" in stages) and "pv" in stages) == name.startswith("key_mask")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("group", [4, 16])
+def test_mta_general_route_is_four_stages(pkg, group, dtype):
+    """All four MTA weights non-trivial (what training produces): QK^T+conv, mix+softmax, conv+mix, P V -- four kernels,
+    the score tensor written twice and read three times; mixing groups of 4 and dense 16x16 weights."""
+    print(f"mta general route group={group} {dtype}", flush=True)
+    h, s, d = 16, 520, 64
+    q, k, v = O.seeded_qkv(1, h, s, d, dtype, seed=97)
+    params = _config_like(h, group, 7, 7, 0.05, dtype, post="random")
+    want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3])
+    for structure in ("infer", "dense"):
+        mod = _mta_module(pkg, h, 7, 7, 3, 3, *params, dtype, structure=structure)
+        stages = []
+        mod._stage_hook = stages.append
+        got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
+        if group <= 8 and structure == "infer":
+            assert stages == ["qk_conv", "mix_softmax", "conv_mix_post", "pv", "end"]
+        else:   # a 16-head mixing group is beyond the one-pass mix/softmax kernel: mix, then softmax
+            assert stages == ["qk_conv", "mix_pre", "softmax", "conv_mix_post", "pv", "end"]
+        torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+
+
 @pytest.mark.parametrize("post", ["identity", "random"])
 def test_mta_use_mask_key_mask_long_rows(pkg, post):
     """Key mask at a size where the 16-bit kernels run several passes per row (one-pass mix/softmax/mix and the

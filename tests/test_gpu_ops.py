@@ -266,6 +266,51 @@ def test_mix_softmax_mix_key_bias(ops, case, dt):
         ops.headmix_softmax(x.cuda(), None, None, True, key_bias=bias.cuda().half())
 
 
+CH_CASES = [
+    # N, C, H(=W), R, S, group (None = dense)
+    (1, 4, 64, 3, 3, 2), (2, 4, 100, 3, 3, 4), (1, 8, 264, 3, 3, 4), (1, 16, 136, 3, 3, None), (1, 16, 200, 7, 7, None),
+    (1, 8, 72, 5, 7, 8), (1, 2, 33, 3, 5, 1), (1, 6, 50, 2, 2, 2), (1, 32, 96, 3, 3, 16),
+]
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("case", CH_CASES)
+def test_conv_headmix_parity(ops, case, causal, dt):
+    """mta_conv_after_sm_triton -> wposm_triton (mta_attention_triton.py:81-85) as one kernel, against the oracle's
+    conv (rounded to the I/O dtype, as the unfused pipeline stores it) followed by its head mixing."""
+    n, c, s, r, sk, group = case
+    dtype = DT[dt]
+    print(f"conv_headmix case={case} causal={causal} dt={dt}", flush=True)
+    g = torch.Generator().manual_seed(21)
+    x = torch.softmax(_randn((n, c, s, s), 20, torch.float32, 2.0).masked_fill(_upper(s, s) if causal else torch.zeros(s, s, dtype=torch.bool), float("-inf")), -1).to(dtype)
+    wc = _randn((c, r, sk), 22, dtype, 0.3)
+    wm = O.block_diag_head_weight(c, group or c, 0.3, g, dtype)
+    t = O.depthwise_conv(x.float(), wc.float(), causal).to(dtype)
+    want = O.head_linear(t, wm, causal, 0.0)
+    for fill in (True, False):
+        got = ops.conv2d_headmix(x.cuda(), wc.cuda(), wm.cuda(), causal, group_size=group, fill_upper=fill)
+        assert got is not None and got.dtype == dtype
+        got = got.cpu()
+        if causal:
+            up = _upper(s, s)
+            if fill:
+                assert (got[..., up] == 0).all() and not torch.signbit(got[..., up]).any()
+            got = torch.tril(got)
+        torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+    # mix weights of another dtype than the data take the plain multiply-add path
+    if dtype != torch.float32:
+        got = ops.conv2d_headmix(x.cuda(), wc.cuda(), wm.float().cuda(), causal, group_size=group).cpu()
+        torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+
+
+def test_conv_headmix_unsupported_group(ops):
+    x = torch.zeros(1, 12, 16, 16, device="cuda")
+    assert ops.conv2d_headmix(x, torch.zeros(12, 3, 3, device="cuda"), torch.eye(12, device="cuda"), True) is None
+    assert ops.conv2d_headmix(x, torch.zeros(12, 3, 3, device="cuda"), torch.eye(12, device="cuda"), True,
+                              group_size=4) is not None
+
+
 def test_error_codes(ops):
     x = torch.zeros(1, 2, 8, 8, device="cuda")
     with pytest.raises(ValueError, match="kernel size"):
