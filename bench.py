@@ -63,10 +63,45 @@ def stage_model(name, b, h, s, d, r=6, sk=11, esize=2):
     return t + full, 0
 
 
-# HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at the benchmark shape
-# (profiles/mta_forward_c4_hbm_traffic.txt); FETCH_SIZE is scaled by 2.0, the factor a plain 1 GiB
-# device copy shows for it on this machine, WRITE_SIZE by 1.0.
-MEASURED_TRAFFIC_BYTES = {"qk_conv": 606.7e6, "mix_softmax_mix": 1111.4e6, "pv": 648.7e6}
+# Which kernel runs a stage of the headline forward, as rocprofv3 names it in profiles/mta_forward_c4_hbm_traffic.txt
+STAGE_KERNEL = {"qk_conv": "conv_attn_fwd_mfma<bf16_t, 128, 6, 11, true, 4>", "mix_softmax_mix": "mix_softmax_mix_packed<",
+                "pv": "causal_pv_kernel<"}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "mta_forward_c4_hbm_traffic.txt")
+
+
+def kernel_sources_digest():
+    """sha256 over the kernel sources the library is built from: names the build a counter profile belongs to."""
+    import hashlib
+    d = os.path.join(ROOT, "multitokenatention_triton_amd", "csrc")
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(d)):
+        if name.endswith((".hip", ".hpp")):
+            h.update(name.encode())
+            with open(os.path.join(d, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(stage):
+    """HBM bytes per launch of the stage's kernel from the committed rocprofv3 counter summary (FETCH_SIZE and
+    WRITE_SIZE, each scaled by what the same counter reads for a plain 1 GiB device copy; the summary states the
+    factors) -- or None when the summary was taken from other kernel sources than the ones in this tree."""
+    pat = STAGE_KERNEL.get(stage)
+    try:
+        lines = open(TRAFFIC_PROFILE).read().splitlines()
+    except OSError:
+        return None
+    digest = [ln.split(":", 1)[1].strip() for ln in lines if ln.startswith("kernel sources sha256")]
+    if not pat or not digest or digest[0] != kernel_sources_digest():
+        return None
+    for ln in lines:
+        f = ln.split(None, 5)
+        if len(f) == 6 and pat in f[5]:
+            try:
+                return float(f[4]) * 1e6
+            except ValueError:
+                pass
+    return None
 
 
 def build_c4(torch, mta, O, device, b=2, h=16, s=4096, d=128, dtype=None, nsets=3):
@@ -83,6 +118,23 @@ def build_c4(torch, mta, O, device, b=2, h=16, s=4096, d=128, dtype=None, nsets=
     # the configuration states the structure (identity wpsm and post conv, groups of 4): read it off the weights once
     mod.infer_weight_structure()
     sets = [tuple(t.to(device) for t in O.seeded_qkv(b, h, s, d, dtype, seed=123 + i)) for i in range(nsets)]
+    return mod, sets
+
+
+def build_general(torch, mta, O, device, b=1, h=16, s=4096, d=128, nsets=2):
+    """The closest shape to the reference's published rows (benchmark_seq_len_results.jsonl: H16 D128 fp16, 7x7 conv
+    before and after the softmax): all four weights non-trivial -- random 7x7 kernels, dense random 16x16 head weights."""
+    dtype = torch.float16
+    g = torch.Generator().manual_seed(321)
+    cfg = mta.MTAConfig(query_kernel_size=7, key_kernel_size=7, after_sm_query_kernel_size=7, after_sm_key_kernel_size=7)
+    mod = mta.MTAAttentionTriton(h, cfg, dropout=0.0, causal=True).to(dtype)
+    with torch.no_grad():
+        mod.mta_conv_triton.weight.copy_(O.seeded_conv_weight(h, 7, 7, 0.05, dtype, seed=5))
+        mod.mta_conv_after_sm_triton.weight.copy_(O.seeded_conv_weight(h, 7, 7, 0.05, dtype, seed=6))
+        mod.wpsm_triton.weight.copy_(torch.eye(h) + 0.1 * torch.randn(h, h, generator=g))
+        mod.wposm_triton.weight.copy_(torch.eye(h) + 0.1 * torch.randn(h, h, generator=g))
+    mod = mod.to(device).eval().requires_grad_(False)   # dense weights: nothing is assumed about their structure
+    sets = [tuple(t.to(device) for t in O.seeded_qkv(b, h, s, d, dtype, seed=400 + i)) for i in range(nsets)]
     return mod, sets
 
 
@@ -178,12 +230,21 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
     out["conv_attn_fused_bf16_1x32x8192x128"] = {"ms": ms, "mfma_useful_flops": mfma_flops,
                                                  "TFLOPs": mfma_flops / ms / 1e9,
                                                  "frac_mfma_peak": mfma_flops / ms / 1e9 / MFMA_BF16_PEAK_TF}
+    del sets, os_
+    # the general four-stage forward (all MTA weights non-trivial), B1 H16 S4096 D128 fp16, 7x7 conv pre and post
+    mod, sets = build_general(torch, mta, O, device)
+    ms = time_steps(torch, lambda i: mod(*sets[i], None, None), len(sets), min(warmup, 3), max(3, steps // 2))
+    stages = stage_breakdown(torch, mod, sets, 3)
+    out["mta_forward_general_fp16_1x16x4096x128_7x7_pre_post_dense"] = {
+        "ms": ms, "stages_ms": stages,
+        "note": "forward only; the reference's published row for this shape (Triton 11.345 ms, PyTorch 43.795 ms, "
+                "hardware unstated) is context, not a baseline"}
     return out
 
 
-def cpu_baseline(torch, O, b, h, s, d, budget_s=15.0):
-    """The oracle's torch MTA forward on the host cores, on a bounded sample of the same workload."""
-    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+def cpu_baseline(torch, O, b, h, s, d, budget_s=12.0):
+    """The oracle's torch MTA forward on all host cores, on a bounded sample of the same workload."""
+    threads = os.cpu_count() or 1
     torch.set_num_threads(threads)
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(125)
@@ -209,7 +270,61 @@ def cpu_baseline(torch, O, b, h, s, d, budget_s=15.0):
     return {"value": t * 1e3 * factor, "unit": "ms", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"oracle.mta_forward bf16 on B=1,H={h},S={ss},D={d} took {t * 1e3:.1f} ms; "
                       f"scaled by {factor:.0f} (score-tensor elements) to B={b},S={s}",
-            "cpu_model": _cpu_model()}
+            "host_cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads(), "cpu_model": _cpu_model()}
+
+
+def cpu_baselines_other(torch, O):
+    """The oracle on the host cores for the other configurations: C1 at its full size, one batch element of the
+    conv-alone and head-mix-alone configurations, and a row slab of the fused conv-attention one.  A few seconds each."""
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    out = {}
+    with torch.no_grad():
+        # C1: B1 H4 S256 D64 fp32, conv 3x5, full size, 10 repetitions
+        q, k, v = O.seeded_qkv(1, 4, 256, 64, torch.float32)
+        g = torch.Generator().manual_seed(125)
+        w_pre = O.seeded_conv_weight(4, 3, 5, 0.1, torch.float32).unsqueeze(1)
+        w_post = O.identity_conv_kernel(4, 3, 3, torch.float32).unsqueeze(1)
+        wpsm, wposm = O.block_diag_head_weight(4, 2, 0.1, g), O.block_diag_head_weight(4, 2, 0.1, g)
+        O.mta_forward(q, k, v, w_pre, wpsm, w_post, wposm)
+        t0 = time.perf_counter()
+        for _ in range(10):
+            O.mta_forward(q, k, v, w_pre, wpsm, w_post, wposm)
+        out["mta_forward_fp32_1x4x256x64"] = {"value": (time.perf_counter() - t0) * 100.0, "unit": "ms", "cores": threads,
+                                              "kind": "port", "sample": "full size, mean of 10 repetitions"}
+        # C2: conv alone (2,16,2048,2048) bf16 6x11: one batch element, scaled by 2
+        bf16 = torch.bfloat16
+        gg = torch.Generator().manual_seed(7)
+        x = torch.tril(torch.randn(1, 16, 2048, 2048, generator=gg)).to(bf16)
+        w = O.seeded_conv_weight(16, 6, 11, 0.05, bf16, identity_tap=False)
+        t0 = time.perf_counter()
+        O.depthwise_conv(x, w, True)
+        t = time.perf_counter() - t0
+        out["conv2d_6x11_bf16_2x16x2048x2048"] = {"value": t * 2e3, "unit": "ms", "cores": threads, "kind": "port",
+                                                  "sample": f"one of the two batch elements took {t * 1e3:.0f} ms; scaled by 2"}
+        del x
+        # C3: head-mix alone (2,32,2048,2048) bf16 groups of 4: one batch element, scaled by 2
+        x = torch.softmax(torch.randn(1, 32, 2048, 2048, generator=gg).masked_fill(
+            torch.triu(torch.ones(2048, 2048, dtype=torch.bool), 1), float("-inf")), -1).to(bf16)
+        wm = O.block_diag_head_weight(32, 4, 0.1, gg, bf16)
+        t0 = time.perf_counter()
+        O.head_linear(x, wm, True, 0.0)
+        t = time.perf_counter() - t0
+        out["headmix_g4_bf16_2x32x2048x2048"] = {"value": t * 2e3, "unit": "ms", "cores": threads, "kind": "port",
+                                                 "sample": f"one of the two batch elements took {t * 1e3:.0f} ms; scaled by 2"}
+        del x
+        # C5: fused conv-attention B1 H32 S8192 D128 bf16: 256 query rows in the middle of the sequence against all
+        # keys, 8 of the 32 heads; scaled by rows and heads (the work per row grows with the row index: the middle
+        # slab stands for the average row)
+        q, k, v = O.seeded_qkv(1, 8, 8192, 128, bf16, seed=200)
+        wc = O.seeded_conv_weight(8, 6, 11, 0.05, bf16)
+        t0 = time.perf_counter()
+        O.conv_attention_rows(q, k, v, wc, 3968, 4224, True)
+        t = time.perf_counter() - t0
+        out["conv_attn_fused_bf16_1x32x8192x128"] = {
+            "value": t * 1e3 * (8192 / 256) * (32 / 8), "unit": "ms", "cores": threads, "kind": "port",
+            "sample": f"query rows 3968..4223 of 8 heads took {t * 1e3:.0f} ms; scaled by 32 (rows) x 4 (heads)"}
+    return out
 
 
 def _cpu_model():
@@ -278,7 +393,7 @@ def main():
                                "identity post-softmax conv, head-mix groups of 4 (BASELINE configs[3])",
                    "global_batch": b, "seq_len": s},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(dom),
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(dom),
                      "algorithmic_bytes": dom_bytes, "avg_kernel_ms": hip_stages[dom],
                      "useful_matrix_TFLOPs": dom_flops / hip_stages[dom] / 1e9},
         "stages_ms": stages,
@@ -287,6 +402,8 @@ def main():
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(torch, O, b, h, s, d)
+        if not args.no_extras:
+            result["cpu_baselines_other_configs"] = cpu_baselines_other(torch, O)
     print(json.dumps(result))
 
 

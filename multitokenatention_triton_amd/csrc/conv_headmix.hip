@@ -47,11 +47,10 @@ __global__ __launch_bounds__(CH_NT) void conv_headmix_kernel(const T *__restrict
     const int R = R_T > 0 ? R_T : R_rt;
     const int S = S_T > 0 ? S_T : S_rt;
     const int pad_h = R - 1, pad_w = (S - 1) / 2;
-    const int LD = CH_TN + S;  // S-1 halo columns + 1 pad
     extern __shared__ float smem[];
     float *wms = smem;                              // G*G mix weights of this group, [o][h]
     float *wcs = wms + G * G;                       // G*R*S conv weights of the group's heads
-    float *tile = wcs + ((G * R * S + 3) & ~3);     // (CH_TM+R-1) x LD
+    float *tile = wcs + ((G * R * S + 3) & ~3);     // two windows of (CH_TM+R-1) x LD
     // mix weights as packed pairs of the I/O dtype, (w[o][2j], w[o][2j+1])
     static_assert(!DOT || (sizeof(T) == 2 && G % 2 == 0), "packed pairs of a 16-bit type");
     __shared__ uint32_t wmp[DOT ? G * (G / 2) : 1];
@@ -122,11 +121,24 @@ __global__ __launch_bounds__(CH_NT) void conv_headmix_kernel(const T *__restrict
 #pragma unroll
         for (int u = 0; u < 8; ++u) out[o][u] = 0.0f;
 
+    // Staging.  Kernel sizes with an instantiation of their own, on tensors whose rows are whole 16-byte vectors: the
+    // window starts at a vector boundary left of the halo, each lane fetches its vectors of head h+1 into registers
+    // before it convolves head h and writes them to the other LDS window afterwards (one barrier per head, the fetch
+    // overlaps the arithmetic).  Anything else: element by element into a single window, two barriers per head.
+    constexpr int VEC = vec_of<T>::n;
+    constexpr bool PRE = R_T > 0 && S_T > 0;
+    constexpr int HL = PRE ? ((S_T - 1) / 2 + VEC - 1) / VEC * VEC : 0;
+    constexpr int HRT = PRE ? ((S_T - 1 - (S_T - 1) / 2) + VEC - 1) / VEC * VEC : 0;
+    constexpr int SW = HL + CH_TN + HRT, VPR = SW / VEC;  // staged columns, vectors per staged row
+    constexpr int ROWS_T = CH_TM + (R_T > 0 ? R_T : 1) - 1, NVECS = ROWS_T * VPR, SLOTS = (NVECS + CH_NT - 1) / CH_NT;
+    const bool vec_in = PRE && (W % VEC == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    const int LD = vec_in ? SW + 1 : CH_TN + S;   // (odd: the 8 rows x 8 key groups of a wavefront read 64 different banks)
+    const int c0 = vec_in ? HL - pad_w : 0;       // window column of the first tap of the lane with tc = 0
     const int rows = CH_TM + R - 1, cols = CH_TN + S - 1;
-    // rounded conv result of head h for this lane's 8 positions
-    auto conv_head = [&](int h, float (&acc)[8]) __attribute__((always_inline)) {
+    float *tile1 = tile + rows * LD;
+
+    auto stage_scalar = [&](int h, float *dst) {
         const T *xp = xg + h * plane;
-        __syncthreads();  // everybody is done with the previous head's window
         for (int rr = tid / 64; rr < rows; rr += CH_NT / 64) {
             const int hh = p0 - pad_h + rr;
             const bool row_ok = hh >= 0 && hh < H;
@@ -134,10 +146,38 @@ __global__ __launch_bounds__(CH_NT) void conv_headmix_kernel(const T *__restrict
                 const int k = q0 - pad_w + cc;
                 float v = 0.0f;
                 if (row_ok && k >= 0 && k < W && (!causal || k <= hh)) v = to_float(xp[(int64_t)hh * W + k]);
-                tile[rr * LD + cc] = v;
+                dst[rr * LD + cc] = v;
             }
         }
-        __syncthreads();
+    };
+    auto fetch = [&](int h, pack16<T> (&pre)[SLOTS]) __attribute__((always_inline)) {
+        const T *xp = xg + h * plane;
+#pragma unroll
+        for (int sl = 0; sl < SLOTS; ++sl) {
+            const int idx = sl * CH_NT + tid;
+            const int rr = idx / VPR, vc = idx % VPR;
+            const int hh = p0 - pad_h + rr, k0 = q0 - HL + vc * VEC;
+            const bool ok = idx < NVECS && hh >= 0 && hh < H && k0 >= 0 && k0 < W && (!causal || k0 <= hh);
+            // (a vector outside the plane or wholly above the diagonal re-reads the plane's first vector: the
+            // load stays unconditional, its value is dropped below)
+            pre[sl] = *reinterpret_cast<const pack16<T> *>(xp + (ok ? (int64_t)hh * W + k0 : 0));
+        }
+    };
+    auto deposit = [&](const pack16<T> (&pre)[SLOTS], float *dst) __attribute__((always_inline)) {
+#pragma unroll
+        for (int sl = 0; sl < SLOTS; ++sl) {
+            const int idx = sl * CH_NT + tid;
+            if (idx >= NVECS) continue;
+            const int rr = idx / VPR, vc = idx % VPR;
+            const int hh = p0 - pad_h + rr, k0 = q0 - HL + vc * VEC;
+            const bool ok = hh >= 0 && hh < H && k0 >= 0 && k0 < W;
+#pragma unroll
+            for (int u = 0; u < VEC; ++u)
+                dst[rr * LD + vc * VEC + u] = (ok && (!causal || k0 + u <= hh)) ? to_float(pre[sl].v[u]) : 0.0f;
+        }
+    };
+    // rounded conv result of head h for this lane's 8 positions, from the staged window `tl`
+    auto conv_head = [&](const float *tl, int h, float (&acc)[8]) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < 8; ++u) acc[u] = 0.0f;
         const float *wch = wcs + h * R * S;
@@ -145,7 +185,7 @@ __global__ __launch_bounds__(CH_NT) void conv_headmix_kernel(const T *__restrict
 #pragma unroll
             for (int i = 0; i < R_T; ++i) {
                 float win[S_T + 7];
-                const float *src = tile + (tr + i) * LD + tc;
+                const float *src = tl + (tr + i) * LD + tc + c0;
 #pragma unroll
                 for (int u = 0; u < S_T + 7; ++u) win[u] = src[u];
 #pragma unroll
@@ -157,7 +197,7 @@ __global__ __launch_bounds__(CH_NT) void conv_headmix_kernel(const T *__restrict
             }
         } else {
             for (int i = 0; i < R; ++i) {
-                const float *src = tile + (tr + i) * LD + tc;
+                const float *src = tl + (tr + i) * LD + tc + c0;
                 for (int j = 0; j < S; ++j) {
                     const float wv = wch[i * S + j];
 #pragma unroll
@@ -169,33 +209,55 @@ __global__ __launch_bounds__(CH_NT) void conv_headmix_kernel(const T *__restrict
 #pragma unroll
         for (int u = 0; u < 8; ++u) acc[u] = (causal && q + u > p) ? 0.0f : round_to<T>(acc[u]);
     };
-    if constexpr (DOT) {
-        for (int h = 0; h < G; h += 2) {
-            float a0[8], a1[8];
-            conv_head(h, a0);
-            uint32_t pp[8];
+    // head h's contribution to the outputs (packed-dot path: heads enter in pairs)
+    uint32_t pp[8];
+    auto mix_in = [&](int h, const float (&acc)[8]) __attribute__((always_inline)) {
+        if constexpr (DOT) {
+            if ((h & 1) == 0) {
 #pragma unroll
-            for (int u = 0; u < 8; ++u) pp[u] = pack2<T>(a0[u], 0.0f) & 0xffffu;  // (exact: already rounded)
-            conv_head(h + 1, a1);
+                for (int u = 0; u < 8; ++u) pp[u] = pack2<T>(acc[u], 0.0f) & 0xffffu;  // (exact: already rounded)
+            } else {
 #pragma unroll
-            for (int u = 0; u < 8; ++u) pp[u] |= pack2<T>(0.0f, a1[u]) & 0xffff0000u;
+                for (int u = 0; u < 8; ++u) pp[u] |= pack2<T>(0.0f, acc[u]) & 0xffff0000u;
 #pragma unroll
-            for (int o = 0; o < G; ++o) {
-                const uint32_t wv = wmp[o * (G / 2) + (h >> 1)];
+                for (int o = 0; o < G; ++o) {
+                    const uint32_t wv = wmp[o * (G / 2) + (h >> 1)];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) out[o][u] = dot2_io<T>(wv, pp[u], out[o][u]);
+                    for (int u = 0; u < 8; ++u) out[o][u] = dot2_io<T>(wv, pp[u], out[o][u]);
+                }
             }
-        }
-    } else {
-        for (int h = 0; h < G; ++h) {
-            float acc[8];
-            conv_head(h, acc);
+        } else {
 #pragma unroll
             for (int o = 0; o < G; ++o) {
                 const float wv = wms[o * G + h];
 #pragma unroll
                 for (int u = 0; u < 8; ++u) out[o][u] = fmaf(wv, acc[u], out[o][u]);
             }
+        }
+    };
+    if (vec_in) {
+        pack16<T> pre[SLOTS];
+        fetch(0, pre);
+        deposit(pre, tile);
+        __syncthreads();  // (also covers the weights)
+#pragma unroll 1
+        for (int h = 0; h < G; ++h) {
+            if (h + 1 < G) fetch(h + 1, pre);
+            float acc[8];
+            conv_head((h & 1) ? tile1 : tile, h, acc);
+            mix_in(h, acc);
+            if (h + 1 < G) deposit(pre, (h & 1) ? tile : tile1);  // last read a head ago, ahead of the barrier below
+            __syncthreads();
+        }
+    } else {
+#pragma unroll 1
+        for (int h = 0; h < G; ++h) {
+            __syncthreads();  // everybody is done with the previous head's window
+            stage_scalar(h, tile);
+            __syncthreads();
+            float acc[8];
+            conv_head(tile, h, acc);
+            mix_in(h, acc);
         }
     }
 #pragma unroll
@@ -214,8 +276,10 @@ int launch(const void *x, const void *wc, const void *wm, void *y, int64_t N, in
            int S, int causal, int fill_upper, int wc_dtype, int wm_dtype, hipStream_t st)
 {
     const int tiles_m = (int)((H + CH_TM - 1) / CH_TM), tiles_n = (int)((W + CH_TN - 1) / CH_TN);
-    const size_t lds = sizeof(float) * ((size_t)G * G + ((G * R * S + 3) & ~3) + (size_t)(CH_TM + R - 1) * (CH_TN + S));
-    if (lds > 60 * 1024) return MTA_ERR_KERNEL_SIZE;
+    // two windows of (32+R-1) rows; a row is at most 64 keys + both halos rounded up to whole vectors + 1
+    const size_t row = (size_t)CH_TN + 2 * ((S + 7) / 8 * 8) + 1;
+    const size_t lds = sizeof(float) * ((size_t)G * G + ((G * R * S + 3) & ~3) + 2 * (size_t)(CH_TM + R - 1) * row);
+    if (lds > 64 * 1024) return MTA_ERR_UNSUPPORTED;
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)(N * (C / G)));
     constexpr bool DOT_OK = sizeof(T) == 2 && G % 2 == 0;
     const bool use_dot = DOT_OK && wm_dtype == (std::is_same<T, bf16_t>::value ? MTA_BF16 : MTA_F16);

@@ -13,8 +13,9 @@ Inference (no input or parameter requires grad, or grad mode is off):
     post-softmax conv kernel is the identity tap -- the post-softmax head mixing run
     as one kernel (``mta_headmix_softmax_fwd``): one pass over the score tensor
     instead of four, and no fp32 copy of it;
-  * otherwise the post-softmax conv and head mixing run as one kernel
-    (``mta_conv2d_headmix_fwd``): the conv result never reaches HBM;
+  * otherwise, for mixing groups of up to 4 heads and 3x3 or 7x7 kernels, the
+    post-softmax conv and head mixing run as one kernel (``mta_conv2d_headmix_fwd``):
+    the conv result never reaches HBM;
   * P V reads only the lower triangle of P (``mta_causal_pv_fwd``).
 
 Training (something requires grad): the stages run one by one through the autograd
@@ -52,6 +53,9 @@ from .triton_linear_head import TritonLinearHead
 
 # largest mixing group the one-pass mix/softmax/mix kernel keeps in registers
 _FUSED_MAX_GROUP = 8
+# where the one-pass post-softmax conv + head mixing kernel is used (see forward)
+_CONV_MIX_MAX_GROUP = 4
+_CONV_MIX_SIZES = ((3, 3), (7, 7))
 
 
 @dataclass
@@ -178,7 +182,10 @@ class MTAAttentionTriton(nn.Module):
                 scores = ops.headmix_softmax(scores, None, None, self.causal, key_bias=key_bias,
                                              fill_upper=post_conv_identity and w2 is None and not own_pv)
             done = None
-            if not post_conv_identity and w2 is not None:   # conv and mix in one pass, the conv result never written
+            # conv and mix in one pass, the conv result never written: taken where it measures at least as fast as the
+            # two kernels (mixing groups of up to 4 heads, kernel sizes with a vector-staged instance: 3x3, 7x7)
+            ks = tuple(self.mta_conv_after_sm_triton.weight.shape[1:])
+            if not post_conv_identity and w2 is not None and g_post <= _CONV_MIX_MAX_GROUP and ks in _CONV_MIX_SIZES:
                 self._mark("conv_mix_post")
                 done = ops.conv2d_headmix(scores, self.mta_conv_after_sm_triton.weight, w_post, self.causal,
                                           group_size=g_post, fill_upper=not own_pv)
