@@ -311,7 +311,7 @@ typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
 // The scores-only kernel pins its conv phase by hand instead (reads issued from assembly, see below).
 constexpr int F_BK = 64;   // keys per iteration
 constexpr int QK_OCC = 3;     // wavefronts per SIMD the scores-only kernel is compiled for (three workgroups per CU)
-constexpr int QK_CHUNK = 32;  // key blocks per work item of the scores-only kernel
+constexpr int QK_CHUNK = 48;  // key blocks per work item of the scores-only kernel (24..128 measured at S = 4096)
 constexpr int F_SLD = 80;  // score-tile row stride (elements): exactly the retained columns + one key block.  A wider
                            // row costs the scores-only kernel its third workgroup per CU, and with this one a fragment
                            // read (16 consecutive rows x 64 bytes) is free of bank conflicts as it is: the LDS serves
@@ -334,6 +334,10 @@ __device__ __forceinline__ void lds_write8_at(unsigned addr, int off, uint32_t l
     const u32x2_t v = {lo, hi};
     asm volatile("ds_write_b64 %0, %1 offset:%2" : : "v"(addr), "v"(v), "n"(off) : "memory");
 }
+__device__ __forceinline__ void lds_write16_at(unsigned addr, int off, u32x4_t v)
+{
+    asm volatile("ds_write_b128 %0, %1 offset:%2" : : "v"(addr), "v"(v), "n"(off) : "memory");
+}
 template <int N> __device__ __forceinline__ void lds_wait_upto(u32x4_t &v)
 {
     asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(N) : "memory");
@@ -348,6 +352,19 @@ template <int N, typename F> __device__ __forceinline__ void static_for(F &&f)
 {
     static_for_impl(std::make_integer_sequence<int, N>{}, f);
 }
+// The scores-only kernel writes the scores of 16-key blocks cb-1 and cb (cb odd, both row blocks: two writes) right
+// after step (cb+1)*KS + LAG - 1 of its score phase; the last pair after the loop.  Number of those writes issued at the
+// end of a step in [lo, hi).
+constexpr int score_writes_between(int lo, int hi, int KS, int NCB, int LAG)
+{
+    int c = 0;
+    for (int cb = 1; cb + 1 < NCB; cb += 2) {
+        const int s = (cb + 1) * KS + LAG - 1;
+        if (s >= lo && s < hi) c += 2;
+    }
+    return c;
+}
+
 // Returns its argument, opaquely: what is derived from the result cannot be hoisted out of the block that computes it.
 __device__ __forceinline__ int opaque_lane(int v)
 {
@@ -568,6 +585,77 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
         if (j < j_end) issue_kv(j + 1, Kn, Vn);  // lands while this block is being worked on
 
         // ---- S^T = K Q^T, zero above the diagonal / outside the sequence, to the score tile ----
+        if constexpr (SCORES_ONLY) {
+            // Pipelined like the conv phase below: K fragments are read from assembly KLD steps (two 16-key blocks)
+            // ahead into a ring of registers, a step being one fragment and the two products it feeds (both row
+            // blocks); a block's scores are rounded, scaled, masked and written LAG steps into the next block.
+            constexpr int NSTEP = NCB * KS, KLD = 2 * KS, KSLOT = KLD + 1, LAG = 2;
+            static_assert(NSTEP > KLD && KS >= LAG && NCB % 2 == 0, "pipeline deeper than the work; blocks are written in pairs");
+            unsigned ka[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                ka[ks] = lds_addr(Kb) + (unsigned)((ln * D + (((ks * 4 + kg) ^ (ln & (CPR - 1))) * 8)) * (int)sizeof(T));
+            const unsigned wa = lds_addr(Sc) + (unsigned)((trow[0] * F_SLD + G::HC + (kg & 1) * 16 + (kg >> 1) * 8) * (int)sizeof(T));
+            u32x4_t kring[KSLOT];
+            f32x4 sacc[2][2];
+            uint32_t held[2][2];
+            auto kissue = [&](auto ic) __attribute__((always_inline)) {
+                constexpr int n = decltype(ic)::value;
+                kring[n % KSLOT] = lds_read16_at(ka[n % KS], (n / KS) * 16 * D * (int)sizeof(T));
+            };
+            auto epilogue = [&](auto cbc) __attribute__((always_inline)) {
+                constexpr int cb = decltype(cbc)::value;
+                // key block wholly inside the sequence and on or below the diagonal for all 32 rows: no masks
+                const bool s_plain = PLAIN || (cbase + cb * 16 >= 0 && cbase + cb * 16 + 16 <= S && (!causal || cbase + cb * 16 + 15 <= pmin));
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb) {
+                    const f32x4 a = sacc[cb & 1][rb];
+                    // MTA scales the scores before the conv, in the I/O dtype: round, scale, round again
+                    float a0, a1, a2, a3;
+                    unpack2<T>(pack2<T>(a[0], a[1]), a0, a1);
+                    unpack2<T>(pack2<T>(a[2], a[3]), a2, a3);
+                    uint32_t lo = pack2<T>(a0 * scale, a1 * scale), hi = pack2<T>(a2 * scale, a3 * scale);
+                    if (!s_plain) {
+                        const int col = cbase + cb * 16 + kg * 4;
+                        const int lim = causal ? (prow[rb] < S - 1 ? prow[rb] : S - 1) : S - 1;  // last key kept
+                        if (col < 0 || col > lim) lo &= 0xffff0000u;
+                        if (col + 1 < 0 || col + 1 > lim) lo &= 0x0000ffffu;
+                        if (col + 2 < 0 || col + 2 > lim) hi &= 0xffff0000u;
+                        if (col + 3 < 0 || col + 3 > lim) hi &= 0x0000ffffu;
+                    }
+                    // (blocks go to the tile in pairs, as 16-byte vectors: see the exchange in the other branch)
+                    if constexpr ((cb & 1) == 0) {
+                        held[rb][0] = lo;
+                        held[rb][1] = hi;
+                    } else {
+                        const u32x2_t s0 = __builtin_amdgcn_permlane16_swap(held[rb][0], lo, false, false);
+                        const u32x2_t s1 = __builtin_amdgcn_permlane16_swap(held[rb][1], hi, false, false);
+                        lds_write16_at(wa, (rb * 16 * F_SLD + (cb - 1) * 16) * (int)sizeof(T), u32x4_t{s0[0], s1[0], s0[1], s1[1]});
+                    }
+                }
+            };
+            static_for<KLD>(kissue);
+            static_for<NSTEP>([&](auto ic) __attribute__((always_inline)) {
+                constexpr int n = decltype(ic)::value;
+                constexpr int cb = n / KS, ks = n % KS;
+                if constexpr (n + KLD < NSTEP) kissue(std::integral_constant<int, n + KLD>{});
+                // LDS operations younger than read n: the reads issued after it and the score writes issued since
+                constexpr int younger = (n + KLD < NSTEP ? n + KLD : NSTEP - 1) - n + score_writes_between(n > KLD ? n - KLD : 0, n, KS, NCB, LAG);
+                lds_wait_upto<(younger < 15 ? younger : 15)>(kring[n % KSLOT]);
+                if constexpr (ks == 0) {
+                    sacc[cb & 1][0] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                    sacc[cb & 1][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                }
+                mma16(sacc[cb & 1][0], __builtin_bit_cast(frag8<T>, kring[n % KSLOT]), qf[0][ks]);
+                mma16(sacc[cb & 1][1], __builtin_bit_cast(frag8<T>, kring[n % KSLOT]), qf[1][ks]);
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (cb >= 1 && ks == LAG - 1) {
+                    epilogue(std::integral_constant<int, cb - 1>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            });
+            epilogue(std::integral_constant<int, NCB - 1>{});
+        } else
         // The K fragments of key block cb+1 are read from LDS while the matrix cores work on block cb.
         {
             frag8<T> kf[2][KS];
