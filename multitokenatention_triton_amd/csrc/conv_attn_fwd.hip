@@ -758,8 +758,10 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
             // Pack and mask output block b.  Blocks leave in pairs, like the scores above: after the exchange a lane
             // holds 8 consecutive keys of one of the two blocks and stores them itself, 16 rows x 64 bytes per
             // instruction; no staging through LDS.
-            // (non-temporal: the scores are written once and next read by another kernel; as ordinary stores they
-            // would push this head's K blocks, which every workgroup of the head re-reads, out of the L2)
+            // (Ordinary stores: a 128-byte line is completed by two instructions a few hundred cycles apart, and the L2
+            // merges them.  Marked non-temporal, each 64-byte half went to memory on its own and the write counter
+            // read 1.38 times the bytes; the price of the merge is that the scores displace some of the head's K blocks
+            // from the L2 - fetches 79 -> 196 MB per launch at the benchmark shape, 825 -> 736 MB in total, 4 % faster.)
             auto finish = [&](auto bc) __attribute__((always_inline)) {
                 constexpr int b = decltype(bc)::value;
                 constexpr int rb = b / NCB, cb = b % NCB;
@@ -784,8 +786,7 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
                     const int kg_o = opaque_lane(kg);
                     const int col = j * F_BK + (cb - 1 + (kg_o & 1)) * 16 + (kg_o >> 1) * 8;
                     if (tr_ >= G::HR && tr_ < wave * 32 + 32 && p_ < S && (PLAIN || (col < S && (!causal || fill_upper || col <= p_))))
-                        __builtin_nontemporal_store(u32x4_t{s0[0], s1[0], s0[1], s1[1]},
-                                                    reinterpret_cast<u32x4_t *>(Op + (int64_t)p_ * S + col));
+                        *reinterpret_cast<u32x4_t *>(Op + (int64_t)p_ * S + col) = u32x4_t{s0[0], s1[0], s0[1], s1[1]};
                 }
             };
             static_for<NLD>(issue);
