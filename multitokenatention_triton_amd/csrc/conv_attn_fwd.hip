@@ -311,7 +311,8 @@ typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
 // The scores-only kernel pins its conv phase by hand instead (reads issued from assembly, see below).
 constexpr int F_BK = 64;   // keys per iteration
 constexpr int QK_OCC = 3;     // wavefronts per SIMD the scores-only kernel is compiled for (three workgroups per CU)
-constexpr int QK_CHUNK = 48;  // key blocks per work item of the scores-only kernel (24..128 measured at S = 4096)
+constexpr int QK_CHUNK = 32;  // key blocks per work item of the scores-only kernel (24..128 measured at S = 4096,
+                              // with the items started longest first)
 constexpr int F_SLD = 80;  // score-tile row stride (elements): exactly the retained columns + one key block.  A wider
                            // row costs the scores-only kernel its third workgroup per CU, and with this one a fragment
                            // read (16 consecutive rows x 64 bytes) is free of bank conflicts as it is: the LDS serves
@@ -365,6 +366,33 @@ constexpr int score_writes_between(int lo, int hi, int KS, int NCB, int LAG)
     return c;
 }
 
+// a.lo*b.lo + a.hi*b.hi + c for two packed pairs of the 16-bit type T, accumulated in fp32
+template <typename T> __device__ __forceinline__ float dot2_io(uint32_t a, uint32_t b, float c)
+{
+    if constexpr (std::is_same<T, bf16_t>::value) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(mta_bf16x2, a), __builtin_bit_cast(mta_bf16x2, b), c, false);
+    } else {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(mta_f16x2, a), __builtin_bit_cast(mta_f16x2, b), c, false);
+    }
+}
+
+// max / sum over the four lane groups (lanes l, l^16, l^32, l^48) that share a query row, in every lane: two
+// exchanges between whole rows of lanes on the vector ALU (no LDS permute, so the LDS counter stays ours to count)
+__device__ __forceinline__ float max_across_groups(float v)
+{
+    u32x2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_across_groups(float v)
+{
+    u32x2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // Returns its argument, opaquely: what is derived from the result cannot be hoisted out of the block that computes it.
 __device__ __forceinline__ int opaque_lane(int v)
 {
@@ -393,6 +421,16 @@ template <int R, int SK, int NW> struct fused_geom {
     static constexpr int WZ_OFF = SHIFT + 16, WZ_LD = WZ_OFF + 32;
 };
 
+// A head's work items (query block, key chunk) in the order they are to be started: longest first, so that the long
+// items all start early and the short ones fill the end of the grid.  Built on the host for every launch (a counting
+// sort over at most ITEM_TABLE_MAX items) and passed by value as a kernel argument; n = 0: no table, the kernel
+// walks the query blocks from the last to the first instead.
+constexpr int ITEM_TABLE_MAX = 1024;
+struct item_table {
+    int n;
+    uint16_t e[ITEM_TABLE_MAX];  // query block (11 bits) | key chunk << 11
+};
+
 // SCORES_ONLY: stop after the conv and write  conv(mask0(scale * Q K^T))  as an (S,S) plane per (batch, head)
 // (`O` is then the score tensor, V is unused).  Only q <= p is written when causal, plus +0 above the
 // diagonal when `fill_upper` is set.
@@ -401,7 +439,8 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
                                                              const T *__restrict__ V, const T *__restrict__ Wt,
                                                              T *__restrict__ O, float *__restrict__ Lse, int S, int causal,
                                                              float scale, int H, int nqb, int fill_upper, int64_t total_wg,
-                                                             int64_t per_xcd, int jc_len, int items_per_bh, int hpx)
+                                                             int64_t per_xcd, int jc_len, int items_per_bh, int hpx,
+                                                             item_table tbl)
 {
     using G = fused_geom<R, SK, NW>;
     constexpr int F_NT = 64 * NW, F_SR = 32 * NW;
@@ -448,13 +487,19 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
     // the attention kernel accumulates over all keys and gets jc_len = all of them.
     const int64_t bh = lid / items_per_bh;
     int item = (int)(lid % items_per_bh), qb = nqb - 1, jc = 0;
-    for (; qb > 0; --qb) {  // longest query blocks first
-        const int ql = (qb * G::BQ + G::BQ - 1 < S - 1) ? qb * G::BQ + G::BQ - 1 : S - 1;
-        const int nch = ((causal ? ql / F_BK : (S - 1) / F_BK) + jc_len) / jc_len;
-        if (item < nch) break;
-        item -= nch;
+    if (tbl.n > 0) {
+        const unsigned e = tbl.e[item];
+        qb = (int)(e & 2047u);
+        jc = (int)(e >> 11);
+    } else {
+        for (; qb > 0; --qb) {  // longest query blocks first
+            const int ql = (qb * G::BQ + G::BQ - 1 < S - 1) ? qb * G::BQ + G::BQ - 1 : S - 1;
+            const int nch = ((causal ? ql / F_BK : (S - 1) / F_BK) + jc_len) / jc_len;
+            if (item < nch) break;
+            item -= nch;
+        }
+        jc = item;
     }
-    jc = item;
     const int head = (int)(bh % H);
     const int q0 = qb * G::BQ;
     const T *Qp = Q + bh * (int64_t)S * D;
@@ -564,6 +609,20 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
     }
     // the two 16-row blocks of this wavefront span rows pmin..pmin+31 of the sequence
     const int pmin = q0 - G::HR + wave * 32;
+    // Rows of the conv (and of everything after it: softmax, P V, the stores).  The first wavefront's rows are taken
+    // R-1 further down than the rows it computes scores for: its conv windows then start at tile row 0 instead of
+    // above the tile, every fragment address is the same affine function of (row block, kernel row), and what it
+    // leaves out are halo rows nobody stores.  Its last R-1 rows belong to the second wavefront too and are not
+    // stored from here.
+    const int cshift = wave == 0 ? R - 1 : 0;
+    int cprow[2];
+    bool row_stored[2];
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+        const int tr_ = trow[rb] + cshift;
+        cprow[rb] = prow[rb] + cshift;
+        row_stored[rb] = tr_ >= G::HR && tr_ < wave * 32 + 32 && cprow[rb] < S;
+    }
 
     // PLAIN: the key block (its scores and its conv outputs) lies inside the sequence and on or below the diagonal
     // for all 32 rows of this wavefront: no masks and no per-sub-block tests (most blocks of a long sequence)
@@ -585,7 +644,7 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
         if (j < j_end) issue_kv(j + 1, Kn, Vn);  // lands while this block is being worked on
 
         // ---- S^T = K Q^T, zero above the diagonal / outside the sequence, to the score tile ----
-        if constexpr (SCORES_ONLY) {
+        {
             // Pipelined like the conv phase below: K fragments are read from assembly KLD steps (two 16-key blocks)
             // ahead into a ring of registers, a step being one fragment and the two products it feeds (both row
             // blocks); a block's scores are rounded, scaled, masked and written LAG steps into the next block.
@@ -610,11 +669,14 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
 #pragma unroll
                 for (int rb = 0; rb < 2; ++rb) {
                     const f32x4 a = sacc[cb & 1][rb];
-                    // MTA scales the scores before the conv, in the I/O dtype: round, scale, round again
-                    float a0, a1, a2, a3;
-                    unpack2<T>(pack2<T>(a[0], a[1]), a0, a1);
-                    unpack2<T>(pack2<T>(a[2], a[3]), a2, a3);
-                    uint32_t lo = pack2<T>(a0 * scale, a1 * scale), hi = pack2<T>(a2 * scale, a3 * scale);
+                    uint32_t lo = pack2<T>(a[0], a[1]), hi = pack2<T>(a[2], a[3]);
+                    if (SCORES_ONLY) {  // MTA scales the scores before the conv, in the I/O dtype: round, scale, round again
+                        float a0, a1, a2, a3;
+                        unpack2<T>(lo, a0, a1);
+                        unpack2<T>(hi, a2, a3);
+                        lo = pack2<T>(a0 * scale, a1 * scale);
+                        hi = pack2<T>(a2 * scale, a3 * scale);
+                    }
                     if (!s_plain) {
                         const int col = cbase + cb * 16 + kg * 4;
                         const int lim = causal ? (prow[rb] < S - 1 ? prow[rb] : S - 1) : S - 1;  // last key kept
@@ -623,7 +685,10 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
                         if (col + 2 < 0 || col + 2 > lim) hi &= 0xffff0000u;
                         if (col + 3 < 0 || col + 3 > lim) hi &= 0x0000ffffu;
                     }
-                    // (blocks go to the tile in pairs, as 16-byte vectors: see the exchange in the other branch)
+                    // Two 16-key blocks go to the tile together.  A lane holds keys 4kg..4kg+3 of each; after the
+                    // exchange between neighbouring lane groups (even groups give their second block's part and take
+                    // the neighbour's first block's part) it holds 8 consecutive keys of one block: one 16-byte write
+                    // per lane and block pair instead of two 8-byte ones, which conflicted four ways in the banks.
                     if constexpr ((cb & 1) == 0) {
                         held[rb][0] = lo;
                         held[rb][1] = hi;
@@ -655,119 +720,50 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
                 }
             });
             epilogue(std::integral_constant<int, NCB - 1>{});
-        } else
-        // The K fragments of key block cb+1 are read from LDS while the matrix cores work on block cb.
-        {
-            frag8<T> kf[2][KS];
-            auto load_kf = [&](int cb, frag8<T> (&dst)[KS]) {
-                const int krow = cb * 16 + ln;
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks)
-                    dst[ks] = *reinterpret_cast<const frag8<T> *>(Kb + krow * D + (((ks * 4 + kg) ^ (krow & (CPR - 1))) * 8));
-            };
-            load_kf(0, kf[0]);
-            uint32_t held[2][2];
-            static_assert(NCB % 2 == 0, "score blocks are written in pairs");
-#pragma unroll
-            for (int cb = 0; cb < NCB; ++cb) {
-                if (cb + 1 < NCB) load_kf(cb + 1, kf[(cb + 1) & 1]);
-                f32x4 sacc[2] = {f32x4{0.0f, 0.0f, 0.0f, 0.0f}, f32x4{0.0f, 0.0f, 0.0f, 0.0f}};
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    mma16(sacc[0], kf[cb & 1][ks], qf[0][ks]);
-                    mma16(sacc[1], kf[cb & 1][ks], qf[1][ks]);
-                }
-                // key block wholly inside the sequence and on or below the diagonal for all 32 rows: no masks
-                const bool s_plain = PLAIN || (cbase + cb * 16 >= 0 && cbase + cb * 16 + 16 <= S && (!causal || cbase + cb * 16 + 15 <= pmin));
-#pragma unroll
-                for (int rb = 0; rb < 2; ++rb) {
-                    uint32_t lo = pack2<T>(sacc[rb][0], sacc[rb][1]), hi = pack2<T>(sacc[rb][2], sacc[rb][3]);
-                    if (SCORES_ONLY) {  // MTA scales the scores before the conv, in the I/O dtype: round, scale, round again
-                        float a0, a1, a2, a3;
-                        unpack2<T>(lo, a0, a1);
-                        unpack2<T>(hi, a2, a3);
-                        lo = pack2<T>(a0 * scale, a1 * scale);
-                        hi = pack2<T>(a2 * scale, a3 * scale);
-                    }
-                    if (!s_plain) {
-                        const int col = cbase + cb * 16 + kg * 4;
-                        const int lim = causal ? (prow[rb] < S - 1 ? prow[rb] : S - 1) : S - 1;  // last key kept
-                        if (col < 0 || col > lim) lo &= 0xffff0000u;
-                        if (col + 1 < 0 || col + 1 > lim) lo &= 0x0000ffffu;
-                        if (col + 2 < 0 || col + 2 > lim) hi &= 0xffff0000u;
-                        if (col + 3 < 0 || col + 3 > lim) hi &= 0x0000ffffu;
-                    }
-                    // Two 16-key blocks go to the tile together.  A lane holds keys 4kg..4kg+3 of each; after the
-                    // exchange between neighbouring lane groups (even groups give their second block's part and take
-                    // the neighbour's first block's part) it holds 8 consecutive keys of one block: one 16-byte write
-                    // per lane and block pair instead of two 8-byte ones, which conflicted four ways in the banks.
-                    if ((cb & 1) == 0) {
-                        held[rb][0] = lo;
-                        held[rb][1] = hi;
-                    } else {
-                        const u32x2_t s0 = __builtin_amdgcn_permlane16_swap(held[rb][0], lo, false, false);
-                        const u32x2_t s1 = __builtin_amdgcn_permlane16_swap(held[rb][1], hi, false, false);
-                        *reinterpret_cast<u32x4_t *>(Sc + trow[rb] * F_SLD + G::HC + (cb - 1 + (kg & 1)) * 16 + (kg >> 1) * 8) =
-                            u32x4_t{s0[0], s1[0], s0[1], s1[1]};
-                    }
-                }
-            }
         }
         // score tile complete for everybody.  Only the LDS counter is waited for: a fence would also wait for the
         // copy of the next key block, in flight since the top of the iteration
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         if (j < j_lo) return;
 
-        // score fragments of block blk = rb*NCB+cb: rows trow-(R-1)+i, the block's 32-key window
-        auto load_xf = [&](int blk, frag8<T> (&dst)[R]) {
-            const int rb = blk / NCB, cb = blk % NCB;
-#pragma unroll
-            for (int i = 0; i < R; ++i) {
-                int srow = trow[rb] - (R - 1) + i;
-                srow = srow < 0 ? 0 : srow;  // only halo rows (discarded) can reach above the tile
-                dst[i] = *reinterpret_cast<const frag8<T> *>(Sc + srow * F_SLD + cb * 16 + kg * 8);
-            }
+        // ---- conv (Toeplitz MFMAs over the score tile) -> global (scores only) / -> online softmax ----
+        // One product needs one fresh 1 KB score fragment from LDS, and a wavefront that waits for each fragment
+        // where it is used spends four times the products' own time here.  The reads are therefore issued NLD
+        // products ahead, from assembly (see lds_read16_at), into a ring of registers; every product is preceded by
+        // a wait that leaves exactly the younger operations outstanding.  The result of an output block is taken up
+        // LAG products into the next block, when it is long complete.
+        constexpr int NB = 2 * NCB, NREAD = NB * R;
+        // score fragments in flight (scores only: 8 and 12 measure the same, 15 spills; the attention kernel, at the
+        // 256-register limit, spills from 6 on)
+        constexpr int NLD = SCORES_ONLY ? 8 : 4;
+        constexpr int NSLOT = NLD + 1;
+        constexpr int LAG = 2;
+        static_assert(NREAD > NLD && R >= LAG && NLD <= 15, "pipeline deeper than the work or than the counter");
+        const unsigned xa = lds_addr(Sc) + (unsigned)(((trow[0] + cshift - (R - 1)) * F_SLD + kg * 8) * (int)sizeof(T));
+        u32x4_t ring[NSLOT];
+        f32x4 cacc[2];
+        auto issue = [&](auto ic) __attribute__((always_inline)) {
+            constexpr int n = decltype(ic)::value;
+            constexpr int blk = n / R, i = n % R;
+            ring[n % NSLOT] = lds_read16_at(xa, (((blk / NCB) * 16 + i) * F_SLD + (blk % NCB) * 16) * (int)sizeof(T));
         };
-
-        if constexpr (SCORES_ONLY) {
-            // ---- conv (Toeplitz MFMAs over the score tile) -> global ----
-            // One product needs one fresh 1 KB score fragment from LDS, and a wavefront that waits for each fragment
-            // where it is used spends four times the products' own time here.  The reads are therefore issued NLD
-            // products ahead, from assembly (see lds_read16_at), into a ring of registers; every product is preceded by
-            // a wait that leaves exactly the younger operations outstanding.  The result of an output block is packed
-            // LAG products into the next block, when it is long complete.
-            constexpr int NB = 2 * NCB, NREAD = NB * R;
-            constexpr int NLD = 8;  // score fragments in flight (8 and 12 measure the same; 15 spills)
-            constexpr int NSLOT = NLD + 1;
-            constexpr int LAG = 2;
-            static_assert(NREAD > NLD && R >= LAG && NLD <= 15, "pipeline deeper than the work or than the counter");
-            // Rows of the conv.  The first wavefront's rows are taken R-1 further down than the rows it computed scores
-            // for: its windows then start at tile row 0 instead of above the tile, every address below is the same
-            // affine function of (row block, kernel row), and what it leaves out are halo rows nobody stores.  Its last
-            // R-1 rows belong to the second wavefront too and are not stored from here.
-            const int cshift = wave == 0 ? R - 1 : 0;
-            const unsigned xa = lds_addr(Sc) + (unsigned)(((trow[0] + cshift - (R - 1)) * F_SLD + kg * 8) * (int)sizeof(T));
-            u32x4_t ring[NSLOT];
-            f32x4 cacc[2];
-            uint32_t held[2];
-            auto issue = [&](auto ic) __attribute__((always_inline)) {
-                constexpr int n = decltype(ic)::value;
-                constexpr int blk = n / R, i = n % R;
-                ring[n % NSLOT] = lds_read16_at(xa, (((blk / NCB) * 16 + i) * F_SLD + (blk % NCB) * 16) * (int)sizeof(T));
-            };
-            // Pack and mask output block b.  Blocks leave in pairs, like the scores above: after the exchange a lane
-            // holds 8 consecutive keys of one of the two blocks and stores them itself, 16 rows x 64 bytes per
-            // instruction; no staging through LDS.
-            // (Ordinary stores: a 128-byte line is completed by two instructions a few hundred cycles apart, and the L2
-            // merges them.  Marked non-temporal, each 64-byte half went to memory on its own and the write counter
-            // read 1.38 times the bytes; the price of the merge is that the scores displace some of the head's K blocks
-            // from the L2 - fetches 79 -> 196 MB per launch at the benchmark shape, 825 -> 736 MB in total, 4 % faster.)
-            auto finish = [&](auto bc) __attribute__((always_inline)) {
-                constexpr int b = decltype(bc)::value;
-                constexpr int rb = b / NCB, cb = b % NCB;
-                const f32x4 a = cacc[b & 1];
+        // what happens to output block b = rb*NCB + cb (rows crow[rb], keys j*64 + 16cb ..) once it is complete
+        uint32_t held[2];           // scores only: the even block of a pair, packed
+        float sv[NCB][4], mloc;     // attention: the row block's scaled logits and their running maximum
+        frag8<T> pf[2][2];          // attention: probabilities, in the operand layout of the P V products
+        auto finish = [&](auto bc) __attribute__((always_inline)) {
+            constexpr int b = decltype(bc)::value;
+            constexpr int rb = b / NCB, cb = b % NCB;
+            const f32x4 a = cacc[b & 1];
+            const int p_ = cprow[rb];
+            if constexpr (SCORES_ONLY) {
+                // Blocks leave in pairs, like the scores above: after the exchange a lane holds 8 consecutive keys of
+                // one of the two blocks and stores them itself, 16 rows x 64 bytes per instruction; no staging through LDS.
+                // (Ordinary stores: a 128-byte line is completed by two instructions a few hundred cycles apart, and the L2
+                // merges them.  Marked non-temporal, each 64-byte half went to memory on its own and the write counter
+                // read 1.38 times the bytes; the price of the merge is that the scores displace some of the head's K blocks
+                // from the L2 - fetches 79 -> 196 MB per launch at the benchmark shape, 825 -> 736 MB in total, 4 % faster.)
                 uint32_t lo = pack2<T>(a[0], a[1]), hi = pack2<T>(a[2], a[3]);
-                const int tr_ = trow[rb] + cshift, p_ = prow[rb] + cshift;
                 if (!PLAIN && causal && j * F_BK + cb * 16 + 15 > pmin) {  // block touches the diagonal for some row
                     const int col = j * F_BK + cb * 16 + kg * 4;
                     if (col > p_) lo &= 0xffff0000u;
@@ -785,90 +781,81 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
                     // of being kept in registers across the key-block loop - the kernel is at its register limit)
                     const int kg_o = opaque_lane(kg);
                     const int col = j * F_BK + (cb - 1 + (kg_o & 1)) * 16 + (kg_o >> 1) * 8;
-                    if (tr_ >= G::HR && tr_ < wave * 32 + 32 && p_ < S && (PLAIN || (col < S && (!causal || fill_upper || col <= p_))))
+                    if (row_stored[rb] && (PLAIN || (col < S && (!causal || fill_upper || col <= p_))))
                         *reinterpret_cast<u32x4_t *>(Op + (int64_t)p_ * S + col) = u32x4_t{s0[0], s1[0], s0[1], s1[1]};
                 }
-            };
-            static_for<NLD>(issue);
-            static_for<NREAD>([&](auto ic) __attribute__((always_inline)) {
-                constexpr int n = decltype(ic)::value;
-                constexpr int blk = n / R, i = n % R;
-                if constexpr (n + NLD < NREAD) issue(std::integral_constant<int, n + NLD>{});
-                // LDS operations younger than read n: exactly the reads issued after it
-                constexpr int younger = (n + NLD < NREAD ? n + NLD : NREAD - 1) - n;
-                lds_wait_upto<younger>(ring[n % NSLOT]);
-                if constexpr (i == 0) cacc[blk & 1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-                mma16(cacc[blk & 1], tz[i], __builtin_bit_cast(frag8<T>, ring[n % NSLOT]));
-                __builtin_amdgcn_sched_barrier(0);
-                if constexpr (blk >= 1 && i == LAG - 1) {
-                    finish(std::integral_constant<int, blk - 1>{});
-                    __builtin_amdgcn_sched_barrier(0);
+            } else {
+                // conv output and scaled logits are rounded to the I/O dtype, as the unfused pipeline stores them
+                float v4[4];
+                unpack2<T>(pack2<T>(a[0], a[1]), v4[0], v4[1]);
+                unpack2<T>(pack2<T>(a[2], a[3]), v4[2], v4[3]);
+                unpack2<T>(pack2<T>(v4[0] * scale, v4[1] * scale), v4[0], v4[1]);
+                unpack2<T>(pack2<T>(v4[2] * scale, v4[3] * scale), v4[2], v4[3]);
+                const bool c_plain = PLAIN || (j * F_BK + cb * 16 + 16 <= S && (!causal || j * F_BK + cb * 16 + 15 <= pmin));
+                if constexpr (cb == 0) mloc = -INFINITY;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    float val = v4[v];
+                    if (!c_plain) {
+                        const int col = j * F_BK + cb * 16 + kg * 4 + v;
+                        if (!(col < S && !(causal && col > p_))) val = -INFINITY;
+                    }
+                    sv[cb][v] = val;
+                    mloc = fmaxf(mloc, val);
                 }
-            });
-            finish(std::integral_constant<int, NB - 1>{});
-            return;
-        }
-
-        // ---- conv (Toeplitz MFMAs over the score tile), scale, mask, online softmax ----
-        frag8<T> pf[2][2];
-        {
-            frag8<T> xf[2][R];
-            load_xf(0, xf[0]);
+                if constexpr (cb == NCB - 1) {  // the row block is complete: online softmax (a row lives in 4 lanes)
+                    mloc = max_across_groups(mloc);
+                    const float m_new = fmaxf(m_i[rb], mloc);
+                    const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+                    // exp(x - m) = exp2(x*log2(e) - m*log2(e)): one multiply-add and one v_exp per element
+                    constexpr float LOG2E = 1.4426950408889634f;
+                    const float mneg = -m_use * LOG2E;
+                    const float alpha = __builtin_amdgcn_exp2f(fmaf(m_i[rb], LOG2E, mneg));
+                    m_i[rb] = m_new;
+                    float lsum = 0.0f;
+                    const uint32_t ones = pack2<T>(1.0f, 1.0f);
 #pragma unroll
-            for (int rb = 0; rb < 2; ++rb) {
-                float sv[NCB][4];
-                float mloc = -INFINITY;
+                    for (int c = 0; c < NCB; ++c) {
+                        float e[4];
 #pragma unroll
-                for (int cb = 0; cb < NCB; ++cb) {
-                    const int blk = rb * NCB + cb;
-                    if (blk + 1 < 2 * NCB) load_xf(blk + 1, xf[(blk + 1) & 1]);
-                        f32x4 cacc = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                        for (int v = 0; v < 4; ++v) e[v] = __builtin_amdgcn_exp2f(fmaf(sv[c][v], LOG2E, mneg));
+                        const uint32_t lo = pack2<T>(e[0], e[1]), hi = pack2<T>(e[2], e[3]);
+                        // the row sum runs over the rounded probabilities (what the P V products see): a packed dot
+                        // product with (1, 1) adds a pair in one instruction
+                        lsum = dot2_io<T>(lo, ones, lsum);
+                        lsum = dot2_io<T>(hi, ones, lsum);
+                        uint32_t *dst = reinterpret_cast<uint32_t *>(&pf[rb][c >> 1]) + (c & 1) * 2;
+                        dst[0] = lo;
+                        dst[1] = hi;
+                    }
+                    l_i[rb] = l_i[rb] * alpha + lsum;
+                    // (once the running maxima have settled, alpha is 1 in every lane for most key blocks: the 4*DB
+                    // multiplications are skipped for the wavefront then)
+                    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-                    for (int i = 0; i < R; ++i) mma16(cacc, tz[i], xf[blk & 1][i]);
-                        // conv output and scaled logits are rounded to the I/O dtype, as the unfused pipeline stores them
-                    float a[4];
-                    unpack2<T>(pack2<T>(cacc[0], cacc[1]), a[0], a[1]);
-                    unpack2<T>(pack2<T>(cacc[2], cacc[3]), a[2], a[3]);
-                    unpack2<T>(pack2<T>(a[0] * scale, a[1] * scale), a[0], a[1]);
-                    unpack2<T>(pack2<T>(a[2] * scale, a[3] * scale), a[2], a[3]);
-                    const bool c_plain = PLAIN || (j * F_BK + cb * 16 + 16 <= S && (!causal || j * F_BK + cb * 16 + 15 <= pmin));
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        float val = a[v];
-                        if (!c_plain) {
-                            const int col = j * F_BK + cb * 16 + kg * 4 + v;
-                            if (!(col < S && !(causal && col > prow[rb]))) val = -INFINITY;
-                        }
-                        sv[cb][v] = val;
-                        mloc = fmaxf(mloc, val);
+                        for (int db = 0; db < DB; ++db) oacc[rb][db] *= alpha;
                     }
                 }
-                mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
-                mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-                const float m_new = fmaxf(m_i[rb], mloc);
-                const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-                const float alpha = __expf(m_i[rb] - m_use);
-                m_i[rb] = m_new;
-                float lsum = 0.0f;
-#pragma unroll
-                for (int cb = 0; cb < NCB; ++cb) {
-                    float e[4];
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) e[v] = __expf(sv[cb][v] - m_use);
-                    const uint32_t lo = pack2<T>(e[0], e[1]), hi = pack2<T>(e[2], e[3]);
-                    float r0, r1, r2, r3;
-                    unpack2<T>(lo, r0, r1);
-                    unpack2<T>(hi, r2, r3);
-                    lsum += (r0 + r1) + (r2 + r3);
-                    uint32_t *dst = reinterpret_cast<uint32_t *>(&pf[rb][cb >> 1]) + (cb & 1) * 2;
-                    dst[0] = lo;
-                    dst[1] = hi;
-                }
-                l_i[rb] = l_i[rb] * alpha + lsum;
-#pragma unroll
-                for (int db = 0; db < DB; ++db) oacc[rb][db] *= alpha;
             }
-        }
+        };
+        static_for<NLD>(issue);
+        static_for<NREAD>([&](auto ic) __attribute__((always_inline)) {
+            constexpr int n = decltype(ic)::value;
+            constexpr int blk = n / R, i = n % R;
+            if constexpr (n + NLD < NREAD) issue(std::integral_constant<int, n + NLD>{});
+            // LDS operations younger than read n: exactly the reads issued after it
+            constexpr int younger = (n + NLD < NREAD ? n + NLD : NREAD - 1) - n;
+            lds_wait_upto<younger>(ring[n % NSLOT]);
+            if constexpr (i == 0) cacc[blk & 1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            mma16(cacc[blk & 1], tz[i], __builtin_bit_cast(frag8<T>, ring[n % NSLOT]));
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (blk >= 1 && i == LAG - 1) {
+                finish(std::integral_constant<int, blk - 1>{});
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        });
+        finish(std::integral_constant<int, NB - 1>{});
+        if constexpr (SCORES_ONLY) return;
 
         // ---- O^T += V^T P^T ; V^T fragments via the LDS transpose read of the row-major V block ----
         {
@@ -930,17 +917,15 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
     // ---- normalise and store (halo rows are dropped) ----
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb) {
-        float l_row = l_i[rb];
-        l_row += __shfl_xor(l_row, 16);
-        l_row += __shfl_xor(l_row, 32);
-        if (trow[rb] >= G::HR && prow[rb] < S) {
+        const float l_row = sum_across_groups(l_i[rb]);
+        if (row_stored[rb]) {
             const float inv = 1.0f / l_row;
-            if (Lse != nullptr && kg == 0) Lse[bh * (int64_t)S + prow[rb]] = m_i[rb] + __logf(l_row);
+            if (Lse != nullptr && kg == 0) Lse[bh * (int64_t)S + cprow[rb]] = m_i[rb] + __logf(l_row);
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 const uint32_t lo = pack2<T>(oacc[rb][db][0] * inv, oacc[rb][db][1] * inv);
                 const uint32_t hi = pack2<T>(oacc[rb][db][2] * inv, oacc[rb][db][3] * inv);
-                *reinterpret_cast<uint2 *>(Op + (int64_t)prow[rb] * D + db * 16 + kg * 4) = make_uint2(lo, hi);
+                *reinterpret_cast<uint2 *>(Op + (int64_t)cprow[rb] * D + db * 16 + kg * 4) = make_uint2(lo, hi);
             }
         }
     }
@@ -965,10 +950,52 @@ int launch_mfma(const void *q, const void *k, const void *v, const void *w, void
     }
     const int64_t total_wg = B * H * items_per_bh, per_xcd = (total_wg + 7) / 8;
     if (per_xcd * 8 > 0x7fffffffLL || items_per_bh > 0x7fffffffLL) return MTA_ERR_SHAPE;
+    // the items of a head, longest first (the number of key blocks an item visits, as the kernel computes it)
+    item_table tbl;
+    tbl.n = 0;
+    if (SCORES_ONLY && items_per_bh <= ITEM_TABLE_MAX && nqb <= 2047 && items_per_bh > 1) {
+        constexpr int MAXLEN = 4096;
+        static thread_local int count[MAXLEN + 2];
+        bool ok = true;
+        auto length = [&](int qb, int jc) {
+            const int64_t ql = std::min<int64_t>((int64_t)qb * G::BQ + G::BQ - 1, S - 1);
+            const int j_last = (int)(causal ? ql / F_BK : (S - 1) / F_BK);
+            const int j_lo = jc * jc_len, j_end = std::min(j_lo + jc_len - 1, j_last);
+            const int j_start = j_lo > 0 ? j_lo - 1 : (G::PWR > 0 ? -1 : 0);
+            return j_end - j_start + 1;
+        };
+        auto chunks = [&](int qb) {
+            const int64_t ql = std::min<int64_t>((int64_t)qb * G::BQ + G::BQ - 1, S - 1);
+            return (int)(((causal ? ql / F_BK : (S - 1) / F_BK) + jc_len) / jc_len);
+        };
+        std::fill(count, count + MAXLEN + 2, 0);
+        for (int qb = 0; qb < nqb && ok; ++qb) {
+            const int nch = chunks(qb);
+            if (nch > 31) ok = false;
+            for (int jc = 0; jc < nch && ok; ++jc) {
+                const int len = length(qb, jc);
+                if (len < 0 || len > MAXLEN) ok = false;
+                else ++count[len];
+            }
+        }
+        if (ok) {
+            // positions: longer items first; among equal lengths later query blocks first
+            int pos = 0;
+            for (int len = MAXLEN; len >= 0; --len) {
+                const int c = count[len];
+                count[len] = pos;
+                pos += c;
+            }
+            for (int qb = nqb - 1; qb >= 0; --qb)
+                for (int jc = 0, nch = chunks(qb); jc < nch; ++jc)
+                    tbl.e[count[length(qb, jc)]++] = (uint16_t)(qb | (jc << 11));
+            tbl.n = (int)items_per_bh;
+        }
+    }
     dim3 grid((unsigned)(per_xcd * 8));
     hipLaunchKernelGGL(kern, grid, dim3(F_NT), 0, st, (const T *)q, (const T *)k, (const T *)v, (const T *)w, (T *)o,
                        lse, (int)S, causal, scale, (int)H, nqb, fill_upper, total_wg, per_xcd, jc_len, (int)items_per_bh,
-                       (B * H) % 8 == 0 ? (int)(B * H / 8) : 0);
+                       (B * H) % 8 == 0 ? (int)(B * H / 8) : 0, tbl);
     return launch_status();
 }
 
