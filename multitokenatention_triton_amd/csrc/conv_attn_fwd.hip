@@ -393,6 +393,11 @@ __device__ __forceinline__ float sum_across_groups(float v)
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// Inside a rarely taken, wavefront-uniform `if`: keeps it a branch.  Without it the compiler turns the masks of the
+// diagonal key blocks into selects that every key block executes (a third of the attention kernel's vector
+// instructions).
+#define MTA_KEEP_BRANCH() asm volatile("" ::: "memory")
+
 // Returns its argument, opaquely: what is derived from the result cannot be hoisted out of the block that computes it.
 __device__ __forceinline__ int opaque_lane(int v)
 {
@@ -455,16 +460,21 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
     // Every buffer is an array of its own, and the key-block loop body is instantiated once per K/V buffer: the
     // compiler then sees that LDS reads never touch the asynchronous copy in flight into the other buffer.  With one
     // block of dynamic LDS it cannot, and waits for the copy ahead of the first LDS read that follows its issue.
-    __shared__ __align__(16) T Kt0[TILE];
-    __shared__ __align__(16) T Kt1[TILE];
-    __shared__ __align__(16) T Vt0[SCORES_ONLY ? 8 : TILE];
-    __shared__ __align__(16) T Vt1[SCORES_ONLY ? 8 : TILE];
+    // The scores-only kernel double-buffers K in B0 / B1.  The attention kernel rotates K and V through three
+    // buffers: in an iteration K(j) sits in one, V(j) in another; K(j+1) is copied into the third from the top of the
+    // iteration on, and V(j+1) into K(j)'s buffer once the score phase is over (the barrier in the middle of the
+    // iteration).  Three 16 KB buffers and the score tile are 68 KB: two workgroups per CU, which overlap each
+    // other's vector-ALU and matrix-core phases (a single workgroup's wavefronts meet at two barriers per key block
+    // and are all in the same phase at the same time).
+    __shared__ __align__(16) T B0[TILE];
+    __shared__ __align__(16) T B1[TILE];
+    __shared__ __align__(16) T B2[SCORES_ONLY ? 8 : TILE];
     __shared__ __align__(16) T Sc[F_SR * F_SLD];                          // score tile
-    // zero-padded kernel rows, only needed until the Toeplitz fragments are built: they borrow the second K buffer,
-    // which receives its first copy after that (LDS is granted in 1280-byte units; the array's own 648 bytes were
-    // the difference between two and three workgroups per CU for the scores-only kernel)
+    // zero-padded kernel rows, only needed until the Toeplitz fragments are built: they borrow a buffer that
+    // receives its first copy after that (LDS is granted in 1280-byte units; the array's own 648 bytes were the
+    // difference between two and three workgroups per CU for the scores-only kernel)
     static_assert(R * G::WZ_LD <= TILE, "kernel rows do not fit the borrowed buffer");
-    T *const wz = Kt1;
+    T *const wz = SCORES_ONLY ? B1 : B2;
 
     const int tid = threadIdx.x;
     // (the wavefront index through readfirstlane: everything derived from it is then scalar, branches included)
@@ -518,27 +528,35 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
     // below 4, which a copy round does not change either)
     static_assert((F_NT / CPR) % 16 == 0, "copy rounds must keep the V swizzle phase");
     const int v_off0 = kv_row0 * D + ((tid % CPR) ^ v_swizzle4<D>(kv_row0)) * 8;
-    auto issue_kv = [&](int j, T *Kdst, T *Vdst) {
+    auto issue_k = [&](int j, T *Kdst) {
         const int cb = j * F_BK + G::PWR;
-        const bool inside = cb >= 0 && cb + F_BK <= S && j >= 0 && (j + 1) * F_BK <= S;  // no key needs clamping
+        const bool inside = cb >= 0 && cb + F_BK <= S;  // no key needs clamping
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r) {
             const int kv_row = kv_row0 + r * (F_NT / CPR), kv_off = kv_off0 + r * (F_NT / CPR) * D;
-            const int v_off = v_off0 + r * (F_NT / CPR) * D;
-            int koff = cb * D + kv_off, voff = j * F_BK * D + v_off;
+            int koff = cb * D + kv_off;
             if (!inside) {
                 int kr = cb + kv_row;
                 kr = kr < 0 ? 0 : (kr >= S ? S - 1 : kr);
-                int vr = j * F_BK + kv_row;
-                vr = vr < 0 ? 0 : (vr >= S ? S - 1 : vr);
                 koff = kv_off + (kr - kv_row) * D;
-                voff = v_off + (vr - kv_row) * D;
             }
             __builtin_amdgcn_global_load_lds((glb_void_t *)(Kp + koff),
                                              (lds_void_t *)(Kdst + (r * F_NT + wave * 64) * 8), 16, 0, 0);
-            if (!SCORES_ONLY)
-                __builtin_amdgcn_global_load_lds((glb_void_t *)(Vp + voff),
-                                                 (lds_void_t *)(Vdst + (r * F_NT + wave * 64) * 8), 16, 0, 0);
+        }
+    };
+    auto issue_v = [&](int j, T *Vdst) {
+        const bool inside = j >= 0 && (j + 1) * F_BK <= S;
+#pragma unroll
+        for (int r = 0; r < ROUNDS; ++r) {
+            const int kv_row = kv_row0 + r * (F_NT / CPR), v_off = v_off0 + r * (F_NT / CPR) * D;
+            int voff = j * F_BK * D + v_off;
+            if (!inside) {
+                int vr = j * F_BK + kv_row;
+                vr = vr < 0 ? 0 : (vr >= S ? S - 1 : vr);
+                voff = v_off + (vr - kv_row) * D;
+            }
+            __builtin_amdgcn_global_load_lds((glb_void_t *)(Vp + voff),
+                                             (lds_void_t *)(Vdst + (r * F_NT + wave * 64) * 8), 16, 0, 0);
         }
     };
 
@@ -548,7 +566,8 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
     const int j_end = (j_lo + jc_len - 1 < j_last) ? j_lo + jc_len - 1 : j_last;
     // one key block earlier only fills the retained score columns (before the first one: the right pad, if any)
     const int j_start = j_lo > 0 ? j_lo - 1 : (G::PWR > 0 ? -1 : 0);
-    issue_kv(j_start, Kt0, Vt0);
+    issue_k(j_start, B0);
+    if (!SCORES_ONLY) issue_v(j_start, B1);
 
     // zero the score tile once (columns past HC+BK are read by the last window but never written)
     for (int e = tid; e < F_SR * F_SLD / 8; e += F_NT) {
@@ -641,14 +660,14 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
 #pragma unroll
         for (int it = 0; it < TAIL_IT; ++it)
             if (tail_off[it] >= 0) *reinterpret_cast<u32x4_t *>(Sc + tail_off[it]) = tailreg[it];
-        if (j < j_end) issue_kv(j + 1, Kn, Vn);  // lands while this block is being worked on
+        if (j < j_end) issue_k(j + 1, Kn);  // lands while this block is being worked on
 
         // ---- S^T = K Q^T, zero above the diagonal / outside the sequence, to the score tile ----
         {
-            // Pipelined like the conv phase below: K fragments are read from assembly KLD steps (two 16-key blocks)
-            // ahead into a ring of registers, a step being one fragment and the two products it feeds (both row
+            // Pipelined like the conv phase below: K fragments are read from assembly KLD steps (one or two 16-key
+            // blocks) ahead into a ring of registers, a step being one fragment and the two products it feeds (both row
             // blocks); a block's scores are rounded, scaled, masked and written LAG steps into the next block.
-            constexpr int NSTEP = NCB * KS, KLD = 2 * KS, KSLOT = KLD + 1, LAG = 2;
+            constexpr int NSTEP = NCB * KS, KLD = SCORES_ONLY ? 2 * KS : KS, KSLOT = KLD + 1, LAG = 2;  // (attention kernel: one block ahead; two spill)
             static_assert(NSTEP > KLD && KS >= LAG && NCB % 2 == 0, "pipeline deeper than the work; blocks are written in pairs");
             unsigned ka[KS];
 #pragma unroll
@@ -678,6 +697,7 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
                         hi = pack2<T>(a2 * scale, a3 * scale);
                     }
                     if (!s_plain) {
+                        MTA_KEEP_BRANCH();
                         const int col = cbase + cb * 16 + kg * 4;
                         const int lim = causal ? (prow[rb] < S - 1 ? prow[rb] : S - 1) : S - 1;  // last key kept
                         if (col < 0 || col > lim) lo &= 0xffff0000u;
@@ -724,6 +744,8 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
         // score tile complete for everybody.  Only the LDS counter is waited for: a fence would also wait for the
         // copy of the next key block, in flight since the top of the iteration
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        // (attention kernel: nobody reads K(j) any more, the next V block may land in its buffer)
+        if (!SCORES_ONLY && j < j_end) issue_v(j + 1, Vn);
         if (j < j_lo) return;
 
         // ---- conv (Toeplitz MFMAs over the score tile) -> global (scores only) / -> online softmax ----
@@ -793,15 +815,18 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
                 unpack2<T>(pack2<T>(v4[2] * scale, v4[3] * scale), v4[2], v4[3]);
                 const bool c_plain = PLAIN || (j * F_BK + cb * 16 + 16 <= S && (!causal || j * F_BK + cb * 16 + 15 <= pmin));
                 if constexpr (cb == 0) mloc = -INFINITY;
+                if (!c_plain) {
+                    MTA_KEEP_BRANCH();
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int col = j * F_BK + cb * 16 + kg * 4 + v;
+                        if (!(col < S && !(causal && col > p_))) v4[v] = -INFINITY;
+                    }
+                }
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
-                    float val = v4[v];
-                    if (!c_plain) {
-                        const int col = j * F_BK + cb * 16 + kg * 4 + v;
-                        if (!(col < S && !(causal && col > p_))) val = -INFINITY;
-                    }
-                    sv[cb][v] = val;
-                    mloc = fmaxf(mloc, val);
+                    sv[cb][v] = v4[v];
+                    mloc = fmaxf(mloc, v4[v]);
                 }
                 if constexpr (cb == NCB - 1) {  // the row block is complete: online softmax (a row lives in 4 lanes)
                     mloc = max_across_groups(mloc);
@@ -882,17 +907,28 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
             }
         }
     };
-    auto plain = [&](int j) {  // (scores-only kernel: the attention kernel has no registers to spare for a second body)
+    auto plain = [&](int j) {  // (scores-only kernel: a second body per buffer rotation makes the attention kernel spill)
         const int cbase = j * F_BK + G::PWR;
         return SCORES_ONLY && j >= 0 && cbase + F_BK <= S && (!causal || cbase + F_BK - 1 <= pmin);
     };
-    for (int j = j_start;;) {
-        if (SCORES_ONLY && plain(j)) block(std::integral_constant<bool, SCORES_ONLY>{}, j, Kt0, Vt0, Kt1, Vt1);
-        else block(std::false_type{}, j, Kt0, Vt0, Kt1, Vt1);
-        if (++j > j_end) break;
-        if (SCORES_ONLY && plain(j)) block(std::integral_constant<bool, SCORES_ONLY>{}, j, Kt1, Vt1, Kt0, Vt0);
-        else block(std::false_type{}, j, Kt1, Vt1, Kt0, Vt0);
-        if (++j > j_end) break;
+    if constexpr (SCORES_ONLY) {
+        for (int j = j_start;;) {  // block(tag, j, K(j), V(j), where K(j+1) goes, where V(j+1) goes)
+            if (plain(j)) block(std::true_type{}, j, B0, B0, B1, B1);
+            else block(std::false_type{}, j, B0, B0, B1, B1);
+            if (++j > j_end) break;
+            if (plain(j)) block(std::true_type{}, j, B1, B1, B0, B0);
+            else block(std::false_type{}, j, B1, B1, B0, B0);
+            if (++j > j_end) break;
+        }
+    } else {
+        for (int j = j_start;;) {
+            block(std::false_type{}, j, B0, B1, B2, B0);
+            if (++j > j_end) break;
+            block(std::false_type{}, j, B2, B0, B1, B2);
+            if (++j > j_end) break;
+            block(std::false_type{}, j, B1, B2, B0, B1);
+            if (++j > j_end) break;
+        }
     }
 
     if constexpr (SCORES_ONLY) {
@@ -915,17 +951,22 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_f
         return;
     }
     // ---- normalise and store (halo rows are dropped) ----
+    // (row and column from a lane index counted afresh: the store addresses are then formed here, after the key-block
+    // loop, and nothing has to be kept - or spilled - across the loop for them)
+    const int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    const int ln_o = lane_e & 15, kg_o = lane_e >> 4;
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb) {
         const float l_row = sum_across_groups(l_i[rb]);
-        if (row_stored[rb]) {
+        const int tr_ = wave * 32 + rb * 16 + ln_o + cshift, p_ = q0 - G::HR + tr_;
+        if (tr_ >= G::HR && tr_ < wave * 32 + 32 && p_ < S) {
             const float inv = 1.0f / l_row;
-            if (Lse != nullptr && kg == 0) Lse[bh * (int64_t)S + cprow[rb]] = m_i[rb] + __logf(l_row);
+            if (Lse != nullptr && kg_o == 0) Lse[bh * (int64_t)S + p_] = m_i[rb] + __logf(l_row);
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 const uint32_t lo = pack2<T>(oacc[rb][db][0] * inv, oacc[rb][db][1] * inv);
                 const uint32_t hi = pack2<T>(oacc[rb][db][2] * inv, oacc[rb][db][3] * inv);
-                *reinterpret_cast<uint2 *>(Op + (int64_t)cprow[rb] * D + db * 16 + kg * 4) = make_uint2(lo, hi);
+                *reinterpret_cast<uint2 *>(Op + (int64_t)p_ * D + db * 16 + kg_o * 4) = make_uint2(lo, hi);
             }
         }
     }
@@ -935,7 +976,7 @@ template <typename T, int D, int R, int SK, bool SCORES_ONLY>
 int launch_mfma(const void *q, const void *k, const void *v, const void *w, void *o, float *lse, int64_t B, int64_t H,
                 int64_t S, int causal, float scale, int fill_upper, hipStream_t st)
 {
-    constexpr int NW = SCORES_ONLY ? 4 : 8;
+    constexpr int NW = 4;
     constexpr int F_NT = 64 * NW;
     using G = fused_geom<R, SK, NW>;
     static_assert(G::fits, "conv window exceeds the 32-key MFMA contraction");
