@@ -385,9 +385,8 @@ __device__ __forceinline__ float max_raw(float a, float b)
     asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
     return r;
 }
-// Wavefront-wide reduction, result in every lane: four DPP steps inside rows of 16 lanes (the operand permuted on the
-// way into the ALU; the two wait states a DPP read of a just-written register needs are part of the asm), then two
-// exchanges across rows.
+// One DPP step of a reduction inside rows of 16 lanes (the operand permuted on the way into the ALU; the two wait states
+// a DPP read of a just-written register needs are part of the asm).
 #define MTA_RS_DPP_STEP(op, ctrl) asm("s_nop 1\n\t" op "_dpp %0, %1, %1 " ctrl " row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v)); v = r;
 // The same for operands that dot-product instructions may just have written: a different vector-ALU instruction
 // may read such a register only three wait states later, and the compiler, which inserts those for its own
@@ -399,41 +398,87 @@ __device__ __forceinline__ float max3_after_dot(float a, float b, float c)
     return r;
 }
 
-template <bool IS_MAX> __device__ __forceinline__ float wave_reduce(float v)
+typedef unsigned int rs_u2 __attribute__((ext_vector_type(2)));
+template <bool IS_MAX> __device__ __forceinline__ float rs_op(float a, float b) { return IS_MAX ? max_raw(a, b) : a + b; }
+
+// The G per-lane values v[0..G) (one per head), each reduced over the wavefront, all at once: an exchange of the two
+// halves of the wavefront leaves head 2j's result-so-far in the lower and head 2j+1's in the upper 32 lanes of one
+// register, an exchange of rows of 16 lanes folds two such registers into one (rows 0..3 then hold heads 4j, 4j+2, 4j+1,
+// 4j+3), and four DPP steps finish inside the rows.  The first lane of each row writes dst[head*NW + wave].
+template <bool IS_MAX, int G, int NW> __device__ __forceinline__ void heads_reduce_store(const float (&val)[G], float *dst, int wave, int lane)
 {
-    float r;
+    static_assert(G == 2 || G == 4 || G == 8, "head groups of the packed kernel");
+    float c[G / 2];
+#pragma unroll
+    for (int j = 0; j < G / 2; ++j) {
+        const rs_u2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(val[2 * j]), __float_as_uint(val[2 * j + 1]), false, false);
+        c[j] = rs_op<IS_MAX>(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    }
+    constexpr int ND = G >= 4 ? G / 4 : 1;
+    float d[ND];
+#pragma unroll
+    for (int j = 0; j < ND; ++j) {
+        const float a = c[G >= 4 ? 2 * j : 0], b = c[G >= 4 ? 2 * j + 1 : 0];
+        const rs_u2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+        d[j] = rs_op<IS_MAX>(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    }
+    const int row = lane >> 4;
+#pragma unroll
+    for (int j = 0; j < ND; ++j) {
+        float v = d[j], r;
+        if constexpr (IS_MAX) {
+            MTA_RS_DPP_STEP("v_max_f32", "quad_perm:[1,0,3,2]")
+            MTA_RS_DPP_STEP("v_max_f32", "quad_perm:[2,3,0,1]")
+            MTA_RS_DPP_STEP("v_max_f32", "row_half_mirror")
+            MTA_RS_DPP_STEP("v_max_f32", "row_mirror")
+        } else {
+            MTA_RS_DPP_STEP("v_add_f32", "quad_perm:[1,0,3,2]")
+            MTA_RS_DPP_STEP("v_add_f32", "quad_perm:[2,3,0,1]")
+            MTA_RS_DPP_STEP("v_add_f32", "row_half_mirror")
+            MTA_RS_DPP_STEP("v_add_f32", "row_mirror")
+        }
+        // rows 0..3 hold heads (G >= 4) 4j + {0, 2, 1, 3}; (G == 2) {0, 0, 1, 1}
+        const int head = G >= 4 ? 4 * j + ((row & 1) << 1) + (row >> 1) : (row >> 1);
+        if ((lane & 15) == 0 && (G >= 4 || (row & 1) == 0)) dst[head * NW + wave] = v;
+    }
+}
+
+// What the first `nlw` wavefronts left in src[head*NW + wave], combined per head, the same in every lane: lane l takes
+// entry l, NW neighbouring lanes fold with DPP steps, and one lane per head is read out as a wavefront-uniform value.
+template <bool IS_MAX, int G, int NW> __device__ __forceinline__ void heads_combine(const float *src, int nlw, int lane, float (&out)[G])
+{
+    static_assert(NW * G <= 64 && (NW == 4 || NW == 8), "one entry per lane");
+    const float neutral = IS_MAX ? -INFINITY : 0.0f;
+    const float got = src[lane & (NW * G - 1)];
+    float v = (lane & (NW - 1)) < nlw ? got : neutral, r;
     if constexpr (IS_MAX) {
         MTA_RS_DPP_STEP("v_max_f32", "quad_perm:[1,0,3,2]")
         MTA_RS_DPP_STEP("v_max_f32", "quad_perm:[2,3,0,1]")
-        MTA_RS_DPP_STEP("v_max_f32", "row_half_mirror")
-        MTA_RS_DPP_STEP("v_max_f32", "row_mirror")
-        v = max_raw(v, __shfl_xor(v, 16));
-        v = max_raw(v, __shfl_xor(v, 32));
+        if constexpr (NW == 8) { MTA_RS_DPP_STEP("v_max_f32", "row_half_mirror") }
     } else {
         MTA_RS_DPP_STEP("v_add_f32", "quad_perm:[1,0,3,2]")
         MTA_RS_DPP_STEP("v_add_f32", "quad_perm:[2,3,0,1]")
-        MTA_RS_DPP_STEP("v_add_f32", "row_half_mirror")
-        MTA_RS_DPP_STEP("v_add_f32", "row_mirror")
-        v += __shfl_xor(v, 16);
-        v += __shfl_xor(v, 32);
+        if constexpr (NW == 8) { MTA_RS_DPP_STEP("v_add_f32", "row_half_mirror") }
     }
-    return v;
+#pragma unroll
+    for (int o = 0; o < G; ++o) out[o] = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), o * NW));
 }
 #undef MTA_RS_DPP_STEP
 
-template <typename T, int G, int NV, bool HAS1, bool HAS2>
-__global__ __launch_bounds__(256, (G * NV == 8) ? RS_OCC : 1) void mix_softmax_mix_packed(
+template <typename T, int G, int NV, bool HAS1, bool HAS2, int NT, int OCC>
+__global__ __launch_bounds__(NT, OCC) void mix_softmax_mix_packed(
     const T *__restrict__ x, const T *__restrict__ w1, const T *__restrict__ w2, T *__restrict__ y, int C, int P, int Q,
     int causal, int fill_upper)
 {
-    constexpr int NT = 256, VEC = 8, NW = NT / 64, H2 = G / 2;
+    constexpr int VEC = 8, NW = NT / 64, H2 = G / 2;
     static_assert(sizeof(T) == 2 && G % 2 == 0, "packed pairs of a 16-bit type");
     __shared__ float red[2][NW * G];  // [0] maxima, [1] sums
-    const int tid = threadIdx.x;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int lane = threadIdx.x & 63;
     const unsigned groups = (unsigned)(C / G);
     unsigned b = blockIdx.x;
     const int p = (int)(b % (unsigned)P); b /= (unsigned)P;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int tid = threadIdx.x;
     const int g = (int)(b % groups);
     const int64_t n = b / groups;
     const int64_t plane = (int64_t)P * Q;
@@ -444,6 +489,23 @@ __global__ __launch_bounds__(256, (G * NV == 8) ? RS_OCC : 1) void mix_softmax_m
     int nlive = 0;
 #pragma unroll
     for (int k = 0; k < NV; ++k) nlive += ((k * NT + wave * 64) * VEC <= last) ? 1 : 0;
+    // Slices wholly above the diagonal: nothing to read and nothing to contribute.  Their wavefronts end here, ahead of
+    // the workgroup barriers (a barrier waits for the surviving wavefronts only), and free their registers for the next
+    // workgroup; the others reduce over the first `nlw` slices.
+    const int nlw = last / (64 * VEC) + 1 < NW ? last / (64 * VEC) + 1 : NW;
+    if (nlive == 0) {
+        if (fill_upper) {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                const int q = (k * NT + tid) * VEC;
+                if (q >= Q) continue;
+                const rs_u4 z = {0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int o = 0; o < G; ++o) __builtin_nontemporal_store(z, reinterpret_cast<rs_u4 *>(y + base + o * plane + q));
+            }
+        }
+        return;
+    }
 
     // packed weights, (w[o][2j], w[o][2j+1]); identical for all lanes
     uint32_t w1p[G][H2], w2p[G][H2];
@@ -521,21 +583,13 @@ __global__ __launch_bounds__(256, (G * NV == 8) ? RS_OCC : 1) void mix_softmax_m
                 }
             }
         }
-#pragma unroll
-        for (int o = 0; o < G; ++o) {
-            const float v = wave_reduce<true>(m[o]);
-            if (lane == 0) red[0][wave * G + o] = v;
-        }
+        heads_reduce_store<true, G, NW>(m, red[0], wave, lane);
         __syncthreads();
-#pragma unroll
-        for (int o = 0; o < G; ++o) {
-            float v = red[0][o];
-#pragma unroll
-            for (int i = 1; i < NW; ++i) v = max_raw(v, red[0][i * G + o]);
+        heads_combine<true, G, NW>(red[0], nlw, lane, m);
+        if constexpr (HAS1) {
             // the maximum of the rounded scores is the rounded maximum (the row's first key is always attended: finite)
-            float dummy = v;
-            if constexpr (HAS1) round_pair<T>(v, dummy);
-            m[o] = v;
+#pragma unroll
+            for (int o = 0; o < G; o += 2) round_pair<T>(m[o], m[o + 1]);
         }
 
         // ---- exp(s - max) = exp2(s*log2(e) - max*log2(e)), running sum ----
@@ -544,7 +598,8 @@ __global__ __launch_bounds__(256, (G * NV == 8) ? RS_OCC : 1) void mix_softmax_m
 #pragma unroll
         for (int o = 0; o < G; ++o) {
             const float mneg = -m[o] * LOG2E;
-            float acc = 0.0f;
+            float &acc = inv[o];
+            acc = 0.0f;
 #pragma unroll
             for (int k = 0; k < L; ++k)
 #pragma unroll
@@ -556,16 +611,14 @@ __global__ __launch_bounds__(256, (G * NV == 8) ? RS_OCC : 1) void mix_softmax_m
                     acc += e[o][k][2 * d];
                     acc += e[o][k][2 * d + 1];
                 }
-            const float v = wave_reduce<false>(acc);
-            if (lane == 0) red[1][wave * G + o] = v;
         }
+        heads_reduce_store<false, G, NW>(inv, red[1], wave, lane);
         __syncthreads();
+        heads_combine<false, G, NW>(red[1], nlw, lane, inv);
 #pragma unroll
-        for (int o = 0; o < G; ++o) {
-            float v = red[1][o];
-#pragma unroll
-            for (int i = 1; i < NW; ++i) v += red[1][i * G + o];
-            inv[o] = 1.0f / v;
+        for (int o = 0; o < G; ++o) {  // 1/sum: the hardware reciprocal and one Newton step (within an ulp of the quotient)
+            const float r = __builtin_amdgcn_rcpf(inv[o]);
+            inv[o] = fmaf(fmaf(-inv[o], r, 1.0f), r, r);
         }
 
         // ---- normalise, round in pairs of heads, second mix, store ----
@@ -628,12 +681,10 @@ __global__ __launch_bounds__(256, (G * NV == 8) ? RS_OCC : 1) void mix_softmax_m
         }
     };
     // does the last live pass reach beyond the last attended key?
-    const bool edge = nlive > 0 && ((nlive - 1) * NT + wave * 64 + 64) * VEC - 1 > last;
+    const bool edge = ((nlive - 1) * NT + wave * 64 + 64) * VEC - 1 > last;
     static_assert(NV <= 4, "live-pass dispatch");
     using std::integral_constant;
-    if (nlive == 0) {
-        run(integral_constant<int, 0>{}, std::false_type{});
-    } else if (edge) {
+    if (edge) {
         if (nlive == 1) run(integral_constant<int, 1>{}, std::true_type{});
         if constexpr (NV >= 2) { if (nlive == 2) run(integral_constant<int, 2>{}, std::true_type{}); }
         if constexpr (NV >= 3) { if (nlive == 3) run(integral_constant<int, 3>{}, std::true_type{}); }
@@ -736,20 +787,24 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb, voi
         const int io_code = std::is_same<T, bf16_t>::value ? MTA_BF16 : MTA_F16;
         if (vec_ok && !kb && !no_packed && w_dtype == io_code && (w1 || w2) && (!w1 || aligned_to(w1, 4)) &&
             (!w2 || aligned_to(w2, 4)) && C % 2 == 0 && Q <= 256 * VEC * 4) {
-#define MTA_RSP_LAUNCH(g, v, h1, h2)                                                                                   \
+#define MTA_RSP_LAUNCH(g, v, h1, h2, nt, occ)                                                                          \
     {                                                                                                                  \
-        hipLaunchKernelGGL((mix_softmax_mix_packed<T, g, v, h1, h2>), dim3((unsigned)(N * (C / g) * P)), dim3(256), 0, \
-                           st, (const T *)x, (const T *)w1, (const T *)w2, (T *)y, (int)C, (int)P, (int)Q, causal,     \
-                           fill_upper);                                                                                \
+        hipLaunchKernelGGL((mix_softmax_mix_packed<T, g, v, h1, h2, nt, occ>), dim3((unsigned)(N * (C / g) * P)),      \
+                           dim3(nt), 0, st, (const T *)x, (const T *)w1, (const T *)w2, (T *)y, (int)C, (int)P,        \
+                           (int)Q, causal, fill_upper);                                                                \
         return launch_status();                                                                                        \
     }
-#define MTA_RSP_CASE(g, v)                                                                                             \
-    if (G == g && nv <= v) {                                                                                           \
-        if (w1 && w2) MTA_RSP_LAUNCH(g, v, true, true)                                                                 \
-        if (w1) MTA_RSP_LAUNCH(g, v, true, false)                                                                      \
-        MTA_RSP_LAUNCH(g, v, false, true)                                                                              \
+#define MTA_RSP_CASE(g, v, nt, occ)                                                                                    \
+    if (G == g && Q <= (int64_t)(nt) * VEC * (v)) {                                                                    \
+        if (w1 && w2) MTA_RSP_LAUNCH(g, v, true, true, nt, occ)                                                        \
+        if (w1) MTA_RSP_LAUNCH(g, v, true, false, nt, occ)                                                             \
+        MTA_RSP_LAUNCH(g, v, false, true, nt, occ)                                                                     \
     }
-            MTA_RSP_CASE(2, 1) MTA_RSP_CASE(2, 2) MTA_RSP_CASE(2, 4) MTA_RSP_CASE(4, 1) MTA_RSP_CASE(4, 2) MTA_RSP_CASE(8, 1)
+            MTA_RSP_CASE(2, 1, 256, 1) MTA_RSP_CASE(2, 2, 256, 1) MTA_RSP_CASE(2, 4, 256, RS_OCC) MTA_RSP_CASE(4, 1, 256, 1)
+            // 4 heads x up to 4096 keys: with one weight, 8 wavefronts of one pass each (63 registers: 8 wavefronts per
+            // SIMD; measured 2 % faster than 4 wavefronts of two passes); with both weights the latter is 4 % faster
+            if (!(w1 && w2)) MTA_RSP_CASE(4, 1, 512, 8)
+            MTA_RSP_CASE(4, 2, 256, RS_OCC) MTA_RSP_CASE(8, 1, 256, RS_OCC)
 #undef MTA_RSP_CASE
 #undef MTA_RSP_LAUNCH
         }
