@@ -8,7 +8,10 @@ configuration the headline metric is quoted on: B=2, H=16, S=4096, D=128, bf16, 
 6x11 pre-softmax conv (N(0,0.05) + identity tap), identity pre-softmax head weights,
 identity 3x3 post-softmax conv, post-softmax head mixing in groups of 4 (I + N(0,0.1)).
 Inputs are synthetic, seeded, and resident in HBM before the timed region.  Prints ONE
-JSON line.  `value` is the latency of one forward in ms.
+JSON line.  `value` is the latency of one forward in ms.  Defaults: 60 warm-up steps, 100
+timed ones - the first forty or so forwards after the device has been idle run up to 20 %
+slower than the ones that follow (0.62-0.68 ms against 0.565 ms), so fewer warm-up steps
+time the run-up, not the forward.
 
 The `roofline` object is for the slowest hand-written kernel of the step; its duration
 is measured live with events recorded on the stream the kernels run on.  `kernels` adds
@@ -224,7 +227,7 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
     sets = [tuple(t.to(device) for t in O.seeded_qkv(b, h, s, d, bf16, seed=200 + i)) for i in range(2)]
     wc = O.seeded_conv_weight(h, 6, 11, 0.05, bf16).to(device)
     os_ = [torch.empty_like(sets[0][0]) for _ in range(2)]
-    ms = time_launches(torch, lambda i: mta.ops.conv_attn_fwd(*sets[i], wc, True, None, out=os_[i]), 2, min(warmup, 2),
+    ms = time_launches(torch, lambda i: mta.ops.conv_attn_fwd(*sets[i], wc, True, None, out=os_[i]), 2, min(warmup, 10),
                     max(2, steps // 4))
     mfma_flops = 4 * b * h * tri(s) * d
     out["conv_attn_fused_bf16_1x32x8192x128"] = {"ms": ms, "mfma_useful_flops": mfma_flops,
@@ -233,7 +236,7 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
     del sets, os_
     # the general four-stage forward (all MTA weights non-trivial), B1 H16 S4096 D128 fp16, 7x7 conv pre and post
     mod, sets = build_general(torch, mta, O, device)
-    ms = time_steps(torch, lambda i: mod(*sets[i], None, None), len(sets), min(warmup, 3), max(3, steps // 2))
+    ms = time_steps(torch, lambda i: mod(*sets[i], None, None), len(sets), min(warmup, 30), max(3, steps // 2))
     stages = stage_breakdown(torch, mod, sets, 3)
     out["mta_forward_general_fp16_1x16x4096x128_7x7_pre_post_dense"] = {
         "ms": ms, "stages_ms": stages,
@@ -341,8 +344,8 @@ def _cpu_model():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=60)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
