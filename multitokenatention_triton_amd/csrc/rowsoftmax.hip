@@ -18,6 +18,12 @@
 
 constexpr int RS_OCC = 5;  // wavefronts per SIMD the G*NV = 8 instances (e.g. 4 heads x 4096 keys) are compiled for
 
+namespace mta {
+// rowsoftmax_dense16.hip: the same pass for groups of 16 heads, both mixes on the matrix cores
+int mix16_softmax_launch(const void *x, const void *w1, const void *w2, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
+                         int causal, int fill_upper, int io_dtype, int w_dtype, hipStream_t st);
+}  // namespace mta
+
 namespace {
 using namespace mta;
 
@@ -785,6 +791,10 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb, voi
         // the general one, for comparisons)
         static const bool no_packed = [] { const char *e_ = getenv("MTA_SOFTMAX_NO_PACKED"); return e_ && e_[0] == '1'; }();
         const int io_code = std::is_same<T, bf16_t>::value ? MTA_BF16 : MTA_F16;
+        if (G == 16 && !kb && !no_packed) {
+            const int rc = mix16_softmax_launch(x, w1, w2, y, N, C, P, Q, causal, fill_upper, io_code, w_dtype, st);
+            if (rc != MTA_ERR_UNSUPPORTED) return rc;
+        }
         if (vec_ok && !kb && !no_packed && w_dtype == io_code && (w1 || w2) && (!w1 || aligned_to(w1, 4)) &&
             (!w2 || aligned_to(w2, 4)) && C % 2 == 0 && Q <= 256 * VEC * 4) {
 #define MTA_RSP_LAUNCH(g, v, h1, h2, nt, occ)                                                                          \

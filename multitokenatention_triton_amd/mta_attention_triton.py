@@ -51,8 +51,20 @@ from . import ops
 from .convolution_2d_trit import Conv2dTriton
 from .triton_linear_head import TritonLinearHead
 
-# largest mixing group the one-pass mix/softmax/mix kernel keeps in registers
+# largest mixing group the one-pass mix/softmax/mix kernel keeps in registers ...
 _FUSED_MAX_GROUP = 8
+# ... and the group size its matrix-core variant takes (16-bit data, rows of up to _FUSED_MFMA_MAX_KEYS keys)
+_FUSED_MFMA_GROUP = 16
+_FUSED_MFMA_MAX_KEYS = 4096
+
+
+def _one_pass_group(group: int, scores_dtype, n_keys: int, *weights) -> bool:
+    """Whether mix -> softmax (-> mix) over mixing groups of ``group`` heads runs as one kernel."""
+    if group <= _FUSED_MAX_GROUP:
+        return True
+    return (group == _FUSED_MFMA_GROUP and scores_dtype in (torch.bfloat16, torch.float16)
+            and n_keys % 8 == 0 and n_keys <= _FUSED_MFMA_MAX_KEYS
+            and all(w is None or w.dtype == scores_dtype for w in weights))
 # where the one-pass post-softmax conv + head mixing kernel is used (see forward)
 _CONV_MIX_MAX_GROUP = 4
 _CONV_MIX_SIZES = ((3, 3), (7, 7))
@@ -149,7 +161,11 @@ class MTAAttentionTriton(nn.Module):
         if w2 is None:
             g_post = 1
         post_conv_identity = st.post_conv_identity
-        one_pass = post_conv_identity and _lcm(g_pre, g_post) <= _FUSED_MAX_GROUP
+        n_keys = xk.size(-2)
+        g_both = _lcm(g_pre, g_post)
+        # (the matrix-core variant for groups of 16 takes no key bias)
+        one_pass = (post_conv_identity and _one_pass_group(g_both, xq.dtype, n_keys, w1, w2)
+                    and (key_bias is None or g_both <= _FUSED_MAX_GROUP))
         # the last stage may leave the upper triangle unwritten only if our own P V kernel consumes it
         own_pv = (xq.size(-2) == xk.size(-2) and xq.dtype == xv.dtype
                   and ops.causal_pv_supported(xq.dtype, xq.size(-2), xv.size(-1)))
@@ -167,10 +183,10 @@ class MTAAttentionTriton(nn.Module):
 
         if one_pass:
             self._mark("mix_softmax_mix")
-            scores = ops.headmix_softmax(scores, w1, w2, self.causal, group_size=_lcm(g_pre, g_post),
+            scores = ops.headmix_softmax(scores, w1, w2, self.causal, group_size=g_both,
                                          fill_upper=not own_pv, key_bias=key_bias)
         else:
-            if g_pre <= _FUSED_MAX_GROUP:
+            if _one_pass_group(g_pre, xq.dtype, n_keys, w1) and (key_bias is None or g_pre <= _FUSED_MAX_GROUP):
                 self._mark("mix_softmax")
                 scores = ops.headmix_softmax(scores, w1, None, self.causal, group_size=g_pre, key_bias=key_bias,
                                              fill_upper=post_conv_identity and w2 is None and not own_pv)

@@ -528,7 +528,7 @@ def test_mta_use_mask_tensor_masks(pkg, name, dtype):
 @pytest.mark.parametrize("group", [4, 16])
 def test_mta_general_route_is_four_stages(pkg, group, dtype):
     """All four MTA weights non-trivial (what training produces).  Mixing groups of 4: QK^T+conv, mix+softmax, conv+mix,
-    P V -- four kernels, the score tensor written three times and read three times.  Dense 16x16 weights: six kernels."""
+    P V -- four kernels, the score tensor written three times and read three times.  Dense 16x16 weights: five kernels."""
     print(f"mta general route group={group} {dtype}", flush=True)
     h, s, d = 16, 520, 64
     q, k, v = O.seeded_qkv(1, h, s, d, dtype, seed=97)
@@ -541,8 +541,8 @@ def test_mta_general_route_is_four_stages(pkg, group, dtype):
         got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
         if group <= 4 and structure == "infer":
             assert stages == ["qk_conv", "mix_softmax", "conv_mix_post", "pv", "end"]
-        else:   # 16-head mixing groups: mix, then softmax; conv, then mix (the one-pass kernels stop at 8 and 4 heads)
-            assert stages == ["qk_conv", "mix_pre", "softmax", "conv_post", "mix_post", "pv", "end"]
+        else:   # 16-head mixing groups (16-bit data): mix + softmax in one pass on the matrix cores; conv, then mix
+            assert stages == ["qk_conv", "mix_softmax", "conv_post", "mix_post", "pv", "end"]
         torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
 
 
