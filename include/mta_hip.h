@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTA_ABI_VERSION 3
+#define MTA_ABI_VERSION 4
 
 enum mta_dtype { MTA_F32 = 0, MTA_BF16 = 1, MTA_F16 = 2 };
 
@@ -59,6 +59,13 @@ const char *mta_strerror(int code);
 int mta_conv2d_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H,
                    int64_t W, int R, int S, int causal, int io_dtype, int w_dtype, void *stream);
 
+/* mta_conv2d_fwd with causal = 1 for a consumer that never reads above the diagonal (mta_headmix_*, mta_causal_pv_fwd):
+ * what lies there in y is unspecified - left alone on square tensors that take the matrix-core kernel, +0.0 otherwise.
+ * A third of the bytes of a causal conv are that fill.  Same citation as mta_conv2d_fwd; the reference zero-fills
+ * (convolution_2d_trit.py:313) whoever reads the result. */
+int mta_conv2d_tril_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H, int64_t W, int R, int S,
+                        int io_dtype, int w_dtype, void *stream);
+
 /* Same op with the input multiplied by `in_scale` as it is read (products are formed
  * in fp32 and, for 16-bit I/O, rounded to the I/O dtype before the taps, which is what
  * a separate elementwise scale in that dtype would produce).  Lets the caller fold
@@ -77,6 +84,12 @@ int mta_conv2d_scaled_fwd(const void *x, const void *w, void *y, int64_t N, int6
 int mta_headmix_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t P,
                     int64_t Q, int group_size, int causal, float fill, int io_dtype, int w_dtype,
                     void *stream);
+
+/* mta_headmix_fwd with causal = 1 for a consumer that never reads above the diagonal: vectors of y wholly above it
+ * are not written (elements above it that share a 16-byte vector with the diagonal are written as +0.0).  Same citation
+ * as mta_headmix_fwd; the reference pre-fills the output (triton_linear_head.py:294-297). */
+int mta_headmix_tril_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
+                         int group_size, int io_dtype, int w_dtype, void *stream);
 
 /* Fused head mixing + row softmax + head mixing over (N,C,P,Q), one pass:
  *   s[o] = w1 ? sum_i w1[o,i] x[i] : x[o]      (fp32, rounded to the I/O dtype;

@@ -651,7 +651,8 @@ __global__ __launch_bounds__(M_WT, 2) void conv2d_mfma(
             }
             younger = interior ? OUT_IT : -1;
         }
-        if (mirror && ctn < ctm / M_SPB) {  // this strip's share of the 128x128 block's image above the diagonal
+        // (mirror == 2: the caller does not want the image written)
+        if (mirror == 1 && ctn < ctm / M_SPB) {  // this strip's share of the 128x128 block's image above the diagonal
             if (fill_full) {
                 zero_fill_strip<T, true>(yp, H, W, q0 + (ctm % M_SPB) * M_TM, (ctm / M_SPB) * M_TN, tid);
                 if (younger > 0) younger += M_TM * (M_TN / VEC) / M_WT;
@@ -683,7 +684,7 @@ int launch_mfma(const void *x, const void *w, void *y, int64_t N, int64_t C, int
     const int tiles_m = (int)((H + M_TM - 1) / M_TM), tiles_n = (int)((W + M_TN - 1) / M_TN);
     // mirror enumeration needs a square grid of whole 128x128 blocks' worth of strips
     const int blocks = (int)((H + M_TN - 1) / M_TN);
-    const int mirror = (causal && H == W) ? 1 : 0;
+    const int mirror = (causal && H == W) ? (causal == 2 ? 2 : 1) : 0;
     const int64_t ipp64 = mirror ? (int64_t)blocks * (blocks + 1) / 2 * M_SPB : (int64_t)tiles_m * tiles_n;
     if (ipp64 > (1 << 24)) return MTA_ERR_SHAPE;  // decode_item's float sqrt is exact well beyond this
     const int ipp = (int)ipp64;
@@ -761,18 +762,26 @@ int conv2d_entry(const void *x, const void *w, void *y, int64_t N, int64_t C, in
 extern "C" int mta_conv2d_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H,
                               int64_t W, int R, int S, int causal, int io_dtype, int w_dtype, void *stream)
 {
-    return conv2d_entry<false>(x, w, y, N, C, H, W, R, S, causal, 1.0f, 0, io_dtype, w_dtype, stream);
+    return conv2d_entry<false>(x, w, y, N, C, H, W, R, S, causal ? 1 : 0, 1.0f, 0, io_dtype, w_dtype, stream);
+}
+
+// (causal == 2 inside this file: causal, and the kernel that enumerates the lower triangle's strips only - the
+// matrix-core one on square tensors - does not write their images above the diagonal; every other path fills as usual)
+extern "C" int mta_conv2d_tril_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H, int64_t W,
+                                   int R, int S, int io_dtype, int w_dtype, void *stream)
+{
+    return conv2d_entry<false>(x, w, y, N, C, H, W, R, S, 2, 1.0f, 0, io_dtype, w_dtype, stream);
 }
 
 extern "C" int mta_conv2d_bwd_input(const void *dy, const void *w, void *dx, int64_t N, int64_t C, int64_t H,
                                     int64_t W, int R, int S, int causal, int io_dtype, int w_dtype, void *stream)
 {
-    return conv2d_entry<true>(dy, w, dx, N, C, H, W, R, S, causal, 1.0f, 0, io_dtype, w_dtype, stream);
+    return conv2d_entry<true>(dy, w, dx, N, C, H, W, R, S, causal ? 1 : 0, 1.0f, 0, io_dtype, w_dtype, stream);
 }
 
 extern "C" int mta_conv2d_scaled_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H,
                                      int64_t W, int R, int S, int causal, float in_scale, int io_dtype,
                                      int w_dtype, void *stream)
 {
-    return conv2d_entry<false>(x, w, y, N, C, H, W, R, S, causal, in_scale, 1, io_dtype, w_dtype, stream);
+    return conv2d_entry<false>(x, w, y, N, C, H, W, R, S, causal ? 1 : 0, in_scale, 1, io_dtype, w_dtype, stream);
 }

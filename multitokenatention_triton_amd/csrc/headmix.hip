@@ -81,8 +81,10 @@ __global__ __launch_bounds__(NT) void headmix_fixed(const T *__restrict__ x, con
     V fillv;
 #pragma unroll
     for (int u = 0; u < VEC; ++u) fillv.v[u] = fill_t;
+    // (causal == 2: causal, and what lies above the diagonal is the caller's to define - vectors wholly above it are
+    // not written)
     if (causal && qc * NT * VEC > p) {  // chunk wholly above the diagonal: fill only, nothing read
-        if (q < Q) {
+        if (q < Q && causal != 2) {
 #pragma unroll
             for (int o = 0; o < G; ++o) store_stream(reinterpret_cast<V *>(y + base + o * plane), fillv);
         }
@@ -101,8 +103,10 @@ __global__ __launch_bounds__(NT) void headmix_fixed(const T *__restrict__ x, con
     __syncthreads();
     if (q >= Q) return;
     if (causal && q > p) {
+        if (causal != 2) {
 #pragma unroll
-        for (int o = 0; o < G; ++o) store_stream(reinterpret_cast<V *>(y + base + o * plane), fillv);
+            for (int o = 0; o < G; ++o) store_stream(reinterpret_cast<V *>(y + base + o * plane), fillv);
+        }
         return;
     }
 #pragma unroll
@@ -159,9 +163,9 @@ __global__ __launch_bounds__(64 * DM_WAVES, 4) void headmix_dense32(const T *__r
     typedef unsigned int u4 __attribute__((ext_vector_type(4)));
     const int key = q0 + ln * 8;
 
-    if (q0 > last) {  // wholly beyond the diagonal: fill only
+    if (q0 > last) {  // wholly beyond the diagonal: fill only (causal == 2: not even that)
         const u4 fv = {fill2, fill2, fill2, fill2};
-        if (key < Q) {
+        if (key < Q && causal != 2) {
 #pragma unroll
             for (int t = 0; t < 8; ++t)
                 __builtin_nontemporal_store(fv, reinterpret_cast<u4 *>(y + base + (kg * 8 + t) * plane + key));
@@ -200,7 +204,7 @@ __global__ __launch_bounds__(64 * DM_WAVES, 4) void headmix_dense32(const T *__r
             mma16(acc[j][ob], wf[ob], xf);
         }
     }
-    if (key >= Q) return;
+    if (key >= Q || (causal == 2 && key > last)) return;
     // acc[j][ob][v]: output head 16ob + 4kg + v, key 8ln + j
 #pragma unroll
     for (int ob = 0; ob < 2; ++ob) {
@@ -326,7 +330,13 @@ extern "C" int mta_headmix_fwd(const void *x, const void *w, void *y, int64_t N,
                                int64_t Q, int group_size, int causal, float fill, int io_dtype, int w_dtype,
                                void *stream)
 {
-    return headmix_entry(x, w, y, N, C, P, Q, group_size, causal, fill, io_dtype, w_dtype, 0, stream);
+    return headmix_entry(x, w, y, N, C, P, Q, group_size, causal ? 1 : 0, fill, io_dtype, w_dtype, 0, stream);
+}
+
+extern "C" int mta_headmix_tril_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
+                                    int group_size, int io_dtype, int w_dtype, void *stream)
+{
+    return headmix_entry(x, w, y, N, C, P, Q, group_size, 2, 0.0f, io_dtype, w_dtype, 0, stream);
 }
 
 // dx[n,i,p,q] = sum_o w[o,i] dy[n,o,p,q]: the forward kernels with the transposed matrix; above the diagonal the
@@ -334,5 +344,5 @@ extern "C" int mta_headmix_fwd(const void *x, const void *w, void *y, int64_t N,
 extern "C" int mta_headmix_bwd_input(const void *dy, const void *w, void *dx, int64_t N, int64_t C, int64_t P,
                                      int64_t Q, int group_size, int causal, int io_dtype, int w_dtype, void *stream)
 {
-    return headmix_entry(dy, w, dx, N, C, P, Q, group_size, causal, 0.0f, io_dtype, w_dtype, 1, stream);
+    return headmix_entry(dy, w, dx, N, C, P, Q, group_size, causal ? 1 : 0, 0.0f, io_dtype, w_dtype, 1, stream);
 }

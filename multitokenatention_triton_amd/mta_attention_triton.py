@@ -193,7 +193,8 @@ class MTAAttentionTriton(nn.Module):
             else:
                 self._mark("mix_pre")
                 fill = float("-inf") if self.causal else 0.0
-                scores = ops.headmix(scores, w_pre, self.causal, fill, group_size=g_pre)
+                # (the softmax kernel that follows never reads above the diagonal)
+                scores = ops.headmix(scores, w_pre, self.causal, fill, group_size=g_pre, fill_upper=False)
                 self._mark("softmax")
                 scores = ops.headmix_softmax(scores, None, None, self.causal, key_bias=key_bias,
                                              fill_upper=post_conv_identity and w2 is None and not own_pv)
@@ -208,12 +209,14 @@ class MTAAttentionTriton(nn.Module):
             if done is not None:
                 scores = done
             else:
+                # neither our head mixing nor our P V reads above the diagonal: whoever feeds them need not write there
                 if not post_conv_identity:
                     self._mark("conv_post")
-                    scores = ops.conv2d_causal(scores, self.mta_conv_after_sm_triton.weight, self.causal)
+                    scores = ops.conv2d_causal(scores, self.mta_conv_after_sm_triton.weight, self.causal,
+                                               fill_upper=w2 is None and not own_pv)
                 if w2 is not None:
                     self._mark("mix_post")
-                    scores = ops.headmix(scores, w_post, self.causal, 0.0, group_size=g_post)
+                    scores = ops.headmix(scores, w_post, self.causal, 0.0, group_size=g_post, fill_upper=not own_pv)
 
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         self._mark("pv")

@@ -43,8 +43,11 @@ def _out_like(x: torch.Tensor, out: Optional[torch.Tensor]) -> torch.Tensor:
 
 
 def conv2d_causal(x: torch.Tensor, weight: torch.Tensor, causal: bool, in_scale: Optional[float] = None,
-                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Depthwise conv over (N,C,H,W) with a (C,R,S) kernel; see mta_conv2d_fwd in include/mta_hip.h."""
+                  out: Optional[torch.Tensor] = None, fill_upper: bool = True) -> torch.Tensor:
+    """Depthwise conv over (N,C,H,W) with a (C,R,S) kernel; see mta_conv2d_fwd in include/mta_hip.h.
+
+    ``fill_upper=False`` (causal, no ``in_scale``): for a consumer that never reads above the diagonal; what lies
+    there is unspecified (mta_conv2d_tril_fwd)."""
     x = _device_tensor(x, "input")
     weight = _device_tensor(weight.detach(), "weight")
     if x.dim() != 4 or weight.dim() != 3:
@@ -56,7 +59,10 @@ def conv2d_causal(x: torch.Tensor, weight: torch.Tensor, causal: bool, in_scale:
     y = _out_like(x, out)
     lib = _lib.load()
     with torch.cuda.device(x.device):
-        if in_scale is None:
+        if in_scale is None and causal and not fill_upper:
+            rc = lib.mta_conv2d_tril_fwd(x.data_ptr(), weight.data_ptr(), y.data_ptr(), n, c, h, w, r, s,
+                                         _code(x, "input"), _code(weight, "weight"), _stream(x))
+        elif in_scale is None:
             rc = lib.mta_conv2d_fwd(x.data_ptr(), weight.data_ptr(), y.data_ptr(), n, c, h, w, r, s, int(bool(causal)),
                                     _code(x, "input"), _code(weight, "weight"), _stream(x))
         else:
@@ -68,8 +74,11 @@ def conv2d_causal(x: torch.Tensor, weight: torch.Tensor, causal: bool, in_scale:
 
 
 def headmix(x: torch.Tensor, weight: torch.Tensor, causal: bool = True, fill: float = 0.0,
-            group_size: Optional[int] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """y[n,o,p,q] = sum_i W[o,i] x[n,i,p,q]; see mta_headmix_fwd in include/mta_hip.h."""
+            group_size: Optional[int] = None, out: Optional[torch.Tensor] = None, fill_upper: bool = True) -> torch.Tensor:
+    """y[n,o,p,q] = sum_i W[o,i] x[n,i,p,q]; see mta_headmix_fwd in include/mta_hip.h.
+
+    ``fill_upper=False`` (causal): for a consumer that never reads above the diagonal; vectors wholly above it are not
+    written (mta_headmix_tril_fwd)."""
     x = _device_tensor(x, "input")
     weight = _device_tensor(weight.detach(), "weight")
     if x.dim() != 4:
@@ -81,9 +90,14 @@ def headmix(x: torch.Tensor, weight: torch.Tensor, causal: bool = True, fill: fl
     assert c == l, f"Channel dimension {c} must match weight dimension {l}"
     y = _out_like(x, out)
     with torch.cuda.device(x.device):
-        rc = _lib.load().mta_headmix_fwd(x.data_ptr(), weight.data_ptr(), y.data_ptr(), n, c, p, q,
-                                         int(group_size or 0), int(bool(causal)), float(fill), _code(x, "input"),
-                                         _code(weight, "weight"), _stream(x))
+        if causal and not fill_upper:
+            rc = _lib.load().mta_headmix_tril_fwd(x.data_ptr(), weight.data_ptr(), y.data_ptr(), n, c, p, q,
+                                                  int(group_size or 0), _code(x, "input"), _code(weight, "weight"),
+                                                  _stream(x))
+        else:
+            rc = _lib.load().mta_headmix_fwd(x.data_ptr(), weight.data_ptr(), y.data_ptr(), n, c, p, q,
+                                             int(group_size or 0), int(bool(causal)), float(fill), _code(x, "input"),
+                                             _code(weight, "weight"), _stream(x))
     _lib.check(rc, "mta_headmix_fwd")
     return y
 

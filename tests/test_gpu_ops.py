@@ -198,6 +198,48 @@ def test_headmix_identity_and_permutation_bit_exact(ops):
     assert torch.equal(got, torch.tril(x[:, perm]) + 0.0)
 
 
+@pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("case", [(1, 2, 384, 6, 11), (2, 3, 200, 3, 3), (1, 2, 1024, 7, 7), (1, 1, 72, 11, 15)])
+def test_conv_tril_leaves_the_upper_triangle_alone(ops, case, dt):
+    """fill_upper=False: the lower triangle (diagonal included) is bit for bit what the filling call writes; above it
+    the output holds either what was there (sentinel) or +0."""
+    n, c, s, r, sk = case
+    dtype = DT[dt]
+    print(f"conv tril case={case} dt={dt}", flush=True)
+    x = torch.tril(_randn((n, c, s, s), 21, dtype)).cuda()
+    w = _randn((c, r, sk), 22, dtype, 0.2).cuda()
+    full = ops.conv2d_causal(x, w, True)
+    out = torch.full_like(x, 7.0)
+    got = ops.conv2d_causal(x, w, True, out=out, fill_upper=False)
+    low = ~_upper(s, s).cuda()
+    assert torch.equal(got[..., low], full[..., low])
+    up = got[..., ~low].float()
+    assert ((up == 7.0) | (up == 0)).all()
+    if dtype != torch.float32 and s % 128 == 0 and (r, sk) != (11, 15):   # the matrix-core kernel: blocks wholly above stay untouched
+        assert (got[..., 0, s - 128:].float() == 7.0).all()
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("case", [(1, 8, 300, 4), (2, 4, 2304, 2), (1, 32, 520, 0), (1, 16, 264, 0), (1, 6, 100, 3)])
+def test_headmix_tril_leaves_the_upper_triangle_alone(ops, case, dt):
+    n, c, s, group = case
+    dtype = DT[dt]
+    print(f"headmix tril case={case} dt={dt}", flush=True)
+    x = _randn((n, c, s, s), 23, dtype).cuda()
+    g = torch.Generator().manual_seed(24)
+    w = (O.block_diag_head_weight(c, group, 0.1, g, dtype) if group else
+         (torch.eye(c) + 0.1 * torch.randn(c, c, generator=g)).to(dtype)).cuda()
+    full = ops.headmix(x, w, True, 0.0, group_size=group or None)
+    out = torch.full_like(x, 7.0)
+    got = ops.headmix(x, w, True, 0.0, group_size=group or None, out=out, fill_upper=False)
+    low = ~_upper(s, s).cuda()
+    assert torch.equal(got[..., low], full[..., low])
+    up = got[..., ~low].float()
+    assert ((up == 7.0) | (up == 0)).all()
+    if s >= 2048:   # whole chunks of a row above the diagonal are never touched
+        assert (got[..., 0, s - 64:].float() == 7.0).all()
+
+
 MS_CASES = [
     # N, C, P(=Q), group, use_w1, use_w2
     (1, 4, 64, 2, True, True), (2, 4, 100, 4, True, False), (1, 8, 257, 4, False, True), (1, 2, 33, 1, False, False),
