@@ -225,6 +225,97 @@ __global__ __launch_bounds__(64 * DM_WAVES, 4) void headmix_dense32(const T *__r
     }
 }
 
+// The same for 16 heads: the contraction of a 16x16x16 product covers the 16 input heads; lane (ln, kg) fetches keys
+// 8ln .. 8ln+7 of the heads 4kg .. 4kg+3 (four 16-byte loads), forms the column of key 8ln + j with two byte permutes,
+// and after eight products holds keys 8ln .. 8ln+7 of the output heads 4kg + v.
+typedef short hm_s4 __attribute__((ext_vector_type(4)));
+typedef _Float16 hm_h4 __attribute__((ext_vector_type(4)));
+typedef unsigned int hm_u2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ f32x4 hm_mma16(bf16_t, hm_u2 a, hm_u2 b)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(hm_s4, a), __builtin_bit_cast(hm_s4, b),
+                                                     f32x4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 hm_mma16(f16_t, hm_u2 a, hm_u2 b)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(hm_h4, a), __builtin_bit_cast(hm_h4, b),
+                                                 f32x4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+}
+
+template <typename T>
+__global__ __launch_bounds__(64 * DM_WAVES, 4) void headmix_dense16(const T *__restrict__ x, const T *__restrict__ w,
+                                                               T *__restrict__ y, int C, int P, int Q, int causal,
+                                                               float fill, int wt, int qchunks)
+{
+    constexpr int HG = 16;  // heads mixed together
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, ln = lane & 15, kg = lane >> 4;
+    const int groups = C / HG;
+    unsigned b = blockIdx.x;
+    const int qc = rotated_chunk(b, qchunks);
+    const int p = (int)(b % (unsigned)P); b /= (unsigned)P;
+    const int g = (int)(b % (unsigned)groups);
+    const int64_t n = b / (unsigned)groups;
+    const int q0 = (qc * DM_WAVES + wave) * DM_KEYS;
+    if (q0 >= Q) return;
+    const int64_t plane = (int64_t)P * Q;
+    const int64_t base = (n * C + (int64_t)g * HG) * plane + (int64_t)p * Q;  // head g*16, row p, key 0
+    const int last = causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;              // last key that is mixed
+    const uint32_t fill2 = pack2<T>(fill, fill);
+    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+    const int key = q0 + ln * 8;
+
+    if (q0 > last) {  // wholly beyond the diagonal: fill only (causal == 2: not even that)
+        const u4 fv = {fill2, fill2, fill2, fill2};
+        if (key < Q && causal != 2) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                __builtin_nontemporal_store(fv, reinterpret_cast<u4 *>(y + base + (kg * 4 + t) * plane + key));
+        }
+        return;
+    }
+
+    const T *xp = x + base + (int64_t)(kg * 4) * plane + (key <= last ? key : 0);
+    u4 xv[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) xv[t] = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(xp + t * plane));
+
+    // w fragment: lane (output head ln, group kg) holds w[o][4kg .. 4kg+3]
+    hm_u2 wf;
+    if (!wt) {
+        wf = *reinterpret_cast<const hm_u2 *>(w + (int64_t)(g * HG + ln) * C + g * HG + kg * 4);
+    } else {  // the transposed matrix: a column of w, gathered element by element (once per wavefront)
+        struct alignas(8) quad { T v[4]; } col;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) col.v[t] = w[(int64_t)(g * HG + kg * 4 + t) * C + g * HG + ln];
+        wf = __builtin_bit_cast(hm_u2, col);
+    }
+
+    f32x4 acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const unsigned sel = (j & 1) ? 0x07060302u : 0x05040100u;
+        const hm_u2 col = {__builtin_amdgcn_perm(xv[1][j >> 1], xv[0][j >> 1], sel),
+                           __builtin_amdgcn_perm(xv[3][j >> 1], xv[2][j >> 1], sel)};  // heads 4kg .. 4kg+3 of key 8ln + j
+        acc[j] = hm_mma16(T{}, wf, col);
+    }
+    if (key >= Q || (causal == 2 && key > last)) return;
+    // acc[j][v]: output head 4kg + v, key 8ln + j
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        u4 o;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) o[u] = pack2<T>(acc[2 * u][v], acc[2 * u + 1][v]);
+        if (key + 7 > last) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (key + 2 * u > last) o[u] = (o[u] & 0xffff0000u) | (fill2 & 0x0000ffffu);
+                if (key + 2 * u + 1 > last) o[u] = (o[u] & 0x0000ffffu) | (fill2 & 0xffff0000u);
+            }
+        }
+        __builtin_nontemporal_store(o, reinterpret_cast<u4 *>(y + base + (int64_t)(kg * 4 + v) * plane + key));
+    }
+}
+
 // Any group size: one (output head, vector) per lane-iteration, inputs re-read per output head.
 template <typename T, int VEC>
 __global__ __launch_bounds__(NT) void headmix_any(const T *__restrict__ x, const void *__restrict__ w,
@@ -271,6 +362,14 @@ int launch(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t 
         // 32 heads mixed densely, 16-bit data and weights of the same dtype: matrix cores (MTA_HEADMIX_NO_MFMA=1 in the
         // environment keeps the vector-ALU kernel, for comparisons)
         static const bool no_mfma = [] { const char *e = getenv("MTA_HEADMIX_NO_MFMA"); return e && e[0] == '1'; }();
+        if (G == 16 && !no_mfma && w_same_dtype && aligned_to(w, 8) && C % 4 == 0) {
+            const int qch = (int)((Q + DM_WAVES * DM_KEYS - 1) / (DM_WAVES * DM_KEYS));
+            const int64_t blocks = N * (C / 16) * P * qch;
+            if (blocks > 0x7fffffffLL) return MTA_ERR_SHAPE;
+            hipLaunchKernelGGL((headmix_dense16<T>), dim3((unsigned)blocks), dim3(64 * DM_WAVES), 0, st, (const T *)x,
+                               (const T *)w, (T *)y, (int)C, (int)P, (int)Q, causal, fill, wt, qch);
+            return launch_status();
+        }
         if (G == 32 && !no_mfma && w_same_dtype && aligned_to(w, 16) && C % 8 == 0) {
             const int qch = (int)((Q + DM_WAVES * DM_KEYS - 1) / (DM_WAVES * DM_KEYS));
             const int64_t blocks = N * (C / 32) * P * qch;
