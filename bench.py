@@ -124,7 +124,7 @@ def build_c4(torch, mta, O, device, b=2, h=16, s=4096, d=128, dtype=None, nsets=
     return mod, sets
 
 
-def build_general(torch, mta, O, device, b=1, h=16, s=4096, d=128, nsets=2):
+def build_general(torch, mta, O, device, b=1, h=16, s=4096, d=128, nsets=2, train=False):
     """The closest shape to the reference's published rows (benchmark_seq_len_results.jsonl: H16 D128 fp16, 7x7 conv
     before and after the softmax): all four weights non-trivial -- random 7x7 kernels, dense random 16x16 head weights."""
     dtype = torch.float16
@@ -136,8 +136,10 @@ def build_general(torch, mta, O, device, b=1, h=16, s=4096, d=128, nsets=2):
         mod.mta_conv_after_sm_triton.weight.copy_(O.seeded_conv_weight(h, 7, 7, 0.05, dtype, seed=6))
         mod.wpsm_triton.weight.copy_(torch.eye(h) + 0.1 * torch.randn(h, h, generator=g))
         mod.wposm_triton.weight.copy_(torch.eye(h) + 0.1 * torch.randn(h, h, generator=g))
-    mod = mod.to(device).eval().requires_grad_(False)   # dense weights: nothing is assumed about their structure
-    sets = [tuple(t.to(device) for t in O.seeded_qkv(b, h, s, d, dtype, seed=400 + i)) for i in range(nsets)]
+    mod = mod.to(device)                                 # dense weights: nothing is assumed about their structure
+    mod = mod.train() if train else mod.eval().requires_grad_(False)
+    sets = [tuple(t.to(device).requires_grad_(train) for t in O.seeded_qkv(b, h, s, d, dtype, seed=400 + i))
+            for i in range(nsets)]
     return mod, sets
 
 
@@ -206,7 +208,17 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
     by = score_pass_bytes(n, c, s, 2)
     out["conv2d_6x11_bf16_2x16x2048x2048"] = {"ms": ms, "algorithmic_bytes": by, "GBps": by / ms / 1e6,
                                               "frac_hbm_peak": by / ms / 1e6 / HBM_PEAK_GBS}
-    del xs, ys
+    del ys
+    # its two gradients at the same shape (convolution_2d_trit.py:336-378): dx reads the lower triangle of dy and
+    # writes all of dx; dw reads the lower triangles of x and dy
+    ms = time_launches(torch, lambda i: mta.ops.conv2d_bwd_input(xs[i], w, True), 3, warmup, steps)
+    out["conv2d_bwd_input_6x11_bf16_2x16x2048x2048"] = {"ms": ms, "algorithmic_bytes": by, "GBps": by / ms / 1e6,
+                                                        "frac_hbm_peak": by / ms / 1e6 / HBM_PEAK_GBS}
+    by2 = 2 * n * c * tri(s) * 2
+    ms = time_launches(torch, lambda i: mta.ops.conv2d_bwd_weight(xs[i], xs[(i + 1) % 3], (6, 11), True), 3, warmup, steps)
+    out["conv2d_bwd_weight_6x11_bf16_2x16x2048x2048"] = {"ms": ms, "algorithmic_bytes": by2, "GBps": by2 / ms / 1e6,
+                                                         "frac_hbm_peak": by2 / ms / 1e6 / HBM_PEAK_GBS}
+    del xs
     # head-mix alone: (2,32,2048,2048) bf16, groups of 4
     n, c, s = 2, 32, 2048
     wm = O.block_diag_head_weight(c, 4, 0.1, g, bf16).to(device)
@@ -221,7 +233,16 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
     for label, grp in (("headmix_g4_bf16_2x32x2048x2048", 4), ("headmix_dense_bf16_2x32x2048x2048", None)):
         ms = time_launches(torch, lambda i: mta.ops.headmix(xs[i], wm, True, 0.0, group_size=grp, out=ys[i]), 2, warmup, steps)
         out[label] = {"ms": ms, "algorithmic_bytes": by, "GBps": by / ms / 1e6, "frac_hbm_peak": by / ms / 1e6 / HBM_PEAK_GBS}
-    del xs, ys
+    del ys
+    # its two gradients (triton_linear_head.py:322-370): dx = W^T dy (groups of 4), dW = dy x^T over the attended positions
+    ms = time_launches(torch, lambda i: mta.ops.headmix_bwd_input(xs[i], wm, True, group_size=4), 2, warmup, steps)
+    out["headmix_bwd_input_g4_bf16_2x32x2048x2048"] = {"ms": ms, "algorithmic_bytes": by, "GBps": by / ms / 1e6,
+                                                       "frac_hbm_peak": by / ms / 1e6 / HBM_PEAK_GBS}
+    by2 = 2 * n * c * tri(s) * 2
+    ms = time_launches(torch, lambda i: mta.ops.headmix_bwd_weight(xs[i], xs[1 - i], True), 2, warmup, steps)
+    out["headmix_bwd_weight_bf16_2x32x2048x2048"] = {"ms": ms, "algorithmic_bytes": by2, "GBps": by2 / ms / 1e6,
+                                                     "frac_hbm_peak": by2 / ms / 1e6 / HBM_PEAK_GBS}
+    del xs
     # fused conv-attention: B1 H32 S8192 D128 bf16, 6x11
     b, h, s, d = 1, 32, 8192, 128
     sets = [tuple(t.to(device) for t in O.seeded_qkv(b, h, s, d, bf16, seed=200 + i)) for i in range(2)]
@@ -241,6 +262,25 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
     out["mta_forward_general_fp16_1x16x4096x128_7x7_pre_post_dense"] = {
         "ms": ms, "stages_ms": stages,
         "note": "forward only; the reference's published row for this shape (Triton 11.345 ms, PyTorch 43.795 ms, "
+                "hardware unstated) is context, not a baseline"}
+    del mod, sets
+    # the same module and shape in training: forward operator by operator (each with its HIP backward kernels; the two
+    # matrix products, the softmax and the dropout are torch's) and backward to q, k, v and the four weights
+    mod, sets = build_general(torch, mta, O, device, train=True)
+    params = [p for p in mod.parameters()]
+    gout = torch.randn(sets[0][0].shape, generator=torch.Generator().manual_seed(9)).to(sets[0][0].dtype).to(device)
+    gout = gout.transpose(1, 2)
+
+    def train_step(i):
+        for t in params + list(sets[i]):
+            t.grad = None
+        with torch.enable_grad():
+            mod(*sets[i], None, None).backward(gout)
+
+    ms = time_steps(torch, train_step, len(sets), min(warmup, 5), max(3, steps // 10))
+    out["mta_forward_backward_general_fp16_1x16x4096x128_7x7_pre_post_dense"] = {
+        "ms": ms,
+        "note": "forward + backward; the reference's published row for this shape (Triton 39.090 ms, PyTorch 253.350 ms, "
                 "hardware unstated) is context, not a baseline"}
     return out
 

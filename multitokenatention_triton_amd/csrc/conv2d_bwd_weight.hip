@@ -10,7 +10,14 @@
 //
 // Work split: the persistent workgroups are divided among the channels; the workgroups of a channel walk that
 // channel's (batch, 32x64 tile) list with a stride.  Tiles wholly above the diagonal are skipped.
+//
+// 16-bit tensors whose rows are a multiple of 8 keys take the matrix cores (conv2d_bwd_weight_mfma): for a fixed
+// key offset j the sums over q of dy[p,q] * x[p',q+j-pad] for 16 rows p and 16 rows p' are one 16x16 product with the
+// keys as contraction index, and the taps (i,j) are the entries p'-p = i-(R-1) of it.  Every 16-row block of dy meets
+// the two 16-row blocks of x that hold its R-1 rows of halo, and all blocks add into the same 2*S accumulators, since
+// only p'-p matters.  The operand of offset j is the lane's 24-key window of x shifted by j keys in registers.
 #include "common.hpp"
+#include "mfma.hpp"
 
 namespace {
 using namespace mta;
@@ -138,6 +145,138 @@ __global__ __launch_bounds__(NT) void conv2d_bwd_weight_fixed(const T *__restric
     }
 }
 
+// ---- matrix-core kernel -------------------------------------------------------------------------------------------
+typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+constexpr int MROWS = 32;  // rows of dy per work item (two 16-row blocks against three 16-row blocks of x)
+
+// Eight consecutive keys k0..k0+7 (k0 a multiple of 8, possibly -8) of row h, with the forward pass's masks: 0 outside
+// the plane and, under the causal rule, for keys beyond the row index.  `edge` = this step may straddle the diagonal.
+template <typename T>
+__device__ __forceinline__ u4 masked_piece(const T *plane, int h, int k0, int H, int W, int causal, bool edge)
+{
+    u4 v = {0u, 0u, 0u, 0u};
+    const bool ok = (unsigned)h < (unsigned)H && (unsigned)k0 < (unsigned)W && !(causal && k0 > h);
+    if (ok) v = *reinterpret_cast<const u4 *>(plane + (int64_t)h * W + k0);
+    if (edge && causal) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int e = k0 + 2 * u;
+            v[u] &= (e <= h ? 0x0000ffffu : 0u) | (e + 1 <= h ? 0xffff0000u : 0u);
+        }
+    }
+    return v;
+}
+
+// One step's operands of a wavefront: keys kb + 8g .. +7 of the lane's rows; for x also the eight keys on either side.
+struct step_operands {
+    u4 dy[2];
+    u4 x[3][3];
+};
+
+template <typename T>
+__device__ __forceinline__ void load_step(step_operands &o, const T *xp, const T *dyp, int p0, int kb, int r, int g,
+                                          int H, int W, int causal)
+{
+    const int k = kb + 8 * g;
+    // rows of this item start at p0 - 16; the step can meet the diagonal if its last key (plus the window) passes that
+    const bool edge = causal && kb + 31 + 8 > p0 - 16;
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) o.dy[mb] = masked_piece(dyp, p0 + 16 * mb + r, k, H, W, causal, edge);
+#pragma unroll
+    for (int nb = 0; nb < 3; ++nb)
+#pragma unroll
+        for (int s = 0; s < 3; ++s) o.x[nb][s] = masked_piece(xp, p0 - 16 + 16 * nb + r, k - 8 + 8 * s, H, W, causal, edge);
+}
+
+template <typename T, int R, int S>
+__global__ __launch_bounds__(NT) void conv2d_bwd_weight_mfma(const T *__restrict__ x, const T *__restrict__ dy,
+                                                             float *__restrict__ partial, int N, int C, int H, int W,
+                                                             int causal, int tiles_m, int nseg, int bpc)
+{
+    static_assert(R <= 17 && S <= 16 && (S - 1) / 2 <= 8, "window of 24 keys, two 16-row blocks of halo");
+    constexpr int PW = (S - 1) / 2;
+    __shared__ float tile[2 * S][16][17];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
+    const int c = blockIdx.x / bpc, sub = blockIdx.x % bpc;
+
+    // acc[half][j]: D[m][n] = sum over keys of dy[p0m + m, q] * x[p0m - 16 + 16*half + n, q + j - PW]
+    f32x4 acc[2][S];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < S; ++j) acc[h][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    const int64_t items = (int64_t)N * tiles_m * nseg;
+    for (int64_t it = (int64_t)sub * (NT / 64) + wave; it < items; it += (int64_t)bpc * (NT / 64)) {
+        const int sg = (int)(it % nseg);
+        const int64_t rest = it / nseg;
+        const int ti = (int)(rest % tiles_m), n = (int)(rest / tiles_m);
+        const int tm = (ti & 1) ? tiles_m - 1 - (ti >> 1) : (ti >> 1);  // long and short rows alternate
+        const int p0 = tm * MROWS;
+        int kend = W;  // dy is zero beyond the diagonal: keys from p0 + MROWS on add nothing
+        if (causal && p0 + MROWS < W) kend = p0 + MROWS;
+        const int nsteps = (kend + 31) / 32, per = (nsteps + nseg - 1) / nseg;
+        const int t0 = sg * per, t1 = (t0 + per < nsteps) ? t0 + per : nsteps;
+        if (t0 >= t1) continue;
+        const int64_t plane = ((int64_t)n * C + c) * H * W;
+        const T *xp = x + plane, *dyp = dy + plane;
+        step_operands cur;
+        load_step(cur, xp, dyp, p0, 32 * t0, r, g, H, W, causal);
+        for (int t = t0; t < t1; ++t) {
+            step_operands nxt;
+            if (t + 1 < t1) load_step(nxt, xp, dyp, p0, 32 * (t + 1), r, g, H, W, causal);
+            else nxt = cur;
+            frag8<T> a[2];
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb) a[mb] = __builtin_bit_cast(frag8<T>, cur.dy[mb]);
+#pragma unroll
+            for (int nb = 0; nb < 3; ++nb) {
+                unsigned w[12];
+#pragma unroll
+                for (int s = 0; s < 3; ++s)
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) w[4 * s + u] = cur.x[nb][s][u];
+#pragma unroll
+                for (int j = 0; j < S; ++j) {
+                    const int o = 8 + j - PW;  // first key of the operand inside the window (compile-time after unrolling)
+                    u4 bv;
+#pragma unroll
+                    for (int d = 0; d < 4; ++d)
+                        bv[d] = (o & 1) ? __builtin_amdgcn_alignbyte(w[(o + 1) / 2 + d], w[(o - 1) / 2 + d], 2) : w[o / 2 + d];
+                    const frag8<T> b = __builtin_bit_cast(frag8<T>, bv);
+                    if (nb <= 1) mma16(acc[0][j], a[nb], b);
+                    if (nb >= 1) mma16(acc[1][j], a[nb - 1], b);
+                }
+            }
+            cur = nxt;
+        }
+    }
+
+    // tap (i,j) = sum over m of D_j[m][m + i - (R-1)] taken from the half that holds that column; the four wavefronts
+    // pass through the LDS tile one after the other and every tap is added up in a fixed order
+    float s = 0.0f;
+    const int ti = tid / S, tj = tid % S;
+    for (int wv = 0; wv < NT / 64; ++wv) {
+        __syncthreads();
+        if (wave == wv) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int j = 0; j < S; ++j)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) tile[h * S + j][4 * g + v][r] = acc[h][j][v];
+        }
+        __syncthreads();
+        if (tid < R * S) {
+            for (int m = 0; m < 16; ++m) {
+                const int n1 = m + ti - (R - 1);
+                s += n1 >= 0 ? tile[S + tj][m][n1] : tile[tj][m][n1 + 16];
+            }
+        }
+    }
+    if (tid < R * S) partial[((int64_t)c * bpc + sub) * (R * S) + tid] = s;
+}
+
 // Any kernel size: x halo tile and dy tile in LDS, the R*S running sums in LDS too; thread t owns taps t, t+256, ...
 // (nothing is unrolled over the taps: the fixed-size kernel above is the fast path).
 template <typename T>
@@ -232,8 +371,40 @@ int launch(const void *x, const void *dy, float *dw, float *partial, int bpc, in
            int R, int S, int causal, hipStream_t st)
 {
     const int tiles_m = (int)((H + TM - 1) / TM), tiles_n = (int)((W + TN - 1) / TN);
-    dim3 grid((unsigned)(C * bpc));
     const int vec_ok = (W % 8 == 0 && aligned_to(dy, 16)) ? 1 : 0;
+    dim3 grid((unsigned)(C * bpc));
+    if constexpr (sizeof(T) == 2) {
+        // 16-bit tensors with rows of whole 16-byte vectors: matrix cores (MTA_CONV_FORCE_VALU=1 in the environment keeps
+        // the fp32-FMA kernel, for comparisons).  Two workgroups per CU; the key range of a row block is cut into
+        // segments until every wavefront has about two items.
+        static const bool force_valu = [] { const char *e = getenv("MTA_CONV_FORCE_VALU"); return e && e[0] == '1'; }();
+        if (!force_valu && vec_ok && aligned_to(x, 16) && R <= MROWS / 2 + 1) {
+            const int rows_m = (int)((H + MROWS - 1) / MROWS);
+            int bm = (int)((512 + C - 1) / C);
+            if (bm > bpc) bm = bpc;
+            int64_t nseg = ((int64_t)8 * bm + N * rows_m - 1) / (N * rows_m);
+            const int64_t seg_cap = W / 256 > 1 ? W / 256 : 1;
+            if (nseg > seg_cap) nseg = seg_cap;
+            if (nseg > 8) nseg = 8;
+            if (bm > N * rows_m * nseg) bm = (int)(N * rows_m * nseg);
+#define MTA_CONV_CASE(r, s)                                                                                          \
+    if (R == r && S == s) {                                                                                          \
+        hipLaunchKernelGGL((conv2d_bwd_weight_mfma<T, r, s>), dim3((unsigned)(C * bm)), dim3(NT), 0, st,              \
+                           (const T *)x, (const T *)dy, partial, (int)N, (int)C, (int)H, (int)W, causal, rows_m,      \
+                           (int)nseg, bm);                                                                           \
+        bpc = bm;                                                                                                    \
+        goto reduce;                                                                                                 \
+    }
+            MTA_CONV_CASE(3, 3)
+            MTA_CONV_CASE(3, 5)
+            MTA_CONV_CASE(5, 5)
+            MTA_CONV_CASE(5, 7)
+            MTA_CONV_CASE(6, 11)
+            MTA_CONV_CASE(7, 7)
+            MTA_CONV_CASE(7, 9)
+#undef MTA_CONV_CASE
+        }
+    }
 #define MTA_CONV_CASE(r, s)                                                                                          \
     if (R == r && S == s) {                                                                                          \
         hipLaunchKernelGGL((conv2d_bwd_weight_fixed<T, r, s>), grid, dim3(NT), 0, st, (const T *)x, (const T *)dy,    \

@@ -359,8 +359,8 @@ int launch(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t 
            float fill, int w_dtype, int wt, bool w_same_dtype, hipStream_t st)
 {
     if constexpr (VEC == 8) {
-        // 32 heads mixed densely, 16-bit data and weights of the same dtype: matrix cores (MTA_HEADMIX_NO_MFMA=1 in the
-        // environment keeps the vector-ALU kernel, for comparisons)
+        // 16 or 32 heads mixed densely, 16-bit data and weights of the same dtype: matrix cores
+        // (MTA_HEADMIX_NO_MFMA=1 in the environment keeps the vector-ALU kernel, for comparisons)
         static const bool no_mfma = [] { const char *e = getenv("MTA_HEADMIX_NO_MFMA"); return e && e[0] == '1'; }();
         if (G == 16 && !no_mfma && w_same_dtype && aligned_to(w, 8) && C % 4 == 0) {
             const int qch = (int)((Q + DM_WAVES * DM_KEYS - 1) / (DM_WAVES * DM_KEYS));

@@ -648,6 +648,34 @@ def test_mta_unfused_16bit_route_never_reads_above_the_diagonal(pkg):
     torch.testing.assert_close(out.transpose(1, 2).cpu().float(), want.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("h,group,dtype", [(8, 4, torch.bfloat16), (16, 16, torch.float16), (32, 32, torch.bfloat16)])
+def test_mta_lower_triangle_route_never_reads_above_the_diagonal(pkg, h, group, dtype):
+    """The inference route writes none of its intermediates above the diagonal (scores kernel and mix + softmax with
+    fill_upper=False, mta_conv2d_tril_fwd, mta_headmix_tril_fwd).  Every stage here writes into a NaN-filled buffer
+    and gets its input with the upper triangle set to NaN again: the result must be the oracle's."""
+    print(f"mta lower-triangle route h={h} group={group} {dtype}", flush=True)
+    b, s, d = 1, 264, 64
+    ops = pkg.ops
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=96)
+    w_pre, wpsm, w_post, wposm = _config_like(h, group, 6, 11, 0.05, dtype, post="random")
+    want = _oracle_mta(q, k, v, [w_pre, wpsm, w_post, wposm])
+    up = torch.triu(torch.ones(s, s, dtype=torch.bool, device="cuda"), 1)
+    nan = lambda: torch.full((b, h, s, s), float("nan"), dtype=dtype, device="cuda")
+    again = lambda t: t.masked_fill(up, float("nan"))
+    scale = float(torch.rsqrt(torch.tensor(float(d))))
+    x = again(ops.qk_conv(q.cuda(), k.cuda(), w_pre.cuda(), True, scale, fill_upper=False, out=nan()))
+    if group <= 16:
+        x = again(ops.headmix_softmax(x, wpsm.cuda(), None, True, group_size=group, out=nan(), fill_upper=False))
+    else:
+        x = again(ops.headmix(x, wpsm.cuda(), True, float("-inf"), group_size=group, out=nan(), fill_upper=False))
+        x = again(ops.headmix_softmax(x, None, None, True, out=nan(), fill_upper=False))
+    x = again(ops.conv2d_causal(x, w_post.cuda(), True, out=nan(), fill_upper=False))
+    x = again(ops.headmix(x, wposm.cuda(), True, 0.0, group_size=group, out=nan(), fill_upper=False))
+    assert torch.isfinite(x[..., ~up].float()).all()
+    out = ops.causal_pv(x, v.cuda(), True)
+    torch.testing.assert_close(out.transpose(1, 2).cpu().float(), want.float(), **tol(dtype))
+
+
 @pytest.mark.parametrize("case", [(1, 2, 300, 64, 6, 11, True, torch.float32), (1, 2, 777, 128, 6, 11, True, torch.bfloat16),
                                   (2, 2, 260, 64, 3, 3, False, torch.float16), (1, 2, 333, 128, 11, 15, True, torch.bfloat16)])
 def test_conv_attention_lse(pkg, case):

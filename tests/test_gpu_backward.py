@@ -53,6 +53,12 @@ CONV_CASES = [
     (1, 2, 264, 264, 7, 7, True),
     (1, 2, 512, 512, 6, 11, True),     # several strips / tiles per plane, interior ones included
     (1, 1, 200, 200, 7, 9, True),
+    # 16-bit: matrix-core weight-gradient kernel (rows of whole 16-byte vectors)
+    (1, 2, 72, 72, 6, 11, False),
+    (2, 2, 40, 96, 5, 5, False),       # not square
+    (1, 2, 96, 40, 3, 5, True),        # causal rule on a tall plane: keys beyond the row index never take part
+    (1, 1, 1040, 1040, 7, 7, True),    # key range cut into segments, many steps per item
+    (3, 5, 136, 136, 5, 7, True),
 ]
 
 
