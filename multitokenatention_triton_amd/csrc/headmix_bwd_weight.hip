@@ -9,8 +9,8 @@
 //
 // 16-bit tensors with C = 16 or 32 take the matrix cores: A = dY (rows = output heads), B = X (columns = input heads),
 // 32 positions per v_mfma_f32_16x16x32.  Which position feeds which contraction slot is free as long as both
-// operands agree, so lane (head r, group g) reads the 64 contiguous bytes of positions 32g..32g+31 of its 128-position
-// chunk and product t takes the t-th 16 bytes of them: a wavefront's load instruction covers 16 heads x 256 bytes.
+// operands agree; product t of a 128-position chunk takes positions 32t..32t+31, lane (head r, group g) the eight from
+// 32t + 8g on: a wavefront's load instruction covers 64 contiguous bytes of each of 16 heads.
 // Everything else (fp32, other head counts, rows that are not a multiple of 8 keys) takes a generic LDS kernel.
 #include "common.hpp"
 #include "mfma.hpp"
@@ -51,12 +51,13 @@ __global__ __launch_bounds__(NT) void headmix_bwd_weight_mfma(const T *__restric
             const int last = causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;  // last position of the row that takes part
             const int64_t rowbase = (int64_t)n * C * plane + (int64_t)p * Q;
             for (int q0 = 0; q0 <= last; q0 += CHUNK) {
-                const int q = q0 + 32 * g;  // this lane's 32 positions: q .. q+31, four 16-byte vectors
+                const int q = q0 + 8 * g;  // this lane's positions: q + 32t .. +7 for product t (a load instruction
+                                           // covers 64 contiguous bytes of each of 16 heads)
                 u4 av[NB][4], bv[NB][4];
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     // a vector wholly beyond `last` re-reads the row start (valid memory) and is zeroed below
-                    const int qq = (q + 8 * t <= last) ? q + 8 * t : 0;
+                    const int qq = (q + 32 * t <= last) ? q + 32 * t : 0;
 #pragma unroll
                     for (int a = 0; a < NB; ++a) {
                         av[a][t] = *reinterpret_cast<const u4 *>(dy + rowbase + (int64_t)(a * 16 + r) * plane + qq);
@@ -69,7 +70,7 @@ __global__ __launch_bounds__(NT) void headmix_bwd_weight_mfma(const T *__restric
                     for (int t = 0; t < 4; ++t)
 #pragma unroll
                         for (int u = 0; u < 4; ++u) {
-                            const int e = q + 8 * t + 2 * u;
+                            const int e = q + 32 * t + 2 * u;
                             const unsigned keep = (e <= last ? 0x0000ffffu : 0u) | (e + 1 <= last ? 0xffff0000u : 0u);
 #pragma unroll
                             for (int a = 0; a < NB; ++a) {
@@ -150,14 +151,28 @@ __global__ __launch_bounds__(NT) void headmix_bwd_weight_any(const T *__restrict
     for (int pair = tid; pair < CC; pair += NT) partial[(int64_t)blockIdx.x * CC + pair] = sums[pair];
 }
 
-__global__ __launch_bounds__(NT) void reduce_partials(const float *__restrict__ partial, float *__restrict__ dw, int CC,
-                                                      int nparts)
+// dw[e] = sum of the partial matrices' entries e, in a fixed order: 64 entries per workgroup, the partial matrices dealt
+// to 16 wavefronts (each adds its share in index order), the 16 sums added in wavefront order
+constexpr int RED_SLICES = 16;
+__global__ __launch_bounds__(64 * RED_SLICES) void reduce_partials(const float *__restrict__ partial,
+                                                                   float *__restrict__ dw, int CC, int nparts)
 {
-    const int e = blockIdx.x * NT + threadIdx.x;
-    if (e >= CC) return;
+    __shared__ float red[RED_SLICES][64];
+    const int le = threadIdx.x & 63, sl = threadIdx.x >> 6;
+    const int e = blockIdx.x * 64 + le;
     float s = 0.0f;
-    for (int b = 0; b < nparts; ++b) s += partial[(int64_t)b * CC + e];
-    dw[e] = s;
+    if (e < CC) {
+#pragma unroll 8
+        for (int b = sl; b < nparts; b += RED_SLICES) s += partial[(int64_t)b * CC + e];
+    }
+    red[sl][le] = s;
+    __syncthreads();
+    if (sl == 0 && e < CC) {
+        float t = 0.0f;
+#pragma unroll
+        for (int k = 0; k < RED_SLICES; ++k) t += red[k][le];
+        dw[e] = t;
+    }
 }
 
 constexpr int64_t MAX_WS_BYTES = 8 << 20;  // partial matrices never take more than this
@@ -165,7 +180,7 @@ constexpr int64_t MAX_WS_BYTES = 8 << 20;  // partial matrices never take more t
 // persistent workgroups (= partial matrices) for a problem
 inline int num_blocks(int64_t N, int64_t C, int64_t P, int64_t Q)
 {
-    int64_t nb = 512;
+    int64_t nb = 1024;
     const int64_t pairs = (N * P + 1) / 2;
     if (nb > pairs) nb = pairs;
     const int64_t cap = MAX_WS_BYTES / (C * C * (int64_t)sizeof(float));
@@ -220,6 +235,7 @@ extern "C" int mta_headmix_bwd_weight(const void *x, const void *dy, void *dw, v
     int rc = launch_status();
     if (rc != MTA_OK) return rc;
     const int CC = (int)(C * C);
-    hipLaunchKernelGGL(reduce_partials, dim3((unsigned)((CC + NT - 1) / NT)), dim3(NT), 0, st, partial, (float *)dw, CC, nb);
+    hipLaunchKernelGGL(reduce_partials, dim3((unsigned)((CC + 63) / 64)), dim3(64 * RED_SLICES), 0, st, partial, (float *)dw,
+                       CC, nb);
     return launch_status();
 }
