@@ -18,9 +18,14 @@ Inference (no input or parameter requires grad, or grad mode is off):
     the conv result never reaches HBM;
   * P V reads only the lower triangle of P (``mta_causal_pv_fwd``).
 
-Training (something requires grad): the stages run one by one through the autograd
-Functions of convolution_2d_trit / triton_linear_head, as in the reference, so that
-``backward()`` works; torch differentiates the two GEMMs, the softmax and the dropout.
+Training (something requires grad): the stages run one by one through autograd
+Functions, as in the reference, so that ``backward()`` works: the two conv and the two
+head-mixing stages with their HIP gradient kernels (convolution_2d_trit /
+triton_linear_head); the 1/sqrt(D) factor folded into the pre-softmax conv and, in
+backward, into the (B,H,S,D) gradients of Q and K; pre-softmax head mixing and softmax as
+one forward kernel where the inference route has one, with torch's softmax gradient taken
+from the stored 16-bit probabilities (no fp32 copy of the score tensor in either
+direction).  torch differentiates the two GEMMs and the dropout.
 
 Weight structure.  By default nothing is assumed about the four weights: every stage runs
 with the dense weight it is given.  Skipping identity stages and applying block-diagonal
@@ -68,6 +73,70 @@ def _one_pass_group(group: int, scores_dtype, n_keys: int, *weights) -> bool:
 # where the one-pass post-softmax conv + head mixing kernel is used (see forward)
 _CONV_MIX_MAX_GROUP = 4
 _CONV_MIX_SIZES = ((3, 3), (7, 7))
+
+
+class _ScaledScoresConv(torch.autograd.Function):
+    """conv(round(Q K^T) * scale) for the training route (mta_attention_triton.py:69-73): the library GEMM, then
+    ``mta_conv2d_scaled_fwd``, which applies the factor (and the rounding to the score dtype that the reference's
+    separate multiplication performs) on the way into the conv.  Backward: the conv's input gradient ``g`` goes through
+    the two GEMMs and the factor is applied to their (B,H,S,D) results; the kernel gradient is taken against the raw
+    scores and scaled afterwards.  Neither direction spends a pass over the (B,H,S,S) tensor on the factor."""
+
+    @staticmethod
+    def forward(ctx, xq, xk, weight, scale, causal, mark):
+        mark("qk")
+        raw = torch.matmul(xq, xk.transpose(2, 3))
+        mark("conv_pre")
+        ctx.save_for_backward(xq, xk, weight, raw)
+        ctx.scale, ctx.causal = scale, causal
+        return ops.conv2d_causal(raw, weight, causal, in_scale=scale)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        xq, xk, weight, raw = ctx.saved_tensors
+        dq = dk = dw = None
+        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+            g = ops.conv2d_bwd_input(grad_output, weight, ctx.causal)
+            if ctx.needs_input_grad[0]:
+                dq = torch.matmul(g, xk) * ctx.scale
+            if ctx.needs_input_grad[1]:
+                dk = torch.matmul(g.transpose(2, 3), xq) * ctx.scale
+        if ctx.needs_input_grad[2]:
+            dw = ops.conv2d_bwd_weight(raw, grad_output.to(raw.dtype), tuple(weight.shape[1:]), ctx.causal)
+            dw = (dw * ctx.scale).to(weight.dtype)
+        return dq, dk, dw, None, None, None
+
+
+class _MixSoftmax(torch.autograd.Function):
+    """softmax(mix(x, weight)) over the keys for the training route (mta_attention_triton.py:75-79), one kernel
+    (``mta_headmix_softmax_fwd``; ``weight=None``: the softmax alone).  The probabilities are computed in fp32 from the
+    mixed scores rounded to the score dtype and stored in it, as ``F.softmax(scores.float()).type_as(scores)`` leaves
+    them.  Backward: torch's softmax gradient from the stored probabilities, then the head mixing's two gradient
+    kernels."""
+
+    @staticmethod
+    def forward(ctx, x, weight, causal, group_size):
+        p = ops.headmix_softmax(x, weight, None, causal, group_size=group_size if weight is not None else None)
+        ctx.save_for_backward(x if weight is not None else None, weight, p)
+        ctx.causal, ctx.group_size = causal, group_size
+        return p
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, weight, p = ctx.saved_tensors
+        ds = torch._softmax_backward_data(grad_output.to(p.dtype), p, -1, p.dtype)
+        if weight is None:
+            return ds, None, None, None
+        dx = dw = None
+        if ctx.needs_input_grad[0]:
+            dx = ops.headmix_bwd_input(ds, weight, ctx.causal, ctx.group_size)
+        if ctx.needs_input_grad[1]:
+            dw = ops.headmix_bwd_weight(x, ds, ctx.causal)
+            if ctx.group_size:
+                blk = torch.arange(weight.shape[0], device=weight.device) // ctx.group_size
+                dw = dw * (blk[:, None] == blk[None, :])
+            dw = dw.to(weight.dtype)
+        return dx, dw, None, None
 
 
 @dataclass
@@ -230,15 +299,18 @@ class MTAAttentionTriton(nn.Module):
         """The reference's own sequence of operators (mta_attention_triton.py:68-92), each differentiable: taken
         whenever a gradient may be asked for.  No weight structure is assumed here, so every entry of the four
         weights receives its gradient."""
-        scale = torch.rsqrt(torch.tensor(float(xq.size(-1)), device=xq.device))
-        self._mark("qk")
-        scores = torch.matmul(xq, xk.transpose(2, 3)) * scale
-        self._mark("conv_pre")
-        scores = self.mta_conv_triton(scores)
-        self._mark("mix_pre")
-        scores = self.wpsm_triton(scores)
-        self._mark("softmax")
-        scores = F.softmax(scores.float(), dim=-1).type_as(xq)
+        scale = float(torch.rsqrt(torch.tensor(float(xq.size(-1)))))
+        scores = _ScaledScoresConv.apply(xq, xk, self.mta_conv_triton.weight, scale, self.causal, self._mark)
+        group = self.wpsm_triton.group_size
+        w_pre = self.wpsm_triton.weight
+        if _one_pass_group(group or self.n_heads, scores.dtype, xk.size(-2), w_pre):
+            self._mark("mix_softmax")
+            scores = _MixSoftmax.apply(scores, w_pre, self.causal, group)
+        else:
+            self._mark("mix_pre")
+            scores = self.wpsm_triton(scores)
+            self._mark("softmax")
+            scores = _MixSoftmax.apply(scores, None, self.causal, None)
         self._mark("conv_post")
         scores = self.mta_conv_after_sm_triton(scores)
         self._mark("mix_post")
@@ -317,7 +389,7 @@ class MTAAttentionTriton(nn.Module):
                 return self._forward_fused(xq, xk.masked_fill(hidden, 0), xv.masked_fill(hidden, 0),
                                            key_bias=bias.contiguous())
         mask = self._update_mask(mask=mask, bsz=xq.size(0), xq=xq, xk_size=xk.size(-2))
-        scale = torch.rsqrt(torch.tensor(float(xq.size(-1)), device=xq.device))
+        scale = float(torch.rsqrt(torch.tensor(float(xq.size(-1)))))  # a host scalar: the product stays one vectorised pass
         scores = torch.matmul(xq, xk.transpose(2, 3)) * scale
         blocked = mask == float("-inf")
         scores = self.mta_conv_triton(scores.masked_fill(blocked, 0))

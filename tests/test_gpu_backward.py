@@ -177,7 +177,7 @@ def _mta_pair(pkg, h, r1, s1, dtype, seed):
     return mod.to(dtype).cuda().eval(), params
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_mta_module_backward(pkg, dtype):
     """compare_mta_attention.py:123-162 restated: gradients with respect to xq, xk, xv and the four MTA weights of
     MTAAttentionTriton against autograd through the PyTorch restatement (seed 123, B2 H16 S128 D64 as in :21-27,
