@@ -149,15 +149,28 @@ __global__ __launch_bounds__(NT) void conv2d_bwd_weight_fixed(const T *__restric
 typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 constexpr int MROWS = 32;  // rows of dy per work item (two 16-row blocks against three 16-row blocks of x)
 
-// Eight consecutive keys k0..k0+7 (k0 a multiple of 8, possibly -8) of row h, with the forward pass's masks: 0 outside
-// the plane and, under the causal rule, for keys beyond the row index.  `edge` = this step may straddle the diagonal.
-template <typename T>
-__device__ __forceinline__ u4 masked_piece(const T *plane, int h, int k0, int H, int W, int causal, bool edge)
+// Eight consecutive keys k0..k0+7 (k0 a multiple of 8, possibly -8) of row h.  The forward pass's masks -- 0 outside the
+// plane and, under the causal rule, for keys beyond the row index -- are applied in two parts: piece_ok() picks the
+// address (a piece that is masked as a whole loads the start of the plane instead, so that every load is unconditional
+// and the compiler can keep a whole step's loads in flight), mask_piece() zeroes what must read as 0 once the data is
+// there.  `edge` = the step may straddle the diagonal (wavefront-uniform).
+__device__ __forceinline__ bool piece_ok(int h, int k0, int H, int W, int causal)
 {
-    u4 v = {0u, 0u, 0u, 0u};
-    const bool ok = (unsigned)h < (unsigned)H && (unsigned)k0 < (unsigned)W && !(causal && k0 > h);
-    if (ok) v = *reinterpret_cast<const u4 *>(plane + (int64_t)h * W + k0);
-    if (edge && causal) {
+    return (unsigned)h < (unsigned)H && (unsigned)k0 < (unsigned)W && !(causal && k0 > h);
+}
+
+template <typename T> __device__ __forceinline__ u4 load_piece(const T *plane, int h, int k0, int H, int W, int causal)
+{
+    const T *src = piece_ok(h, k0, H, W, causal) ? plane + (int64_t)h * W + k0 : plane;
+    return *reinterpret_cast<const u4 *>(src);
+}
+
+__device__ __forceinline__ u4 mask_piece(u4 v, int h, int k0, int H, int W, int causal, bool edge)
+{
+    const unsigned keep = piece_ok(h, k0, H, W, causal) ? 0xffffffffu : 0u;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] &= keep;
+    if (edge) {
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int e = k0 + 2 * u;
@@ -178,14 +191,56 @@ __device__ __forceinline__ void load_step(step_operands &o, const T *xp, const T
                                           int H, int W, int causal)
 {
     const int k = kb + 8 * g;
-    // rows of this item start at p0 - 16; the step can meet the diagonal if its last key (plus the window) passes that
-    const bool edge = causal && kb + 31 + 8 > p0 - 16;
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb) o.dy[mb] = masked_piece(dyp, p0 + 16 * mb + r, k, H, W, causal, edge);
+    for (int mb = 0; mb < 2; ++mb) o.dy[mb] = load_piece(dyp, p0 + 16 * mb + r, k, H, W, causal);
 #pragma unroll
     for (int nb = 0; nb < 3; ++nb)
 #pragma unroll
-        for (int s = 0; s < 3; ++s) o.x[nb][s] = masked_piece(xp, p0 - 16 + 16 * nb + r, k - 8 + 8 * s, H, W, causal, edge);
+        for (int s = 0; s < 3; ++s) o.x[nb][s] = load_piece(xp, p0 - 16 + 16 * nb + r, k - 8 + 8 * s, H, W, causal);
+}
+
+__device__ __forceinline__ void mask_step(step_operands &o, int p0, int kb, int r, int g, int H, int W, int causal)
+{
+    const int k = kb + 8 * g;
+    // rows of this item start at p0 - 16, the step's last key (with the window) is kb + 39
+    const bool edge = causal && kb + 39 > p0 - 16;
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) o.dy[mb] = mask_piece(o.dy[mb], p0 + 16 * mb + r, k, H, W, causal, edge);
+#pragma unroll
+    for (int nb = 0; nb < 3; ++nb)
+#pragma unroll
+        for (int s = 0; s < 3; ++s)
+            o.x[nb][s] = mask_piece(o.x[nb][s], p0 - 16 + 16 * nb + r, k - 8 + 8 * s, H, W, causal, edge);
+}
+
+// The 4*S products of a step: block mb of dy against blocks mb and mb+1 of x, every key offset j.  The operand of
+// offset j is the lane's 24-key window of x from key 8 + j - pad on (a byte shift of two registers for odd starts).
+template <typename T, int S>
+__device__ __forceinline__ void accumulate_step(f32x4 (&acc)[2][S], const step_operands &o)
+{
+    constexpr int PW = (S - 1) / 2;
+    frag8<T> a[2];
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) a[mb] = __builtin_bit_cast(frag8<T>, o.dy[mb]);
+#pragma unroll
+    for (int nb = 0; nb < 3; ++nb) {
+        unsigned w[12];
+#pragma unroll
+        for (int s = 0; s < 3; ++s)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) w[4 * s + u] = o.x[nb][s][u];
+#pragma unroll
+        for (int j = 0; j < S; ++j) {
+            const int st = 8 + j - PW;  // compile-time after unrolling
+            u4 bv;
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+                bv[d] = (st & 1) ? __builtin_amdgcn_alignbyte(w[(st + 1) / 2 + d], w[(st - 1) / 2 + d], 2) : w[st / 2 + d];
+            const frag8<T> b = __builtin_bit_cast(frag8<T>, bv);
+            if (nb <= 1) mma16(acc[0][j], a[nb], b);
+            if (nb >= 1) mma16(acc[1][j], a[nb - 1], b);
+        }
+    }
 }
 
 template <typename T, int R, int S>
@@ -194,7 +249,6 @@ __global__ __launch_bounds__(NT) void conv2d_bwd_weight_mfma(const T *__restrict
                                                              int causal, int tiles_m, int nseg, int bpc)
 {
     static_assert(R <= 17 && S <= 16 && (S - 1) / 2 <= 8, "window of 24 keys, two 16-row blocks of halo");
-    constexpr int PW = (S - 1) / 2;
     __shared__ float tile[2 * S][16][17];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int c = blockIdx.x / bpc, sub = blockIdx.x % bpc;
@@ -220,35 +274,18 @@ __global__ __launch_bounds__(NT) void conv2d_bwd_weight_mfma(const T *__restrict
         if (t0 >= t1) continue;
         const int64_t plane = ((int64_t)n * C + c) * H * W;
         const T *xp = x + plane, *dyp = dy + plane;
-        step_operands cur;
-        load_step(cur, xp, dyp, p0, 32 * t0, r, g, H, W, causal);
-        for (int t = t0; t < t1; ++t) {
-            step_operands nxt;
-            if (t + 1 < t1) load_step(nxt, xp, dyp, p0, 32 * (t + 1), r, g, H, W, causal);
-            else nxt = cur;
-            frag8<T> a[2];
-#pragma unroll
-            for (int mb = 0; mb < 2; ++mb) a[mb] = __builtin_bit_cast(frag8<T>, cur.dy[mb]);
-#pragma unroll
-            for (int nb = 0; nb < 3; ++nb) {
-                unsigned w[12];
-#pragma unroll
-                for (int s = 0; s < 3; ++s)
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) w[4 * s + u] = cur.x[nb][s][u];
-#pragma unroll
-                for (int j = 0; j < S; ++j) {
-                    const int o = 8 + j - PW;  // first key of the operand inside the window (compile-time after unrolling)
-                    u4 bv;
-#pragma unroll
-                    for (int d = 0; d < 4; ++d)
-                        bv[d] = (o & 1) ? __builtin_amdgcn_alignbyte(w[(o + 1) / 2 + d], w[(o - 1) / 2 + d], 2) : w[o / 2 + d];
-                    const frag8<T> b = __builtin_bit_cast(frag8<T>, bv);
-                    if (nb <= 1) mma16(acc[0][j], a[nb], b);
-                    if (nb >= 1) mma16(acc[1][j], a[nb - 1], b);
-                }
-            }
-            cur = nxt;
+        // two operand sets take turns, so that a step's loads stay in flight through the whole of the step before it;
+        // the last step fetches itself again: the number of loads in flight never depends on a branch
+        step_operands oa, ob;
+        load_step(oa, xp, dyp, p0, 32 * t0, r, g, H, W, causal);
+        for (int t = t0; t < t1; t += 2) {
+            load_step(ob, xp, dyp, p0, 32 * (t + 1 < t1 ? t + 1 : t), r, g, H, W, causal);
+            mask_step(oa, p0, 32 * t, r, g, H, W, causal);
+            accumulate_step<T, S>(acc, oa);
+            if (t + 1 >= t1) break;
+            load_step(oa, xp, dyp, p0, 32 * (t + 2 < t1 ? t + 2 : t + 1), r, g, H, W, causal);
+            mask_step(ob, p0, 32 * (t + 1), r, g, H, W, causal);
+            accumulate_step<T, S>(acc, ob);
         }
     }
 
