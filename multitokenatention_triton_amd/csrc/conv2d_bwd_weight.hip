@@ -159,12 +159,6 @@ __device__ __forceinline__ bool piece_ok(int h, int k0, int H, int W, int causal
     return (unsigned)h < (unsigned)H && (unsigned)k0 < (unsigned)W && !(causal && k0 > h);
 }
 
-template <typename T> __device__ __forceinline__ u4 load_piece(const T *plane, int h, int k0, int H, int W, int causal)
-{
-    const T *src = piece_ok(h, k0, H, W, causal) ? plane + (int64_t)h * W + k0 : plane;
-    return *reinterpret_cast<const u4 *>(src);
-}
-
 __device__ __forceinline__ u4 mask_piece(u4 v, int h, int k0, int H, int W, int causal, bool edge)
 {
     const unsigned keep = piece_ok(h, k0, H, W, causal) ? 0xffffffffu : 0u;
@@ -186,17 +180,43 @@ struct step_operands {
     u4 x[3][3];
 };
 
-template <typename T>
-__device__ __forceinline__ void load_step(step_operands &o, const T *xp, const T *dyp, int p0, int kb, int r, int g,
-                                          int H, int W, int causal)
+// The rows a lane reads in a work item, as element offsets into the plane (which the host keeps below 2^31 elements):
+// x rows p0 - 16 + 16 nb + r from key 8g - 8 on, dy rows p0 + 16 mb + r from key 8g on.  The offset of a row outside
+// the plane wraps around and is never used.
+struct lane_rows {
+    unsigned x[3];
+    unsigned dy[2];
+};
+
+template <typename T> __device__ __forceinline__ u4 load16(const T *plane, unsigned off)
 {
-    const int k = kb + 8 * g;
+    return *reinterpret_cast<const u4 *>(plane + (size_t)off);
+}
+
+// `inner` (wavefront-uniform): every piece of the step lies inside the plane and on or below the diagonal
+template <typename T>
+__device__ __forceinline__ void load_step(step_operands &o, const T *xp, const T *dyp, const lane_rows &rows, int p0,
+                                          int kb, int r, int g, int H, int W, int causal, bool inner)
+{
+    if (inner) {
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb) o.dy[mb] = load_piece(dyp, p0 + 16 * mb + r, k, H, W, causal);
+        for (int mb = 0; mb < 2; ++mb) o.dy[mb] = load16(dyp, rows.dy[mb] + kb);
 #pragma unroll
-    for (int nb = 0; nb < 3; ++nb)
+        for (int nb = 0; nb < 3; ++nb)
 #pragma unroll
-        for (int s = 0; s < 3; ++s) o.x[nb][s] = load_piece(xp, p0 - 16 + 16 * nb + r, k - 8 + 8 * s, H, W, causal);
+            for (int s = 0; s < 3; ++s) o.x[nb][s] = load16(xp, rows.x[nb] + kb + 8 * s);
+    } else {
+        const int k = kb + 8 * g;
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+            o.dy[mb] = load16(dyp, piece_ok(p0 + 16 * mb + r, k, H, W, causal) ? rows.dy[mb] + kb : 0u);
+#pragma unroll
+        for (int nb = 0; nb < 3; ++nb)
+#pragma unroll
+            for (int s = 0; s < 3; ++s)
+                o.x[nb][s] = load16(xp, piece_ok(p0 - 16 + 16 * nb + r, k - 8 + 8 * s, H, W, causal) ? rows.x[nb] + kb + 8 * s
+                                                                                                   : 0u);
+    }
 }
 
 __device__ __forceinline__ void mask_step(step_operands &o, int p0, int kb, int r, int g, int H, int W, int causal)
@@ -260,12 +280,15 @@ __global__ __launch_bounds__(NT) void conv2d_bwd_weight_mfma(const T *__restrict
 #pragma unroll
         for (int j = 0; j < S; ++j) acc[h][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
+    // Items in order of falling length (under the causal rule a row block further down has more keys), dealt to the
+    // channel's wavefronts forwards and backwards in turn, so that every wavefront gets about the same number of steps.
     const int64_t items = (int64_t)N * tiles_m * nseg;
-    for (int64_t it = (int64_t)sub * (NT / 64) + wave; it < items; it += (int64_t)bpc * (NT / 64)) {
-        const int sg = (int)(it % nseg);
-        const int64_t rest = it / nseg;
-        const int ti = (int)(rest % tiles_m), n = (int)(rest / tiles_m);
-        const int tm = (ti & 1) ? tiles_m - 1 - (ti >> 1) : (ti >> 1);  // long and short rows alternate
+    const int nwv = bpc * (NT / 64), wv = sub * (NT / 64) + wave, per_tm = N * nseg;
+    for (int64_t k = 0; k * nwv < items; ++k) {
+        const int64_t it = k * nwv + ((k & 1) ? nwv - 1 - wv : wv);
+        if (it >= items) continue;
+        const int tm = tiles_m - 1 - (int)(it / per_tm), rem = (int)(it % per_tm);
+        const int n = rem / nseg, sg = rem % nseg;
         const int p0 = tm * MROWS;
         int kend = W;  // dy is zero beyond the diagonal: keys from p0 + MROWS on add nothing
         if (causal && p0 + MROWS < W) kend = p0 + MROWS;
@@ -274,17 +297,29 @@ __global__ __launch_bounds__(NT) void conv2d_bwd_weight_mfma(const T *__restrict
         if (t0 >= t1) continue;
         const int64_t plane = ((int64_t)n * C + c) * H * W;
         const T *xp = x + plane, *dyp = dy + plane;
+        lane_rows rows;
+#pragma unroll
+        for (int nb = 0; nb < 3; ++nb) rows.x[nb] = (unsigned)((p0 - 16 + 16 * nb + r) * W + 8 * g - 8);
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) rows.dy[mb] = (unsigned)((p0 + 16 * mb + r) * W + 8 * g);
+        // steps whose pieces all lie inside the plane and on or below the diagonal need neither selects nor masks:
+        // rows p0-16 .. p0+31 inside the plane, keys kb-8 .. kb+39 inside it and (causal) not beyond row p0-16
+        const bool rows_in = p0 >= 16 && p0 + MROWS <= H;
+        const int last_inner = causal ? (p0 - 16 - 39 < W - 40 ? p0 - 16 - 39 : W - 40) : W - 40;  // largest such kb
+        auto inner = [&](int t) { return rows_in && 32 * t >= 8 && 32 * t <= last_inner; };
         // two operand sets take turns, so that a step's loads stay in flight through the whole of the step before it;
         // the last step fetches itself again: the number of loads in flight never depends on a branch
         step_operands oa, ob;
-        load_step(oa, xp, dyp, p0, 32 * t0, r, g, H, W, causal);
+        load_step(oa, xp, dyp, rows, p0, 32 * t0, r, g, H, W, causal, inner(t0));
         for (int t = t0; t < t1; t += 2) {
-            load_step(ob, xp, dyp, p0, 32 * (t + 1 < t1 ? t + 1 : t), r, g, H, W, causal);
-            mask_step(oa, p0, 32 * t, r, g, H, W, causal);
+            const int tb = t + 1 < t1 ? t + 1 : t;
+            load_step(ob, xp, dyp, rows, p0, 32 * tb, r, g, H, W, causal, inner(tb));
+            if (!inner(t)) mask_step(oa, p0, 32 * t, r, g, H, W, causal);
             accumulate_step<T, S>(acc, oa);
             if (t + 1 >= t1) break;
-            load_step(oa, xp, dyp, p0, 32 * (t + 2 < t1 ? t + 2 : t + 1), r, g, H, W, causal);
-            mask_step(ob, p0, 32 * (t + 1), r, g, H, W, causal);
+            const int ta = t + 2 < t1 ? t + 2 : t + 1;
+            load_step(oa, xp, dyp, rows, p0, 32 * ta, r, g, H, W, causal, inner(ta));
+            if (!inner(t + 1)) mask_step(ob, p0, 32 * (t + 1), r, g, H, W, causal);
             accumulate_step<T, S>(acc, ob);
         }
     }
@@ -415,7 +450,7 @@ int launch(const void *x, const void *dy, float *dw, float *partial, int bpc, in
         // the fp32-FMA kernel, for comparisons).  Two workgroups per CU; the key range of a row block is cut into
         // segments until every wavefront has about two items.
         static const bool force_valu = [] { const char *e = getenv("MTA_CONV_FORCE_VALU"); return e && e[0] == '1'; }();
-        if (!force_valu && vec_ok && aligned_to(x, 16) && R <= MROWS / 2 + 1) {
+        if (!force_valu && vec_ok && aligned_to(x, 16) && R <= MROWS / 2 + 1 && (H + MROWS) * W < 0x7fffffffLL) {
             const int rows_m = (int)((H + MROWS - 1) / MROWS);
             int bm = (int)((512 + C - 1) / C);
             if (bm > bpc) bm = bpc;
