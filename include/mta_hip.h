@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTA_ABI_VERSION 4
+#define MTA_ABI_VERSION 5
 
 enum mta_dtype { MTA_F32 = 0, MTA_BF16 = 1, MTA_F16 = 2 };
 
@@ -90,6 +90,17 @@ int mta_headmix_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C,
  * as mta_headmix_fwd; the reference pre-fills the output (triton_linear_head.py:294-297). */
 int mta_headmix_tril_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
                          int group_size, int io_dtype, int w_dtype, void *stream);
+
+/* Gradient of the row softmax over the keys of an (N,C,P,Q) tensor, from the stored probabilities:
+ *   dx[q] = p[q] * (dp[q] - sum_k p[k] * dp[k])      fp32 arithmetic, p / dp / dx in the I/O dtype
+ * causal: keys q > row index take no part and are never read; dx there is written as +0.0 when
+ * fill_upper != 0 and left alone otherwise.
+ * Replaces torch's autograd through F.softmax(scores.float(), dim=-1).type_as(xq)
+ * (mta_attention_triton.py:79), which keeps an fp32 copy of the probabilities and writes the product
+ * p * dp before it reduces it; with p stored in 16 bits the result differs from that path by the
+ * rounding of p. */
+int mta_softmax_bwd(const void *p, const void *dp, void *dx, int64_t N, int64_t C, int64_t P, int64_t Q,
+                    int causal, int fill_upper, int io_dtype, void *stream);
 
 /* Fused head mixing + row softmax + head mixing over (N,C,P,Q), one pass:
  *   s[o] = w1 ? sum_i w1[o,i] x[i] : x[o]      (fp32, rounded to the I/O dtype;

@@ -23,9 +23,9 @@ Functions, as in the reference, so that ``backward()`` works: the two conv and t
 head-mixing stages with their HIP gradient kernels (convolution_2d_trit /
 triton_linear_head); the 1/sqrt(D) factor folded into the pre-softmax conv and, in
 backward, into the (B,H,S,D) gradients of Q and K; pre-softmax head mixing and softmax as
-one forward kernel where the inference route has one, with torch's softmax gradient taken
-from the stored 16-bit probabilities (no fp32 copy of the score tensor in either
-direction).  torch differentiates the two GEMMs and the dropout.
+one forward kernel where the inference route has one, with the softmax gradient taken from
+the stored 16-bit probabilities (``mta_softmax_bwd``; no fp32 copy of the score tensor in
+either direction).  torch differentiates the two GEMMs and the dropout.
 
 Weight structure.  By default nothing is assumed about the four weights: every stage runs
 with the dense weight it is given.  Skipping identity stages and applying block-diagonal
@@ -111,8 +111,8 @@ class _MixSoftmax(torch.autograd.Function):
     """softmax(mix(x, weight)) over the keys for the training route (mta_attention_triton.py:75-79), one kernel
     (``mta_headmix_softmax_fwd``; ``weight=None``: the softmax alone).  The probabilities are computed in fp32 from the
     mixed scores rounded to the score dtype and stored in it, as ``F.softmax(scores.float()).type_as(scores)`` leaves
-    them.  Backward: torch's softmax gradient from the stored probabilities, then the head mixing's two gradient
-    kernels."""
+    them.  Backward: the softmax gradient from the stored probabilities (``mta_softmax_bwd``), then the head mixing's
+    two gradient kernels."""
 
     @staticmethod
     def forward(ctx, x, weight, causal, group_size):
@@ -124,7 +124,8 @@ class _MixSoftmax(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         x, weight, p = ctx.saved_tensors
-        ds = torch._softmax_backward_data(grad_output.to(p.dtype), p, -1, p.dtype)
+        # the head mixing's gradient kernels never read above the diagonal; autograd's next consumer might
+        ds = ops.softmax_bwd(p, grad_output.to(p.dtype), ctx.causal, fill_upper=weight is None)
         if weight is None:
             return ds, None, None, None
         dx = dw = None

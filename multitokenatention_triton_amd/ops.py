@@ -214,6 +214,22 @@ def headmix_softmax(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optional[to
     return y
 
 
+def softmax_bwd(p: torch.Tensor, dp: torch.Tensor, causal: bool = True, fill_upper: bool = True) -> torch.Tensor:
+    """Gradient of the row softmax from its stored output ``p`` (N,C,P,Q) and the incoming gradient ``dp``; see
+    mta_softmax_bwd.  ``fill_upper=False`` (causal) leaves the result above the diagonal unwritten."""
+    p = _device_tensor(p, "probabilities")
+    dp = _device_tensor(dp, "grad_output")
+    if p.dim() != 4 or p.shape != dp.shape or p.dtype != dp.dtype:
+        raise ValueError("probabilities and grad_output must be (N,C,P,Q) tensors of one shape and dtype")
+    n, c, rows, q = p.shape
+    dx = torch.empty_like(p, memory_format=torch.contiguous_format)
+    with torch.cuda.device(p.device):
+        rc = _lib.load().mta_softmax_bwd(p.data_ptr(), dp.data_ptr(), dx.data_ptr(), n, c, rows, q, int(bool(causal)),
+                                         int(bool(fill_upper)), _code(p, "probabilities"), _stream(p))
+    _lib.check(rc, "mta_softmax_bwd")
+    return dx
+
+
 def conv2d_headmix(x: torch.Tensor, w_conv: torch.Tensor, w_mix: torch.Tensor, causal: bool = True,
                    group_size: Optional[int] = None, out: Optional[torch.Tensor] = None,
                    fill_upper: bool = True) -> Optional[torch.Tensor]:

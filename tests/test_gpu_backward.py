@@ -129,6 +129,57 @@ def test_headmix_backward_parity(pkg, case, dtype):
     assert torch.equal(dw, pkg.ops.headmix_bwd_weight(x_dev, dy_dev, causal))
 
 
+SM_CASES = [
+    # N, C, P, Q, causal
+    (1, 2, 40, 40, True),
+    (2, 3, 264, 264, True),        # rows of whole 16-byte vectors: one read of p and dp
+    (1, 2, 100, 104, False),
+    (1, 1, 33, 65, False),         # ragged
+    (1, 2, 2304, 2304, True),      # two vectors per thread
+    (1, 1, 300, 4360, False),      # four vectors per thread
+    (1, 1, 3, 8200, False),        # longer than the register path holds
+    (1, 1, 1, 1, True),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", SM_CASES)
+def test_softmax_backward_parity(pkg, case, dtype):
+    """mta_softmax_bwd against torch.autograd through F.softmax(x.float()).type_as(x), the expression the reference
+    differentiates (mta_attention_triton.py:79).  The kernel sees the probabilities rounded to the score dtype, autograd
+    their fp32 originals: for 16-bit data the bar is atol 2e-2 * max|dx| (each rounded p is within 2^-9 of its
+    original); fp32: rtol 1e-4.  Above the diagonal: +0 with fill_upper, untouched without."""
+    n, c, rows, q, causal = case
+    print(f"softmax bwd case={case} {dtype}", flush=True)
+    x, dp = _rand((n, c, rows, q), 5, dtype), _rand((n, c, rows, q), 6, dtype)
+    up = torch.triu(torch.ones(rows, q, dtype=torch.bool), 1)
+    leaf = x.float().masked_fill(up, float("-inf")) if causal else x.float()
+    leaf.requires_grad_(True)
+    probs = torch.softmax(leaf, -1)
+    probs.backward(dp.float().masked_fill(up, 0.0) if causal else dp.float())
+    want = leaf.grad
+    p_dev, dp_dev = probs.detach().to(dtype).cuda(), dp.cuda()
+    if causal:   # what lies above the diagonal must never be read
+        p_dev, dp_dev = p_dev.masked_fill(up.cuda(), float("nan")), dp_dev.masked_fill(up.cuda(), float("nan"))
+    got = pkg.ops.softmax_bwd(p_dev, dp_dev, causal)
+    assert got.dtype == dtype and got.shape == x.shape
+    _close(got, want, dtype, "dx")
+    if causal:
+        g = got.cpu()
+        assert (g[..., up] == 0).all() and not torch.signbit(g[..., up]).any()
+        # fill_upper=False: the same below the diagonal, nothing written in vectors wholly above it
+        sentinel = torch.full_like(p_dev, 7.0)
+        lib = pkg._lib.load()
+        rc = lib.mta_softmax_bwd(p_dev.data_ptr(), dp_dev.data_ptr(), sentinel.data_ptr(), n, c, rows, q, 1, 0,
+                                 {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}[dtype],
+                                 torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        low = ~up
+        assert torch.equal(sentinel.cpu()[..., low], g[..., low])
+        far = torch.triu(torch.ones(rows, q, dtype=torch.bool), 8)   # beyond any vector that touches the diagonal
+        assert (sentinel.cpu()[..., far] == 7.0).all()
+
+
 def test_operator_functions_backward(pkg):
     """Conv2dTritonFunction / TritonLinearHeadFunction under torch.autograd, fp32, against the oracle's grads."""
     print("operator Functions backward", flush=True)
