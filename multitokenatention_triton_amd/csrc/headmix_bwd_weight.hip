@@ -25,6 +25,64 @@ constexpr int CHUNK = 128;  // positions per wavefront step (MFMA kernel)
 // mask a pair of consecutive rows always carries P+1 positions.
 __device__ __forceinline__ int interleaved_row(int j, int P) { return (j & 1) ? P - 1 - (j >> 1) : (j >> 1); }
 
+typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+
+// One 128-position chunk of one query row: where it starts and where the row's attended positions end.
+struct hm_unit {
+    int64_t rowbase;
+    int q0, last;
+};
+
+// The chunk's operands of a lane: for product t the eight positions from q0 + 32t + 8g on, of head 16a + r.
+template <int NB> struct hm_operands {
+    u4 dy[NB][4], x[NB][4];
+};
+
+template <typename T, int NB>
+__device__ __forceinline__ void hm_load(hm_operands<NB> &o, const T *x, const T *dy, const hm_unit &u, int64_t plane, int r,
+                                        int g)
+{
+    const int q = u.q0 + 8 * g;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        // every load is unconditional: a vector wholly beyond `last` re-reads the row start and is zeroed before use
+        const int qq = (q + 32 * t <= u.last) ? q + 32 * t : 0;
+#pragma unroll
+        for (int a = 0; a < NB; ++a) {
+            o.dy[a][t] = *reinterpret_cast<const u4 *>(dy + u.rowbase + (int64_t)(a * 16 + r) * plane + qq);
+            o.x[a][t] = *reinterpret_cast<const u4 *>(x + u.rowbase + (int64_t)(a * 16 + r) * plane + qq);
+        }
+    }
+}
+
+template <typename T, int NB>
+__device__ __forceinline__ void hm_consume(f32x4 (&acc)[NB][NB], hm_operands<NB> &o, const hm_unit &u, int g)
+{
+    if (u.q0 + CHUNK - 1 > u.last) {  // the chunk straddles the end of the row: zero what lies beyond it, in both
+                                      // operands (what x holds there need not even be finite)
+        const int q = u.q0 + 8 * g;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int e = q + 32 * t + 2 * v;
+                const unsigned keep = (e <= u.last ? 0x0000ffffu : 0u) | (e + 1 <= u.last ? 0xffff0000u : 0u);
+#pragma unroll
+                for (int a = 0; a < NB; ++a) {
+                    o.dy[a][t][v] &= keep;
+                    o.x[a][t][v] &= keep;
+                }
+            }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int a = 0; a < NB; ++a)
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+                mma16(acc[a][b], __builtin_bit_cast(frag8<T>, o.dy[a][t]), __builtin_bit_cast(frag8<T>, o.x[b][t]));
+}
+
 template <typename T, int NB>  // NB = C / 16
 __global__ __launch_bounds__(NT) void headmix_bwd_weight_mfma(const T *__restrict__ x, const T *__restrict__ dy,
                                                               float *__restrict__ partial, int N, int P, int Q, int causal)
@@ -39,55 +97,46 @@ __global__ __launch_bounds__(NT) void headmix_bwd_weight_mfma(const T *__restric
 #pragma unroll
         for (int b = 0; b < NB; ++b) acc[a][b] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
     const int64_t rows = (int64_t)N * P;
     const int64_t nwaves = (int64_t)gridDim.x * (NT / 64), wid = (int64_t)blockIdx.x * (NT / 64) + wave;
-    // a wavefront takes pairs of rows (2k, 2k+1) of the interleaved order
-    for (int64_t pr = wid; pr * 2 < rows; pr += nwaves) {
-        for (int half = 0; half < 2; ++half) {
-            const int64_t rid = pr * 2 + half;
-            if (rid >= rows) break;
-            const int n = (int)(rid / P), p = interleaved_row((int)(rid % P), P);
-            const int last = causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;  // last position of the row that takes part
-            const int64_t rowbase = (int64_t)n * C * plane + (int64_t)p * Q;
-            for (int q0 = 0; q0 <= last; q0 += CHUNK) {
-                const int q = q0 + 8 * g;  // this lane's positions: q + 32t .. +7 for product t (a load instruction
-                                           // covers 64 contiguous bytes of each of 16 heads)
-                u4 av[NB][4], bv[NB][4];
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    // a vector wholly beyond `last` re-reads the row start (valid memory) and is zeroed below
-                    const int qq = (q + 32 * t <= last) ? q + 32 * t : 0;
-#pragma unroll
-                    for (int a = 0; a < NB; ++a) {
-                        av[a][t] = *reinterpret_cast<const u4 *>(dy + rowbase + (int64_t)(a * 16 + r) * plane + qq);
-                        bv[a][t] = *reinterpret_cast<const u4 *>(x + rowbase + (int64_t)(a * 16 + r) * plane + qq);
-                    }
-                }
-                if (q0 + CHUNK - 1 > last) {  // the chunk straddles the end of the row: zero what lies beyond it, in both
-                                              // operands (what x holds there need not even be finite)
-#pragma unroll
-                    for (int t = 0; t < 4; ++t)
-#pragma unroll
-                        for (int u = 0; u < 4; ++u) {
-                            const int e = q + 32 * t + 2 * u;
-                            const unsigned keep = (e <= last ? 0x0000ffffu : 0u) | (e + 1 <= last ? 0xffff0000u : 0u);
-#pragma unroll
-                            for (int a = 0; a < NB; ++a) {
-                                av[a][t][u] &= keep;
-                                bv[a][t][u] &= keep;
-                            }
-                        }
-                }
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-#pragma unroll
-                    for (int a = 0; a < NB; ++a)
-#pragma unroll
-                        for (int b = 0; b < NB; ++b)
-                            mma16(acc[a][b], __builtin_bit_cast(frag8<T>, av[a][t]), __builtin_bit_cast(frag8<T>, bv[b][t]));
-            }
+    // A wavefront takes pairs of rows (2k, 2k+1) of the interleaved order, k = wid, wid + nwaves, ...; j counts its
+    // rows.  The chunks of all its rows form one sequence, and the loads of a chunk are issued before the products of
+    // the chunk ahead of it (two operand sets take turns).  (Four wavefronts sharing a row chunk by chunk measured
+    // slower: short rows leave most of them without work.)
+    int64_t j = 0;
+    int q0 = 0;
+    auto unit_at = [&](hm_unit &u) -> bool {
+        const int64_t rid = 2 * (wid + (j >> 1) * nwaves) + (j & 1);
+        if (rid >= rows) return false;
+        const int n = (int)(rid / P), p = interleaved_row((int)(rid % P), P);
+        u.last = causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;  // last position of the row that takes part
+        u.rowbase = (int64_t)n * C * plane + (int64_t)p * Q;
+        u.q0 = q0;
+        return true;
+    };
+    auto advance = [&](const hm_unit &u) {
+        q0 += CHUNK;
+        if (q0 > u.last) {
+            q0 = 0;
+            ++j;
         }
+    };
+    hm_unit ua, ub;
+    hm_operands<NB> oa, ob;
+    bool ha = unit_at(ua);
+    if (ha) hm_load<T, NB>(oa, x, dy, ua, plane, r, g);
+    while (ha) {
+        advance(ua);
+        const bool hb = unit_at(ub);
+        if (!hb) ub = ua;  // nothing follows: fetch the same chunk again, so that the loads in flight never depend on a branch
+        hm_load<T, NB>(ob, x, dy, ub, plane, r, g);
+        hm_consume<T, NB>(acc, oa, ua, g);
+        if (!hb) break;
+        advance(ub);
+        ha = unit_at(ua);
+        if (!ha) ua = ub;
+        hm_load<T, NB>(oa, x, dy, ua, plane, r, g);
+        hm_consume<T, NB>(acc, ob, ub, g);
     }
     // acc[a][b][v] = dw[16a + 4g + v][16b + r]
 #pragma unroll
