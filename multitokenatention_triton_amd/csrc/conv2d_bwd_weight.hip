@@ -147,7 +147,10 @@ __global__ __launch_bounds__(NT) void conv2d_bwd_weight_fixed(const T *__restric
 
 // ---- matrix-core kernel -------------------------------------------------------------------------------------------
 typedef unsigned int u4 __attribute__((ext_vector_type(4)));
-constexpr int MROWS = 32;  // rows of dy per work item (two 16-row blocks against three 16-row blocks of x)
+constexpr int MB = 2;            // 16-row blocks of dy per work item (against MB + 1 blocks of x)
+constexpr int HV = 1;            // 32-key half steps per step
+constexpr int MROWS = 16 * MB;   // rows of dy per work item
+constexpr int KSTEP = 32 * HV;   // keys per step
 
 // Eight consecutive keys k0..k0+7 (k0 a multiple of 8, possibly -8) of row h.  The forward pass's masks -- 0 outside the
 // plane and, under the causal rule, for keys beyond the row index -- are applied in two parts: piece_ok() picks the
@@ -174,18 +177,22 @@ __device__ __forceinline__ u4 mask_piece(u4 v, int h, int k0, int H, int W, int 
     return v;
 }
 
-// One step's operands of a wavefront: keys kb + 8g .. +7 of the lane's rows; for x also the eight keys on either side.
+// One step of a wavefront: HV half steps of 32 keys each (lane: keys kb + 32 hv + 8g .. +7) over MB 16-row blocks of dy
+// and the MB + 1 blocks of x around them; for x also the eight keys on either side of the lane's eight.  MB = 2, HV = 1
+// is the fastest measured: 11 loads per 4*S products.  MB = 1, HV = 2 (whole 128-byte lines of every row per step, 14
+// loads per 4*S products) fetches 40 % less from memory, since no line is asked for twice a step apart, and still takes
+// 20 % longer: the time follows the number of load instructions, not the bytes.
 struct step_operands {
-    u4 dy[2];
-    u4 x[3][3];
+    u4 dy[MB][HV];
+    u4 x[MB + 1][HV][3];
 };
 
 // The rows a lane reads in a work item, as element offsets into the plane (which the host keeps below 2^31 elements):
 // x rows p0 - 16 + 16 nb + r from key 8g - 8 on, dy rows p0 + 16 mb + r from key 8g on.  The offset of a row outside
 // the plane wraps around and is never used.
 struct lane_rows {
-    unsigned x[3];
-    unsigned dy[2];
+    unsigned x[MB + 1];
+    unsigned dy[MB];
 };
 
 template <typename T> __device__ __forceinline__ u4 load16(const T *plane, unsigned off)
@@ -200,65 +207,78 @@ __device__ __forceinline__ void load_step(step_operands &o, const T *xp, const T
 {
     if (inner) {
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) o.dy[mb] = load16(dyp, rows.dy[mb] + kb);
+        for (int hv = 0; hv < HV; ++hv) {
 #pragma unroll
-        for (int nb = 0; nb < 3; ++nb)
+            for (int mb = 0; mb < MB; ++mb) o.dy[mb][hv] = load16(dyp, rows.dy[mb] + kb + 32 * hv);
 #pragma unroll
-            for (int s = 0; s < 3; ++s) o.x[nb][s] = load16(xp, rows.x[nb] + kb + 8 * s);
+            for (int nb = 0; nb < MB + 1; ++nb)
+#pragma unroll
+                for (int s = 0; s < 3; ++s) o.x[nb][hv][s] = load16(xp, rows.x[nb] + kb + 32 * hv + 8 * s);
+        }
     } else {
-        const int k = kb + 8 * g;
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
-            o.dy[mb] = load16(dyp, piece_ok(p0 + 16 * mb + r, k, H, W, causal) ? rows.dy[mb] + kb : 0u);
+        for (int hv = 0; hv < HV; ++hv) {
+            const int k = kb + 32 * hv + 8 * g;
 #pragma unroll
-        for (int nb = 0; nb < 3; ++nb)
+            for (int mb = 0; mb < MB; ++mb)
+                o.dy[mb][hv] = load16(dyp, piece_ok(p0 + 16 * mb + r, k, H, W, causal) ? rows.dy[mb] + kb + 32 * hv : 0u);
 #pragma unroll
-            for (int s = 0; s < 3; ++s)
-                o.x[nb][s] = load16(xp, piece_ok(p0 - 16 + 16 * nb + r, k - 8 + 8 * s, H, W, causal) ? rows.x[nb] + kb + 8 * s
-                                                                                                   : 0u);
+            for (int nb = 0; nb < MB + 1; ++nb)
+#pragma unroll
+                for (int s = 0; s < 3; ++s)
+                    o.x[nb][hv][s] = load16(xp, piece_ok(p0 - 16 + 16 * nb + r, k - 8 + 8 * s, H, W, causal)
+                                                    ? rows.x[nb] + kb + 32 * hv + 8 * s
+                                                    : 0u);
+        }
     }
 }
 
 __device__ __forceinline__ void mask_step(step_operands &o, int p0, int kb, int r, int g, int H, int W, int causal)
 {
-    const int k = kb + 8 * g;
-    // rows of this item start at p0 - 16, the step's last key (with the window) is kb + 39
-    const bool edge = causal && kb + 39 > p0 - 16;
+    // rows of this item start at p0 - 16, the step's last key (with the window) is kb + KSTEP + 7
+    const bool edge = causal && kb + KSTEP + 7 > p0 - 16;
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb) o.dy[mb] = mask_piece(o.dy[mb], p0 + 16 * mb + r, k, H, W, causal, edge);
+    for (int hv = 0; hv < HV; ++hv) {
+        const int k = kb + 32 * hv + 8 * g;
 #pragma unroll
-    for (int nb = 0; nb < 3; ++nb)
+        for (int mb = 0; mb < MB; ++mb) o.dy[mb][hv] = mask_piece(o.dy[mb][hv], p0 + 16 * mb + r, k, H, W, causal, edge);
 #pragma unroll
-        for (int s = 0; s < 3; ++s)
-            o.x[nb][s] = mask_piece(o.x[nb][s], p0 - 16 + 16 * nb + r, k - 8 + 8 * s, H, W, causal, edge);
+        for (int nb = 0; nb < MB + 1; ++nb)
+#pragma unroll
+            for (int s = 0; s < 3; ++s)
+                o.x[nb][hv][s] = mask_piece(o.x[nb][hv][s], p0 - 16 + 16 * nb + r, k - 8 + 8 * s, H, W, causal, edge);
+    }
 }
 
-// The 4*S products of a step: block mb of dy against blocks mb and mb+1 of x, every key offset j.  The operand of
-// offset j is the lane's 24-key window of x from key 8 + j - pad on (a byte shift of two registers for odd starts).
+// The 2*MB*HV*S products of a step: block mb of dy against blocks mb and mb+1 of x, every key offset j.  The operand
+// of offset j is the lane's 24-key window of x from key 8 + j - pad on (a byte shift of two registers for odd starts).
 template <typename T, int S>
 __device__ __forceinline__ void accumulate_step(f32x4 (&acc)[2][S], const step_operands &o)
 {
     constexpr int PW = (S - 1) / 2;
-    frag8<T> a[2];
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb) a[mb] = __builtin_bit_cast(frag8<T>, o.dy[mb]);
+    for (int hv = 0; hv < HV; ++hv) {
+        frag8<T> a[MB];
 #pragma unroll
-    for (int nb = 0; nb < 3; ++nb) {
-        unsigned w[12];
+        for (int mb = 0; mb < MB; ++mb) a[mb] = __builtin_bit_cast(frag8<T>, o.dy[mb][hv]);
 #pragma unroll
-        for (int s = 0; s < 3; ++s)
+        for (int nb = 0; nb < MB + 1; ++nb) {
+            unsigned w[12];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) w[4 * s + u] = o.x[nb][s][u];
+            for (int s = 0; s < 3; ++s)
 #pragma unroll
-        for (int j = 0; j < S; ++j) {
-            const int st = 8 + j - PW;  // compile-time after unrolling
-            u4 bv;
+                for (int u = 0; u < 4; ++u) w[4 * s + u] = o.x[nb][hv][s][u];
 #pragma unroll
-            for (int d = 0; d < 4; ++d)
-                bv[d] = (st & 1) ? __builtin_amdgcn_alignbyte(w[(st + 1) / 2 + d], w[(st - 1) / 2 + d], 2) : w[st / 2 + d];
-            const frag8<T> b = __builtin_bit_cast(frag8<T>, bv);
-            if (nb <= 1) mma16(acc[0][j], a[nb], b);
-            if (nb >= 1) mma16(acc[1][j], a[nb - 1], b);
+            for (int j = 0; j < S; ++j) {
+                const int st = 8 + j - PW;  // compile-time after unrolling
+                u4 bv;
+#pragma unroll
+                for (int d = 0; d < 4; ++d)
+                    bv[d] = (st & 1) ? __builtin_amdgcn_alignbyte(w[(st + 1) / 2 + d], w[(st - 1) / 2 + d], 2) : w[st / 2 + d];
+                const frag8<T> b = __builtin_bit_cast(frag8<T>, bv);
+                if (nb <= MB - 1) mma16(acc[0][j], a[nb < MB ? nb : 0], b);
+                if (nb >= 1) mma16(acc[1][j], a[nb - 1 >= 0 ? nb - 1 : 0], b);
+            }
         }
     }
 }
@@ -292,34 +312,35 @@ __global__ __launch_bounds__(NT) void conv2d_bwd_weight_mfma(const T *__restrict
         const int p0 = tm * MROWS;
         int kend = W;  // dy is zero beyond the diagonal: keys from p0 + MROWS on add nothing
         if (causal && p0 + MROWS < W) kend = p0 + MROWS;
-        const int nsteps = (kend + 31) / 32, per = (nsteps + nseg - 1) / nseg;
+        const int nsteps = (kend + KSTEP - 1) / KSTEP, per = (nsteps + nseg - 1) / nseg;
         const int t0 = sg * per, t1 = (t0 + per < nsteps) ? t0 + per : nsteps;
         if (t0 >= t1) continue;
         const int64_t plane = ((int64_t)n * C + c) * H * W;
         const T *xp = x + plane, *dyp = dy + plane;
         lane_rows rows;
 #pragma unroll
-        for (int nb = 0; nb < 3; ++nb) rows.x[nb] = (unsigned)((p0 - 16 + 16 * nb + r) * W + 8 * g - 8);
+        for (int nb = 0; nb < MB + 1; ++nb) rows.x[nb] = (unsigned)((p0 - 16 + 16 * nb + r) * W + 8 * g - 8);
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) rows.dy[mb] = (unsigned)((p0 + 16 * mb + r) * W + 8 * g);
-        // steps whose pieces all lie inside the plane and on or below the diagonal need neither selects nor masks:
-        // rows p0-16 .. p0+31 inside the plane, keys kb-8 .. kb+39 inside it and (causal) not beyond row p0-16
+        for (int mb = 0; mb < MB; ++mb) rows.dy[mb] = (unsigned)((p0 + 16 * mb + r) * W + 8 * g);
+        // steps whose pieces all lie inside the plane and on or below the diagonal need neither selects nor masks: rows
+        // p0-16 .. p0+MROWS-1 inside the plane, keys kb-8 .. kb+KSTEP+7 inside it and (causal) not beyond row p0-16
         const bool rows_in = p0 >= 16 && p0 + MROWS <= H;
-        const int last_inner = causal ? (p0 - 16 - 39 < W - 40 ? p0 - 16 - 39 : W - 40) : W - 40;  // largest such kb
-        auto inner = [&](int t) { return rows_in && 32 * t >= 8 && 32 * t <= last_inner; };
+        const int in_plane = W - KSTEP - 8, below = p0 - 16 - KSTEP - 7;
+        const int last_inner = causal ? (below < in_plane ? below : in_plane) : in_plane;  // largest such kb
+        auto inner = [&](int t) { return rows_in && KSTEP * t >= 8 && KSTEP * t <= last_inner; };
         // two operand sets take turns, so that a step's loads stay in flight through the whole of the step before it;
         // the last step fetches itself again: the number of loads in flight never depends on a branch
         step_operands oa, ob;
-        load_step(oa, xp, dyp, rows, p0, 32 * t0, r, g, H, W, causal, inner(t0));
+        load_step(oa, xp, dyp, rows, p0, KSTEP * t0, r, g, H, W, causal, inner(t0));
         for (int t = t0; t < t1; t += 2) {
             const int tb = t + 1 < t1 ? t + 1 : t;
-            load_step(ob, xp, dyp, rows, p0, 32 * tb, r, g, H, W, causal, inner(tb));
-            if (!inner(t)) mask_step(oa, p0, 32 * t, r, g, H, W, causal);
+            load_step(ob, xp, dyp, rows, p0, KSTEP * tb, r, g, H, W, causal, inner(tb));
+            if (!inner(t)) mask_step(oa, p0, KSTEP * t, r, g, H, W, causal);
             accumulate_step<T, S>(acc, oa);
             if (t + 1 >= t1) break;
             const int ta = t + 2 < t1 ? t + 2 : t + 1;
-            load_step(oa, xp, dyp, rows, p0, 32 * ta, r, g, H, W, causal, inner(ta));
-            if (!inner(t + 1)) mask_step(ob, p0, 32 * (t + 1), r, g, H, W, causal);
+            load_step(oa, xp, dyp, rows, p0, KSTEP * ta, r, g, H, W, causal, inner(ta));
+            if (!inner(t + 1)) mask_step(ob, p0, KSTEP * (t + 1), r, g, H, W, causal);
             accumulate_step<T, S>(acc, ob);
         }
     }
@@ -450,7 +471,7 @@ int launch(const void *x, const void *dy, float *dw, float *partial, int bpc, in
         // the fp32-FMA kernel, for comparisons).  Two workgroups per CU; the key range of a row block is cut into
         // segments until every wavefront has about two items.
         static const bool force_valu = [] { const char *e = getenv("MTA_CONV_FORCE_VALU"); return e && e[0] == '1'; }();
-        if (!force_valu && vec_ok && aligned_to(x, 16) && R <= MROWS / 2 + 1 && (H + MROWS) * W < 0x7fffffffLL) {
+        if (!force_valu && vec_ok && aligned_to(x, 16) && R <= 17 && (H + MROWS + 16) * W < 0x7fffffffLL) {
             const int rows_m = (int)((H + MROWS - 1) / MROWS);
             int bm = (int)((512 + C - 1) / C);
             if (bm > bpc) bm = bpc;
