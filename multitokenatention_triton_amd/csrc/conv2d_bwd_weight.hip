@@ -302,12 +302,12 @@ __global__ __launch_bounds__(NT) void conv2d_bwd_weight_mfma(const T *__restrict
 
     // Items in order of falling length (under the causal rule a row block further down has more keys), dealt to the
     // channel's wavefronts forwards and backwards in turn, so that every wavefront gets about the same number of steps.
-    const int64_t items = (int64_t)N * tiles_m * nseg;
+    const int items = N * tiles_m * nseg;  // the host keeps this below 2^31
     const int nwv = bpc * (NT / 64), wv = sub * (NT / 64) + wave, per_tm = N * nseg;
-    for (int64_t k = 0; k * nwv < items; ++k) {
-        const int64_t it = k * nwv + ((k & 1) ? nwv - 1 - wv : wv);
+    for (int k = 0; k * nwv < items; ++k) {
+        const int it = k * nwv + ((k & 1) ? nwv - 1 - wv : wv);
         if (it >= items) continue;
-        const int tm = tiles_m - 1 - (int)(it / per_tm), rem = (int)(it % per_tm);
+        const int tm = tiles_m - 1 - it / per_tm, rem = it % per_tm;
         const int n = rem / nseg, sg = rem % nseg;
         const int p0 = tm * MROWS;
         int kend = W;  // dy is zero beyond the diagonal: keys from p0 + MROWS on add nothing
@@ -480,6 +480,7 @@ int launch(const void *x, const void *dy, float *dw, float *partial, int bpc, in
             if (nseg > seg_cap) nseg = seg_cap;
             if (nseg > 8) nseg = 8;
             if (bm > N * rows_m * nseg) bm = (int)(N * rows_m * nseg);
+            if (N * rows_m * nseg > 0x3fffffffLL) return MTA_ERR_SHAPE;  // the kernel counts items in 32 bits
 #define MTA_CONV_CASE(r, s)                                                                                          \
     if (R == r && S == s) {                                                                                          \
         hipLaunchKernelGGL((conv2d_bwd_weight_mfma<T, r, s>), dim3((unsigned)(C * bm)), dim3(NT), 0, st,              \
