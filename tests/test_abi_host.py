@@ -57,6 +57,10 @@ def test_argument_validation_needs_no_gpu():
     assert lib.mta_conv2d_fwd(p, p, p, 1, 1, 8, 8, 3, 3, 1, 7, 0, None) == -2
     # shape
     assert lib.mta_conv2d_fwd(p, p, p, 0, 1, 8, 8, 3, 3, 1, 0, 0, None) == -3
+    # softmax gradient: null pointer, dtype, shape
+    assert lib.mta_softmax_bwd(p, None, p, 1, 1, 8, 8, 1, 1, 0, None) == -1
+    assert lib.mta_softmax_bwd(p, p, p, 1, 1, 8, 8, 1, 1, 9, None) == -2
+    assert lib.mta_softmax_bwd(p, p, p, 1, 1, 8, 0, 1, 1, 0, None) == -3
     assert lib.mta_headmix_fwd(p, p, p, 1, 2, 0, 8, 0, 1, 0.0, 0, 0, None) == -3
     assert lib.mta_conv_attn_fwd(p, p, p, p, p, 1, 1, 0, 64, 3, 3, 1, 0.1, 0, 0, None) == -3
     # kernel size
