@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTA_ABI_VERSION 5
+#define MTA_ABI_VERSION 6
 
 enum mta_dtype { MTA_F32 = 0, MTA_BF16 = 1, MTA_F16 = 2 };
 
@@ -44,6 +44,12 @@ enum mta_error {
 };
 
 /* Largest conv kernel the entry points accept. */
+/* `causal` of mta_conv2d_fwd, mta_conv2d_scaled_fwd, mta_conv2d_bwd_input, mta_headmix_fwd and mta_headmix_bwd_input:
+ * 0 = no mask; MTA_CAUSAL_LOWER_ONLY = causal, for a consumer that never reads above the diagonal (what lies there
+ * in the output is left alone, except where a vector or tile straddles the diagonal: +0.0 / fill); any other value =
+ * causal with the output above the diagonal written (+0.0 / fill).  The other entry points read `causal` as a flag. */
+#define MTA_CAUSAL_LOWER_ONLY 2
+
 #define MTA_MAX_KERNEL_R 32
 #define MTA_MAX_KERNEL_S 63
 

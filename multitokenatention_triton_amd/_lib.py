@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libmta_hip.so")
 
 # dtype codes of include/mta_hip.h
 MTA_F32, MTA_BF16, MTA_F16 = 0, 1, 2
+MTA_CAUSAL_LOWER_ONLY = 2  # `causal` of the conv / head-mixing entry points: nothing written above the diagonal
 
 _c = ctypes
 _vp, _i64, _int, _f32 = _c.c_void_p, _c.c_int64, _c.c_int, _c.c_float

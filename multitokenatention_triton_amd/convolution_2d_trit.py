@@ -16,13 +16,18 @@ from . import ops
 
 
 class Conv2dTritonFunction(torch.autograd.Function):
-    """apply(input (N,C,H,W), weight (C,R,S), causal) -> (N,C,H,W), same dtype as input."""
+    """apply(input (N,C,H,W), weight (C,R,S), causal) -> (N,C,H,W), same dtype as input.
+
+    Two optional flags for callers that know who reads the results (both only matter when ``causal``):
+    ``fill_upper=False`` -- the output is only read on and below the diagonal; ``grad_fill_upper=False`` -- so is the
+    input gradient that backward returns.  What lies above the diagonal is then left unwritten."""
 
     @staticmethod
-    def forward(ctx, input, weight, causal):
+    def forward(ctx, input, weight, causal, fill_upper=True, grad_fill_upper=True):
         ctx.save_for_backward(input, weight)
         ctx.causal = causal
-        return ops.conv2d_causal(input, weight, causal)
+        ctx.grad_fill_upper = grad_fill_upper
+        return ops.conv2d_causal(input, weight, causal, fill_upper=fill_upper)
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -31,11 +36,11 @@ class Conv2dTritonFunction(torch.autograd.Function):
         input, weight = ctx.saved_tensors
         grad_input = grad_weight = None
         if ctx.needs_input_grad[0]:
-            grad_input = ops.conv2d_bwd_input(grad_output, weight, ctx.causal)
+            grad_input = ops.conv2d_bwd_input(grad_output, weight, ctx.causal, fill_upper=ctx.grad_fill_upper)
         if ctx.needs_input_grad[1]:
             grad_weight = ops.conv2d_bwd_weight(input, grad_output.to(input.dtype), tuple(weight.shape[1:]),
                                                 ctx.causal).to(weight.dtype)
-        return grad_input, grad_weight, None
+        return grad_input, grad_weight, None, None, None
 
 
 class Conv2dTriton(nn.Module):

@@ -757,12 +757,15 @@ int conv2d_entry(const void *x, const void *w, void *y, int64_t N, int64_t C, in
     });
     return MTA_ERR_DTYPE;
 }
+// the `causal` argument of the entry points: 0 = no mask, 2 = causal with the output above the diagonal left to the
+// caller (MTA_CAUSAL_LOWER_ONLY), anything else = causal with +0 written there
+inline int causal_mode(int causal) { return causal == MTA_CAUSAL_LOWER_ONLY ? 2 : (causal ? 1 : 0); }
 }  // namespace
 
 extern "C" int mta_conv2d_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H,
                               int64_t W, int R, int S, int causal, int io_dtype, int w_dtype, void *stream)
 {
-    return conv2d_entry<false>(x, w, y, N, C, H, W, R, S, causal ? 1 : 0, 1.0f, 0, io_dtype, w_dtype, stream);
+    return conv2d_entry<false>(x, w, y, N, C, H, W, R, S, causal_mode(causal), 1.0f, 0, io_dtype, w_dtype, stream);
 }
 
 // (causal == 2 inside this file: causal, and the kernel that enumerates the lower triangle's strips only - the
@@ -776,12 +779,12 @@ extern "C" int mta_conv2d_tril_fwd(const void *x, const void *w, void *y, int64_
 extern "C" int mta_conv2d_bwd_input(const void *dy, const void *w, void *dx, int64_t N, int64_t C, int64_t H,
                                     int64_t W, int R, int S, int causal, int io_dtype, int w_dtype, void *stream)
 {
-    return conv2d_entry<true>(dy, w, dx, N, C, H, W, R, S, causal ? 1 : 0, 1.0f, 0, io_dtype, w_dtype, stream);
+    return conv2d_entry<true>(dy, w, dx, N, C, H, W, R, S, causal_mode(causal), 1.0f, 0, io_dtype, w_dtype, stream);
 }
 
 extern "C" int mta_conv2d_scaled_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H,
                                      int64_t W, int R, int S, int causal, float in_scale, int io_dtype,
                                      int w_dtype, void *stream)
 {
-    return conv2d_entry<false>(x, w, y, N, C, H, W, R, S, causal ? 1 : 0, in_scale, 1, io_dtype, w_dtype, stream);
+    return conv2d_entry<false>(x, w, y, N, C, H, W, R, S, causal_mode(causal), in_scale, 1, io_dtype, w_dtype, stream);
 }

@@ -429,7 +429,8 @@ extern "C" int mta_headmix_fwd(const void *x, const void *w, void *y, int64_t N,
                                int64_t Q, int group_size, int causal, float fill, int io_dtype, int w_dtype,
                                void *stream)
 {
-    return headmix_entry(x, w, y, N, C, P, Q, group_size, causal ? 1 : 0, fill, io_dtype, w_dtype, 0, stream);
+    return headmix_entry(x, w, y, N, C, P, Q, group_size, causal == MTA_CAUSAL_LOWER_ONLY ? 2 : (causal ? 1 : 0), fill,
+                         io_dtype, w_dtype, 0, stream);
 }
 
 extern "C" int mta_headmix_tril_fwd(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
@@ -443,5 +444,6 @@ extern "C" int mta_headmix_tril_fwd(const void *x, const void *w, void *y, int64
 extern "C" int mta_headmix_bwd_input(const void *dy, const void *w, void *dx, int64_t N, int64_t C, int64_t P,
                                      int64_t Q, int group_size, int causal, int io_dtype, int w_dtype, void *stream)
 {
-    return headmix_entry(dy, w, dx, N, C, P, Q, group_size, causal ? 1 : 0, 0.0f, io_dtype, w_dtype, 1, stream);
+    return headmix_entry(dy, w, dx, N, C, P, Q, group_size, causal == MTA_CAUSAL_LOWER_ONLY ? 2 : (causal ? 1 : 0), 0.0f,
+                         io_dtype, w_dtype, 1, stream);
 }

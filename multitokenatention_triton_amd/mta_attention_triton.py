@@ -53,8 +53,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import ops
-from .convolution_2d_trit import Conv2dTriton
-from .triton_linear_head import TritonLinearHead
+from .convolution_2d_trit import Conv2dTriton, Conv2dTritonFunction
+from .triton_linear_head import TritonLinearHead, TritonLinearHeadFunction
 
 # largest mixing group the one-pass mix/softmax/mix kernel keeps in registers ...
 _FUSED_MAX_GROUP = 8
@@ -89,7 +89,8 @@ class _ScaledScoresConv(torch.autograd.Function):
         mark("conv_pre")
         ctx.save_for_backward(xq, xk, weight, raw)
         ctx.scale, ctx.causal = scale, causal
-        return ops.conv2d_causal(raw, weight, causal, in_scale=scale)
+        # (the stage that follows, head mixing or mixing + softmax, never reads above the diagonal)
+        return ops.conv2d_causal(raw, weight, causal, in_scale=scale, fill_upper=False)
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -115,29 +116,31 @@ class _MixSoftmax(torch.autograd.Function):
     two gradient kernels."""
 
     @staticmethod
-    def forward(ctx, x, weight, causal, group_size):
-        p = ops.headmix_softmax(x, weight, None, causal, group_size=group_size if weight is not None else None)
+    def forward(ctx, x, weight, causal, group_size, fill_upper=True, grad_fill_upper=True):
+        p = ops.headmix_softmax(x, weight, None, causal, group_size=group_size if weight is not None else None,
+                                fill_upper=fill_upper)
         ctx.save_for_backward(x if weight is not None else None, weight, p)
-        ctx.causal, ctx.group_size = causal, group_size
+        ctx.causal, ctx.group_size, ctx.grad_fill_upper = causal, group_size, grad_fill_upper
         return p
 
     @staticmethod
     def backward(ctx, grad_output):
         x, weight, p = ctx.saved_tensors
-        # the head mixing's gradient kernels never read above the diagonal; autograd's next consumer might
-        ds = ops.softmax_bwd(p, grad_output.to(p.dtype), ctx.causal, fill_upper=weight is None)
+        # the head mixing's gradient kernels never read above the diagonal; whoever takes the gradient we return might
+        ds = ops.softmax_bwd(p, grad_output.to(p.dtype), ctx.causal,
+                             fill_upper=weight is None and ctx.grad_fill_upper)
         if weight is None:
-            return ds, None, None, None
+            return ds, None, None, None, None, None
         dx = dw = None
         if ctx.needs_input_grad[0]:
-            dx = ops.headmix_bwd_input(ds, weight, ctx.causal, ctx.group_size)
+            dx = ops.headmix_bwd_input(ds, weight, ctx.causal, ctx.group_size, fill_upper=ctx.grad_fill_upper)
         if ctx.needs_input_grad[1]:
             dw = ops.headmix_bwd_weight(x, ds, ctx.causal)
             if ctx.group_size:
                 blk = torch.arange(weight.shape[0], device=weight.device) // ctx.group_size
                 dw = dw * (blk[:, None] == blk[None, :])
             dw = dw.to(weight.dtype)
-        return dx, dw, None, None
+        return dx, dw, None, None, None, None
 
 
 @dataclass
@@ -304,18 +307,25 @@ class MTAAttentionTriton(nn.Module):
         scores = _ScaledScoresConv.apply(xq, xk, self.mta_conv_triton.weight, scale, self.causal, self._mark)
         group = self.wpsm_triton.group_size
         w_pre = self.wpsm_triton.weight
+        # Between two of these stages nothing reads above the diagonal (causal kernels never do, in either direction),
+        # so nothing is written there: only the last stage's output, which torch's GEMM reads in full, and the score
+        # gradient that goes into torch's GEMMs (inside _ScaledScoresConv) are filled.
+        lower = not self.causal   # value of the fill flags: False (leave alone) when causal
         if _one_pass_group(group or self.n_heads, scores.dtype, xk.size(-2), w_pre):
             self._mark("mix_softmax")
-            scores = _MixSoftmax.apply(scores, w_pre, self.causal, group)
+            scores = _MixSoftmax.apply(scores, w_pre, self.causal, group, lower, lower)
         else:
             self._mark("mix_pre")
-            scores = self.wpsm_triton(scores)
+            scores = TritonLinearHeadFunction.apply(scores, w_pre, self.wpsm_triton.causal, self.wpsm_triton.output_value,
+                                                    group, lower, lower)
             self._mark("softmax")
-            scores = _MixSoftmax.apply(scores, None, self.causal, None)
+            scores = _MixSoftmax.apply(scores, None, self.causal, None, lower, lower)
         self._mark("conv_post")
-        scores = self.mta_conv_after_sm_triton(scores)
+        scores = Conv2dTritonFunction.apply(scores, self.mta_conv_after_sm_triton.weight, self.causal, lower, lower)
         self._mark("mix_post")
-        scores = self.wposm_triton(scores)
+        post = self.wposm_triton
+        scores = TritonLinearHeadFunction.apply(scores, post.weight, post.causal, post.output_value, post.group_size,
+                                                True, lower)
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         self._mark("pv")
         output = torch.matmul(scores, xv)

@@ -34,6 +34,13 @@ def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+def _causal_mode(causal: bool, fill_upper: bool) -> int:
+    """The `causal` argument of the conv / head-mixing entry points: 0, 1, or MTA_CAUSAL_LOWER_ONLY."""
+    if not causal:
+        return 0
+    return 1 if fill_upper else _lib.MTA_CAUSAL_LOWER_ONLY
+
+
 def _out_like(x: torch.Tensor, out: Optional[torch.Tensor]) -> torch.Tensor:
     if out is None:
         return torch.empty_like(x, memory_format=torch.contiguous_format)
@@ -67,7 +74,7 @@ def conv2d_causal(x: torch.Tensor, weight: torch.Tensor, causal: bool, in_scale:
                                     _code(x, "input"), _code(weight, "weight"), _stream(x))
         else:
             rc = lib.mta_conv2d_scaled_fwd(x.data_ptr(), weight.data_ptr(), y.data_ptr(), n, c, h, w, r, s,
-                                           int(bool(causal)), float(in_scale), _code(x, "input"),
+                                           _causal_mode(causal, fill_upper), float(in_scale), _code(x, "input"),
                                            _code(weight, "weight"), _stream(x))
     _lib.check(rc, "mta_conv2d_fwd")
     return y
@@ -106,17 +113,19 @@ def _workspace(nbytes: int, device) -> torch.Tensor:
     return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
 
 
-def conv2d_bwd_input(dy: torch.Tensor, weight: torch.Tensor, causal: bool) -> torch.Tensor:
-    """Gradient of ``conv2d_causal`` with respect to its input; see mta_conv2d_bwd_input."""
+def conv2d_bwd_input(dy: torch.Tensor, weight: torch.Tensor, causal: bool, fill_upper: bool = True,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Gradient of ``conv2d_causal`` with respect to its input; see mta_conv2d_bwd_input.  ``fill_upper=False``
+    (causal): for a consumer that never reads above the diagonal."""
     dy = _device_tensor(dy, "grad_output")
     weight = _device_tensor(weight.detach(), "weight")
     n, c, h, w = dy.shape
     c_out, r, s = weight.shape
     assert c == c_out, "This implementation assumes depthwise convolution (C_in == C_out)"
-    dx = torch.empty_like(dy, memory_format=torch.contiguous_format)
+    dx = _out_like(dy, out)
     with torch.cuda.device(dy.device):
         rc = _lib.load().mta_conv2d_bwd_input(dy.data_ptr(), weight.data_ptr(), dx.data_ptr(), n, c, h, w, r, s,
-                                              int(bool(causal)), _code(dy, "grad_output"), _code(weight, "weight"),
+                                              _causal_mode(causal, fill_upper), _code(dy, "grad_output"), _code(weight, "weight"),
                                               _stream(dy))
     _lib.check(rc, "mta_conv2d_bwd_input")
     return dx
@@ -142,16 +151,18 @@ def conv2d_bwd_weight(x: torch.Tensor, dy: torch.Tensor, kernel_size, causal: bo
 
 
 def headmix_bwd_input(dy: torch.Tensor, weight: torch.Tensor, causal: bool = True,
-                      group_size: Optional[int] = None) -> torch.Tensor:
-    """Gradient of ``headmix`` with respect to its input (+0 above the diagonal); see mta_headmix_bwd_input."""
+                      group_size: Optional[int] = None, fill_upper: bool = True,
+                      out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Gradient of ``headmix`` with respect to its input (+0 above the diagonal); see mta_headmix_bwd_input.
+    ``fill_upper=False`` (causal): for a consumer that never reads above the diagonal."""
     dy = _device_tensor(dy, "grad_output")
     weight = _device_tensor(weight.detach(), "weight")
     n, c, p, q = dy.shape
     assert tuple(weight.shape) == (c, c), f"Weight must be ({c},{c}), got {tuple(weight.shape)}"
-    dx = torch.empty_like(dy, memory_format=torch.contiguous_format)
+    dx = _out_like(dy, out)
     with torch.cuda.device(dy.device):
         rc = _lib.load().mta_headmix_bwd_input(dy.data_ptr(), weight.data_ptr(), dx.data_ptr(), n, c, p, q,
-                                               int(group_size or 0), int(bool(causal)), _code(dy, "grad_output"),
+                                               int(group_size or 0), _causal_mode(causal, fill_upper), _code(dy, "grad_output"),
                                                _code(weight, "weight"), _stream(dy))
     _lib.check(rc, "mta_headmix_bwd_input")
     return dx

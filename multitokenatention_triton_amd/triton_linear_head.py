@@ -17,14 +17,20 @@ from . import ops
 
 
 class TritonLinearHeadFunction(torch.autograd.Function):
-    """apply(input (N,C,P,Q), weight (C,C), causal=True, output_value=0.0[, group_size])."""
+    """apply(input (N,C,P,Q), weight (C,C), causal=True, output_value=0.0[, group_size]).
+
+    Two optional flags for callers that know who reads the results (both only matter when ``causal``):
+    ``fill_upper=False`` -- the output is only read on and below the diagonal; ``grad_fill_upper=False`` -- so is the
+    input gradient that backward returns.  What lies above the diagonal is then left unwritten."""
 
     @staticmethod
-    def forward(ctx, input, weight, causal=True, output_value=0.0, group_size=None):
+    def forward(ctx, input, weight, causal=True, output_value=0.0, group_size=None, fill_upper=True,
+                grad_fill_upper=True):
         ctx.save_for_backward(input, weight)
         ctx.causal = causal
         ctx.group_size = group_size
-        return ops.headmix(input, weight, causal, output_value, group_size)
+        ctx.grad_fill_upper = grad_fill_upper
+        return ops.headmix(input, weight, causal, output_value, group_size, fill_upper=fill_upper)
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -33,14 +39,15 @@ class TritonLinearHeadFunction(torch.autograd.Function):
         input, weight = ctx.saved_tensors
         grad_input = grad_weight = None
         if ctx.needs_input_grad[0]:
-            grad_input = ops.headmix_bwd_input(grad_output, weight, ctx.causal, ctx.group_size)
+            grad_input = ops.headmix_bwd_input(grad_output, weight, ctx.causal, ctx.group_size,
+                                               fill_upper=ctx.grad_fill_upper)
         if ctx.needs_input_grad[1]:
             grad_weight = ops.headmix_bwd_weight(input, grad_output.to(input.dtype), ctx.causal)
             if ctx.group_size:
                 blk = torch.arange(weight.shape[0], device=weight.device) // ctx.group_size
                 grad_weight = grad_weight * (blk[:, None] == blk[None, :])
             grad_weight = grad_weight.to(weight.dtype)
-        return grad_input, grad_weight, None, None, None
+        return grad_input, grad_weight, None, None, None, None, None
 
 
 class TritonLinearHead(nn.Module):

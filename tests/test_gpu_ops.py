@@ -240,6 +240,34 @@ def test_headmix_tril_leaves_the_upper_triangle_alone(ops, case, dt):
         assert (got[..., 0, s - 64:].float() == 7.0).all()
 
 
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32"])
+@pytest.mark.parametrize("case", [(1, 2, 384, 6, 11), (2, 2, 264, 7, 7), (1, 3, 100, 3, 3)])
+def test_lower_only_mode_of_the_other_conv_and_headmix_entries(ops, case, dt):
+    """`causal` = MTA_CAUSAL_LOWER_ONLY in mta_conv2d_scaled_fwd, mta_conv2d_bwd_input and mta_headmix_bwd_input: on and
+    below the diagonal bit for bit the filling call's result, above it the buffer's old content (sentinel) or +0."""
+    n, c, s, r, sk = case
+    dtype = DT[dt]
+    print(f"lower-only case={case} dt={dt}", flush=True)
+    x = torch.tril(_randn((n, c, s, s), 31, dtype)).cuda()
+    w = _randn((c, r, sk), 32, dtype, 0.2).cuda()
+    g = torch.Generator().manual_seed(33)
+    wm = (torch.eye(c) + 0.1 * torch.randn(c, c, generator=g)).to(dtype).cuda()
+    low = ~_upper(s, s).cuda()
+    sent = lambda: torch.full_like(x, 7.0)
+    pairs = [
+        (ops.conv2d_causal(x, w, True, in_scale=0.125), ops.conv2d_causal(x, w, True, in_scale=0.125, out=sent(), fill_upper=False)),
+        (ops.conv2d_bwd_input(x, w, True), ops.conv2d_bwd_input(x, w, True, fill_upper=False, out=sent())),
+        (ops.headmix_bwd_input(x, wm, True), ops.headmix_bwd_input(x, wm, True, fill_upper=False, out=sent())),
+    ]
+    for full, got in pairs:
+        assert torch.equal(got[..., low], full[..., low])
+        up = got[..., ~low].float()
+        assert ((up == 7.0) | (up == 0)).all()
+    if dtype != torch.float32 and s % 128 == 0:   # matrix-core conv kernels: blocks wholly above the diagonal stay untouched
+        for _, got in pairs[:2]:
+            assert (got[..., 0, s - 128:].float() == 7.0).all()
+
+
 MS_CASES = [
     # N, C, P(=Q), group, use_w1, use_w2
     (1, 4, 64, 2, True, True), (2, 4, 100, 4, True, False), (1, 8, 257, 4, False, True), (1, 2, 33, 1, False, False),
