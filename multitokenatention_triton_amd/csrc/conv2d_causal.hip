@@ -244,6 +244,25 @@ __device__ __forceinline__ void zero_fill_strip(T *yp, int H, int W, int p0, int
     }
 }
 
+// The part of a square causal output above the diagonal's 128x128 blocks, written as +0 by workgroups of their own
+// (mirror == 3): row p of a plane gets keys (p / M_TN + 1) * M_TN .. W-1, a contiguous run.  Workgroup `fid` of `nfill`
+// takes rows fid, fid + nfill, ... of all planes.
+template <typename T>
+__device__ __forceinline__ void fill_above_blocks(T *y, int64_t planes, int H, int W, int fid, int nfill, int tid)
+{
+    constexpr int VEC = 8;
+    pack16<T> z;
+#pragma unroll
+    for (int u = 0; u < VEC; ++u) z.v[u] = from_float<T>(0.0f);
+    const int64_t rows = planes * H;
+    for (int64_t rr = fid; rr < rows; rr += nfill) {
+        const int p = (int)(rr % H);
+        T *row = y + rr * W;
+        for (int q = (p / M_TN + 1) * M_TN + tid * VEC; q < W; q += M_WT * VEC)
+            MTA_CONV_STORE(reinterpret_cast<u32x4 *>(row + q), __builtin_bit_cast(u32x4, z));
+    }
+}
+
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef const __attribute__((address_space(1))) void glb_void_t;
 
@@ -316,8 +335,14 @@ __device__ __forceinline__ void wg_barrier() { asm volatile("s_barrier" : : : "m
 template <typename T, int R, int S, bool SCALED, bool BWD>
 __global__ __launch_bounds__(M_WT, 2) void conv2d_mfma(
     const T *__restrict__ x, const T *__restrict__ w, T *__restrict__ y, int C, int H, int W, int causal, float in_scale,
-    int tiles_n, int ipp, int64_t total, int64_t per_xcd, int nw, int mirror)
+    int tiles_n, int ipp, int64_t total, int64_t per_xcd, int nw, int mirror, int nfill)
 {
+    // mirror == 3: the image above the diagonal is written by nfill workgroups of their own, which the device runs
+    // beside the persistent ones (they hold no registers or LDS traffic to speak of)
+    if (mirror == 3 && (int)blockIdx.x >= nw * 8) {
+        fill_above_blocks<T>(y, total / ipp, H, W, (int)blockIdx.x - nw * 8, nfill, (int)threadIdx.x);
+        return;
+    }
     using G = mfma_geom<R, S>;
     static_assert(!BWD || (S % 2 == 1 && !SCALED), "the backward instance assumes symmetric key halos and no scale");
     constexpr int TOP = BWD ? 0 : R - 1;                    // halo rows above the strip (the others lie below it)
@@ -684,7 +709,9 @@ int launch_mfma(const void *x, const void *w, void *y, int64_t N, int64_t C, int
     const int tiles_m = (int)((H + M_TM - 1) / M_TM), tiles_n = (int)((W + M_TN - 1) / M_TN);
     // mirror enumeration needs a square grid of whole 128x128 blocks' worth of strips
     const int blocks = (int)((H + M_TN - 1) / M_TN);
-    const int mirror = (causal && H == W) ? (causal == 2 ? 2 : 1) : 0;
+    // (MTA_CONV_INLINE_FILL=1 in the environment: the strips' own workgroups write the image, for comparisons)
+    static const bool inline_fill = [] { const char *e = getenv("MTA_CONV_INLINE_FILL"); return e && e[0] == '1'; }();
+    const int mirror = (causal && H == W) ? (causal == 2 ? 2 : ((inline_fill || W % 8 != 0 || blocks < 2) ? 1 : 3)) : 0;
     const int64_t ipp64 = mirror ? (int64_t)blocks * (blocks + 1) / 2 * M_SPB : (int64_t)tiles_m * tiles_n;
     if (ipp64 > (1 << 24)) return MTA_ERR_SHAPE;  // decode_item's float sqrt is exact well beyond this
     const int ipp = (int)ipp64;
@@ -693,16 +720,17 @@ int launch_mfma(const void *x, const void *w, void *y, int64_t N, int64_t C, int
     int nw = device_cu_count() * M_WG_PER_CU / 8;  // persistent workgroups per XCD
     if (nw < 1) nw = 1;
     if (per_xcd < nw) nw = (int)per_xcd;
-    dim3 grid((unsigned)(nw * 8));
+    const int nfill = mirror == 3 ? device_cu_count() * 2 : 0;  // two more workgroups per CU fit beside the persistent four
+    dim3 grid((unsigned)(nw * 8 + nfill));
     if constexpr (BWD) {
         hipLaunchKernelGGL((conv2d_mfma<T, R, S, false, true>), grid, dim3(M_WT), 0, st, (const T *)x, (const T *)w, (T *)y,
-                           (int)C, (int)H, (int)W, causal, in_scale, tiles_n, ipp, total, per_xcd, nw, mirror);
+                           (int)C, (int)H, (int)W, causal, in_scale, tiles_n, ipp, total, per_xcd, nw, mirror, nfill);
     } else if (use_scale) {
         hipLaunchKernelGGL((conv2d_mfma<T, R, S, true, false>), grid, dim3(M_WT), 0, st, (const T *)x, (const T *)w, (T *)y,
-                           (int)C, (int)H, (int)W, causal, in_scale, tiles_n, ipp, total, per_xcd, nw, mirror);
+                           (int)C, (int)H, (int)W, causal, in_scale, tiles_n, ipp, total, per_xcd, nw, mirror, nfill);
     } else {
         hipLaunchKernelGGL((conv2d_mfma<T, R, S, false, false>), grid, dim3(M_WT), 0, st, (const T *)x, (const T *)w, (T *)y,
-                           (int)C, (int)H, (int)W, causal, in_scale, tiles_n, ipp, total, per_xcd, nw, mirror);
+                           (int)C, (int)H, (int)W, causal, in_scale, tiles_n, ipp, total, per_xcd, nw, mirror, nfill);
     }
     return launch_status();
 }
