@@ -1,0 +1,37 @@
+"""The comparison switches of the library (environment variables read once per process) select kernels that the default
+dispatch only takes for other dtypes or shapes.  Each group of switches is set for a child process that runs the
+parity tests of the operators concerned: the alternative kernels must meet the same bars on the 16-bit cases too."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+GROUPS = [
+    # the conv's own workgroups write the +0 above the diagonal; vector-ALU head mixing for 16 and 32 heads; the
+    # general softmax and fused kernels for 16-bit data
+    ({"MTA_CONV_INLINE_FILL": "1", "MTA_HEADMIX_NO_MFMA": "1", "MTA_SOFTMAX_NO_PACKED": "1", "MTA_FUSED_FORCE_GENERAL": "1"},
+     ["tests/test_gpu_ops.py", "tests/test_gpu_attention.py"],
+     "test_conv_parity or test_conv_identity_tap or test_conv_tril or test_headmix_parity or test_mix_softmax_mix_parity "
+     "or test_conv_attention_parity or test_mta_general"),
+    # fp32-FMA conv kernels (forward, input gradient, weight gradient) for 16-bit data
+    ({"MTA_CONV_FORCE_VALU": "1"},
+     ["tests/test_gpu_ops.py", "tests/test_gpu_backward.py"],
+     "test_conv_parity or test_conv_identity_tap or test_conv_backward_parity"),
+]
+
+
+@pytest.mark.parametrize("group", range(len(GROUPS)))
+def test_comparison_switches_meet_the_same_bars(group):
+    env, files, select = GROUPS[group]
+    print(f"switches {sorted(env)}", flush=True)
+    cmd = [sys.executable, "-u", "-m", "pytest", *files, "-x", "-q", "-k", select, "-p", "no:cacheprovider",
+           "--timeout", "120", "--timeout-method", "thread"]
+    r = subprocess.run(cmd, cwd=ROOT, env={**os.environ, **env}, capture_output=True, text=True, timeout=900)
+    tail = (r.stdout or "")[-3000:] + (r.stderr or "")[-1000:]
+    assert r.returncode == 0, tail
+    assert " passed" in r.stdout, tail
