@@ -76,20 +76,29 @@ _CONV_MIX_SIZES = ((3, 3), (7, 7))
 
 
 class _ScaledScoresConv(torch.autograd.Function):
-    """conv(round(Q K^T) * scale) for the training route (mta_attention_triton.py:69-73): the library GEMM, then
-    ``mta_conv2d_scaled_fwd``, which applies the factor (and the rounding to the score dtype that the reference's
-    separate multiplication performs) on the way into the conv.  Backward: the conv's input gradient ``g`` goes through
-    the two GEMMs and the factor is applied to their (B,H,S,D) results; the kernel gradient is taken against the raw
-    scores and scaled afterwards.  Neither direction spends a pass over the (B,H,S,S) tensor on the factor."""
+    """conv(round(Q K^T) * scale) for the training route (mta_attention_triton.py:69-73).  Forward: the inference
+    route's one kernel (``mta_qk_conv_fwd``, the raw scores never reach memory) where it exists; otherwise the library
+    GEMM, then ``mta_conv2d_scaled_fwd``, which applies the factor (and the rounding to the score dtype that the
+    reference's separate multiplication performs) on the way into the conv.  Backward: the conv's input gradient ``g``
+    goes through the two GEMMs and the factor is applied to their (B,H,S,D) results; the kernel gradient is taken
+    against the raw scores -- kept by the second forward, recomputed with one GEMM after the first, which so saves a
+    (B,H,S,S) activation -- and scaled afterwards.  Neither direction spends a pass over a (B,H,S,S) tensor on the
+    factor."""
 
     @staticmethod
     def forward(ctx, xq, xk, weight, scale, causal, mark):
+        ctx.scale, ctx.causal = scale, causal
+        # (the stage that follows, head mixing or mixing + softmax, never reads above the diagonal)
+        if xq.shape == xk.shape and xq.dtype != torch.float32:
+            mark("qk_conv")
+            out = ops.qk_conv(xq, xk, weight, causal, scale, fill_upper=False)
+            if out is not None:
+                ctx.save_for_backward(xq, xk, weight, None)
+                return out
         mark("qk")
         raw = torch.matmul(xq, xk.transpose(2, 3))
         mark("conv_pre")
         ctx.save_for_backward(xq, xk, weight, raw)
-        ctx.scale, ctx.causal = scale, causal
-        # (the stage that follows, head mixing or mixing + softmax, never reads above the diagonal)
         return ops.conv2d_causal(raw, weight, causal, in_scale=scale, fill_upper=False)
 
     @staticmethod
@@ -103,6 +112,8 @@ class _ScaledScoresConv(torch.autograd.Function):
             if ctx.needs_input_grad[1]:
                 dk = torch.matmul(g.transpose(2, 3), xq) * ctx.scale
         if ctx.needs_input_grad[2]:
+            if raw is None:
+                raw = torch.matmul(xq, xk.transpose(2, 3))
             dw = ops.conv2d_bwd_weight(raw, grad_output.to(raw.dtype), tuple(weight.shape[1:]), ctx.causal)
             dw = (dw * ctx.scale).to(weight.dtype)
         return dq, dk, dw, None, None, None
