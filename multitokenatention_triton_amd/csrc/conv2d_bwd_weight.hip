@@ -148,9 +148,8 @@ __global__ __launch_bounds__(NT) void conv2d_bwd_weight_fixed(const T *__restric
 // ---- matrix-core kernel -------------------------------------------------------------------------------------------
 typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 constexpr int MB = 2;            // 16-row blocks of dy per work item (against MB + 1 blocks of x)
-constexpr int HV = 1;            // 32-key half steps per step
 constexpr int MROWS = 16 * MB;   // rows of dy per work item
-constexpr int KSTEP = 32 * HV;   // keys per step
+constexpr int KSTEP = 32;        // keys per step
 
 // Eight consecutive keys k0..k0+7 (k0 a multiple of 8, possibly -8) of row h.  The forward pass's masks -- 0 outside the
 // plane and, under the causal rule, for keys beyond the row index -- are applied in two parts: piece_ok() picks the
@@ -177,19 +176,20 @@ __device__ __forceinline__ u4 mask_piece(u4 v, int h, int k0, int H, int W, int 
     return v;
 }
 
-// One step of a wavefront: HV half steps of 32 keys each (lane: keys kb + 32 hv + 8g .. +7) over MB 16-row blocks of dy
-// and the MB + 1 blocks of x around them; for x also the eight keys on either side of the lane's eight.  MB = 2, HV = 1
-// is the fastest measured: 11 loads per 4*S products.  MB = 1, HV = 2 (whole 128-byte lines of every row per step, 14
-// loads per 4*S products) fetches 40 % less from memory, since no line is asked for twice a step apart, and still takes
-// 20 % longer: the time follows the number of load instructions, not the bytes.
-struct step_operands {
-    u4 dy[MB][HV];
-    u4 x[MB + 1][HV][3];
+// One step of a wavefront covers 32 keys: lane (r, g) loads the eight keys kb + 8g .. +7 of its rows -- MB 16-row blocks
+// of dy and the MB + 1 blocks of x around them -- and nothing else.  The products pair the dy keys of the lane group to
+// the LEFT (k-8 .. k-1, k = kb + 8g) with the 24-key window k-16 .. k+7 of x, whose first two thirds are the pieces of
+// the two lane groups to the left as well: those come over ds_bpermute (for the first groups of a step, from the step
+// before, which stays in registers), not from memory.  With every lane loading its whole window itself (three pieces
+// per block of x: 11 loads per step instead of 5) the kernel's time followed the number of load instructions.
+struct step_pieces {
+    u4 dy[MB];
+    u4 x[MB + 1];
 };
 
 // The rows a lane reads in a work item, as element offsets into the plane (which the host keeps below 2^31 elements):
-// x rows p0 - 16 + 16 nb + r from key 8g - 8 on, dy rows p0 + 16 mb + r from key 8g on.  The offset of a row outside
-// the plane wraps around and is never used.
+// x rows p0 - 16 + 16 nb + r and dy rows p0 + 16 mb + r, both from key 8g on.  The offset of a row outside the plane
+// wraps around and is never used.
 struct lane_rows {
     unsigned x[MB + 1];
     unsigned dy[MB];
@@ -200,85 +200,80 @@ template <typename T> __device__ __forceinline__ u4 load16(const T *plane, unsig
     return *reinterpret_cast<const u4 *>(plane + (size_t)off);
 }
 
-// `inner` (wavefront-uniform): every piece of the step lies inside the plane and on or below the diagonal
+// `inner` (wavefront-uniform): every piece of the step lies inside the plane and on or below the diagonal.  kb may be
+// -32 (the step ahead of a row's first, whose pieces all read as 0).
 template <typename T>
-__device__ __forceinline__ void load_step(step_operands &o, const T *xp, const T *dyp, const lane_rows &rows, int p0,
-                                          int kb, int r, int g, int H, int W, int causal, bool inner)
+__device__ __forceinline__ void load_step(step_pieces &o, const T *xp, const T *dyp, const lane_rows &rows, int p0, int kb,
+                                          int r, int g, int H, int W, int causal, bool inner)
 {
     if (inner) {
 #pragma unroll
-        for (int hv = 0; hv < HV; ++hv) {
+        for (int mb = 0; mb < MB; ++mb) o.dy[mb] = load16(dyp, rows.dy[mb] + kb);
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) o.dy[mb][hv] = load16(dyp, rows.dy[mb] + kb + 32 * hv);
-#pragma unroll
-            for (int nb = 0; nb < MB + 1; ++nb)
-#pragma unroll
-                for (int s = 0; s < 3; ++s) o.x[nb][hv][s] = load16(xp, rows.x[nb] + kb + 32 * hv + 8 * s);
-        }
+        for (int nb = 0; nb < MB + 1; ++nb) o.x[nb] = load16(xp, rows.x[nb] + kb);
     } else {
+        const int k = kb + 8 * g;
 #pragma unroll
-        for (int hv = 0; hv < HV; ++hv) {
-            const int k = kb + 32 * hv + 8 * g;
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-                o.dy[mb][hv] = load16(dyp, piece_ok(p0 + 16 * mb + r, k, H, W, causal) ? rows.dy[mb] + kb + 32 * hv : 0u);
-#pragma unroll
-            for (int nb = 0; nb < MB + 1; ++nb)
-#pragma unroll
-                for (int s = 0; s < 3; ++s)
-                    o.x[nb][hv][s] = load16(xp, piece_ok(p0 - 16 + 16 * nb + r, k - 8 + 8 * s, H, W, causal)
-                                                    ? rows.x[nb] + kb + 32 * hv + 8 * s
-                                                    : 0u);
-        }
-    }
-}
-
-__device__ __forceinline__ void mask_step(step_operands &o, int p0, int kb, int r, int g, int H, int W, int causal)
-{
-    // rows of this item start at p0 - 16, the step's last key (with the window) is kb + KSTEP + 7
-    const bool edge = causal && kb + KSTEP + 7 > p0 - 16;
-#pragma unroll
-    for (int hv = 0; hv < HV; ++hv) {
-        const int k = kb + 32 * hv + 8 * g;
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) o.dy[mb][hv] = mask_piece(o.dy[mb][hv], p0 + 16 * mb + r, k, H, W, causal, edge);
+        for (int mb = 0; mb < MB; ++mb)
+            o.dy[mb] = load16(dyp, piece_ok(p0 + 16 * mb + r, k, H, W, causal) ? rows.dy[mb] + kb : 0u);
 #pragma unroll
         for (int nb = 0; nb < MB + 1; ++nb)
-#pragma unroll
-            for (int s = 0; s < 3; ++s)
-                o.x[nb][hv][s] = mask_piece(o.x[nb][hv][s], p0 - 16 + 16 * nb + r, k - 8 + 8 * s, H, W, causal, edge);
+            o.x[nb] = load16(xp, piece_ok(p0 - 16 + 16 * nb + r, k, H, W, causal) ? rows.x[nb] + kb : 0u);
     }
 }
 
-// The 2*MB*HV*S products of a step: block mb of dy against blocks mb and mb+1 of x, every key offset j.  The operand
-// of offset j is the lane's 24-key window of x from key 8 + j - pad on (a byte shift of two registers for odd starts).
+__device__ __forceinline__ void mask_step(step_pieces &o, int p0, int kb, int r, int g, int H, int W, int causal)
+{
+    const int k = kb + 8 * g;
+    // rows of this item start at p0 - 16, the step's last key is kb + 31
+    const bool edge = causal && kb + 31 > p0 - 16;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) o.dy[mb] = mask_piece(o.dy[mb], p0 + 16 * mb + r, k, H, W, causal, edge);
+#pragma unroll
+    for (int nb = 0; nb < MB + 1; ++nb) o.x[nb] = mask_piece(o.x[nb], p0 - 16 + 16 * nb + r, k, H, W, causal, edge);
+}
+
+// the piece that lane (r, g - back) holds in `cur`, or, for the first `back` lane groups, lane (r, g - back + 4) in `prev`
+__device__ __forceinline__ u4 piece_from_left(const u4 &prev, const u4 &cur, int lane, int back)
+{
+    const bool from_prev = lane >= 64 - 16 * back;  // as a source: these lanes are read by the first groups of this step
+    const int src = ((lane - 16 * back) & 63) * 4;
+    u4 v;
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+        v[d] = (unsigned)__builtin_amdgcn_ds_bpermute(src, (int)(from_prev ? prev[d] : cur[d]));
+    return v;
+}
+
+// The 2*MB*S products of a step: block mb of dy against blocks mb and mb+1 of x, every key offset j.  The operand of
+// offset j is the 24-key window of x from key 8 + j - pad on (a byte shift of two registers for odd starts).
 template <typename T, int S>
-__device__ __forceinline__ void accumulate_step(f32x4 (&acc)[2][S], const step_operands &o)
+__device__ __forceinline__ void accumulate_step(f32x4 (&acc)[2][S], const step_pieces &prev, const step_pieces &cur, int lane)
 {
     constexpr int PW = (S - 1) / 2;
+    frag8<T> a[MB];
 #pragma unroll
-    for (int hv = 0; hv < HV; ++hv) {
-        frag8<T> a[MB];
+    for (int mb = 0; mb < MB; ++mb) a[mb] = __builtin_bit_cast(frag8<T>, piece_from_left(prev.dy[mb], cur.dy[mb], lane, 1));
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) a[mb] = __builtin_bit_cast(frag8<T>, o.dy[mb][hv]);
+    for (int nb = 0; nb < MB + 1; ++nb) {
+        const u4 ll = piece_from_left(prev.x[nb], cur.x[nb], lane, 2), l = piece_from_left(prev.x[nb], cur.x[nb], lane, 1);
+        unsigned w[12];
 #pragma unroll
-        for (int nb = 0; nb < MB + 1; ++nb) {
-            unsigned w[12];
+        for (int u = 0; u < 4; ++u) {
+            w[u] = ll[u];
+            w[4 + u] = l[u];
+            w[8 + u] = cur.x[nb][u];
+        }
 #pragma unroll
-            for (int s = 0; s < 3; ++s)
+        for (int j = 0; j < S; ++j) {
+            const int st = 8 + j - PW;  // compile-time after unrolling
+            u4 bv;
 #pragma unroll
-                for (int u = 0; u < 4; ++u) w[4 * s + u] = o.x[nb][hv][s][u];
-#pragma unroll
-            for (int j = 0; j < S; ++j) {
-                const int st = 8 + j - PW;  // compile-time after unrolling
-                u4 bv;
-#pragma unroll
-                for (int d = 0; d < 4; ++d)
-                    bv[d] = (st & 1) ? __builtin_amdgcn_alignbyte(w[(st + 1) / 2 + d], w[(st - 1) / 2 + d], 2) : w[st / 2 + d];
-                const frag8<T> b = __builtin_bit_cast(frag8<T>, bv);
-                if (nb <= MB - 1) mma16(acc[0][j], a[nb < MB ? nb : 0], b);
-                if (nb >= 1) mma16(acc[1][j], a[nb - 1 >= 0 ? nb - 1 : 0], b);
-            }
+            for (int d = 0; d < 4; ++d)
+                bv[d] = (st & 1) ? __builtin_amdgcn_alignbyte(w[(st + 1) / 2 + d], w[(st - 1) / 2 + d], 2) : w[st / 2 + d];
+            const frag8<T> b = __builtin_bit_cast(frag8<T>, bv);
+            if (nb <= MB - 1) mma16(acc[0][j], a[nb < MB ? nb : 0], b);
+            if (nb >= 1) mma16(acc[1][j], a[nb - 1 >= 0 ? nb - 1 : 0], b);
         }
     }
 }
@@ -312,37 +307,48 @@ __global__ __launch_bounds__(NT) void conv2d_bwd_weight_mfma(const T *__restrict
         const int p0 = tm * MROWS;
         int kend = W;  // dy is zero beyond the diagonal: keys from p0 + MROWS on add nothing
         if (causal && p0 + MROWS < W) kend = p0 + MROWS;
-        const int nsteps = (kend + KSTEP - 1) / KSTEP, per = (nsteps + nseg - 1) / nseg;
+        // a step pairs the dy keys kb-8 .. kb+23 with their windows of x: the row's keys end at kend-1
+        const int nsteps = (kend + 8 + KSTEP - 1) / KSTEP, per = (nsteps + nseg - 1) / nseg;
         const int t0 = sg * per, t1 = (t0 + per < nsteps) ? t0 + per : nsteps;
         if (t0 >= t1) continue;
         const int64_t plane = ((int64_t)n * C + c) * H * W;
         const T *xp = x + plane, *dyp = dy + plane;
         lane_rows rows;
 #pragma unroll
-        for (int nb = 0; nb < MB + 1; ++nb) rows.x[nb] = (unsigned)((p0 - 16 + 16 * nb + r) * W + 8 * g - 8);
+        for (int nb = 0; nb < MB + 1; ++nb) rows.x[nb] = (unsigned)((p0 - 16 + 16 * nb + r) * W + 8 * g);
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) rows.dy[mb] = (unsigned)((p0 + 16 * mb + r) * W + 8 * g);
         // steps whose pieces all lie inside the plane and on or below the diagonal need neither selects nor masks: rows
-        // p0-16 .. p0+MROWS-1 inside the plane, keys kb-8 .. kb+KSTEP+7 inside it and (causal) not beyond row p0-16
+        // p0-16 .. p0+MROWS-1 inside the plane, keys kb .. kb+31 inside it and (causal) not beyond row p0-16
         const bool rows_in = p0 >= 16 && p0 + MROWS <= H;
-        const int in_plane = W - KSTEP - 8, below = p0 - 16 - KSTEP - 7;
+        const int in_plane = W - KSTEP, below = p0 - 16 - (KSTEP - 1);
         const int last_inner = causal ? (below < in_plane ? below : in_plane) : in_plane;  // largest such kb
-        auto inner = [&](int t) { return rows_in && KSTEP * t >= 8 && KSTEP * t <= last_inner; };
-        // two operand sets take turns, so that a step's loads stay in flight through the whole of the step before it;
-        // the last step fetches itself again: the number of loads in flight never depends on a branch
-        step_operands oa, ob;
-        load_step(oa, xp, dyp, rows, p0, KSTEP * t0, r, g, H, W, causal, inner(t0));
-        for (int t = t0; t < t1; t += 2) {
-            const int tb = t + 1 < t1 ? t + 1 : t;
-            load_step(ob, xp, dyp, rows, p0, KSTEP * tb, r, g, H, W, causal, inner(tb));
-            if (!inner(t)) mask_step(oa, p0, KSTEP * t, r, g, H, W, causal);
-            accumulate_step<T, S>(acc, oa);
-            if (t + 1 >= t1) break;
-            const int ta = t + 2 < t1 ? t + 2 : t + 1;
-            load_step(oa, xp, dyp, rows, p0, KSTEP * ta, r, g, H, W, causal, inner(ta));
-            if (!inner(t + 1)) mask_step(ob, p0, KSTEP * (t + 1), r, g, H, W, causal);
-            accumulate_step<T, S>(acc, ob);
+        auto inner = [&](int t) { return rows_in && t >= 0 && KSTEP * t <= last_inner; };
+        // Three sets of pieces take turns as (step before, this step, next step): the next step's loads stay in flight
+        // through this step's products, and the step before supplies the left neighbours of this step's first lane
+        // groups.  The last step fetches itself again, so that the loads in flight never depend on a branch; the step
+        // ahead of the segment's first is fetched for its pieces only.
+        step_pieces sa, sb, sc;
+        load_step(sa, xp, dyp, rows, p0, KSTEP * (t0 - 1), r, g, H, W, causal, inner(t0 - 1));
+        load_step(sb, xp, dyp, rows, p0, KSTEP * t0, r, g, H, W, causal, inner(t0));
+        if (!inner(t0 - 1)) mask_step(sa, p0, KSTEP * (t0 - 1), r, g, H, W, causal);
+        int t = t0;
+#define MTA_CBW_STEP(PV, CU, NX)                                                                        \
+        {                                                                                               \
+            const int tn = t + 1 < t1 ? t + 1 : t;                                                      \
+            load_step(NX, xp, dyp, rows, p0, KSTEP * tn, r, g, H, W, causal, inner(tn));                \
+            if (!inner(t)) mask_step(CU, p0, KSTEP * t, r, g, H, W, causal);                            \
+            accumulate_step<T, S>(acc, PV, CU, lane);                                                   \
         }
+        for (;;) {
+            MTA_CBW_STEP(sa, sb, sc)
+            if (++t >= t1) break;
+            MTA_CBW_STEP(sb, sc, sa)
+            if (++t >= t1) break;
+            MTA_CBW_STEP(sc, sa, sb)
+            if (++t >= t1) break;
+        }
+#undef MTA_CBW_STEP
     }
 
     // tap (i,j) = sum over m of D_j[m][m + i - (R-1)] taken from the half that holds that column; the four wavefronts
