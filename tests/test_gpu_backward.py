@@ -87,6 +87,28 @@ def test_conv_backward_parity(pkg, case, dtype):
     assert torch.equal(dw, pkg.ops.conv2d_bwd_weight(x_dev, dy_dev, (r, s), causal))
 
 
+def test_conv_backward_full_size(pkg):
+    """BASELINE config 2 at full size, (2,16,2048,2048) bf16 6x11 causal: the kernel gradient of every channel is the sum
+    of the two batch elements' (linearity, all channels), and two channels are compared with the oracle on their own
+    slices; the input gradient of those channels likewise."""
+    print("conv bwd full size", flush=True)
+    n, c, s, r, sk = 2, 16, 2048, 6, 11
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(71)
+    x = torch.tril(torch.randn(n, c, s, s, generator=g).to(dtype))
+    dy = torch.tril(torch.randn(n, c, s, s, generator=g).to(dtype))
+    wt = (0.2 * torch.randn(c, r, sk, generator=g)).to(dtype)
+    xd, dyd = x.cuda(), dy.cuda()
+    dw = pkg.ops.conv2d_bwd_weight(xd, dyd, (r, sk), True)
+    parts = sum(pkg.ops.conv2d_bwd_weight(xd[b:b + 1].contiguous(), dyd[b:b + 1].contiguous(), (r, sk), True) for b in range(n))
+    _close(dw, parts, dtype, "dw = sum over the batch", weight_grad=True)
+    dx = pkg.ops.conv2d_bwd_input(dyd, wt.cuda(), True)
+    for ch in (3, 12):
+        want_dx, want_dw = O.depthwise_conv_grads(x[:, ch:ch + 1].float(), wt[ch:ch + 1].float(), True, dy[:, ch:ch + 1].float())
+        _close(dw[ch:ch + 1], want_dw, dtype, f"dw channel {ch}", weight_grad=True)
+        _close(dx[:, ch:ch + 1], want_dx, dtype, f"dx channel {ch}")
+
+
 HM_CASES = [
     # N, C, P, Q, group, causal
     (2, 4, 40, 40, None, True),
