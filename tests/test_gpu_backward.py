@@ -202,6 +202,33 @@ def test_softmax_backward_parity(pkg, case, dtype):
         assert (sentinel.cpu()[..., far] == 7.0).all()
 
 
+def test_headmix_and_softmax_backward_full_size(pkg):
+    """(2,32,2048,2048) bf16, BASELINE config 3's shape: the head-mixing weight gradient is the sum of the two batch
+    elements' (linearity) and symmetric in its arguments (dW(x, dy) = dW(dy, x)^T); the softmax gradient, whose rows are
+    independent, is compared with autograd on slabs of rows of two planes."""
+    print("headmix / softmax bwd full size", flush=True)
+    n, c, s = 2, 32, 2048
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(72)
+    xd = torch.randn(n, c, s, s, generator=g).to(dtype).cuda()
+    dyd = torch.randn(n, c, s, s, generator=g).to(dtype).cuda()
+    dw = pkg.ops.headmix_bwd_weight(xd, dyd, True)
+    parts = sum(pkg.ops.headmix_bwd_weight(xd[b:b + 1].contiguous(), dyd[b:b + 1].contiguous(), True) for b in range(n))
+    _close(dw, parts, dtype, "dw = sum over the batch", weight_grad=True)
+    _close(pkg.ops.headmix_bwd_weight(dyd, xd, True).t(), dw, dtype, "dw(dy, x)^T", weight_grad=True)
+    # softmax gradient: p from the CPU softmax of the same logits, rows 0-63 and the last 96 of planes (0,5) and (1,30)
+    up = torch.triu(torch.ones(s, s, dtype=torch.bool), 1)
+    for b, ch in ((0, 5), (1, 30)):
+        logits = xd[b, ch].cpu().float().masked_fill(up, float("-inf")).requires_grad_(True)
+        probs = torch.softmax(logits, -1)
+        probs.backward(dyd[b, ch].cpu().float().masked_fill(up, 0.0))
+        p_dev = torch.zeros(1, 1, s, s, dtype=dtype, device="cuda")
+        p_dev[0, 0] = probs.detach().to(dtype).cuda()
+        got = pkg.ops.softmax_bwd(p_dev, dyd[b:b + 1, ch:ch + 1].contiguous(), True)[0, 0].cpu()
+        for rows in (slice(0, 64), slice(s - 96, s)):
+            _close(got[rows], logits.grad[rows], dtype, f"softmax dx plane {(b, ch)} rows {rows}")
+
+
 def test_operator_functions_backward(pkg):
     """Conv2dTritonFunction / TritonLinearHeadFunction under torch.autograd, fp32, against the oracle's grads."""
     print("operator Functions backward", flush=True)
