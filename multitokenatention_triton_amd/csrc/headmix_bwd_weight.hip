@@ -43,13 +43,17 @@ __device__ __forceinline__ void hm_load(hm_operands<NB> &o, const T *x, const T 
                                         int g)
 {
     const int q = u.q0 + 8 * g;
+    // every load is unconditional: a vector wholly beyond `last` re-reads the row start and is zeroed before use
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        // every load is unconditional: a vector wholly beyond `last` re-reads the row start and is zeroed before use
-        const int qq = (q + 32 * t <= u.last) ? q + 32 * t : 0;
+    for (int a = 0; a < NB; ++a) {
 #pragma unroll
-        for (int a = 0; a < NB; ++a) {
+        for (int t = 0; t < 4; ++t) {
+            const int qq = (q + 32 * t <= u.last) ? q + 32 * t : 0;
             o.dy[a][t] = *reinterpret_cast<const u4 *>(dy + u.rowbase + (int64_t)(a * 16 + r) * plane + qq);
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int qq = (q + 32 * t <= u.last) ? q + 32 * t : 0;
             o.x[a][t] = *reinterpret_cast<const u4 *>(x + u.rowbase + (int64_t)(a * 16 + r) * plane + qq);
         }
     }
