@@ -19,7 +19,9 @@ namespace {
 using namespace mta;
 
 constexpr int NT = 256;
-constexpr int CHUNK = 128;  // positions per wavefront step (MFMA kernel)
+// positions per wavefront step of the MFMA kernel: 512 contiguous bytes of every head's row with 16 heads, 256 with 32
+// (registers)
+template <int NB> constexpr int chunk_of() { return NB == 1 ? 256 : 128; }
 
 // Rows are visited in an order that interleaves short and long ones (0, P-1, 1, P-2, ...), so that under the causal
 // mask a pair of consecutive rows always carries P+1 positions.
@@ -35,7 +37,7 @@ struct hm_unit {
 
 // The chunk's operands of a lane: for product t the eight positions from q0 + 32t + 8g on, of head 16a + r.
 template <int NB> struct hm_operands {
-    u4 dy[NB][4], x[NB][4];
+    u4 dy[NB][chunk_of<NB>() / 32], x[NB][chunk_of<NB>() / 32];
 };
 
 template <typename T, int NB>
@@ -47,12 +49,12 @@ __device__ __forceinline__ void hm_load(hm_operands<NB> &o, const T *x, const T 
 #pragma unroll
     for (int a = 0; a < NB; ++a) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < chunk_of<NB>() / 32; ++t) {
             const int qq = (q + 32 * t <= u.last) ? q + 32 * t : 0;
             o.dy[a][t] = *reinterpret_cast<const u4 *>(dy + u.rowbase + (int64_t)(a * 16 + r) * plane + qq);
         }
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < chunk_of<NB>() / 32; ++t) {
             const int qq = (q + 32 * t <= u.last) ? q + 32 * t : 0;
             o.x[a][t] = *reinterpret_cast<const u4 *>(x + u.rowbase + (int64_t)(a * 16 + r) * plane + qq);
         }
@@ -62,11 +64,11 @@ __device__ __forceinline__ void hm_load(hm_operands<NB> &o, const T *x, const T 
 template <typename T, int NB>
 __device__ __forceinline__ void hm_consume(f32x4 (&acc)[NB][NB], hm_operands<NB> &o, const hm_unit &u, int g)
 {
-    if (u.q0 + CHUNK - 1 > u.last) {  // the chunk straddles the end of the row: zero what lies beyond it, in both
+    if (u.q0 + chunk_of<NB>() - 1 > u.last) {  // the chunk straddles the end of the row: zero what lies beyond it, in both
                                       // operands (what x holds there need not even be finite)
         const int q = u.q0 + 8 * g;
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+        for (int t = 0; t < chunk_of<NB>() / 32; ++t)
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int e = q + 32 * t + 2 * v;
@@ -79,7 +81,7 @@ __device__ __forceinline__ void hm_consume(f32x4 (&acc)[NB][NB], hm_operands<NB>
             }
     }
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int t = 0; t < chunk_of<NB>() / 32; ++t)
 #pragma unroll
         for (int a = 0; a < NB; ++a)
 #pragma unroll
@@ -119,7 +121,7 @@ __global__ __launch_bounds__(NT) void headmix_bwd_weight_mfma(const T *__restric
         return true;
     };
     auto advance = [&](const hm_unit &u) {
-        q0 += CHUNK;
+        q0 += chunk_of<NB>();
         if (q0 > u.last) {
             q0 = 0;
             ++j;
