@@ -148,8 +148,10 @@ __global__ __launch_bounds__(NT) void conv2d_bwd_weight_fixed(const T *__restric
 // ---- matrix-core kernel -------------------------------------------------------------------------------------------
 typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 constexpr int MB = 2;            // 16-row blocks of dy per work item (against MB + 1 blocks of x)
+constexpr int HV = 2;            // 32-key halves per step: a step takes whole 128-byte lines of its rows, the two
+                                 // halves of a line in load instructions issued back to back
 constexpr int MROWS = 16 * MB;   // rows of dy per work item
-constexpr int KSTEP = 32;        // keys per step
+constexpr int KSTEP = 32 * HV;   // keys per step
 
 // Eight consecutive keys k0..k0+7 (k0 a multiple of 8, possibly -8) of row h.  The forward pass's masks -- 0 outside the
 // plane and, under the causal rule, for keys beyond the row index -- are applied in two parts: piece_ok() picks the
@@ -183,8 +185,8 @@ __device__ __forceinline__ u4 mask_piece(u4 v, int h, int k0, int H, int W, int 
 // before, which stays in registers), not from memory.  With every lane loading its whole window itself (three pieces
 // per block of x: 11 loads per step instead of 5) the kernel's time followed the number of load instructions.
 struct step_pieces {
-    u4 dy[MB];
-    u4 x[MB + 1];
+    u4 dy[MB][HV];
+    u4 x[MB + 1][HV];
 };
 
 // The rows a lane reads in a work item, as element offsets into the plane (which the host keeps below 2^31 elements):
@@ -208,29 +210,44 @@ __device__ __forceinline__ void load_step(step_pieces &o, const T *xp, const T *
 {
     if (inner) {
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) o.dy[mb] = load16(dyp, rows.dy[mb] + kb);
-#pragma unroll
-        for (int nb = 0; nb < MB + 1; ++nb) o.x[nb] = load16(xp, rows.x[nb] + kb);
-    } else {
-        const int k = kb + 8 * g;
-#pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-            o.dy[mb] = load16(dyp, piece_ok(p0 + 16 * mb + r, k, H, W, causal) ? rows.dy[mb] + kb : 0u);
+#pragma unroll
+            for (int hv = 0; hv < HV; ++hv) o.dy[mb][hv] = load16(dyp, rows.dy[mb] + kb + 32 * hv);
 #pragma unroll
         for (int nb = 0; nb < MB + 1; ++nb)
-            o.x[nb] = load16(xp, piece_ok(p0 - 16 + 16 * nb + r, k, H, W, causal) ? rows.x[nb] + kb : 0u);
+#pragma unroll
+            for (int hv = 0; hv < HV; ++hv) o.x[nb][hv] = load16(xp, rows.x[nb] + kb + 32 * hv);
+    } else {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int hv = 0; hv < HV; ++hv) {
+                const int k = kb + 32 * hv + 8 * g;
+                o.dy[mb][hv] = load16(dyp, piece_ok(p0 + 16 * mb + r, k, H, W, causal) ? rows.dy[mb] + kb + 32 * hv : 0u);
+            }
+#pragma unroll
+        for (int nb = 0; nb < MB + 1; ++nb)
+#pragma unroll
+            for (int hv = 0; hv < HV; ++hv) {
+                const int k = kb + 32 * hv + 8 * g;
+                o.x[nb][hv] = load16(xp, piece_ok(p0 - 16 + 16 * nb + r, k, H, W, causal) ? rows.x[nb] + kb + 32 * hv : 0u);
+            }
     }
 }
 
 __device__ __forceinline__ void mask_step(step_pieces &o, int p0, int kb, int r, int g, int H, int W, int causal)
 {
-    const int k = kb + 8 * g;
-    // rows of this item start at p0 - 16, the step's last key is kb + 31
-    const bool edge = causal && kb + 31 > p0 - 16;
+    // rows of this item start at p0 - 16, the step's last key is kb + KSTEP - 1
+    const bool edge = causal && kb + KSTEP - 1 > p0 - 16;
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) o.dy[mb] = mask_piece(o.dy[mb], p0 + 16 * mb + r, k, H, W, causal, edge);
+    for (int hv = 0; hv < HV; ++hv) {
+        const int k = kb + 32 * hv + 8 * g;
 #pragma unroll
-    for (int nb = 0; nb < MB + 1; ++nb) o.x[nb] = mask_piece(o.x[nb], p0 - 16 + 16 * nb + r, k, H, W, causal, edge);
+        for (int mb = 0; mb < MB; ++mb) o.dy[mb][hv] = mask_piece(o.dy[mb][hv], p0 + 16 * mb + r, k, H, W, causal, edge);
+#pragma unroll
+        for (int nb = 0; nb < MB + 1; ++nb)
+            o.x[nb][hv] = mask_piece(o.x[nb][hv], p0 - 16 + 16 * nb + r, k, H, W, causal, edge);
+    }
 }
 
 // the piece that lane (r, g - back) holds in `cur`, or, for the first `back` lane groups, lane (r, g - back + 4) in `prev`
@@ -251,29 +268,38 @@ template <typename T, int S>
 __device__ __forceinline__ void accumulate_step(f32x4 (&acc)[2][S], const step_pieces &prev, const step_pieces &cur, int lane)
 {
     constexpr int PW = (S - 1) / 2;
-    frag8<T> a[MB];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) a[mb] = __builtin_bit_cast(frag8<T>, piece_from_left(prev.dy[mb], cur.dy[mb], lane, 1));
+    for (int hv = 0; hv < HV; ++hv) {
+        // what lies to the left of this half's first lane groups: the last half of the step before, or this step's
+        // half before this one
+        frag8<T> a[MB];
 #pragma unroll
-    for (int nb = 0; nb < MB + 1; ++nb) {
-        const u4 ll = piece_from_left(prev.x[nb], cur.x[nb], lane, 2), l = piece_from_left(prev.x[nb], cur.x[nb], lane, 1);
-        unsigned w[12];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            w[u] = ll[u];
-            w[4 + u] = l[u];
-            w[8 + u] = cur.x[nb][u];
+        for (int mb = 0; mb < MB; ++mb) {
+            const u4 &before = hv == 0 ? prev.dy[mb][HV - 1] : cur.dy[mb][hv > 0 ? hv - 1 : 0];
+            a[mb] = __builtin_bit_cast(frag8<T>, piece_from_left(before, cur.dy[mb][hv], lane, 1));
         }
 #pragma unroll
-        for (int j = 0; j < S; ++j) {
-            const int st = 8 + j - PW;  // compile-time after unrolling
-            u4 bv;
+        for (int nb = 0; nb < MB + 1; ++nb) {
+            const u4 &before = hv == 0 ? prev.x[nb][HV - 1] : cur.x[nb][hv > 0 ? hv - 1 : 0];
+            const u4 ll = piece_from_left(before, cur.x[nb][hv], lane, 2), l = piece_from_left(before, cur.x[nb][hv], lane, 1);
+            unsigned w[12];
 #pragma unroll
-            for (int d = 0; d < 4; ++d)
-                bv[d] = (st & 1) ? __builtin_amdgcn_alignbyte(w[(st + 1) / 2 + d], w[(st - 1) / 2 + d], 2) : w[st / 2 + d];
-            const frag8<T> b = __builtin_bit_cast(frag8<T>, bv);
-            if (nb <= MB - 1) mma16(acc[0][j], a[nb < MB ? nb : 0], b);
-            if (nb >= 1) mma16(acc[1][j], a[nb - 1 >= 0 ? nb - 1 : 0], b);
+            for (int u = 0; u < 4; ++u) {
+                w[u] = ll[u];
+                w[4 + u] = l[u];
+                w[8 + u] = cur.x[nb][hv][u];
+            }
+#pragma unroll
+            for (int j = 0; j < S; ++j) {
+                const int st = 8 + j - PW;  // compile-time after unrolling
+                u4 bv;
+#pragma unroll
+                for (int d = 0; d < 4; ++d)
+                    bv[d] = (st & 1) ? __builtin_amdgcn_alignbyte(w[(st + 1) / 2 + d], w[(st - 1) / 2 + d], 2) : w[st / 2 + d];
+                const frag8<T> b = __builtin_bit_cast(frag8<T>, bv);
+                if (nb <= MB - 1) mma16(acc[0][j], a[nb < MB ? nb : 0], b);
+                if (nb >= 1) mma16(acc[1][j], a[nb - 1 >= 0 ? nb - 1 : 0], b);
+            }
         }
     }
 }
@@ -307,7 +333,7 @@ __global__ __launch_bounds__(NT) void conv2d_bwd_weight_mfma(const T *__restrict
         const int p0 = tm * MROWS;
         int kend = W;  // dy is zero beyond the diagonal: keys from p0 + MROWS on add nothing
         if (causal && p0 + MROWS < W) kend = p0 + MROWS;
-        // a step pairs the dy keys kb-8 .. kb+23 with their windows of x: the row's keys end at kend-1
+        // a step pairs the dy keys kb-8 .. kb+KSTEP-9 with their windows of x: the row's keys end at kend-1
         const int nsteps = (kend + 8 + KSTEP - 1) / KSTEP, per = (nsteps + nseg - 1) / nseg;
         const int t0 = sg * per, t1 = (t0 + per < nsteps) ? t0 + per : nsteps;
         if (t0 >= t1) continue;
@@ -319,7 +345,7 @@ __global__ __launch_bounds__(NT) void conv2d_bwd_weight_mfma(const T *__restrict
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) rows.dy[mb] = (unsigned)((p0 + 16 * mb + r) * W + 8 * g);
         // steps whose pieces all lie inside the plane and on or below the diagonal need neither selects nor masks: rows
-        // p0-16 .. p0+MROWS-1 inside the plane, keys kb .. kb+31 inside it and (causal) not beyond row p0-16
+        // p0-16 .. p0+MROWS-1 inside the plane, keys kb .. kb+KSTEP-1 inside it and (causal) not beyond row p0-16
         const bool rows_in = p0 >= 16 && p0 + MROWS <= H;
         const int in_plane = W - KSTEP, below = p0 - 16 - (KSTEP - 1);
         const int last_inner = causal ? (below < in_plane ? below : in_plane) : in_plane;  // largest such kb
