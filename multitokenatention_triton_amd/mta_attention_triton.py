@@ -75,6 +75,50 @@ _CONV_MIX_MAX_GROUP = 4
 _CONV_MIX_SIZES = ((3, 3), (7, 7))
 
 
+_IDENTITY_KERNELS = {}
+
+
+def _lower_scores(a: torch.Tensor, b: torch.Tensor) -> Optional[torch.Tensor]:
+    """round(a b^T) on and below the diagonal of a (B,H,S,S) tensor, nothing written above it, for consumers that
+    never read there: the scores kernel (``mta_qk_conv_fwd``) with factor 1 and a 3x3 kernel that is the pass-through
+    tap, which copies its input exactly.  Half the output traffic of the library GEMM.  None where that kernel does not
+    apply (fp32, ragged lengths): the caller then takes the GEMM."""
+    if a.shape != b.shape or a.dtype == torch.float32 or a.dtype != b.dtype:
+        return None
+    h = a.size(1)
+    key = (h, a.dtype, a.device)
+    w = _IDENTITY_KERNELS.get(key)
+    if w is None:
+        w = torch.zeros(h, 3, 3, dtype=a.dtype, device=a.device)
+        w[:, 2, 1] = 1.0
+        _IDENTITY_KERNELS[key] = w
+    return ops.qk_conv(a, b, w, True, 1.0, fill_upper=False)
+
+
+class _ProbsTimesValues(torch.autograd.Function):
+    """P V of the training route (mta_attention_triton.py:89).  Forward is the library GEMM.  Backward: dV = P^T dO is
+    one too; dP = dO V^T is only ever read on and below the diagonal when ``lower`` (the head mixing's gradient kernels
+    take it from here) and then comes from ``_lower_scores``."""
+
+    @staticmethod
+    def forward(ctx, p, v, lower):
+        ctx.save_for_backward(p, v)
+        ctx.lower = lower
+        return torch.matmul(p, v)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        p, v = ctx.saved_tensors
+        dp = dv = None
+        if ctx.needs_input_grad[0]:
+            dp = _lower_scores(grad_output, v) if ctx.lower else None
+            if dp is None:
+                dp = torch.matmul(grad_output, v.transpose(2, 3))
+        if ctx.needs_input_grad[1]:
+            dv = torch.matmul(p.transpose(2, 3), grad_output)
+        return dp, dv, None
+
+
 class _ScaledScoresConv(torch.autograd.Function):
     """conv(round(Q K^T) * scale) for the training route (mta_attention_triton.py:69-73).  Forward: the inference
     route's one kernel (``mta_qk_conv_fwd``, the raw scores never reach memory) where it exists; otherwise the library
@@ -112,8 +156,10 @@ class _ScaledScoresConv(torch.autograd.Function):
             if ctx.needs_input_grad[1]:
                 dk = torch.matmul(g.transpose(2, 3), xq) * ctx.scale
         if ctx.needs_input_grad[2]:
-            if raw is None:
-                raw = torch.matmul(xq, xk.transpose(2, 3))
+            if raw is None:  # (the kernel gradient reads its first argument on and below the diagonal only)
+                raw = _lower_scores(xq, xk) if ctx.causal else None
+                if raw is None:
+                    raw = torch.matmul(xq, xk.transpose(2, 3))
             dw = ops.conv2d_bwd_weight(raw, grad_output.to(raw.dtype), tuple(weight.shape[1:]), ctx.causal)
             dw = (dw * ctx.scale).to(weight.dtype)
         return dq, dk, dw, None, None, None
@@ -339,7 +385,9 @@ class MTAAttentionTriton(nn.Module):
                                                 True, lower)
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         self._mark("pv")
-        output = torch.matmul(scores, xv)
+        # (the gradient with respect to the probabilities goes back into the head mixing's gradient kernels, through the
+        # dropout's elementwise mask at most: nothing there reads above the diagonal when causal)
+        output = _ProbsTimesValues.apply(scores, xv, self.causal and post.causal)
         self._mark("end")
         return output.transpose(1, 2)
 
