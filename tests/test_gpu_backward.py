@@ -312,6 +312,33 @@ def test_mta_module_backward(pkg, dtype):
             _close(p_.grad, wt, dtype, f"grad {name}")
 
 
+@pytest.mark.parametrize("shape", [(1, 8, 100, 32, 6, 11), (2, 4, 264, 128, 7, 7), (1, 32, 136, 64, 3, 5)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mta_module_backward_other_shapes(pkg, shape, dtype):
+    """The training route where its single-kernel stages do not apply and where they do: a head size and a sequence
+    length without a scores kernel (library GEMM + scaled conv, GEMM for dP), 8 heads (packed mix + softmax), 32 dense
+    heads (mixing and softmax as two kernels), head size 128 with a 7x7 kernel."""
+    b, h, s, d, r1, s1 = shape
+    print(f"mta module backward shape={shape} {dtype}", flush=True)
+    mod, params = _mta_pair(pkg, h, r1, s1, dtype, seed=321)
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=322)
+    go = _rand((b, s, h, d), 323, dtype)
+    leaves = [t.detach().clone().float().requires_grad_(True) for t in (q, k, v)]
+    wl = [p.detach().clone().float().requires_grad_(True) for p in params]
+    out = O.mta_forward(*leaves, wl[0].unsqueeze(1), wl[1], wl[2].unsqueeze(1), wl[3])
+    out.backward(go.float())
+    qd, kd, vd = [t.detach().clone().cuda().requires_grad_(True) for t in (q, k, v)]
+    got = mod(qd, kd, vd, None, None)
+    _close(got, out, dtype, "forward")
+    got.backward(go.cuda())
+    for name, gt, wt in (("xq", qd.grad, leaves[0].grad), ("xk", kd.grad, leaves[1].grad), ("xv", vd.grad, leaves[2].grad)):
+        _close(gt, wt, dtype, f"grad {name}")
+    for name, p_, wt in (("pre conv", mod.mta_conv_triton.weight, wl[0].grad), ("wpsm", mod.wpsm_triton.weight, wl[1].grad),
+                         ("post conv", mod.mta_conv_after_sm_triton.weight, wl[2].grad),
+                         ("wposm", mod.wposm_triton.weight, wl[3].grad)):
+        _close(p_.grad, wt, dtype, f"grad {name}")
+
+
 def test_mta_module_backward_reference_bar(pkg):
     """The reference script's own configuration and bar: identity parameters after reset_mta_parameters(), fp32,
     allclose(rtol=1e-3, atol=1e-5) on the three input gradients (compare_mta_attention.py:21-27, 60-74, 113, 136-138)."""
