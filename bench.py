@@ -242,6 +242,12 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
     ms = time_launches(torch, lambda i: mta.ops.headmix_bwd_weight(xs[i], xs[1 - i], True), 2, warmup, steps)
     out["headmix_bwd_weight_bf16_2x32x2048x2048"] = {"ms": ms, "algorithmic_bytes": by2, "GBps": by2 / ms / 1e6,
                                                      "frac_hbm_peak": by2 / ms / 1e6 / HBM_PEAK_GBS}
+    # the softmax gradient of the training route from the stored probabilities (what torch's autograd through
+    # mta_attention_triton.py:79 is replaced by): reads p and dp below the diagonal, writes dx everywhere
+    ms = time_launches(torch, lambda i: mta.ops.softmax_bwd(xs[i], xs[1 - i], True), 2, warmup, steps)
+    by3 = 2 * n * c * tri(s) * 2 + n * c * s * s * 2
+    out["softmax_bwd_bf16_2x32x2048x2048"] = {"ms": ms, "algorithmic_bytes": by3, "GBps": by3 / ms / 1e6,
+                                              "frac_hbm_peak": by3 / ms / 1e6 / HBM_PEAK_GBS}
     del xs
     # fused conv-attention: B1 H32 S8192 D128 bf16, 6x11
     b, h, s, d = 1, 32, 8192, 128
