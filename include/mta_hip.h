@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTA_ABI_VERSION 6
+#define MTA_ABI_VERSION 7
 
 enum mta_dtype { MTA_F32 = 0, MTA_BF16 = 1, MTA_F16 = 2 };
 
@@ -182,12 +182,25 @@ int mta_qk_conv_fwd(const void *q, const void *k, const void *w, void *s_out, in
                     int64_t S, int64_t D, int R, int Sk, int causal, float scale, int fill_upper,
                     int io_dtype, int w_dtype, void *stream);
 
+/* 1 when mta_qk_conv_fwd has a kernel for these sizes and dtypes, 0 when it would return MTA_ERR_UNSUPPORTED: lets the
+ * caller choose between the one-kernel stage and matmul -> conv (mta_attention_triton.py:69-73) before it launches
+ * anything.  Host-side only; needs no GPU. */
+int mta_qk_conv_supported(int64_t S, int64_t D, int R, int Sk, int io_dtype, int w_dtype);
+
 /* O = P V with P (B,H,S,S), V (B,H,S,D), O (B,H,S,D).  When causal only keys q <= p of P are read
  * (what lies above the diagonal may be uninitialised).  Replaces torch.matmul(scores, xv) of
  * mta_attention_triton.py:89 and halves its traffic.  16-bit I/O, D in {64,128}, S % 8 == 0; anything
  * else returns MTA_ERR_UNSUPPORTED. */
 int mta_causal_pv_fwd(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int64_t D,
                       int causal, int io_dtype, void *stream);
+
+/* The transposed product, O[k,:] = sum_p P[p,k] X[p,:] with P (B,H,S,S), X and O (B,H,S,D); when causal only query rows
+ * p >= k take part and nothing of P above the diagonal is read.  These are the gradients the two matrix products of the
+ * attention leave on their right-hand operands, dV = P^T dO (mta_attention_triton.py:89) and dK = G^T Q (:69, G the
+ * gradient of the raw scores), which the reference leaves to torch's autograd as full-square GEMMs.  Same conditions as
+ * mta_causal_pv_fwd. */
+int mta_causal_ptx_fwd(const void *p, const void *x, void *o, int64_t B, int64_t H, int64_t S, int64_t D,
+                       int causal, int io_dtype, void *stream);
 
 /* ---- backward of the two standalone operators -------------------------------------------------------------
  * Gradients flow through the same masks as the forward pass: with `causal`, entries of dy above the diagonal are

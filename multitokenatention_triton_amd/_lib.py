@@ -30,10 +30,12 @@ SIGNATURES = {
     "mta_headmix_softmax_bias_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _vp]),
     "mta_conv2d_headmix_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _int, _int, _int, _vp]),
     "mta_qk_conv_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _int, _int, _int, _vp]),
+    "mta_qk_conv_supported": (_int, [_i64, _i64, _int, _int, _int, _int]),
     "mta_conv2d_tril_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _vp]),
     "mta_headmix_tril_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _vp]),
     "mta_softmax_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _vp]),
     "mta_causal_pv_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
+    "mta_causal_ptx_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "mta_conv_attn_fwd_lse": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _f32, _int, _int, _vp]),
     "mta_conv2d_bwd_input": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _vp]),
     "mta_conv2d_bwd_weight_workspace": (_i64, [_i64, _i64, _i64, _i64, _int, _int]),

@@ -11,6 +11,8 @@
 // 16-byte chunks XOR-swizzled by key) and V^T fragments come out of them through the LDS transpose
 // read: within 16 lanes, lane c supplies the address of 4 head-dim values of key c/4 and lane i
 // receives head-dim value i of 4 consecutive keys.
+#include <type_traits>
+
 #include "common.hpp"
 #include "mfma.hpp"
 
@@ -185,6 +187,172 @@ __global__ __launch_bounds__(P_NT, P_OCC) void causal_pv_kernel(const T *__restr
   }
 }
 
+// ---- the transposed product --------------------------------------------------------------------------------------
+// O[k, :] = sum over p of P[p, k] X[p, :], p >= k only when causal: the gradients that the two matrix products of the
+// attention leave on their right-hand operands (dV = P^T dO, dK = G^T Q), whose left factor is only defined - and only
+// read - on and below the diagonal.
+//
+// A workgroup owns 128 keys (output rows; 32 per wavefront, two blocks of 16) and walks the query rows from its first
+// key downwards in blocks of 64.  O^T += X^T P on 16x16x32 MFMAs with the query rows as contraction index: both
+// operands are copied global -> LDS asynchronously as row-major blocks (64 rows of X, 64 rows x 128 keys of P; double
+// buffered, 16-byte chunks XOR-swizzled by row) and both fragments come out of them through the LDS transpose read,
+// which hands a lane four consecutive rows of one column: X^T with the head dim as operand row, P with the key as
+// operand column.  P is streamed from memory once; the X blocks are re-read from L2 by every key block above them.
+constexpr int T_KB = 32 * P_WAVES;  // keys per workgroup
+constexpr int T_PB = 64;            // query rows per step
+constexpr int T_KS = T_PB / 32;
+
+template <typename T, int D>
+__global__ __launch_bounds__(P_NT, P_OCC) void causal_ptx_kernel(const T *__restrict__ P, const T *__restrict__ X,
+                                                                 T *__restrict__ O, int S, int causal, int nkb, int64_t total_wg,
+                                                                 int64_t per_xcd)
+{
+    constexpr int XT = T_PB * D, PT = T_PB * T_KB;  // elements per X block / P tile
+    constexpr int XC = D / 8, PC = T_KB / 8;        // 16-byte chunks per row
+    constexpr int XR = XT / 8 / P_NT, PR = PT / 8 / P_NT;
+    static_assert(XT / 8 % P_NT == 0 && PT / 8 % P_NT == 0, "whole copy rounds");
+    constexpr int DB = D / 16;
+    __shared__ __align__(16) T x_a[XT];
+    __shared__ __align__(16) T x_b[XT];
+    __shared__ __align__(16) T p_a[PT];
+    __shared__ __align__(16) T p_b[PT];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, ln = lane & 15, kg = lane >> 4;
+    const int64_t lid = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (lid >= total_wg) return;
+    // two key blocks per workgroup, pi and nkb-1-pi: under the causal rule the first has the most query rows and the
+    // second the fewest, so that every workgroup gets the same amount of work
+    const int npairs = (nkb + 1) / 2;
+    const int pi = (int)(lid % npairs);
+    const int64_t bh = lid / npairs;
+    const T *Pp = P + bh * (int64_t)S * S;
+    const T *Xp = X + bh * (int64_t)S * D;
+    T *Op = O + bh * (int64_t)S * D;
+  for (int half = 0; half < 2; ++half) {
+    const int kb = half == 0 ? pi : nkb - 1 - pi;
+    if (half == 1 && kb == pi) break;  // odd number of blocks: the middle one is alone
+    const int k0 = kb * T_KB;
+    if (half == 1) __syncthreads();    // the buffers are reused: everybody has finished reading them
+
+    // block j = query rows 64j ..; rows past the sequence re-read the last row, keys past it the block's first chunk:
+    // what they bring in is masked (rows) or belongs to output rows that are not stored (keys)
+    auto issue = [&](int j, T *xdst, T *pdst) {
+#pragma unroll
+        for (int r = 0; r < XR; ++r) {
+            const int slot = r * P_NT + tid;
+            const int row = slot / XC, c = (slot % XC) ^ v_swizzle<D>(row);
+            int pr = j * T_PB + row;
+            pr = pr >= S ? S - 1 : pr;
+            __builtin_amdgcn_global_load_lds((glb_void_t *)(Xp + (int64_t)pr * D + c * 8),
+                                             (lds_void_t *)(xdst + (r * P_NT + wave * 64) * 8), 16, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < PR; ++r) {
+            const int slot = r * P_NT + tid;
+            const int row = slot / PC;
+            int c = (slot % PC) ^ v_swizzle<T_KB>(row);
+            if (k0 + c * 8 >= S) c = 0;
+            int pr = j * T_PB + row;
+            pr = pr >= S ? S - 1 : pr;
+            __builtin_amdgcn_global_load_lds((glb_void_t *)(Pp + (int64_t)pr * S + k0 + c * 8),
+                                             (lds_void_t *)(pdst + (r * P_NT + wave * 64) * 8), 16, 0, 0);
+        }
+    };
+    // operand fragment out of a row-major block of LD columns: contraction slots t = 0..7 of step ks are the block's rows
+    // 32ks + 8kg + t, the operand's row / column is column 16*blk + ln of the block
+    auto frag_of = [&](const T *tile, auto ldc, int ks, int blk) {
+        constexpr int LD = decltype(ldc)::value;
+        const int row_a = ks * 32 + kg * 8 + (ln >> 2), row_b = row_a + 4;
+        const int ch = blk * 2 + ((ln & 3) >> 1);
+        const int sub = (ln & 1) * 4;
+        const T *pa = tile + row_a * LD + ((ch ^ v_swizzle<LD>(row_a)) * 8) + sub;
+        const T *pb = tile + row_b * LD + ((ch ^ v_swizzle<LD>(row_b)) * 8) + sub;
+        struct { v4s_t a, b; } both = {__builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)pa),
+                                       __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t *)pb)};
+        return __builtin_bit_cast(frag8<T>, both);
+    };
+
+    // this lane's two output rows (keys)
+    int krow[2];
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) krow[rb] = k0 + (wave * 2 + rb) * 16 + ln;
+    const int j_start = causal ? k0 / T_PB : 0, j_end = (S - 1) / T_PB;
+    f32x4 oacc[2][DB];
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) oacc[rb][db] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    issue(j_start, x_a, p_a);
+
+    auto step = [&](int j, const T *Xb, const T *Pb, T *Xn, T *Pn) __attribute__((always_inline)) {
+        __builtin_amdgcn_s_waitcnt(0);  // block j has arrived
+        __syncthreads();                // for every wavefront; reads of the other buffers are finished
+        if (j < j_end) issue(j + 1, Xn, Pn);
+        // P fragments of this wavefront's two key blocks; query rows above the key (causal: P is undefined there) or
+        // past the sequence count as 0
+        frag8<T> pf[2][T_KS];
+        const int pbase = j * T_PB;
+        const bool edge = pbase + T_PB > S || (causal && pbase < k0 + T_KB - 1);  // (wavefront-uniform)
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+            for (int ks = 0; ks < T_KS; ++ks) {
+                pf[rb][ks] = frag_of(Pb, std::integral_constant<int, T_KB>{}, ks, wave * 2 + rb);
+                if (edge) {
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) {
+                        const int p = pbase + ks * 32 + kg * 8 + t;
+                        if (p >= S || (causal && p < krow[rb])) pf[rb][ks].v[t] = from_float<T>(0.0f);
+                    }
+                }
+            }
+        frag8<T> xf[2];
+        xf[0] = frag_of(Xb, std::integral_constant<int, D>{}, 0, 0);
+#pragma unroll
+        for (int blk = 0; blk < T_KS * DB; ++blk) {
+            const int ks = blk / DB, db = blk % DB;
+            if (blk + 1 < T_KS * DB) xf[(blk + 1) & 1] = frag_of(Xb, std::integral_constant<int, D>{}, (blk + 1) / DB, (blk + 1) % DB);
+            __builtin_amdgcn_sched_barrier(0);  // (the instruction scheduler would move the reads back behind the products)
+            mma16(oacc[0][db], xf[blk & 1], pf[0][ks]);
+            mma16(oacc[1][db], xf[blk & 1], pf[1][ks]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    for (int j = j_start;;) {
+        step(j, x_a, p_a, x_b, p_b);
+        if (++j > j_end) break;
+        step(j, x_b, p_b, x_a, p_a);
+        if (++j > j_end) break;
+    }
+
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+        if (krow[rb] >= S) continue;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            struct alignas(8) quad { T v[4]; } out;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) out.v[v] = from_float<T>(oacc[rb][db][v]);
+            *reinterpret_cast<quad *>(Op + (int64_t)krow[rb] * D + db * 16 + kg * 4) = out;
+        }
+    }
+  }
+}
+
+template <typename T, int D>
+int launch_t(const void *p, const void *x, void *o, int64_t B, int64_t H, int64_t S, int causal, hipStream_t st)
+{
+    const int nkb = (int)((S + T_KB - 1) / T_KB);
+    const int64_t total_wg = B * H * ((nkb + 1) / 2), per_xcd = (total_wg + 7) / 8;
+    if (per_xcd * 8 > 0x7fffffffLL) return MTA_ERR_SHAPE;
+    dim3 grid((unsigned)(per_xcd * 8));
+    auto kern = causal_ptx_kernel<T, D>;
+    hipLaunchKernelGGL(kern, grid, dim3(P_NT), 0, st, (const T *)p, (const T *)x, (T *)o, (int)S, causal, nkb, total_wg,
+                       per_xcd);
+    return launch_status();
+}
+
 template <typename T, int D>
 int launch(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int causal, hipStream_t st)
 {
@@ -212,4 +380,19 @@ extern "C" int mta_causal_pv_fwd(const void *p, const void *v, void *o, int64_t 
     if (io_dtype == MTA_BF16)
         return D == 64 ? launch<bf16_t, 64>(p, v, o, B, H, S, causal, st) : launch<bf16_t, 128>(p, v, o, B, H, S, causal, st);
     return D == 64 ? launch<f16_t, 64>(p, v, o, B, H, S, causal, st) : launch<f16_t, 128>(p, v, o, B, H, S, causal, st);
+}
+
+extern "C" int mta_causal_ptx_fwd(const void *p, const void *x, void *o, int64_t B, int64_t H, int64_t S, int64_t D,
+                                  int causal, int io_dtype, void *stream)
+{
+    if (!p || !x || !o) return MTA_ERR_NULL;
+    if (!dtype_size(io_dtype)) return MTA_ERR_DTYPE;
+    if (B <= 0 || H <= 0 || S <= 0 || S > (1 << 24) || B * H > 65535) return MTA_ERR_SHAPE;
+    if (D != 64 && D != 128) return MTA_ERR_HEAD_DIM;
+    if (!aligned_to(p, 16) || !aligned_to(x, 16) || !aligned_to(o, 16)) return MTA_ERR_ALIGN;
+    if (io_dtype == MTA_F32 || S % 8 != 0) return MTA_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    if (io_dtype == MTA_BF16)
+        return D == 64 ? launch_t<bf16_t, 64>(p, x, o, B, H, S, causal, st) : launch_t<bf16_t, 128>(p, x, o, B, H, S, causal, st);
+    return D == 64 ? launch_t<f16_t, 64>(p, x, o, B, H, S, causal, st) : launch_t<f16_t, 128>(p, x, o, B, H, S, causal, st);
 }

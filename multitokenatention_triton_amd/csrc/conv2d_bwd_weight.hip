@@ -16,6 +16,8 @@
 // keys as contraction index, and the taps (i,j) are the entries p'-p = i-(R-1) of it.  Every 16-row block of dy meets
 // the two 16-row blocks of x that hold its R-1 rows of halo, and all blocks add into the same 2*S accumulators, since
 // only p'-p matters.  The operand of offset j is the lane's 24-key window of x shifted by j keys in registers.
+#include <atomic>
+
 #include "common.hpp"
 #include "mfma.hpp"
 
@@ -528,6 +530,7 @@ int launch(const void *x, const void *dy, float *dw, float *partial, int bpc, in
             MTA_CONV_CASE(6, 11)
             MTA_CONV_CASE(7, 7)
             MTA_CONV_CASE(7, 9)
+            MTA_CONV_CASE(11, 15)
 #undef MTA_CONV_CASE
         }
     }
@@ -576,19 +579,21 @@ static __device__ __align__(256) float scratch[STATIC_FLOATS];
 
 float *static_scratch(int *err)
 {
-    static float *ptr[64] = {nullptr};
+    // (atomic slots: two host threads making their first call on a device may both look the address up and both store
+    // it - the same value - without a data race)
+    static std::atomic<float *> ptr[64];
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) { *err = (int)e; return nullptr; }
     if (dev < 0 || dev >= 64) { *err = MTA_ERR_DEVICE; return nullptr; }
-    if (!ptr[dev]) {
-        float *p = nullptr;
+    float *p = ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
         e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch));
         if (e != hipSuccess) { *err = (int)e; return nullptr; }
-        ptr[dev] = p;
+        ptr[dev].store(p, std::memory_order_release);
     }
     *err = MTA_OK;
-    return ptr[dev];
+    return p;
 }
 }  // namespace
 

@@ -26,6 +26,10 @@
 
 #include <stdlib.h>
 
+#include <atomic>
+#include <type_traits>
+#include <utility>
+
 namespace {
 using namespace mta;
 
@@ -175,13 +179,16 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // rows that neighbouring strips re-read (halos) in the L2.
 #define MTA_CONV_STORE(ptr, val) __builtin_nontemporal_store((val), (ptr))
 
-constexpr int M_NW = 2;            // wavefronts per workgroup; each owns one 16-row block of the workgroup's strip
+constexpr int M_NW = 4;            // wavefronts per workgroup: (16-row block, 128-key half) of the workgroup's strip each
 constexpr int M_WT = 64 * M_NW;    // threads per workgroup
-constexpr int M_TM = 16 * M_NW;    // strip rows
-constexpr int M_TN = 128;          // strip cols: 8 column blocks of 16
-constexpr int M_SPB = M_TN / M_TM;  // strips per 128x128 block
-constexpr int M_WG_PER_CU = 4;     // persistent workgroups per CU (two 12 KB strip buffers each); 3, 5 and 6 measured slower
-static_assert(M_TN % M_TM == 0 && (M_SPB & (M_SPB - 1)) == 0, "strip geometry");
+constexpr int M_TM = 32;           // strip rows
+constexpr int M_TN = 256;          // strip cols: two halves of 8 column blocks of 16
+constexpr int M_HALF = M_TN / 2;   // keys per wavefront
+constexpr int M_RPB = M_TN / M_TM;  // row strips per M_TN x M_TN block of the lower triangle
+// persistent workgroups per CU (two 24 KB strip buffers each); kernels of more than 7 rows keep that many more Toeplitz
+// fragments in registers and are compiled for two
+template <int R> constexpr int wg_per_cu() { return R > 7 ? 2 : 3; }
+static_assert(M_NW == 4 && M_TM == 32 && M_TN % M_TM == 0 && M_RPB % 2 == 0, "strip geometry");
 
 // 16 outputs + S-1 taps (+ alignment shift) must fit the 32-key contraction of one 16x16x32 MFMA
 template <int R, int S> struct mfma_geom {
@@ -192,21 +199,26 @@ template <int R, int S> struct mfma_geom {
     static constexpr int TW = M_TN - 16 + 32;              // staged columns
     static constexpr int LD = TW + ((24 - TW % 16) % 16);  // row stride = 8 (mod 16) elements: conflict-free b128 reads
     static constexpr int ROWS = M_TM + R - 1;
+    // results of the wavefronts that own key half `h` go back to LDS columns h * RES_OFF .. + M_HALF - 1, which no
+    // wavefront of the other half reads as input (half 0 reads columns 0 .. M_HALF+15, half 1 columns M_HALF ..)
+    static constexpr int RES_OFF = M_HALF + 16;
+    static_assert(RES_OFF + M_HALF <= LD, "result columns of the second half");
 };
 
-// position t of a work item inside its plane -> (strip row tm (M_TM rows), strip col tn (128 keys)).
-// `mirror` (causal, square): only strips that touch the lower triangle are enumerated, by 128x128
-// block in row-major lower-triangular order, M_SPB strips per block; each strip of an off-diagonal
-// block also zero-fills its share (1/M_SPB) of the block's mirror image above the diagonal.
-__device__ __forceinline__ void decode_item(int t, int tiles_n, int mirror, int &tm, int &tn)
+// Position t of a work item inside its plane -> (strip row tm (M_TM rows), strip col tn (M_TN keys)).
+// `tri` (causal, square, lower triangle only): the strips that touch the lower triangle, row strip by row strip from
+// the top, each from the left up to the diagonal: row strip tm has tm / M_RPB + 1 of them, so M_RPB/2 * b * (b+1) items
+// precede block row b.  Otherwise: all strips, row-major.
+__device__ __forceinline__ void decode_item(int t, int tiles_n, int tri, int &tm, int &tn)
 {
-    if (mirror) {
-        const int blk = t / M_SPB;
-        int bm = (int)((sqrtf(8.0f * (float)blk + 1.0f) - 1.0f) * 0.5f);
-        while ((bm + 1) * (bm + 2) / 2 <= blk) ++bm;
-        while (bm * (bm + 1) / 2 > blk) --bm;
-        tn = blk - bm * (bm + 1) / 2;
-        tm = bm * M_SPB + (t % M_SPB);
+    if (tri) {
+        constexpr int HB = M_RPB / 2;
+        int b = (int)((sqrtf((float)t / (float)HB + 0.25f) - 0.5f));
+        while (HB * (b + 1) * (b + 2) <= t) ++b;
+        while (HB * b * (b + 1) > t) --b;
+        const int rem = t - HB * b * (b + 1);
+        tm = b * M_RPB + rem / (b + 1);
+        tn = rem % (b + 1);
     } else {
         tm = t / tiles_n;
         tn = t % tiles_n;
@@ -226,50 +238,31 @@ __device__ __forceinline__ int opaque(int v)
 template <typename T, bool FULL = false>
 __device__ __forceinline__ void zero_fill_strip(T *yp, int H, int W, int p0, int q0, int tid)
 {
-    constexpr int VEC = 8;
+    constexpr int VEC = 8, VPRW = M_TN / VEC, RPP = M_WT / VPRW;  // vectors per row, rows per pass
     pack16<T> z;
 #pragma unroll
     for (int u = 0; u < VEC; ++u) z.v[u] = from_float<T>(0.0f);
     tid = opaque(tid);
-    // thread t covers rows t/16 + 8k, vector t%16: a uniform base, one 32-bit per-lane byte offset, uniform row steps
-    static_assert(M_WT == 128 && M_TN / VEC == 16, "region rows per pass");
+    // thread t covers rows t/VPRW + RPP*k, vector t%VPRW: a uniform base, one 32-bit per-lane byte offset, uniform row steps
+    static_assert(M_WT % VPRW == 0 && M_TM % RPP == 0, "region rows per pass");
     char *base = reinterpret_cast<char *>(yp + (int64_t)p0 * W + q0);
-    const int r0 = tid >> 4, cv = (tid & 15) * VEC;
+    const int r0 = tid / VPRW, cv = (tid % VPRW) * VEC;
     const unsigned off = (unsigned)(r0 * W + cv) * (unsigned)sizeof(T);
-    const int64_t rstep = (int64_t)(M_WT / 16) * W * (int64_t)sizeof(T);
+    const int64_t rstep = (int64_t)RPP * W * (int64_t)sizeof(T);
 #pragma unroll
-    for (int k = 0; k < M_TM / (M_WT / 16); ++k) {
-        if (FULL || (p0 + r0 + k * (M_WT / 16) < H && q0 + cv < W))
+    for (int k = 0; k < M_TM / RPP; ++k) {
+        if (FULL || (p0 + r0 + k * RPP < H && q0 + cv < W))
             MTA_CONV_STORE(reinterpret_cast<u32x4 *>(base + k * rstep + off), __builtin_bit_cast(u32x4, z));
-    }
-}
-
-// The part of a square causal output above the diagonal's 128x128 blocks, written as +0 by workgroups of their own
-// (mirror == 3): row p of a plane gets keys (p / M_TN + 1) * M_TN .. W-1, a contiguous run.  Workgroup `fid` of `nfill`
-// takes rows fid, fid + nfill, ... of all planes.
-template <typename T>
-__device__ __forceinline__ void fill_above_blocks(T *y, int64_t planes, int H, int W, int fid, int nfill, int tid)
-{
-    constexpr int VEC = 8;
-    pack16<T> z;
-#pragma unroll
-    for (int u = 0; u < VEC; ++u) z.v[u] = from_float<T>(0.0f);
-    const int64_t rows = planes * H;
-    for (int64_t rr = fid; rr < rows; rr += nfill) {
-        const int p = (int)(rr % H);
-        T *row = y + rr * W;
-        for (int q = (p / M_TN + 1) * M_TN + tid * VEC; q < W; q += M_WT * VEC)
-            MTA_CONV_STORE(reinterpret_cast<u32x4 *>(row + q), __builtin_bit_cast(u32x4, z));
     }
 }
 
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef const __attribute__((address_space(1))) void glb_void_t;
 
-// The staged strips are read and written through these, not through C++ accesses: the compiler cannot tell an access
-// to one half of the double buffer from the asynchronous copy in flight into the other half and would wait for the
-// copy first (the copy would then never overlap the matrix products).  LDS operations of a wavefront complete in
-// order; lds_wait() waits for all of them and ties the loaded values to that point.
+// LDS is read and written through these, not through C++ accesses: the compiler cannot tell an access to one half of
+// the double buffer from the asynchronous copy in flight into the other half and would wait for the copy first (the copy
+// would then never overlap the matrix products).  LDS operations of a wavefront complete in order; lds_wait() waits for
+// all of them and ties the loaded values to that point.
 __device__ __forceinline__ u32x4 lds_load16(unsigned addr)
 {
     u32x4 v;
@@ -284,6 +277,12 @@ __device__ __forceinline__ u32x4 lds_load16_at(unsigned addr, int off)
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(off) : "memory");
     return v;
 }
+__device__ __forceinline__ unsigned lds_load_u16(unsigned addr)
+{
+    unsigned v;
+    asm volatile("ds_read_u16 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+}
 __device__ __forceinline__ void lds_store8_at(unsigned addr, int off, unsigned lo, unsigned hi)
 {
     typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
@@ -294,38 +293,57 @@ __device__ __forceinline__ void lds_store16(unsigned addr, u32x4 v)
 {
     asm volatile("ds_write_b128 %0, %1" : : "v"(addr), "v"(v) : "memory");
 }
-__device__ __forceinline__ void lds_store8(unsigned addr, unsigned lo, unsigned hi)
-{
-    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-    const u32x2 v = {lo, hi};
-    asm volatile("ds_write_b64 %0, %1" : : "v"(addr), "v"(v) : "memory");
-}
 __device__ __forceinline__ void lds_wait() { asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory"); }
 __device__ __forceinline__ void lds_wait(u32x4 &a) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a) : : "memory"); }
 // workgroup barrier without the memory fence __syncthreads() carries (which would wait for the copy in flight)
 __device__ __forceinline__ void wg_barrier() { asm volatile("s_barrier" : : : "memory"); }
 
-// Persistent two-wavefront workgroups: each walks a run of M_TM x 128 strips dealt round-robin within its XCD's share
-// of the item list.  Wavefront w owns row block w (16 rows) of the strip: it issues half of the staging copies, computes
-// its row block and stores it.  The wavefronts meet at one barrier per strip (the strip has landed; the previous
-// strip's buffer may be overwritten); latency is hidden by the other workgroups resident on the CU, each in its own
-// phase (loading / matrix cores / storing) with its own two 11.6 KB LDS strip buffers.
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), in order
+template <int... I, typename F> __device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F &&f)
+{
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F> __device__ __forceinline__ void static_for(F &&f)
+{
+    static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+// Persistent four-wavefront workgroups: each walks a run of M_TM x M_TN strips dealt round-robin within its XCD's share
+// of the item list.  Wavefront w owns row block w & 1 (16 rows) and key half w >> 1 (128 keys) of the strip: it issues a
+// quarter of the staging copies, computes its 16 x 128 outputs and stores them.  The wavefronts meet at one barrier per
+// strip (the strip has landed; the previous strip's buffer may be overwritten); latency is hidden by the other
+// workgroups resident on the CU, each in its own phase (loading / matrix cores / storing) with its own two 24 KB LDS
+// strip buffers.
+//
+// Item order.  Strips are taken row strip by row strip, each from the left, so that an XCD's workgroups sweep whole
+// rows of the output together, zero strips included: under the causal rule a strip wholly above the diagonal is an
+// item like the others, whose workgroup stores +0 over it (no copy, no products).  Written this way - every row of the
+// output completed within a short time, 512 contiguous bytes per row and strip - the tensor moves through memory a tenth
+// faster than with 32 x 128 strips taken block by block and the part above the diagonal filled by workgroups of their
+// own.  Odd planes are walked backwards, so that a workgroup's share alternates between the cheap strips above the
+// diagonal and the others.  MTA_CAUSAL_LOWER_ONLY on a square tensor enumerates the strips that touch the lower
+// triangle only.
 //
 // Per 16x16 output block and kernel row i:  out^T[q, p] += T_i^T[q, k] X^T[k, p+i-(R-1)], one
 // v_mfma_f32_16x16x32 whose 32-key contraction window holds the 16 outputs' taps.  A operand =
 // Toeplitz fragment (4 VGPRs per kernel row, kept while the channel is unchanged), B operand = 16 contiguous
 // bytes of one staged row per lane.  A wavefront sustains about one such 1 KB LDS operand per 35 cycles whatever the
-// addresses, against 16 cycles for the product: the products of a strip are therefore split over two wavefronts (on
-// two SIMDs).  Results go back through LDS rows that only the owning wavefront reads (row block 0: the strip's first
-// 16 staged rows; row block w > 0: the last 16 staged rows of its window) so that the global stores are whole
-// 256-byte row segments.
+// addresses, against 16 cycles for the product: the products of a strip are therefore split over four wavefronts (on
+// four SIMDs).  Results go back through LDS rows and columns that only the owning wavefront reads (row block 0: the
+// strip's first 16 staged rows; row block 1: the last 16 staged rows of its window; see mfma_geom::RES_OFF for the
+// columns) so that the global stores are whole 256-byte row segments.
 //
 // Staging.  A strip whose halo lies wholly inside the tensor and on or below the diagonal (the
 // common case, decided per workgroup) is copied global -> LDS by global_load_lds_dwordx4: no
-// registers, no masks, no LDS store instructions.  The LDS row stride is 19 16-byte slots (18 of
-// data + 1 of padding), so thread t of copy `it` simply owns slot it*128+t.  Diagonal and border strips
+// registers, no masks, no LDS store instructions.  The LDS row stride is 35 16-byte slots (34 of
+// data + 1 of padding), so thread t of copy `it` simply owns slot it*256+t.  Diagonal and border strips
 // are copied the same way and fixed up in LDS; the rare strips whose copy could leave the tensor go
 // through registers, where bounds and the causal col<=row rule are applied.
+//
+// Kernel rows.  The channel's R*S taps are copied global -> LDS the same way, one strip ahead, as the dwords that hold
+// them (from the 4-byte aligned address at or below the first tap: such a dword holds at least one tap, so it lies in
+// mapped memory); the copy is older than the strip's, so the wait for the strip covers it, and no register carries a
+// value that is still in flight.  The Toeplitz fragments are gathered from there when the channel changes.
 //
 // SCALED: every strip is staged through registers, where x*in_scale is rounded to the I/O dtype before it
 // reaches LDS (what a separate elementwise scale pass would have produced).
@@ -333,31 +351,26 @@ __device__ __forceinline__ void wg_barrier() { asm volatile("s_barrier" : : : "m
 // BWD: the gradient with respect to the input (see conv2d_valu): kernel rows reversed in both axes, the R-1 halo rows
 // below the strip instead of above it.  Key sizes are odd here, so the key halos are the same on both sides.
 template <typename T, int R, int S, bool SCALED, bool BWD>
-__global__ __launch_bounds__(M_WT, 2) void conv2d_mfma(
+__global__ __launch_bounds__(M_WT, wg_per_cu<R>()) void conv2d_mfma(
     const T *__restrict__ x, const T *__restrict__ w, T *__restrict__ y, int C, int H, int W, int causal, float in_scale,
-    int tiles_n, int ipp, int64_t total, int64_t per_xcd, int nw, int mirror, int nfill)
+    int tiles_n, int ipp, int64_t total, int64_t per_xcd, int nw, int tri)
 {
-    // mirror == 3: the image above the diagonal is written by nfill workgroups of their own, which the device runs
-    // beside the persistent ones (they hold no registers or LDS traffic to speak of)
-    if (mirror == 3 && (int)blockIdx.x >= nw * 8) {
-        fill_above_blocks<T>(y, total / ipp, H, W, (int)blockIdx.x - nw * 8, nfill, (int)threadIdx.x);
-        return;
-    }
     using G = mfma_geom<R, S>;
     static_assert(!BWD || (S % 2 == 1 && !SCALED), "the backward instance assumes symmetric key halos and no scale");
+    static_assert(sizeof(T) == 2, "16-bit data");
     constexpr int TOP = BWD ? 0 : R - 1;                    // halo rows above the strip (the others lie below it)
     constexpr int LD = G::LD, VEC = 8;
-    constexpr int VPR = G::TW / VEC;                        // data vectors per staged row (18)
-    constexpr int SPR = LD / VEC;                           // 16-byte slots per LDS row (19)
+    constexpr int VPR = G::TW / VEC;                        // data vectors per staged row (34)
+    constexpr int SPR = LD / VEC;                           // 16-byte slots per LDS row (35)
     constexpr int SLOTS = G::ROWS * SPR;
-    constexpr int STAGE_IT = (SLOTS + M_WT - 1) / M_WT;     // copies per strip and lane
+    constexpr int STAGE_IT = (SLOTS + M_WT - 1) / M_WT;     // copies per strip and lane (the last round may be partial)
     static_assert(SPR == VPR + 1, "one padding slot per row");
-    // weights of the current channel, each kernel row zero-padded on both sides so that the
-    // Toeplitz fragments can be gathered without range checks
-    constexpr int WZ_OFF = G::SHIFT + 16, WZ_LD = WZ_OFF + 32;
     constexpr int BUF = STAGE_IT * M_WT * VEC;               // elements per LDS strip buffer
     __shared__ __align__(16) T tiles[2 * BUF];               // double buffer: strip n is computed while strip n+1 lands
-    __shared__ T wz[2][R * WZ_LD];                           // by strip parity: a wavefront may run one strip ahead
+    // the channel's kernel as it lies in memory (see above), by strip parity
+    constexpr int WRAW_DW = (R * S + 2) / 2;                 // dwords that cover R*S taps starting in either half of the first
+    constexpr int WRAW_IT = (WRAW_DW + 63) / 64;
+    __shared__ __align__(16) unsigned wraw[2][WRAW_IT * 64];
     using V16 = pack16<T>;
 
     // XCD-aware split: workgroup ids are dealt round-robin to the 8 XCDs; each XCD gets one
@@ -376,11 +389,14 @@ __global__ __launch_bounds__(M_WT, 2) void conv2d_mfma(
     const int tid = threadIdx.x, lane = tid & 63, ln = lane & 15, kg = lane >> 4;
     // (the wavefront index through readfirstlane: everything derived from it is then scalar)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rb0 = (wave & 1) * 16;         // first strip row of this wavefront's row block
+    const int ch = wave >> 1;                // its key half
     frag8<T> tz[R];
     int cur_channel = -1;
+    const bool reflect = causal != 0 && !tri;  // odd planes backwards
 
     // per-thread geometry of the staging copies, fixed for the whole kernel: slot it*M_WT+tid is row srow,
-    // vector svc of the strip; padding slots and slots past the strip re-read a neighbouring valid vector
+    // vector svc of the strip; padding slots re-read a neighbouring valid vector
     unsigned goff[STAGE_IT];  // byte offsets from the strip's first staged element (uniform base + 32-bit lane offset)
 #pragma unroll
     for (int it = 0; it < STAGE_IT; ++it) {
@@ -397,137 +413,134 @@ __global__ __launch_bounds__(M_WT, 2) void conv2d_mfma(
         const int h0 = p0_ - TOP, k0 = q0_ - G::HL;
         return h0 >= 0 && h0 + G::ROWS <= H && k0 >= 0 && k0 + G::TW <= W && (!causal || k0 + G::TW - 1 <= h0);
     };
-    // A strip is `copyable` when the same copy can be issued for it without faulting: its rows lie inside the plane
-    // and the bytes its slots address (left halo of the first column strip = tail of the previous row, right halo of
-    // the last one = head of the next row) lie inside the tensor.  What such a copy brings in from outside the plane
-    // or from above the diagonal is zeroed in LDS afterwards (diagonal and border strips: a quarter of all strips,
-    // which would otherwise load synchronously through registers).
     // (a plane is named by the offset of its first element, `pbase`: kept up to date by additions, no 64-bit divisions)
-    const int64_t total_elems = (int64_t)(total / ipp) * HW;  // planes * H * W
-    auto is_copyable = [&](int64_t pbase_, int p0_, int q0_) {
-        if (SCALED) return false;
-        const int h0 = p0_ - TOP, k0 = q0_ - G::HL;
-        if (h0 < 0 || h0 + G::ROWS > H) return false;
-        const int64_t e0 = pbase_ + (int64_t)h0 * W + k0;
-        return e0 >= 0 && e0 + (int64_t)(G::ROWS - 1) * W + G::TW <= total_elems;
+    // 0: a strip to convolve, 1: wholly above the diagonal, +0 to be stored, 2: wholly above it, nothing to do
+    auto kind_of = [&](int p0_, int q0_) { return (causal && q0_ > p0_ + M_TM - 1) ? (causal == 2 ? 2 : 1) : 0; };
+    // Asynchronous copy of a strip into LDS buffer `buf` (this wavefront's quarter of the slots).  Interior strip: every
+    // slot is copied.  Any other strip: a slot is copied only if it lies inside the plane and on or below the diagonal;
+    // the others - what lies outside the plane (borders), above the diagonal (which is then not read from memory at
+    // all), and the padding slots - are written as zeros right here, while the buffer is still waiting for its data.
+    // What remains to be done once the copy has landed is the one vector of a row that straddles the diagonal.
+    auto slot_valid = [&](int slot, int h0_, int k0_) {
+        const int rr = slot / SPR, vc = slot % SPR;
+        const int h = h0_ + rr, col = k0_ + vc * VEC;
+        return rr < G::ROWS && vc < VPR && h >= 0 && h < H && col >= 0 && col < W && !(causal && col > h);
     };
-    // asynchronous copy of an interior or copyable strip into LDS buffer `buf` (this wavefront's half of the slots)
-    auto prefetch = [&](int64_t pbase_, int p0_, int q0_, T *buf) {
-        const char *base = reinterpret_cast<const char *>(x + pbase_ + (int64_t)(p0_ - TOP) * W + (q0_ - G::HL));
+    auto prefetch = [&](int64_t pbase_, int p0_, int q0_, T *buf, bool interior_) {
+        const char *base = reinterpret_cast<const char *>(x) +
+                           (pbase_ + (int64_t)(p0_ - TOP) * W + (q0_ - G::HL)) * (int64_t)sizeof(T);
+        if (interior_) {
 #pragma unroll
-        for (int it = 0; it < STAGE_IT; ++it)
-            __builtin_amdgcn_global_load_lds((glb_void_t *)(base + goff[it]),
-                                             (lds_void_t *)(buf + (it * M_WT + wave * 64) * VEC), 16, 0, 0);
+            for (int it = 0; it < STAGE_IT; ++it)
+                if ((it + 1) * M_WT <= SLOTS || it * M_WT + tid < SLOTS)
+                    __builtin_amdgcn_global_load_lds((glb_void_t *)(base + goff[it]),
+                                                     (lds_void_t *)(buf + (it * M_WT + wave * 64) * VEC), 16, 0, 0);
+        } else {
+            const int tid_ = opaque(tid);
+            const int h0_ = p0_ - TOP, k0_ = q0_ - G::HL;
+            const unsigned buf_lds = (unsigned)(uintptr_t)(lds_void_t *)buf;
+            const u32x4 zero4 = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int it = 0; it < STAGE_IT; ++it) {
+                const int slot = it * M_WT + tid_;
+                if (slot_valid(slot, h0_, k0_))
+                    __builtin_amdgcn_global_load_lds((glb_void_t *)(base + goff[it]),
+                                                     (lds_void_t *)(buf + (it * M_WT + wave * 64) * VEC), 16, 0, 0);
+                else
+                    lds_store16(buf_lds + (unsigned)slot * 16u, zero4);
+            }
+        }
     };
-
-    // The (zero-padded) kernel rows of a strip's channel are fetched one strip ahead into WPL registers per lane and
-    // written to `wz` at the top of that strip's iteration: the items of a plane are dealt out over all workgroups of
-    // an XCD, so a workgroup changes channel every few strips, and a fetch at the point of use would expose a full
-    // memory latency each time.  The loads are issued from inline assembly, before the strip's copy, and are covered
-    // by the wait for that copy at the top of the next iteration: seen by the compiler, they would make it wait for
-    // every outstanding memory operation - the previous strip's stores included - before the values' first use.
-    // (The build fails if this kernel spills registers: a spill between the load and that wait would save a value
-    // that has not arrived yet.)
-    constexpr int WPL = (R * WZ_LD + M_WT - 1) / M_WT;
-    static_assert(sizeof(T) == 2, "16-bit loads");
-    unsigned wnext[WPL];
-    unsigned woff[WPL];   // byte offset of this lane's tap inside a channel's kernel (0 where the slot is padding)
-    unsigned wvalid = 0;  // bit it: slot it*M_WT+tid of the padded kernel rows holds a tap
+    // asynchronous copy of a channel's kernel into wraw[par] (first wavefront); returns nothing: the taps start
+    // wshift(channel) 16-bit elements into the buffer
+    auto wshift = [&](int channel_) { return (int)((reinterpret_cast<uintptr_t>(w + (int64_t)channel_ * (R * S)) >> 1) & 1u); };
+    auto fetch_weights = [&](int channel_, int par) {
+        if (wave != 0) return;
+        const uintptr_t a0 = reinterpret_cast<uintptr_t>(w + (int64_t)channel_ * (R * S));
+        const char *base = reinterpret_cast<const char *>(a0 & ~(uintptr_t)3);
+        const int ndw = ((int)((a0 >> 1) & 1u) + R * S + 1) / 2;  // dwords that hold a tap (at most WRAW_DW)
 #pragma unroll
-    for (int it = 0; it < WPL; ++it) {
-        const int e = it * M_WT + tid;
-        const int i = e / WZ_LD, j = e % WZ_LD - WZ_OFF;
-        const bool ok = e < R * WZ_LD && j >= 0 && j < S;
-        woff[it] = ok ? (unsigned)(BWD ? (R - 1 - i) * S + (S - 1 - j) : i * S + j) * (unsigned)sizeof(T) : 0u;
-        wvalid |= ok ? (1u << it) : 0u;
-    }
-    auto fetch_weights = [&](int channel_) {
-        const char *wc = reinterpret_cast<const char *>(w + channel_ * R * S);
-#pragma unroll
-        for (int it = 0; it < WPL; ++it)
-            asm volatile("global_load_ushort %0, %1, %2" : "=v"(wnext[it]) : "v"(woff[it]), "s"(wc) : "memory");
+        for (int k = 0; k < WRAW_IT; ++k)
+            if (k * 64 + lane < ndw)
+                __builtin_amdgcn_global_load_lds((glb_void_t *)(base + (k * 64 + lane) * 4), (lds_void_t *)(&wraw[par][k * 64]), 4, 0, 0);
     };
-    // current and next work item: position inside the plane, plane (as element offset) and channel
+    // current and next work item: position inside the plane, plane (as element offset, and its parity) and channel
     int t_nx;
     int64_t pbase_nx;
-    int chan_nx;
+    int chan_nx, podd_nx;
     {
         const int64_t plane0 = first / ipp;
         t_nx = (int)(first - plane0 * ipp);
         pbase_nx = plane0 * HW;
         chan_nx = (int)(plane0 % C);
+        podd_nx = (int)(plane0 & 1);
     }
     int tm, tn;
-    decode_item(t_nx, tiles_n, mirror, tm, tn);
-    fetch_weights(chan_nx);
-    if (is_copyable(pbase_nx, tm * M_TM, tn * M_TN)) prefetch(pbase_nx, tm * M_TM, tn * M_TN, tiles);
+    decode_item((reflect && podd_nx) ? ipp - 1 - t_nx : t_nx, tiles_n, tri, tm, tn);
+    if (kind_of(tm * M_TM, tn * M_TN) == 0) {
+        fetch_weights(chan_nx, 0);
+        if (!SCALED) prefetch(pbase_nx, tm * M_TM, tn * M_TN, tiles, is_interior(tm * M_TM, tn * M_TN));
+    }
 
+    constexpr int ST = 16 * (M_HALF / VEC) / 64;  // stores per strip and lane (a wavefront's 16 x 128 outputs) ...
+    static_assert(ST == M_TM * (M_TN / VEC) / M_WT, "... and per zero strip");
     int younger = -1;                      // stores certainly issued after the copy in flight (-1: unknown)
-    const bool fill_full = H % M_TN == 0;  // mirror images of whole 128x128 blocks lie inside the (square) tensor
     int parity = 0;
     for (int item = 0; item < n_items; ++item, parity ^= 1) {
         T *tile = tiles + parity * BUF;
         T *other = tiles + (parity ^ 1) * BUF;
-        T *wzp = wz[parity];
         const int p0 = tm * M_TM, q0 = tn * M_TN;
-        const int ctm = tm, ctn = tn;
         const int64_t pbase = pbase_nx;
         const T *xp = x + pbase;
         T *yp = y + pbase;
         const int channel = chan_nx;
-        const bool above = causal && q0 > p0 + M_TM - 1;  // wholly above the diagonal (only reachable when !mirror)
-        const bool interior = is_interior(p0, q0);
-        const bool copyable = interior || is_copyable(pbase, p0, q0);
+        const int kind = kind_of(p0, q0);
+        const bool interior = kind == 0 && is_interior(p0, q0);
         const int h0 = p0 - TOP, k0 = q0 - G::HL;
+        // the strip's outputs all lie inside the tensor: its stores are unconditional then, and their number is known
+        const bool full_out = p0 + M_TM <= H && q0 + M_TN <= W;
         // (opaque: the addresses derived from it are then formed where they are used instead of being kept, dozens of
         // them, in registers across the loop)
         const unsigned tile_lds = (unsigned)opaque((int)(unsigned)(uintptr_t)(lds_void_t *)tile);
 
-        // This wavefront's half of the strip's copy (if any) has landed.  Vector-memory operations complete in issue
-        // order, and the only ones this wavefront issued after that copy are the previous strip's stores: when their
-        // number is known exactly (`younger`), they may stay in flight.
-        {
-            constexpr int ST = M_TM * (M_TN / VEC) / M_WT;  // stores per strip and lane, and per mirror share
-            if (younger == 2 * ST) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * ST) : "memory");
-            else if (younger == ST) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(ST) : "memory");
-            else asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
-        }
+        // This wavefront's part of the strip's copy (if any) and of its kernel rows has landed.  Vector-memory operations
+        // complete in issue order, and the only ones this wavefront issued after that copy are the previous strip's
+        // stores: when their number is known exactly (`younger`), they may stay in flight.
+        if (younger == ST) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(ST) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
         younger = 0;
 
-        // this strip's kernel rows, fetched during the previous iteration, go to LDS (every strip: see fetch_weights)
-#pragma unroll
-        for (int it = 0; it < WPL; ++it) {
-            asm volatile("" : "+v"(wnext[it]));  // (the value is defined from the wait above on)
-            const int e = it * M_WT + tid;
-            if (e < R * WZ_LD) wzp[e] = ((wvalid >> it) & 1u) ? __builtin_bit_cast(T, (unsigned short)wnext[it]) : from_float<T>(0.0f);
-        }
-
-        if (!above && copyable && !interior) {
-            // the copy has landed: zero what lies outside the plane or above the diagonal (whole vectors, except the one
-            // vector of a row that straddles the diagonal)
+        if (!SCALED && kind == 0 && !interior && causal && k0 + G::TW - 1 > h0) {
+            // the copy has landed: in the one vector of a row that straddles the diagonal, zero the keys beyond it (all
+            // reads first, one wait, then the writes)
             const int tid_ = opaque(tid);
-            const u32x4 zero4 = {0u, 0u, 0u, 0u};
+            constexpr int GRP = 3;  // slots per batch (each holds four registers between its read and its write)
 #pragma unroll
-            for (int it = 0; it < STAGE_IT; ++it) {
-                const int slot = it * M_WT + tid_;
-                const int rr = slot / SPR, vc = slot % SPR;
-                const int h = h0 + rr, col = k0 + vc * VEC;
-                const bool ok = rr < G::ROWS && vc < VPR && col >= 0 && col < W && !(causal && col > h);
-                const unsigned addr = tile_lds + (unsigned)slot * 16u;
-                if (!ok) {
-                    lds_store16(addr, zero4);
-                } else if (causal && col + VEC - 1 > h) {
-                    u32x4 raw = lds_load16(addr);
-                    lds_wait(raw);
-                    V16 v = __builtin_bit_cast(V16, raw);
+            for (int g0 = 0; g0 < STAGE_IT; g0 += GRP) {
+                u32x4 raw[GRP];
 #pragma unroll
-                    for (int u = 0; u < VEC; ++u)
-                        if (col + u > h) v.v[u] = from_float<T>(0.0f);
-                    lds_store16(addr, __builtin_bit_cast(u32x4, v));
+                for (int it = g0; it < g0 + GRP && it < STAGE_IT; ++it) {
+                    const int slot = it * M_WT + tid_;
+                    const int h = h0 + slot / SPR, col = k0 + (slot % SPR) * VEC;
+                    if (slot_valid(slot, h0, k0) && col + VEC - 1 > h) raw[it - g0] = lds_load16(tile_lds + (unsigned)slot * 16u);
+                }
+                lds_wait();
+#pragma unroll
+                for (int it = g0; it < g0 + GRP && it < STAGE_IT; ++it) {
+                    const int slot = it * M_WT + tid_;
+                    const int h = h0 + slot / SPR, col = k0 + (slot % SPR) * VEC;
+                    if (slot_valid(slot, h0, k0) && col + VEC - 1 > h) {
+                        asm volatile("" : "+v"(raw[it - g0]));  // (the value is defined from the wait above on)
+                        V16 v = __builtin_bit_cast(V16, raw[it - g0]);
+#pragma unroll
+                        for (int u = 0; u < VEC; ++u)
+                            if (col + u > h) v.v[u] = from_float<T>(0.0f);
+                        lds_store16(tile_lds + (unsigned)slot * 16u, __builtin_bit_cast(u32x4, v));
+                    }
                 }
             }
-        } else if (!above && !interior) {
-            // edge strip: through registers.  Loads are unconditional and issued back to back (an invalid
+        } else if (SCALED && kind == 0) {
+            // through registers.  Loads are unconditional and issued back to back (an invalid
             // slot re-reads a valid address); what a slot really holds is decided on the way to LDS
             V16 stage[STAGE_IT];
             const int tid_ = opaque(tid);
@@ -536,20 +549,17 @@ __global__ __launch_bounds__(M_WT, 2) void conv2d_mfma(
                 const int slot = it * M_WT + tid_;
                 const int rr = slot / SPR, vc = slot % SPR;
                 const int h = h0 + rr, col = k0 + vc * VEC;
-                const bool ok = rr < G::ROWS && vc < VPR && h >= 0 && h < H && col >= 0 && col < W && !(causal && col > h);
-                stage[it] = *reinterpret_cast<const V16 *>(xp + (ok ? (int64_t)h * W + col : 0));
+                stage[it] = *reinterpret_cast<const V16 *>(xp + (slot_valid(slot, h0, k0) ? (int64_t)h * W + col : 0));
             }
 #pragma unroll
             for (int it = 0; it < STAGE_IT; ++it) {
                 const int slot = it * M_WT + tid_;
                 const int rr = slot / SPR, vc = slot % SPR;
                 const int h = h0 + rr, col = k0 + vc * VEC;
-                const bool ok = rr < G::ROWS && vc < VPR && h >= 0 && h < H && col >= 0 && col < W && !(causal && col > h);
+                const bool ok = slot_valid(slot, h0, k0);
                 V16 v = stage[it];
-                if (SCALED) {
 #pragma unroll
-                    for (int u = 0; u < VEC; ++u) v.v[u] = from_float<T>(to_float(v.v[u]) * in_scale);
-                }
+                for (int u = 0; u < VEC; ++u) v.v[u] = from_float<T>(to_float(v.v[u]) * in_scale);
                 if (!ok) {
 #pragma unroll
                     for (int u = 0; u < VEC; ++u) v.v[u] = from_float<T>(0.0f);
@@ -564,6 +574,36 @@ __global__ __launch_bounds__(M_WT, 2) void conv2d_mfma(
         lds_wait();    // this wavefront's LDS stores above are complete
         wg_barrier();  // the strip and its kernel rows are in LDS; every wavefront is done with the previous strip
 
+        if (kind == 0 && channel != cur_channel) {  // Toeplitz fragments T_i^T for this lane's accumulator row
+            cur_channel = channel;
+            const int lane_ = opaque(lane);
+            const int ln_ = lane_ & 15, kg_ = lane_ >> 4;
+            const unsigned wa = (unsigned)(uintptr_t)(lds_void_t *)&wraw[parity][0] + 2u * (unsigned)wshift(channel);
+#pragma unroll
+            for (int i = 0; i < R; ++i) {  // row m = ln, slots k = 8*kg + t, tap j = k-SHIFT-m
+                unsigned tap[8];
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const int j = kg_ * 8 + t - G::SHIFT - ln_;
+                    const bool ok = j >= 0 && j < S;
+                    const int idx = BWD ? (R - 1 - i) * S + (S - 1 - j) : i * S + j;
+                    tap[t] = lds_load_u16(wa + 2u * (unsigned)(ok ? idx : 0));
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)"
+                             : "+v"(tap[0]), "+v"(tap[1]), "+v"(tap[2]), "+v"(tap[3]), "+v"(tap[4]), "+v"(tap[5]), "+v"(tap[6]), "+v"(tap[7])
+                             :
+                             : "memory");
+                unsigned pk[4];
+#pragma unroll
+                for (int t = 0; t < 8; t += 2) {
+                    const int j = kg_ * 8 + t - G::SHIFT - ln_;
+                    const unsigned lo = (j >= 0 && j < S) ? tap[t] : 0u, hi = (j + 1 >= 0 && j + 1 < S) ? tap[t + 1] : 0u;
+                    pk[t / 2] = lo | (hi << 16);
+                }
+                tz[i] = __builtin_bit_cast(frag8<T>, u32x4{pk[0], pk[1], pk[2], pk[3]});
+            }
+        }
+
         // put the next strip's copy in flight (into the buffer the previous iteration has just released)
         if (item + 1 < n_items) {
             t_nx += step;
@@ -571,73 +611,67 @@ __global__ __launch_bounds__(M_WT, 2) void conv2d_mfma(
                 t_nx -= ipp;
                 pbase_nx += HW;
                 chan_nx = chan_nx + 1 == C ? 0 : chan_nx + 1;
+                podd_nx ^= 1;
             }
-            decode_item(t_nx, tiles_n, mirror, tm, tn);
-            fetch_weights(chan_nx);  // (before the copy: the loop-top wait counts what is younger than the copy)
-            if (is_copyable(pbase_nx, tm * M_TM, tn * M_TN)) prefetch(pbase_nx, tm * M_TM, tn * M_TN, other);
+            decode_item((reflect && podd_nx) ? ipp - 1 - t_nx : t_nx, tiles_n, tri, tm, tn);
+            if (kind_of(tm * M_TM, tn * M_TN) == 0) {
+                fetch_weights(chan_nx, parity ^ 1);  // (before the copy: the loop-top wait counts what is younger than the copy)
+                if (!SCALED) prefetch(pbase_nx, tm * M_TM, tn * M_TN, other, is_interior(tm * M_TM, tn * M_TN));
+            }
         }
-        if (above) {
-            zero_fill_strip<T>(yp, H, W, p0, q0, tid);
-            younger = -1;
+        if (kind != 0) {
+            if (kind == 1) {
+                if (full_out) {
+                    zero_fill_strip<T, true>(yp, H, W, p0, q0, tid);
+                    younger = ST;
+                } else {
+                    zero_fill_strip<T>(yp, H, W, p0, q0, tid);
+                    younger = -1;
+                }
+            }
             continue;
         }
 
-        if (channel != cur_channel) {  // Toeplitz fragments T_i^T for this lane's accumulator row
-            cur_channel = channel;
-#pragma unroll
-            for (int i = 0; i < R; ++i) {  // row m = ln, slots k = 8*kg + t, tap j = k-SHIFT-m
-                const T *src = wzp + i * WZ_LD + WZ_OFF + kg * 8 - G::SHIFT - ln;
-#pragma unroll
-                for (int t = 0; t < 8; ++t) tz[i].v[t] = src[t];
-            }
-        }
-
-        // ---- this wavefront's row block: 8 column blocks of 16x16 outputs on 16x16x32 MFMAs (one per kernel row: the
+        // ---- this wavefront's 16 x 128 outputs: 8 column blocks of 16x16 on 16x16x32 MFMAs (one per kernel row: the
         // 32-key window holds the 16 outputs' taps).  Lane (row ln, group kg) holds keys 4*kg..4*kg+3 of each block.
-        const int rb0 = wave * 16;                                   // first strip row of the block
-        const int res0 = wave == 0 ? 0 : wave * 16 + R - 1;          // staged rows that receive the results
+        const int res0 = rb0 == 0 ? 0 : rb0 + R - 1;                 // staged rows that receive the results
+        const int qw = q0 + ch * M_HALF;                             // first key of this wavefront's outputs
         {
-            f32x4 acc[M_TN / 16];
-            const unsigned xa = tile_lds + (unsigned)((rb0 + ln) * LD + kg * 8) * sizeof(T);
-            // Column blocks in pairs.  A wavefront issues in order, so a run of LDS reads followed by a run of
-            // products leaves the matrix cores idle during the first and the LDS idle during the second; here one read
-            // of the next pair's operands is issued per product of this pair, and a product waits only for its
-            // own operand, issued 2R reads earlier (LDS operations complete in order: lgkmcnt(2R) at every
-            // step).  Source order is pinned (the scheduler would regroup reads and products).  Blocks above the
-            // diagonal are computed like the others and masked below.
-            constexpr int NPAIR = M_TN / 32, NLD = 2 * R;
-            static_assert(NLD <= 15, "lgkmcnt field");
-            u32x4 xf[2][2][R];
-            auto xoff = [&](int pr, int c2, int i) { return (int)((i * LD + (pr * 2 + c2) * 16) * sizeof(T)); };
-#pragma unroll
-            for (int i = 0; i < R; ++i)
-#pragma unroll
-                for (int c2 = 0; c2 < 2; ++c2) xf[0][c2][i] = lds_load16_at(xa, xoff(0, c2, i));
-#pragma unroll
-            for (int pr = 0; pr < NPAIR; ++pr) {
-                acc[2 * pr] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-                acc[2 * pr + 1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-                for (int i = 0; i < R; ++i)
-#pragma unroll
-                    for (int c2 = 0; c2 < 2; ++c2) {
-                        u32x4 &cur = xf[pr & 1][c2][i];
-                        if (pr + 1 < NPAIR) {
-                            xf[(pr + 1) & 1][c2][i] = lds_load16_at(xa, xoff(pr + 1, c2, i));
-                            asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(cur) : "n"(NLD) : "memory");
-                        } else {  // last pair: only this pair's later reads are newer
-                            asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(cur) : "n"(NLD - 1 - (2 * i + c2)) : "memory");
-                        }
-                        mma16(acc[2 * pr + c2], tz[i], __builtin_bit_cast(frag8<T>, cur));
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-            }
+            constexpr int NCB = M_HALF / 16;
+            f32x4 acc[NCB];
+            const unsigned xa = tile_lds + (unsigned)((rb0 + ln) * LD + ch * M_HALF + kg * 8) * sizeof(T);
+            // Column blocks in pairs, kernel row by kernel row (two independent accumulation chains).  A wavefront issues
+            // in order, so a run of LDS reads followed by a run of products leaves the matrix cores idle during the first
+            // and the LDS idle during the second: the operand of product n + NLD is read right before product n is issued,
+            // into a ring of registers, and a product waits only for its own operand (LDS operations complete in order:
+            // exactly the reads issued after it may be outstanding).  Source order is pinned (the scheduler would regroup
+            // reads and products).  Blocks above the diagonal are computed like the others and masked below.
+            constexpr int NPROD = NCB * R, NLD = 2 * R < 12 ? 2 * R : 12, NSLOT = NLD + 1;
+            static_assert(NLD <= 15 && NPROD > NLD, "lgkmcnt field; pipeline deeper than the work");
+            u32x4 ring[NSLOT];
+            // product n: column block 2*(n / 2R) + n % 2, kernel row (n % 2R) / 2
+            auto issue = [&](auto ic) __attribute__((always_inline)) {
+                constexpr int n = decltype(ic)::value;
+                constexpr int cb = 2 * (n / (2 * R)) + n % 2, i = (n % (2 * R)) / 2;
+                ring[n % NSLOT] = lds_load16_at(xa, (int)((i * LD + cb * 16) * sizeof(T)));
+            };
+            static_for<NLD>(issue);
+            static_for<NPROD>([&](auto ic) __attribute__((always_inline)) {
+                constexpr int n = decltype(ic)::value;
+                constexpr int cb = 2 * (n / (2 * R)) + n % 2, i = (n % (2 * R)) / 2;
+                if constexpr (n + NLD < NPROD) issue(std::integral_constant<int, n + NLD>{});
+                constexpr int newer = (n + NLD < NPROD ? n + NLD : NPROD - 1) - n;
+                asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(ring[n % NSLOT]) : "n"(newer) : "memory");
+                if constexpr (i == 0) acc[cb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                mma16(acc[cb], tz[i], __builtin_bit_cast(frag8<T>, ring[n % NSLOT]));
+                __builtin_amdgcn_sched_barrier(0);
+            });
             // results into the staged rows res0.. (read by this wavefront only, and no longer needed by it)
             const int prow = p0 + rb0 + ln;
-            const unsigned ra = tile_lds + (unsigned)((res0 + ln) * LD + kg * 4) * sizeof(T);
+            const unsigned ra = tile_lds + (unsigned)((res0 + ln) * LD + ch * G::RES_OFF + kg * 4) * sizeof(T);
 #pragma unroll
-            for (int cb = 0; cb < M_TN / 16; ++cb) {
-                const int q = q0 + cb * 16 + kg * 4;
+            for (int cb = 0; cb < NCB; ++cb) {
+                const int q = qw + cb * 16 + kg * 4;
                 uint32_t lo = pack2<T>(acc[cb][0], acc[cb][1]), hi = pack2<T>(acc[cb][2], acc[cb][3]);
                 if (!interior && causal && q + 3 > prow) {
                     if (q > prow) lo &= 0xffff0000u;
@@ -652,85 +686,72 @@ __global__ __launch_bounds__(M_WT, 2) void conv2d_mfma(
         // above precede these reads in the wavefront's LDS queue) ----
         {
             // (uniform row base + one 32-bit per-lane byte offset: no 64-bit address arithmetic per store)
-            char *ybase = reinterpret_cast<char *>(yp + (int64_t)(p0 + rb0) * W + q0);
+            char *ybase = reinterpret_cast<char *>(yp + (int64_t)(p0 + rb0) * W + qw);
             const int lane_o = opaque(lane);  // (row offsets formed here, not kept in registers across the loop)
             const int r_l = lane_o >> 4, cv = (lane_o & 15) * VEC;
             const unsigned yoff = (unsigned)(r_l * W + cv) * (unsigned)sizeof(T);
             const int64_t ystep = (int64_t)4 * W * (int64_t)sizeof(T);
-            constexpr int OUT_IT = 16 * (M_TN / VEC) / 64;
-            static_assert(OUT_IT == 4, "four row groups per wavefront");
+            static_assert(ST == 4, "four row groups per wavefront");
             u32x4 v[4];
-            const unsigned va = tile_lds + (unsigned)((res0 + r_l) * LD + cv) * sizeof(T);
+            const unsigned va = tile_lds + (unsigned)((res0 + r_l) * LD + ch * G::RES_OFF + cv) * sizeof(T);
 #pragma unroll
             for (int k = 0; k < 4; ++k) v[k] = lds_load16_at(va, (int)(k * 4 * LD * sizeof(T)));
             asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : : "memory");
-            if (interior) {  // unconditional: exactly OUT_IT vector-memory instructions
+            if (full_out) {  // unconditional: exactly ST vector-memory instructions
 #pragma unroll
                 for (int k = 0; k < 4; ++k) MTA_CONV_STORE(reinterpret_cast<u32x4 *>(ybase + k * ystep + yoff), v[k]);
             } else {
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const int r = k * 4 + r_l;
-                    if (p0 + rb0 + r < H && q0 + cv < W) MTA_CONV_STORE(reinterpret_cast<u32x4 *>(ybase + k * ystep + yoff), v[k]);
+                    if (p0 + rb0 + r < H && qw + cv < W) MTA_CONV_STORE(reinterpret_cast<u32x4 *>(ybase + k * ystep + yoff), v[k]);
                 }
             }
-            younger = interior ? OUT_IT : -1;
-        }
-        // (mirror == 2: the caller does not want the image written)
-        if (mirror == 1 && ctn < ctm / M_SPB) {  // this strip's share of the 128x128 block's image above the diagonal
-            if (fill_full) {
-                zero_fill_strip<T, true>(yp, H, W, q0 + (ctm % M_SPB) * M_TM, (ctm / M_SPB) * M_TN, tid);
-                if (younger > 0) younger += M_TM * (M_TN / VEC) / M_WT;
-            } else {
-                zero_fill_strip<T>(yp, H, W, q0 + (ctm % M_SPB) * M_TM, (ctm / M_SPB) * M_TN, tid);
-                younger = -1;
-            }
+            younger = full_out ? ST : -1;
         }
     }
 }
 
 inline int device_cu_count()
 {
-    static int cached[64] = {0};
+    // (atomic slots: concurrent first calls on a device both query and both store the same value, without a data race)
+    static std::atomic<int> cached[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cached[dev] == 0) {
-        int n = 0;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cached[dev] = n;
+        cached[dev].store(n, std::memory_order_relaxed);
     }
-    return cached[dev];
+    return n;
 }
 
 template <typename T, int R, int S, bool BWD>
 int launch_mfma(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t H, int64_t W, int causal,
                 float in_scale, int use_scale, hipStream_t st)
 {
-    const int tiles_m = (int)((H + M_TM - 1) / M_TM), tiles_n = (int)((W + M_TN - 1) / M_TN);
-    // mirror enumeration needs a square grid of whole 128x128 blocks' worth of strips
-    const int blocks = (int)((H + M_TN - 1) / M_TN);
-    // (MTA_CONV_INLINE_FILL=1 in the environment: the strips' own workgroups write the image, for comparisons)
-    static const bool inline_fill = [] { const char *e = getenv("MTA_CONV_INLINE_FILL"); return e && e[0] == '1'; }();
-    const int mirror = (causal && H == W) ? (causal == 2 ? 2 : ((inline_fill || W % 8 != 0 || blocks < 2) ? 1 : 3)) : 0;
-    const int64_t ipp64 = mirror ? (int64_t)blocks * (blocks + 1) / 2 * M_SPB : (int64_t)tiles_m * tiles_n;
+    const int64_t tiles_m = (H + M_TM - 1) / M_TM, tiles_n = (W + M_TN - 1) / M_TN;
+    // causal, square, and the caller wants nothing written above the diagonal: only the strips that touch the lower triangle
+    const int tri = (causal == 2 && H == W) ? 1 : 0;
+    const int64_t nbf = tiles_m / M_RPB, kl = tiles_m % M_RPB;
+    const int64_t ipp64 = tri ? (M_RPB / 2) * nbf * (nbf + 1) + kl * (nbf + 1) : tiles_m * tiles_n;
     if (ipp64 > (1 << 24)) return MTA_ERR_SHAPE;  // decode_item's float sqrt is exact well beyond this
     const int ipp = (int)ipp64;
     const int64_t total = N * C * ipp64;
     const int64_t per_xcd = (total + 7) / 8;
-    int nw = device_cu_count() * M_WG_PER_CU / 8;  // persistent workgroups per XCD
+    int nw = device_cu_count() * wg_per_cu<R>() / 8;  // persistent workgroups per XCD
     if (nw < 1) nw = 1;
     if (per_xcd < nw) nw = (int)per_xcd;
-    const int nfill = mirror == 3 ? device_cu_count() * 2 : 0;  // two more workgroups per CU fit beside the persistent four
-    dim3 grid((unsigned)(nw * 8 + nfill));
+    dim3 grid((unsigned)(nw * 8));
     if constexpr (BWD) {
         hipLaunchKernelGGL((conv2d_mfma<T, R, S, false, true>), grid, dim3(M_WT), 0, st, (const T *)x, (const T *)w, (T *)y,
-                           (int)C, (int)H, (int)W, causal, in_scale, tiles_n, ipp, total, per_xcd, nw, mirror, nfill);
+                           (int)C, (int)H, (int)W, causal, in_scale, (int)tiles_n, ipp, total, per_xcd, nw, tri);
     } else if (use_scale) {
         hipLaunchKernelGGL((conv2d_mfma<T, R, S, true, false>), grid, dim3(M_WT), 0, st, (const T *)x, (const T *)w, (T *)y,
-                           (int)C, (int)H, (int)W, causal, in_scale, tiles_n, ipp, total, per_xcd, nw, mirror, nfill);
+                           (int)C, (int)H, (int)W, causal, in_scale, (int)tiles_n, ipp, total, per_xcd, nw, tri);
     } else {
         hipLaunchKernelGGL((conv2d_mfma<T, R, S, false, false>), grid, dim3(M_WT), 0, st, (const T *)x, (const T *)w, (T *)y,
-                           (int)C, (int)H, (int)W, causal, in_scale, tiles_n, ipp, total, per_xcd, nw, mirror, nfill);
+                           (int)C, (int)H, (int)W, causal, in_scale, (int)tiles_n, ipp, total, per_xcd, nw, tri);
     }
     return launch_status();
 }
@@ -752,6 +773,7 @@ int dispatch_mfma(const void *x, const void *w, void *y, int64_t N, int64_t C, i
     MTA_CONV_CASE(6, 11)
     MTA_CONV_CASE(7, 7)
     MTA_CONV_CASE(7, 9)
+    MTA_CONV_CASE(11, 15)
 #undef MTA_CONV_CASE
     return 1;
     }

@@ -440,7 +440,7 @@ struct item_table {
 // (`O` is then the score tensor, V is unused).  Only q <= p is written when causal, plus +0 above the
 // diagonal when `fill_upper` is set.
 template <typename T, int D, int R, int SK, bool SCORES_ONLY, int NW>
-__global__ __launch_bounds__(64 * NW, SCORES_ONLY ? QK_OCC : 2) void conv_attn_fwd_mfma(const T *__restrict__ Q, const T *__restrict__ K,
+__global__ __launch_bounds__(64 * NW, SCORES_ONLY ? (R > 7 ? 2 : QK_OCC) : 2) void conv_attn_fwd_mfma(const T *__restrict__ Q, const T *__restrict__ K,
                                                              const T *__restrict__ V, const T *__restrict__ Wt,
                                                              T *__restrict__ O, float *__restrict__ Lse, int S, int causal,
                                                              float scale, int H, int nqb, int fill_upper, int64_t total_wg,
@@ -1053,6 +1053,9 @@ int dispatch_mfma(const void *q, const void *k, const void *v, const void *w, vo
         MTA_FUSED_CASE(5, 7)
         MTA_FUSED_CASE(6, 11)
         MTA_FUSED_CASE(7, 7)
+        // (the 44 registers of its Toeplitz fragments leave the scores kernel two workgroups per CU; the attention
+        // kernel, at the register limit with 6 kernel rows, has no such instance and takes the general kernel)
+        if constexpr (SCORES_ONLY) { MTA_FUSED_CASE(11, 15) }
 #undef MTA_FUSED_CASE
     }
     return 1;
@@ -1118,6 +1121,21 @@ extern "C" int mta_conv_attn_fwd(const void *q, const void *k, const void *v, co
     return mta_conv_attn_fwd_lse(q, k, v, w, o, nullptr, B, H, S, D, R, Sk, causal, scale, io_dtype, w_dtype, stream);
 }
 
+// kernel sizes with a scores-only instance (the cases of dispatch_mfma<.., true>)
+static bool scores_instance(int R, int Sk)
+{
+    return (R == 3 && Sk == 3) || (R == 5 && Sk == 5) || (R == 5 && Sk == 7) || (R == 6 && Sk == 11) || (R == 7 && Sk == 7) ||
+           (R == 11 && Sk == 15);
+}
+
+extern "C" int mta_qk_conv_supported(int64_t S, int64_t D, int R, int Sk, int io_dtype, int w_dtype)
+{
+    return (io_dtype == MTA_BF16 || io_dtype == MTA_F16) && w_dtype == io_dtype && S > 0 && S % 8 == 0 && (D == 64 || D == 128) &&
+                   scores_instance(R, Sk)
+               ? 1
+               : 0;
+}
+
 extern "C" int mta_qk_conv_fwd(const void *q, const void *k, const void *w, void *s_out, int64_t B, int64_t H, int64_t S,
                                int64_t D, int R, int Sk, int causal, float scale, int fill_upper, int io_dtype,
                                int w_dtype, void *stream)
@@ -1136,5 +1154,7 @@ extern "C" int mta_qk_conv_fwd(const void *q, const void *k, const void *w, void
         rc = D == 64 ? dispatch_mfma<io_t, 64, true>(q, k, nullptr, w, s_out, nullptr, B, H, S, R, Sk, causal, scale, fill_upper, st)
                      : dispatch_mfma<io_t, 128, true>(q, k, nullptr, w, s_out, nullptr, B, H, S, R, Sk, causal, scale, fill_upper, st);
     });
+    // (mta_qk_conv_supported must agree with the dispatch: a kernel size it names always has an instance)
+    if (rc == 1 && scores_instance(R, Sk)) return MTA_ERR_KERNEL_SIZE;
     return rc == 1 ? MTA_ERR_UNSUPPORTED : rc;
 }

@@ -96,15 +96,18 @@ def _lower_scores(a: torch.Tensor, b: torch.Tensor) -> Optional[torch.Tensor]:
 
 
 class _ProbsTimesValues(torch.autograd.Function):
-    """P V of the training route (mta_attention_triton.py:89).  Forward is the library GEMM.  Backward: dV = P^T dO is
-    one too; dP = dO V^T is only ever read on and below the diagonal when ``lower`` (the head mixing's gradient kernels
-    take it from here) and then comes from ``_lower_scores``."""
+    """P V of the training route (mta_attention_triton.py:89).  When ``lower`` (causal: the producer of P wrote nothing
+    above the diagonal, and the head mixing's gradient kernels, which take dP from here, read nothing there) all three
+    products touch the lower triangle of their (B,H,S,S) operand only: forward ``mta_causal_pv_fwd``, dV = P^T dO
+    ``mta_causal_ptx_fwd``, dP = dO V^T ``_lower_scores``.  Where those kernels do not apply (fp32, ragged lengths, other
+    head sizes) the caller has filled P and the library GEMMs run."""
 
     @staticmethod
     def forward(ctx, p, v, lower):
         ctx.save_for_backward(p, v)
         ctx.lower = lower
-        return torch.matmul(p, v)
+        out = ops.causal_pv(p, v, True) if lower else None
+        return out if out is not None else torch.matmul(p, v)
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -115,8 +118,15 @@ class _ProbsTimesValues(torch.autograd.Function):
             if dp is None:
                 dp = torch.matmul(grad_output, v.transpose(2, 3))
         if ctx.needs_input_grad[1]:
-            dv = torch.matmul(p.transpose(2, 3), grad_output)
+            dv = ops.causal_ptx(p, grad_output.contiguous(), True) if ctx.lower else None
+            if dv is None:
+                dv = torch.matmul(p.transpose(2, 3), grad_output)
         return dp, dv, None
+
+
+def _lower_products_supported(x: torch.Tensor, s_keys: int) -> bool:
+    """Whether P V, P^T X and round(a b^T) run as kernels that read / write the lower triangle only."""
+    return x.size(-2) == s_keys and ops.causal_pv_supported(x.dtype, s_keys, x.size(-1))
 
 
 class _ScaledScoresConv(torch.autograd.Function):
@@ -124,8 +134,10 @@ class _ScaledScoresConv(torch.autograd.Function):
     route's one kernel (``mta_qk_conv_fwd``, the raw scores never reach memory) where it exists; otherwise the library
     GEMM, then ``mta_conv2d_scaled_fwd``, which applies the factor (and the rounding to the score dtype that the
     reference's separate multiplication performs) on the way into the conv.  Backward: the conv's input gradient ``g``
-    goes through the two GEMMs and the factor is applied to their (B,H,S,D) results; the kernel gradient is taken
-    against the raw scores -- kept by the second forward, recomputed with one GEMM after the first, which so saves a
+    goes through the two products dQ = G K and dK = G^T Q and the factor is applied to their (B,H,S,D) results - under
+    the causal rule with ``mta_causal_pv_fwd`` and ``mta_causal_ptx_fwd``, which read the lower triangle of ``g`` only (it
+    is then not written above the diagonal either), else with the library GEMMs; the kernel gradient is taken against
+    the raw scores -- kept by the second forward, recomputed with one product after the first, which so saves a
     (B,H,S,S) activation -- and scaled afterwards.  Neither direction spends a pass over a (B,H,S,S) tensor on the
     factor."""
 
@@ -133,7 +145,7 @@ class _ScaledScoresConv(torch.autograd.Function):
     def forward(ctx, xq, xk, weight, scale, causal, mark):
         ctx.scale, ctx.causal = scale, causal
         # (the stage that follows, head mixing or mixing + softmax, never reads above the diagonal)
-        if xq.shape == xk.shape and xq.dtype != torch.float32:
+        if ops.qk_conv_supported(xq, xk, weight):
             mark("qk_conv")
             out = ops.qk_conv(xq, xk, weight, causal, scale, fill_upper=False)
             if out is not None:
@@ -150,11 +162,20 @@ class _ScaledScoresConv(torch.autograd.Function):
         xq, xk, weight, raw = ctx.saved_tensors
         dq = dk = dw = None
         if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
-            g = ops.conv2d_bwd_input(grad_output, weight, ctx.causal)
+            lower = ctx.causal and xq.shape == xk.shape and _lower_products_supported(xq, xk.size(-2))
+            g = ops.conv2d_bwd_input(grad_output, weight, ctx.causal, fill_upper=not lower)
             if ctx.needs_input_grad[0]:
-                dq = torch.matmul(g, xk) * ctx.scale
+                dq = ops.causal_pv(g, xk, True) if lower else None
+                if dq is None:
+                    assert not lower
+                    dq = torch.matmul(g, xk)
+                dq = dq * ctx.scale
             if ctx.needs_input_grad[1]:
-                dk = torch.matmul(g.transpose(2, 3), xq) * ctx.scale
+                dk = ops.causal_ptx(g, xq, True) if lower else None
+                if dk is None:
+                    assert not lower
+                    dk = torch.matmul(g.transpose(2, 3), xq)
+                dk = dk * ctx.scale
         if ctx.needs_input_grad[2]:
             if raw is None:  # (the kernel gradient reads its first argument on and below the diagonal only)
                 raw = _lower_scores(xq, xk) if ctx.causal else None
@@ -264,6 +285,7 @@ class MTAAttentionTriton(nn.Module):
         if self._stage_hook is not None:
             self._stage_hook(name)
 
+
     def forward(self, xq, xk, xv, mask, chunk_start_ids):
         assert chunk_start_ids is None, "MTAAttentionTriton does not support chunked attention"
         wants_grad = torch.is_grad_enabled() and (xq.requires_grad or xk.requires_grad or xv.requires_grad
@@ -301,9 +323,9 @@ class MTAAttentionTriton(nn.Module):
                   and ops.causal_pv_supported(xq.dtype, xq.size(-2), xv.size(-1)))
 
         # QK^T -> *1/sqrt(d) -> conv: one kernel when it exists for this dtype / size, else GEMM + conv
-        self._mark("qk_conv")
         scores = None
-        if xq.shape == xk.shape:
+        if ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight):
+            self._mark("qk_conv")
             scores = ops.qk_conv(xq, xk, self.mta_conv_triton.weight, self.causal, scale, fill_upper=False)
         if scores is None:
             self._mark("qk")
@@ -381,13 +403,16 @@ class MTAAttentionTriton(nn.Module):
         scores = Conv2dTritonFunction.apply(scores, self.mta_conv_after_sm_triton.weight, self.causal, lower, lower)
         self._mark("mix_post")
         post = self.wposm_triton
+        # the last stage's output is read by P V: in full by the library GEMM, on and below the diagonal by our kernels
+        lower_pv = (self.causal and post.causal and scores.dtype == xv.dtype
+                    and _lower_products_supported(xv, scores.size(-1)) and scores.size(-2) == scores.size(-1))
         scores = TritonLinearHeadFunction.apply(scores, post.weight, post.causal, post.output_value, post.group_size,
-                                                True, lower)
+                                                not lower_pv, lower)
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         self._mark("pv")
         # (the gradient with respect to the probabilities goes back into the head mixing's gradient kernels, through the
         # dropout's elementwise mask at most: nothing there reads above the diagonal when causal)
-        output = _ProbsTimesValues.apply(scores, xv, self.causal and post.causal)
+        output = _ProbsTimesValues.apply(scores, xv, lower_pv)
         self._mark("end")
         return output.transpose(1, 2)
 

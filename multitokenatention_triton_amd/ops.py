@@ -323,6 +323,16 @@ def qk_conv(q: torch.Tensor, k: torch.Tensor, weight: torch.Tensor, causal: bool
     return out
 
 
+def qk_conv_supported(q: torch.Tensor, k: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether ``qk_conv`` has a kernel for these tensors (a host-side question to the library: nothing is launched)."""
+    if q.dim() != 4 or q.shape != k.shape or q.dtype != k.dtype or weight.dim() != 3:
+        return False
+    if q.dtype not in _DTYPE_CODE or weight.dtype not in _DTYPE_CODE:
+        return False
+    return bool(_lib.load().mta_qk_conv_supported(q.size(2), q.size(3), weight.size(1), weight.size(2),
+                                                  _DTYPE_CODE[q.dtype], _DTYPE_CODE[weight.dtype]))
+
+
 def causal_pv(p: torch.Tensor, v: torch.Tensor, causal: bool) -> Optional[torch.Tensor]:
     """P V for P (B,H,S,S), V (B,H,S,D), reading only the lower triangle of P when causal; see mta_causal_pv_fwd.
 
@@ -339,6 +349,25 @@ def causal_pv(p: torch.Tensor, v: torch.Tensor, causal: bool) -> Optional[torch.
     if rc in (_lib.MTA_ERR_UNSUPPORTED, -7):
         return None
     _lib.check(rc, "mta_causal_pv_fwd")
+    return out
+
+
+def causal_ptx(p: torch.Tensor, x: torch.Tensor, causal: bool) -> Optional[torch.Tensor]:
+    """P^T X for P (B,H,S,S), X (B,H,S,D): out[k] = sum_p P[p,k] X[p], over p >= k only when causal (nothing of P above
+    the diagonal is read); see mta_causal_ptx_fwd.  Returns ``None`` when unsupported (the caller then uses
+    torch.matmul on a fully defined P)."""
+    p = _device_tensor(p, "P")
+    x = _device_tensor(x, "X")
+    if p.dim() != 4 or x.dim() != 4 or p.shape[:3] != x.shape[:3] or p.shape[2] != p.shape[3] or p.dtype != x.dtype:
+        return None
+    b, h, s, d = x.shape
+    out = torch.empty_like(x)
+    with torch.cuda.device(p.device):
+        rc = _lib.load().mta_causal_ptx_fwd(p.data_ptr(), x.data_ptr(), out.data_ptr(), b, h, s, d, int(bool(causal)),
+                                            _code(p, "P"), _stream(p))
+    if rc in (_lib.MTA_ERR_UNSUPPORTED, -7):
+        return None
+    _lib.check(rc, "mta_causal_ptx_fwd")
     return out
 
 

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/mta_hip.h but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes signatures out of sync with the header"
-    assert lib.mta_abi_version() == 6
+    assert lib.mta_abi_version() == 7
 
 
 def test_no_torch_symbols_in_the_library():
@@ -132,11 +132,30 @@ def test_reset_and_copy_parameters():
     mod.copy_mta_parameters(Src)
     assert torch.equal(mod.mta_conv_triton.weight, Src.mta_kernel.squeeze(1))
     assert torch.equal(mod.wposm_triton.weight, Src.wposm.weight)
+    # the other init modes (mta_attention_triton.py:150-183), each by its pattern
     for method in ("uniform", "normal", "diagonal", "const"):
-        cfg.init_method = method
-        m2 = mta.MTAAttentionTriton(4, cfg, 0.0, True)
-        m2.reset_mta_parameters()
-        assert torch.isfinite(m2.mta_conv_triton.weight).all()
+        for r, sk in ((3, 5), (6, 11), (3, 3)):
+            cfg = mta.MTAConfig(query_kernel_size=r, key_kernel_size=sk, init_method=method)
+            m2 = mta.MTAAttentionTriton(4, cfg, 0.0, True)
+            torch.manual_seed(7)
+            m2.reset_mta_parameters()
+            w, w2 = m2.mta_conv_triton.weight.detach(), m2.mta_conv_after_sm_triton.weight.detach()
+            assert w.shape == (4, r, sk) and w2.shape == (4, 3, 3)
+            assert torch.equal(m2.wpsm_triton.weight, torch.eye(4)) and torch.equal(m2.wposm_triton.weight, torch.eye(4))
+            if method == "const":
+                assert (w == 0.3).all() and (w2 == 0.3).all()
+            elif method == "diagonal":
+                # ones on the diagonal j - i = (S+1)//2 - R, which ends at the identity tap [R-1, S//2]; zero elsewhere
+                i, j = torch.meshgrid(torch.arange(r), torch.arange(sk), indexing="ij")
+                want = (j - i == (sk + 1) // 2 - r).float()
+                assert want[r - 1, sk // 2] == 1 and want.sum() == min(r, sk // 2 + 1)
+                assert torch.equal(w, want.expand(4, r, sk))
+            elif method == "uniform":
+                assert w.min() >= -1.0 and w.max() <= 1.0 and w.unique().numel() == w.numel()
+                assert abs(float(w.mean())) < 0.5 and float(w.abs().max()) > 0.5
+            else:   # "normal": std 0.3, truncated at three standard deviations
+                assert w.abs().max() <= 0.9 and w.unique().numel() == w.numel() and 0.1 < float(w.std()) < 0.5
+    cfg = mta.MTAConfig(query_kernel_size=3, key_kernel_size=5)
     cfg.init_method = "nope"
     with pytest.raises(ValueError):
         mta.MTAAttentionTriton(4, cfg, 0.0, True).reset_mta_parameters()
@@ -169,27 +188,36 @@ def test_weight_structure_is_an_opt_in():
 
 def test_forward_route_follows_grad_mode():
     """With grad enabled and parameters that require grad the module runs operator by operator (so that a graph is
-    recorded); otherwise it takes the fused route.  Neither has a CPU path, so both stop at their first kernel."""
-    mod = mta.MTAAttentionTriton(4, mta.MTAConfig(), 0.0, True)
-    x = torch.zeros(1, 4, 8, 64)
-    seen = []
-    mod._stage_hook = seen.append
-    with pytest.raises(RuntimeError, match="no CPU path"):
-        mod(x, x, x, None, None)
-    assert seen == ["qk", "conv_pre"]
-    seen.clear()
-    with torch.no_grad(), pytest.raises(RuntimeError, match="no CPU path"):
-        mod(x, x, x, None, None)
-    assert seen == ["qk_conv"]
-    seen.clear()
-    mod.requires_grad_(False)
-    with pytest.raises(RuntimeError, match="no CPU path"):
-        mod(x, x, x, None, None)
-    assert seen == ["qk_conv"]
-    seen.clear()
-    with pytest.raises(RuntimeError, match="no CPU path"):
-        mod(x.clone().requires_grad_(True), x, x, None, None)
-    assert seen == ["qk", "conv_pre"]
+    recorded); otherwise it takes the fused route.  Neither has a CPU path, so both stop at their first kernel - which is
+    announced to the stage hook only if the library has it: the one-kernel scores stage for 16-bit data, the matrix
+    product and the scaled conv for fp32 (mta_qk_conv_supported is a host-side question)."""
+    lib = _lib.load()
+    assert lib.mta_qk_conv_supported(4096, 128, 6, 11, 1, 1) == 1 and lib.mta_qk_conv_supported(4096, 128, 11, 15, 2, 2) == 1
+    assert lib.mta_qk_conv_supported(4096, 128, 6, 11, 0, 0) == 0      # fp32
+    assert lib.mta_qk_conv_supported(4096, 128, 6, 11, 1, 0) == 0      # weights of another dtype
+    assert lib.mta_qk_conv_supported(4100, 128, 6, 11, 1, 1) == 0      # rows not whole 16-byte vectors
+    assert lib.mta_qk_conv_supported(4096, 96, 6, 11, 1, 1) == 0 and lib.mta_qk_conv_supported(4096, 128, 9, 9, 1, 1) == 0
+    for dtype, first in ((torch.float32, ["qk", "conv_pre"]), (torch.bfloat16, ["qk_conv"])):
+        mod = mta.MTAAttentionTriton(4, mta.MTAConfig(), 0.0, True).to(dtype)
+        x = torch.zeros(1, 4, 8, 64, dtype=dtype)
+        seen = []
+        mod._stage_hook = seen.append
+        with pytest.raises(RuntimeError, match="no CPU path"):
+            mod(x, x, x, None, None)                  # parameters require grad: operator by operator
+        assert seen == first
+        seen.clear()
+        with torch.no_grad(), pytest.raises(RuntimeError, match="no CPU path"):
+            mod(x, x, x, None, None)                  # fused route
+        assert seen == first
+        seen.clear()
+        mod.requires_grad_(False)
+        with pytest.raises(RuntimeError, match="no CPU path"):
+            mod(x, x, x, None, None)
+        assert seen == first
+        seen.clear()
+        with pytest.raises(RuntimeError, match="no CPU path"):
+            mod(x.clone().requires_grad_(True), x, x, None, None)
+        assert seen == first
 
 
 def test_dropin_shims_resolve():

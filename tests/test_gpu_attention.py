@@ -213,6 +213,10 @@ QKC_CASES = [
     (1, 1, 2048, 128, 6, 11, True, torch.bfloat16),
     (1, 2, 1800, 64, 3, 3, True, torch.float16),
     (1, 1, 1544, 128, 5, 5, False, torch.bfloat16),
+    # 11x15, the kernel size of the reference's own benchmark script (benchmark_mta_attention.py:12-15): 112-row query blocks
+    (1, 2, 520, 64, 11, 15, True, torch.bfloat16),
+    (1, 1, 1160, 128, 11, 15, True, torch.float16),
+    (1, 1, 264, 128, 11, 15, False, torch.bfloat16),
 ]
 
 
@@ -250,7 +254,7 @@ def test_qk_conv_reports_unsupported(pkg):
     q = torch.zeros(1, 2, 64, 64, device="cuda")
     assert pkg.ops.qk_conv(q, q, torch.zeros(2, 3, 3, device="cuda"), True, 0.1) is None          # fp32
     qb = q.bfloat16()
-    assert pkg.ops.qk_conv(qb, qb, torch.zeros(2, 11, 15, device="cuda").bfloat16(), True, 0.1) is None  # no 11x15 instance
+    assert pkg.ops.qk_conv(qb, qb, torch.zeros(2, 9, 9, device="cuda").bfloat16(), True, 0.1) is None  # no 9x9 instance
 
 
 PV_CASES = [(1, 2, 256, 128, True, torch.bfloat16), (2, 3, 520, 64, True, torch.float16), (1, 2, 1000, 128, True, torch.bfloat16),
@@ -274,6 +278,29 @@ def test_causal_pv_parity(pkg, case):
     got = pkg.ops.causal_pv(p_dev, v.cuda(), causal)
     assert got is not None
     torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dtype))
+
+
+PTX_CASES = [(1, 2, 256, 128, True, torch.bfloat16), (2, 3, 520, 64, True, torch.float16), (1, 2, 1000, 128, True, torch.bfloat16),
+             (1, 1, 264, 64, False, torch.bfloat16), (1, 2, 8, 128, True, torch.float16), (1, 1, 2304, 128, True, torch.bfloat16),
+             (1, 3, 136, 64, True, torch.bfloat16), (1, 1, 392, 128, False, torch.float16)]
+
+
+@pytest.mark.parametrize("case", PTX_CASES)
+def test_causal_ptx_parity(pkg, case):
+    """out[k] = sum_{p >= k} P[p,k] X[p] (mta_causal_ptx_fwd: dV = P^T dO and dK = G^T Q of the training route) against
+    the fp32 product of the same 16-bit values, with NaN above the diagonal of P: nothing there may be read."""
+    b, h, s, d, causal, dtype = case
+    print(f"causal_ptx case={case}", flush=True)
+    g = torch.Generator().manual_seed(17)
+    p = torch.randn(b, h, s, s, generator=g).to(dtype)
+    x = torch.randn(b, h, s, d, generator=g).to(dtype)
+    pm = torch.tril(p) if causal else p
+    want = torch.matmul(pm.float().transpose(2, 3), x.float())
+    p_dev = p.masked_fill(torch.triu(torch.ones(s, s, dtype=torch.bool), 1), float("nan")).cuda() if causal else p.cuda()
+    got = pkg.ops.causal_ptx(p_dev, x.cuda(), causal)
+    assert got is not None and got.dtype == dtype and got.shape == (b, h, s, d)
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    torch.testing.assert_close(got.cpu().float(), want, rtol=2 * ulp, atol=1e-3 * float(s) ** 0.5)
 
 
 def test_mta_headline_config_small(pkg):
@@ -693,3 +720,30 @@ def test_conv_attention_lse(pkg, case):
     torch.testing.assert_close(lse.cpu(), want, **t)
     o2 = pkg.ops.conv_attn_fwd(q.cuda(), k.cuda(), v.cuda(), w.cuda(), causal, None)
     assert torch.equal(o, o2)
+
+
+@pytest.mark.parametrize("structure", ["infer", "dense"])
+def test_mta_general_route_published_shape(pkg, structure):
+    """The reference's published shape (benchmark_seq_len_results.jsonl: B1 H16 S4096 D128 fp16, 7x7 kernels before and
+    after the softmax) with all four weights non-trivial and dense 16x16 head weights - what bench.py times as the
+    general forward.  Three row slabs against the slab form of the oracle: the first rows; rows that cross an edge
+    between two 120-row query blocks of the scores kernel (17*120 = 2040), the edge between two 128-row blocks of P V
+    and the 2048-key boundary between two instances of the 16-head mix + softmax kernel; the last rows."""
+    print(f"mta general route, published shape, structure={structure}", flush=True)
+    dtype = torch.float16
+    b, h, s, d = 1, 16, 4096, 128
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=400)
+    g = torch.Generator().manual_seed(321)
+    params = [O.seeded_conv_weight(h, 7, 7, 0.05, dtype, seed=5), (torch.eye(h) + 0.1 * torch.randn(h, h, generator=g)).to(dtype),
+              O.seeded_conv_weight(h, 7, 7, 0.05, dtype, seed=6), (torch.eye(h) + 0.1 * torch.randn(h, h, generator=g)).to(dtype)]
+    mod = _mta_module(pkg, h, 7, 7, 7, 7, *params, dtype, structure=structure)
+    stages = []
+    mod._stage_hook = stages.append
+    got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
+    assert stages[0] == "qk_conv" and "qk" not in stages and stages[-2:] == ["pv", "end"]
+    assert "mix_softmax" in stages     # dense groups of 16 heads: mix + softmax on the matrix cores, one pass
+    assert torch.isfinite(got.float()).all()
+    for r0, r1 in [(0, 64), (2008, 2072), (4032, 4096)]:
+        print(f"  slab {r0}:{r1}", flush=True)
+        want = O.mta_forward_rows(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3], r0, r1)
+        torch.testing.assert_close(got[:, r0:r1].float(), want.float(), **tol(dtype))

@@ -9,6 +9,11 @@ Tolerances.  fp32: rtol 1e-4, atol 1e-5 times the largest expected magnitude (we
 up to 10^6 products, so the absolute floor scales with them).  bf16/fp16: inputs and the input gradient are
 stored in 16 bits: 2e-2 times the largest expected magnitude; weight gradients are accumulated and returned
 in fp32 from 16-bit inputs that the oracle sees as the same 16-bit values, so they keep rtol 1e-3.
+Softmax gradients of 16-bit data are small numbers (|dx| <= p |dp - sum|, p of the order 1 / row length), which an
+absolute bar never reaches: they are compared element by element with the value the same rounded probabilities give
+(`_softmax_grad_close`).  Module gradients in 16 bits also meet a bar on the relative error norm per tensor
+(`_rel_norm`): what the oracle's own pipeline run in that dtype on the CPU deviates from its fp32 run is 0.5-0.8 %
+(bf16) and 0.06-0.09 % (fp16); the bars are 2 % and 0.4 %.
 """
 import pytest
 import torch
@@ -33,6 +38,38 @@ def _close(got, want, dtype, what, weight_grad=False):
         torch.testing.assert_close(got, want, rtol=1e-3, atol=1e-3 * scale, msg=lambda m: f"{what}: {m}")
     else:
         torch.testing.assert_close(got, want, rtol=0.0, atol=2e-2 * scale, msg=lambda m: f"{what}: {m}")
+
+
+def _rel_norm(got, want, dtype, what):
+    """||got - want|| / ||want|| per tensor: a bar that an all-zero or a half-wrong result cannot pass."""
+    got, want = got.detach().cpu().float(), want.detach().cpu().float()
+    bar = {torch.float32: 1e-4, torch.bfloat16: 2e-2, torch.float16: 4e-3}[dtype]
+    rel = float((got - want).norm() / want.norm().clamp_min(1e-30))
+    assert rel < bar, f"{what}: relative error norm {rel:.3e} >= {bar:.0e}"
+
+
+def _softmax_grad_close(got, p16, dp, up, dtype, what):
+    """dx = p (dp - sum_k p dp) from the probabilities as the kernel sees them (rounded to the score dtype).  The kernel
+    works in fp32 and rounds once: |got - want| <= one unit in the last place of want (2^-8 / 2^-11 relative) + p times
+    the fp32 summation error of the bracket + half a subnormal step of the format."""
+    p = p16.detach().cpu().float()
+    g = dp.detach().cpu().float()
+    if up is not None:
+        p, g = p.masked_fill(up, 0.0), g.masked_fill(up, 0.0)
+    dot = (p * g).sum(-1, keepdim=True)
+    absdot = (p * g.abs()).sum(-1, keepdim=True)
+    want = p * (g - dot)
+    got = got.detach().cpu().float()
+    if dtype == torch.float32:
+        bound = 1e-4 * want.abs() + p * 1e-5 * (g.abs() + absdot) + 1e-30
+    else:
+        ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+        tiny = 0.0 if dtype == torch.bfloat16 else 2.0 ** -24
+        bound = ulp * want.abs() + p * 1e-5 * (g.abs() + absdot) + tiny + 1e-30
+    bad = (got - want).abs() > bound
+    assert not bad.any(), (f"{what}: {int(bad.sum())} of {bad.numel()} entries off; worst "
+                           f"{float(((got - want).abs() - bound).max()):.3e} beyond its bound")
+    assert float(got.abs().sum()) >= 0.5 * float(want.abs().sum())   # (not an all-zero result)
 
 
 def _rand(shape, seed, dtype):
@@ -186,6 +223,7 @@ def test_softmax_backward_parity(pkg, case, dtype):
     got = pkg.ops.softmax_bwd(p_dev, dp_dev, causal)
     assert got.dtype == dtype and got.shape == x.shape
     _close(got, want, dtype, "dx")
+    _softmax_grad_close(got, probs.detach().to(dtype), dp, up if causal else None, dtype, "dx from the rounded p")
     if causal:
         g = got.cpu()
         assert (g[..., up] == 0).all() and not torch.signbit(g[..., up]).any()
@@ -227,6 +265,8 @@ def test_headmix_and_softmax_backward_full_size(pkg):
         got = pkg.ops.softmax_bwd(p_dev, dyd[b:b + 1, ch:ch + 1].contiguous(), True)[0, 0].cpu()
         for rows in (slice(0, 64), slice(s - 96, s)):
             _close(got[rows], logits.grad[rows], dtype, f"softmax dx plane {(b, ch)} rows {rows}")
+            _softmax_grad_close(got[rows], probs.detach().to(dtype)[rows], dyd[b, ch].cpu()[rows], up[rows], dtype,
+                                f"softmax dx from the rounded p, plane {(b, ch)} rows {rows}")
 
 
 def test_operator_functions_backward(pkg):
@@ -262,7 +302,7 @@ def test_operator_functions_backward(pkg):
         _close(lin.weight.grad, want_dw, torch.float32, "headmix dw")
 
 
-def _mta_pair(pkg, h, r1, s1, dtype, seed):
+def _mta_pair(pkg, h, r1, s1, dtype, seed, causal=True):
     g = torch.Generator().manual_seed(seed)
     params = [O.seeded_conv_weight(h, r1, s1, 0.1, torch.float32, seed=seed + 1),
               torch.eye(h) + 0.1 * torch.randn(h, h, generator=g),
@@ -270,7 +310,7 @@ def _mta_pair(pkg, h, r1, s1, dtype, seed):
               torch.eye(h) + 0.1 * torch.randn(h, h, generator=g)]
     params = [p.to(dtype) for p in params]
     cfg = pkg.MTAConfig(query_kernel_size=r1, key_kernel_size=s1)
-    mod = pkg.MTAAttentionTriton(h, cfg, dropout=0.0, causal=True)
+    mod = pkg.MTAAttentionTriton(h, cfg, dropout=0.0, causal=causal)
     with torch.no_grad():
         for dst, src in zip((mod.mta_conv_triton, mod.wpsm_triton, mod.mta_conv_after_sm_triton, mod.wposm_triton), params):
             dst.weight.copy_(src)
@@ -302,14 +342,15 @@ def test_mta_module_backward(pkg, dtype):
     for name, gt, wt in (("xq", qd.grad, leaves[0].grad), ("xk", kd.grad, leaves[1].grad), ("xv", vd.grad, leaves[2].grad)):
         assert gt is not None and gt.dtype == dtype
         _close(gt, wt, dtype, f"grad {name}")
+        _rel_norm(gt, wt, dtype, f"grad {name}")
     for name, p_, wt in (("pre conv", mod.mta_conv_triton.weight, wl[0].grad), ("wpsm", mod.wpsm_triton.weight, wl[1].grad),
                          ("post conv", mod.mta_conv_after_sm_triton.weight, wl[2].grad),
                          ("wposm", mod.wposm_triton.weight, wl[3].grad)):
         assert p_.grad is not None and p_.grad.dtype == dtype
-        if dtype == torch.float32:
-            _close(p_.grad, wt, dtype, f"grad {name}")
-        else:   # intermediate score tensors are stored in bf16 along the way: 16-bit tolerance on the sums
-            _close(p_.grad, wt, dtype, f"grad {name}")
+        # (intermediate score tensors are stored in 16 bits along the way: the element bar is the 16-bit one, on sums
+        # of magnitude ~100; the norm bar is what pins them)
+        _close(p_.grad, wt, dtype, f"grad {name}")
+        _rel_norm(p_.grad, wt, dtype, f"grad {name}")
 
 
 @pytest.mark.parametrize("shape", [(1, 8, 100, 32, 6, 11), (2, 4, 264, 128, 7, 7), (1, 32, 136, 64, 3, 5)])
@@ -333,10 +374,12 @@ def test_mta_module_backward_other_shapes(pkg, shape, dtype):
     got.backward(go.cuda())
     for name, gt, wt in (("xq", qd.grad, leaves[0].grad), ("xk", kd.grad, leaves[1].grad), ("xv", vd.grad, leaves[2].grad)):
         _close(gt, wt, dtype, f"grad {name}")
+        _rel_norm(gt, wt, dtype, f"grad {name}")
     for name, p_, wt in (("pre conv", mod.mta_conv_triton.weight, wl[0].grad), ("wpsm", mod.wpsm_triton.weight, wl[1].grad),
                          ("post conv", mod.mta_conv_after_sm_triton.weight, wl[2].grad),
                          ("wposm", mod.wposm_triton.weight, wl[3].grad)):
         _close(p_.grad, wt, dtype, f"grad {name}")
+        _rel_norm(p_.grad, wt, dtype, f"grad {name}")
 
 
 def test_mta_module_backward_reference_bar(pkg):
@@ -384,3 +427,156 @@ def test_mta_module_backward_with_mask(pkg):
     _close(vd.grad, leaves[2].grad, dtype, "grad xv")
     _close(mod.mta_conv_triton.weight.grad, wl[0].grad, dtype, "grad pre conv")
     _close(mod.wposm_triton.weight.grad, wl[3].grad, dtype, "grad wposm")
+
+
+# ------------------------------------------------------------------------------------------------------
+# the pieces that exist only on the 16-bit training route, and that route at the sizes the benchmark times
+# ------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_lower_scores_is_the_rounded_product(pkg, d, dtype):
+    """_lower_scores(a, b) = round(a b^T) on and below the diagonal (the scores kernel with factor 1 and the pass-through
+    tap as 3x3 kernel; the training route's dP = dO V^T and its recomputed raw scores).  (1) Operands of small integers:
+    every partial sum and the result are exact in fp32 and in the 16-bit type, so the result is the product bit for bit
+    whatever the order of summation - a conv stage that did anything but copy would show.  (2) N(0,1) operands: within
+    one unit in the last place of the fp64 product (fp32 accumulation in another order, then one rounding; 1e-4 absolute
+    for entries that cancel to almost nothing), and equal to it on all but a few entries.  (3) The same call into a buffer that holds NaN: the lower triangle is unchanged."""
+    from multitokenatention_triton_amd.mta_attention_triton import _lower_scores
+    print(f"_lower_scores d={d} {dtype}", flush=True)
+    b, h, s = 1, 3, 520
+    g = torch.Generator().manual_seed(11)
+    low = torch.tril(torch.ones(s, s, dtype=torch.bool))
+    a = torch.randint(-1, 2, (b, h, s, d), generator=g).to(dtype)
+    c = torch.randint(-1, 2, (b, h, s, d), generator=g).to(dtype)
+    got = _lower_scores(a.cuda(), c.cuda())
+    assert got is not None and got.dtype == dtype and got.shape == (b, h, s, s)
+    want = torch.matmul(a.float(), c.float().transpose(2, 3)).to(dtype)
+    assert torch.equal(got.cpu()[..., low], want[..., low])
+
+    a, c = _rand((b, h, s, d), 12, dtype), _rand((b, h, s, d), 13, dtype)
+    got = _lower_scores(a.cuda(), c.cuda()).cpu()
+    exact = torch.matmul(a.double(), c.double().transpose(2, 3))
+    want = exact.to(dtype)
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    diff = (got.double() - want.double()).abs()[..., low]
+    assert (diff <= ulp * exact.abs()[..., low] + 1e-4).all()   # (+ the fp32 accumulation error of up to 128 terms)
+    assert float((diff == 0).double().mean()) > 0.99
+
+    w = torch.zeros(h, 3, 3, dtype=dtype)
+    w[:, 2, 1] = 1.0
+    buf = torch.full((b, h, s, s), float("nan"), dtype=dtype, device="cuda")
+    out = pkg.ops.qk_conv(a.cuda(), c.cuda(), w.cuda(), True, 1.0, fill_upper=False, out=buf)
+    assert out is buf and torch.equal(buf.cpu()[..., low], got[..., low])
+
+
+def _oracle_grads(q, k, v, params, go, mask=None):
+    leaves = [t.detach().clone().float().requires_grad_(True) for t in (q, k, v)]
+    wl = [p.detach().clone().float().requires_grad_(True) for p in params]
+    out = O.mta_forward(*leaves, wl[0].unsqueeze(1), wl[1], wl[2].unsqueeze(1), wl[3], mask=mask)
+    out.backward(go.float())
+    return out.detach(), [t.grad for t in leaves], [t.grad for t in wl]
+
+
+def _module_grads(mod, q, k, v, go, mask=None):
+    qd, kd, vd = [t.detach().clone().cuda().requires_grad_(True) for t in (q, k, v)]
+    for p_ in mod.parameters():
+        p_.grad = None
+    got = mod(qd, kd, vd, None if mask is None else mask.cuda(), None)
+    got.backward(go.cuda())
+    ws = (mod.mta_conv_triton.weight, mod.wpsm_triton.weight, mod.mta_conv_after_sm_triton.weight, mod.wposm_triton.weight)
+    return got.detach(), [qd.grad, kd.grad, vd.grad], [w.grad for w in ws]
+
+
+_GRAD_NAMES = ("xq", "xk", "xv", "pre conv", "wpsm", "post conv", "wposm")
+
+
+def _check_all(dtype, out, want_out, grads, want_grads):
+    _close(out, want_out, dtype, "forward")
+    _rel_norm(out, want_out, dtype, "forward")
+    for name, gt, wt in zip(_GRAD_NAMES, grads, want_grads):
+        assert gt is not None and gt.dtype == dtype, name
+        _close(gt, wt, dtype, f"grad {name}")
+        _rel_norm(gt, wt, dtype, f"grad {name}")
+
+
+@pytest.mark.parametrize("shape", [(1, 4, 2048, 128, 6, 11, torch.bfloat16), (1, 16, 1024, 128, 7, 7, torch.float16)])
+def test_mta_module_backward_long_sequence(pkg, shape):
+    """The training route at sequence lengths where its kernels run as they do at the benchmark shape: several work
+    items per query block and a split key range in the scores kernel (forward, dP and the recomputed raw scores), rows of
+    several passes in the softmax and its gradient, long key segments in the two weight-gradient kernels, dense 4 / 16
+    head weights.  All seven gradients against autograd through the fp32 oracle on the same 16-bit values."""
+    b, h, s, d, r1, s1, dtype = shape
+    print(f"mta module backward long shape={shape}", flush=True)
+    mod, params = _mta_pair(pkg, h, r1, s1, dtype, seed=331)
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=332)
+    go = _rand((b, s, h, d), 333, dtype)
+    want_out, want_in, want_w = _oracle_grads(q, k, v, params, go)
+    stages = []
+    mod._stage_hook = stages.append
+    out, gin, gw = _module_grads(mod, q, k, v, go)
+    assert stages[0] == "qk_conv" and "qk" not in stages
+    _check_all(dtype, out, want_out, gin + gw, want_in + want_w)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_mta_module_backward_non_causal(pkg, dtype):
+    """MTAAttentionTriton(causal=False) in training: every stage and every gradient kernel in its unmasked form, chained;
+    against autograd through the oracle with an all-visible mask."""
+    print(f"mta module backward causal=False {dtype}", flush=True)
+    b, h, s, d = 2, 4, 136, 64
+    mod, params = _mta_pair(pkg, h, 3, 5, dtype, seed=341, causal=False)
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=342)
+    go = _rand((b, s, h, d), 343, dtype)
+    want_out, want_in, want_w = _oracle_grads(q, k, v, params, go, mask=torch.zeros(1, 1, s, s))
+    out, gin, gw = _module_grads(mod, q, k, v, go)
+    _check_all(dtype, out, want_out, gin + gw, want_in + want_w)
+
+
+def test_mta_module_backward_key_mask_16bit(pkg):
+    """use_mask=True with a key mask, bf16, in training (the mask tensor route through the operator Functions)."""
+    print("mta module backward use_mask bf16", flush=True)
+    dtype = torch.bfloat16
+    b, h, s, d = 1, 4, 136, 64
+    mod, params = _mta_pair(pkg, h, 3, 5, dtype, seed=351)
+    mod.use_mask = True
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=352)
+    keep = torch.ones(1, s, dtype=torch.bool)
+    keep[0, 5:9] = False
+    keep[0, 70] = False
+    go = _rand((b, s, h, d), 353, dtype)
+    want_out, want_in, want_w = _oracle_grads(q, k, v, params, go, mask=keep)
+    out, gin, gw = _module_grads(mod, q, k, v, go, mask=keep)
+    _check_all(dtype, out, want_out, gin + gw, want_in + want_w)
+
+
+def test_mta_module_backward_with_dropout(pkg, monkeypatch):
+    """Training mode with dropout 0.5 under a fixed seed.  The gradient with respect to the probabilities comes from the
+    scores kernel, which writes nothing above the diagonal; the dropout's backward multiplies that buffer elementwise
+    before the head mixing's gradient kernels read its lower triangle.  The result must be finite and agree with a run
+    in which that gradient comes from the library GEMM (fully defined) - also when the memory the buffer is allocated
+    from holds NaN."""
+    import multitokenatention_triton_amd.mta_attention_triton as glue
+    print("mta module backward dropout", flush=True)
+    dtype = torch.bfloat16
+    b, h, s, d = 1, 8, 264, 64
+    mod, params = _mta_pair(pkg, h, 3, 3, dtype, seed=361)
+    mod.dropout = 0.5
+    mod.train()
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=362)
+    go = _rand((b, s, h, d), 363, dtype)
+
+    def run():
+        torch.manual_seed(99)
+        junk = [torch.full((b, h, s, s), float("nan"), dtype=dtype, device="cuda") for _ in range(4)]
+        del junk   # the allocator hands these blocks to the next (B,H,S,S) tensors
+        return _module_grads(mod, q, k, v, go)
+
+    out1, gin1, gw1 = run()
+    for t in [out1] + gin1 + gw1:
+        assert torch.isfinite(t.float()).all()
+    assert float((out1 == 0).float().mean()) < 0.5   # (dropout acts on the probabilities, not on the output)
+    monkeypatch.setattr(glue, "_lower_scores", lambda a, c: None)
+    out2, gin2, gw2 = run()
+    assert torch.equal(out1, out2)                   # same seed, same dropout mask
+    for name, a_, c_ in zip(_GRAD_NAMES, gin1 + gw1, gin2 + gw2):
+        _rel_norm(a_, c_.float(), dtype, f"grad {name}, kernel against GEMM for dP")

@@ -45,6 +45,8 @@ CONV_CASES = [
     # widths divisible by 8: 16-bit inputs take the MFMA (Toeplitz) kernel
     (1, 2, 136, 6, 11), (2, 2, 520, 6, 11), (1, 1, 128, 7, 9), (1, 2, 264, 5, 7), (1, 1, 1032, 3, 3),
     (1, 3, 8, 6, 11), (1, 1, 392, 7, 7), (1, 2, 200, 5, 5),
+    # several 256-key strips per row strip, ragged last one; 11x15 on the matrix cores
+    (1, 2, 776, 6, 11), (1, 1, 128, 11, 15), (1, 2, 520, 11, 15), (3, 1, 264, 6, 11),
 ]
 
 
@@ -97,19 +99,22 @@ def test_conv_delta_is_shift(ops):
         assert torch.equal(got, O.depthwise_conv(x, w, True))
 
 
-MFMA_KERNEL_SIZES = [(3, 3), (3, 5), (5, 5), (5, 7), (6, 11), (7, 7), (7, 9)]
+MFMA_KERNEL_SIZES = [(3, 3), (3, 5), (5, 5), (5, 7), (6, 11), (7, 7), (7, 9), (11, 15)]
 
 
+@pytest.mark.parametrize("plane", [(32, 128), (32, 256), (64, 512)])
 @pytest.mark.parametrize("rs", MFMA_KERNEL_SIZES)
-def test_conv_channel_changes_on_every_strip(ops, rs):
+def test_conv_channel_changes_on_every_strip(ops, rs, plane):
     """Every kernel size with a matrix-core instance, forward and input gradient, on planes that hold a single strip
-    (32 rows x 128 keys) each: consecutive work items of a workgroup then always belong to different channels, so the
-    kernel rows fetched one strip ahead are consumed on every iteration.  Channels get very different weights so that
-    a kernel row applied to the wrong strip cannot pass."""
+    (32 rows x 256 keys; half a strip; four strips) each: consecutive work items of a workgroup then belong to different
+    channels all the time, so the kernel rows fetched one strip ahead are consumed on every iteration, with odd tap counts
+    (3x3, 5x5, ... : every other channel's kernel starts in the middle of a 32-bit word).  Channels get very different
+    weights so that a kernel row applied to the wrong strip cannot pass."""
     r, s = rs
-    print(f"conv channel change rs={rs}", flush=True)
+    print(f"conv channel change rs={rs} plane={plane}", flush=True)
     dtype = torch.bfloat16
-    n, c, h, wd = 3, 24, 32, 128
+    n, c = 3, 24
+    h, wd = plane
     x = _randn((n, c, h, wd), 31, dtype)
     w = (_randn((c, r, s), 32, torch.float32, 0.2) * (1.0 + torch.arange(c)[:, None, None])).to(dtype)
     for causal in (False, True):

@@ -12,12 +12,10 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 GROUPS = [
-    # the conv's own workgroups write the +0 above the diagonal; vector-ALU head mixing for 16 and 32 heads; the
-    # general softmax and fused kernels for 16-bit data
-    ({"MTA_CONV_INLINE_FILL": "1", "MTA_HEADMIX_NO_MFMA": "1", "MTA_SOFTMAX_NO_PACKED": "1", "MTA_FUSED_FORCE_GENERAL": "1"},
+    # vector-ALU head mixing for 16 and 32 heads; the general softmax and fused kernels for 16-bit data
+    ({"MTA_HEADMIX_NO_MFMA": "1", "MTA_SOFTMAX_NO_PACKED": "1", "MTA_FUSED_FORCE_GENERAL": "1"},
      ["tests/test_gpu_ops.py", "tests/test_gpu_attention.py"],
-     "test_conv_parity or test_conv_identity_tap or test_conv_tril or test_headmix_parity or test_mix_softmax_mix_parity "
-     "or test_conv_attention_parity or test_mta_general"),
+     "test_headmix_parity or test_mix_softmax_mix_parity or test_conv_attention_parity or test_mta_general"),
     # fp32-FMA conv kernels (forward, input gradient, weight gradient) for 16-bit data
     ({"MTA_CONV_FORCE_VALU": "1"},
      ["tests/test_gpu_ops.py", "tests/test_gpu_backward.py"],
