@@ -9,9 +9,10 @@ configuration the headline metric is quoted on: B=2, H=16, S=4096, D=128, bf16, 
 identity 3x3 post-softmax conv, post-softmax head mixing in groups of 4 (I + N(0,0.1)).
 Inputs are synthetic, seeded, and resident in HBM before the timed region.  Prints ONE
 JSON line.  `value` is the latency of one forward in ms.  Defaults: 60 warm-up steps, 100
-timed ones - the first forty or so forwards after the device has been idle run up to 20 %
-slower than the ones that follow (0.62-0.68 ms against 0.565 ms), so fewer warm-up steps
-time the run-up, not the forward.
+timed ones.  The first forty or so forwards after the device has been idle run up to 20 %
+slower than the ones that follow (0.62-0.68 ms against 0.565 ms): every timed loop here is
+therefore preceded by 80 ms of the same work (`ramp`), then by the W warm-up steps, then by
+exactly K timed steps.
 
 The `roofline` object is for the slowest hand-written kernel of the step; its duration
 is measured live with events recorded on the stream the kernels run on.  `kernels` adds
@@ -143,7 +144,24 @@ def build_general(torch, mta, O, device, b=1, h=16, s=4096, d=128, nsets=2, trai
     return mod, sets
 
 
+RAMP_MS = 80.0
+
+
+def ramp(torch, fn, nsets, min_ms=RAMP_MS):
+    """Keep the device busy with the work that is about to be timed for `min_ms` of wall time.  After an idle spell
+    (the host preparing inputs takes seconds) the first 25 ms or so of kernels run up to 20 % slower than what follows;
+    the W warm-up steps of the contract come after this and are too few to cover it when W is small."""
+    t0 = time.perf_counter()
+    i = 0
+    while (time.perf_counter() - t0) * 1e3 < min_ms:
+        for _ in range(10):
+            fn(i % nsets)
+            i += 1
+        torch.cuda.synchronize()
+
+
 def time_steps(torch, fn, nsets, warmup, steps):
+    ramp(torch, fn, nsets)
     for i in range(warmup):
         fn(i % nsets)
     torch.cuda.synchronize()
@@ -158,6 +176,7 @@ def time_launches(torch, fn, nsets, warmup, steps):
     """Average duration of one launch of a single-kernel operator: an event pair around every launch, on the stream
     the kernel is launched on (what `rocprofv3 --kernel-trace` reports per dispatch, plus the event overhead; the
     wall clock over a loop of launches also counts the gaps between them)."""
+    ramp(torch, fn, nsets)
     for i in range(warmup):
         fn(i % nsets)
     torch.cuda.synchronize()

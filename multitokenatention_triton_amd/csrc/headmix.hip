@@ -225,6 +225,105 @@ __global__ __launch_bounds__(64 * DM_WAVES, 4) void headmix_dense32(const T *__r
     }
 }
 
+// Dense mixing of HG = 64 or 128 heads on the matrix cores: the same scheme with the contraction run over HG/32 blocks
+// of 32 input heads, one after the other.  A wavefront again owns 128 keys of one (batch, query row) and four blocks of
+// 16 output heads (32 accumulators of 4 registers: what fits); with 128 heads two wavefronts share a key chunk, one per
+// half of the output heads, and each reads all 128 input rows (the second read hits the cache).  The weight fragments of
+// an input block are fetched ahead of its eight input vectors, straight from memory (the matrix is at most 32 KB and
+// stays in cache).
+template <typename T, int HG>
+__global__ __launch_bounds__(64 * DM_WAVES, 2) void headmix_dense_wide(const T *__restrict__ x, const T *__restrict__ w,
+                                                                  T *__restrict__ y, int C, int P, int Q, int causal,
+                                                                  float fill, int wt, int qchunks)
+{
+    static_assert(HG == 64 || HG == 128, "blocks of 32 input heads, four blocks of 16 output heads per wavefront");
+    constexpr int IB = HG / 32;               // blocks of 32 input heads
+    constexpr int OW = 4;                     // blocks of 16 output heads per wavefront
+    constexpr int SPLIT = HG / (16 * OW);     // wavefronts that share a key chunk (1 or 2)
+    constexpr int CHUNKS = DM_WAVES / SPLIT;  // key chunks per workgroup
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, ln = lane & 15, kg = lane >> 4;
+    const int groups = C / HG;
+    unsigned b = blockIdx.x;
+    const int qc = rotated_chunk(b, qchunks);
+    const int p = (int)(b % (unsigned)P); b /= (unsigned)P;
+    const int g = (int)(b % (unsigned)groups);
+    const int64_t n = b / (unsigned)groups;
+    const int q0 = (qc * CHUNKS + wave / SPLIT) * DM_KEYS;
+    const int ob0 = (wave % SPLIT) * OW;      // first block of output heads of this wavefront
+    if (q0 >= Q) return;
+    const int64_t plane = (int64_t)P * Q;
+    const int64_t base = (n * C + (int64_t)g * HG) * plane + (int64_t)p * Q;  // head g*HG, row p, key 0
+    const int last = causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;              // last key that is mixed
+    const uint32_t fill2 = pack2<T>(fill, fill);
+    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+    const int key = q0 + ln * 8;
+
+    if (q0 > last) {  // wholly beyond the diagonal: fill only (causal == 2: not even that)
+        const u4 fv = {fill2, fill2, fill2, fill2};
+        if (key < Q && causal != 2) {
+#pragma unroll
+            for (int t = 0; t < 16; ++t)  // this lane's share of the wavefront's 64 output heads: 16kg .. 16kg+15
+                __builtin_nontemporal_store(fv, reinterpret_cast<u4 *>(y + base + (int64_t)(ob0 * 16 + kg * 16 + t) * plane + key));
+        }
+        return;
+    }
+
+    f32x4 acc[8][OW];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int ob = 0; ob < OW; ++ob) acc[j][ob] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    const T *xp = x + base + (int64_t)(kg * 8) * plane + (key <= last ? key : 0);
+#pragma unroll 1
+    for (int ib = 0; ib < IB; ++ib) {
+        // w fragments of this input block: lane (output head ln of block ob, group kg) holds w[o][32ib + 8kg .. + 7]
+        frag8<T> wf[OW];
+#pragma unroll
+        for (int ob = 0; ob < OW; ++ob) {
+            const int o = g * HG + (ob0 + ob) * 16 + ln, i0 = g * HG + ib * 32 + kg * 8;
+            if (!wt) {
+                wf[ob] = *reinterpret_cast<const frag8<T> *>(w + (int64_t)o * C + i0);
+            } else {  // the transposed matrix: a column of w, gathered element by element
+#pragma unroll
+                for (int t = 0; t < 8; ++t) wf[ob].v[t] = w[(int64_t)(i0 + t) * C + o];
+            }
+        }
+        u4 xv[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+            xv[t] = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(xp + (int64_t)(ib * 32 + t) * plane));
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            u4 xt;  // heads 32ib + 8kg .. + 7 of key 8ln + j
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                xt[u] = __builtin_amdgcn_perm(xv[2 * u + 1][j >> 1], xv[2 * u][j >> 1], (j & 1) ? 0x07060302u : 0x05040100u);
+            const frag8<T> xf = __builtin_bit_cast(frag8<T>, xt);
+#pragma unroll
+            for (int ob = 0; ob < OW; ++ob) mma16(acc[j][ob], wf[ob], xf);
+        }
+    }
+    if (key >= Q || (causal == 2 && key > last)) return;
+    // acc[j][ob][v]: output head 16(ob0 + ob) + 4kg + v, key 8ln + j
+#pragma unroll
+    for (int ob = 0; ob < OW; ++ob) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            u4 o;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) o[u] = pack2<T>(acc[2 * u][ob][v], acc[2 * u + 1][ob][v]);
+            if (key + 7 > last) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (key + 2 * u > last) o[u] = (o[u] & 0xffff0000u) | (fill2 & 0x0000ffffu);
+                    if (key + 2 * u + 1 > last) o[u] = (o[u] & 0x0000ffffu) | (fill2 & 0xffff0000u);
+                }
+            }
+            __builtin_nontemporal_store(o, reinterpret_cast<u4 *>(y + base + (int64_t)((ob0 + ob) * 16 + kg * 4 + v) * plane + key));
+        }
+    }
+}
+
 // The same for 16 heads: the contraction of a 16x16x16 product covers the 16 input heads; lane (ln, kg) fetches keys
 // 8ln .. 8ln+7 of the heads 4kg .. 4kg+3 (four 16-byte loads), forms the column of key 8ln + j with two byte permutes,
 // and after eight products holds keys 8ln .. 8ln+7 of the output heads 4kg + v.
@@ -376,6 +475,19 @@ int launch(const void *x, const void *w, void *y, int64_t N, int64_t C, int64_t 
             if (blocks > 0x7fffffffLL) return MTA_ERR_SHAPE;
             hipLaunchKernelGGL((headmix_dense32<T>), dim3((unsigned)blocks), dim3(64 * DM_WAVES), 0, st, (const T *)x,
                                (const T *)w, (T *)y, (int)C, (int)P, (int)Q, causal, fill, wt, qch);
+            return launch_status();
+        }
+        if ((G == 64 || G == 128) && !no_mfma && w_same_dtype && aligned_to(w, 16) && C % 8 == 0) {
+            const int chunks = G == 64 ? DM_WAVES : DM_WAVES / 2;  // key chunks per workgroup
+            const int qch = (int)((Q + chunks * DM_KEYS - 1) / (chunks * DM_KEYS));
+            const int64_t blocks = N * (C / G) * P * qch;
+            if (blocks > 0x7fffffffLL) return MTA_ERR_SHAPE;
+            if (G == 64)
+                hipLaunchKernelGGL((headmix_dense_wide<T, 64>), dim3((unsigned)blocks), dim3(64 * DM_WAVES), 0, st, (const T *)x,
+                                   (const T *)w, (T *)y, (int)C, (int)P, (int)Q, causal, fill, wt, qch);
+            else
+                hipLaunchKernelGGL((headmix_dense_wide<T, 128>), dim3((unsigned)blocks), dim3(64 * DM_WAVES), 0, st, (const T *)x,
+                                   (const T *)w, (T *)y, (int)C, (int)P, (int)Q, causal, fill, wt, qch);
             return launch_status();
         }
     }

@@ -158,6 +158,8 @@ HM_CASES = [
     (1, 16, 300, 304, None, False),
     (1, 1, 1, 1, None, True),
     (1, 48, 64, 64, None, True),
+    (1, 64, 136, 136, None, True),     # wide matrix-core mixing kernel with the transposed matrix (input gradient)
+    (1, 128, 72, 264, None, False),
 ]
 
 

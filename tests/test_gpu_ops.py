@@ -158,6 +158,10 @@ HM_CASES = [
     # 32 heads mixed densely (matrix-core kernel for 16-bit data): several wavefronts and workgroups per row, ragged
     # last wavefront, rows longer and shorter than the key range, two groups of 32
     (1, 32, 300, 296, None), (1, 32, 40, 1160, None), (2, 64, 136, 136, 32), (1, 32, 600, 64, None),
+    # 64 and 128 heads mixed densely (the head counts of the reference's own benchmark rows,
+    # benchmark_seq_len_results.jsonl:198-213): contraction over 2 / 4 blocks of 32 input heads, two wavefronts per key
+    # chunk for 128 heads; ragged last chunk; two groups of 64
+    (1, 64, 200, 200, None), (1, 128, 136, 136, None), (1, 128, 24, 520, None), (1, 128, 264, 264, 64), (2, 64, 40, 1032, None),
 ]
 
 
