@@ -125,16 +125,19 @@ def build_c4(torch, mta, O, device, b=2, h=16, s=4096, d=128, dtype=None, nsets=
     return mod, sets
 
 
-def build_general(torch, mta, O, device, b=1, h=16, s=4096, d=128, nsets=2, train=False):
-    """The closest shape to the reference's published rows (benchmark_seq_len_results.jsonl: H16 D128 fp16, 7x7 conv
-    before and after the softmax): all four weights non-trivial -- random 7x7 kernels, dense random 16x16 head weights."""
-    dtype = torch.float16
+def build_general(torch, mta, O, device, b=1, h=16, s=4096, d=128, nsets=2, train=False, dtype=None, ks=(7, 7)):
+    """The closest shapes to the reference's published rows (benchmark_seq_len_results.jsonl: H16 D128 fp16, 7x7 conv
+    before and after the softmax; benchmark_mta_attention.py: bf16, 11x15; benchmark_seq_len.py: 128 heads) with all four
+    weights non-trivial -- random kernels, dense random head weights (the reference's scripts run identity weights
+    through kernels that take no advantage of them)."""
+    dtype = dtype or torch.float16
     g = torch.Generator().manual_seed(321)
-    cfg = mta.MTAConfig(query_kernel_size=7, key_kernel_size=7, after_sm_query_kernel_size=7, after_sm_key_kernel_size=7)
+    cfg = mta.MTAConfig(query_kernel_size=ks[0], key_kernel_size=ks[1], after_sm_query_kernel_size=ks[0],
+                        after_sm_key_kernel_size=ks[1])
     mod = mta.MTAAttentionTriton(h, cfg, dropout=0.0, causal=True).to(dtype)
     with torch.no_grad():
-        mod.mta_conv_triton.weight.copy_(O.seeded_conv_weight(h, 7, 7, 0.05, dtype, seed=5))
-        mod.mta_conv_after_sm_triton.weight.copy_(O.seeded_conv_weight(h, 7, 7, 0.05, dtype, seed=6))
+        mod.mta_conv_triton.weight.copy_(O.seeded_conv_weight(h, ks[0], ks[1], 0.05, dtype, seed=5))
+        mod.mta_conv_after_sm_triton.weight.copy_(O.seeded_conv_weight(h, ks[0], ks[1], 0.05, dtype, seed=6))
         mod.wpsm_triton.weight.copy_(torch.eye(h) + 0.1 * torch.randn(h, h, generator=g))
         mod.wposm_triton.weight.copy_(torch.eye(h) + 0.1 * torch.randn(h, h, generator=g))
     mod = mod.to(device)                                 # dense weights: nothing is assumed about their structure
@@ -289,7 +292,22 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
         "note": "forward only; the reference's published row for this shape (Triton 11.345 ms, PyTorch 43.795 ms, "
                 "hardware unstated) is context, not a baseline"}
     del mod, sets
-    # the same module and shape in training: forward operator by operator (each with its HIP backward kernels; the two
+    # two more of the reference's own benchmark shapes, forward only: its benchmark script's configuration (bf16, 11x15
+    # kernels before and after the softmax, B1 H16 S4096 D64: benchmark_mta_attention.py:12-38) and the 128-head sweep's
+    # first row (B1 H128 S2048 D64 fp16 7x7: benchmark_seq_len.py:22-30, benchmark_seq_len_results.jsonl:198)
+    for label, kw, note in (
+            ("mta_forward_general_bf16_1x16x4096x64_11x15_pre_post_dense",
+             dict(b=1, h=16, s=4096, d=64, dtype=torch.bfloat16, ks=(11, 15)),
+             "the reference's benchmark script runs this shape (benchmark_mta_attention.py:12-38); it publishes no number for it"),
+            ("mta_forward_general_fp16_1x128x2048x64_7x7_pre_post_dense",
+             dict(b=1, h=128, s=2048, d=64, dtype=torch.float16, ks=(7, 7)),
+             "the reference's published row for this shape (Triton 22.579 ms, PyTorch 115.382 ms, hardware unstated) is "
+             "context, not a baseline")):
+        mod, sets = build_general(torch, mta, O, device, **kw)
+        ms = time_steps(torch, lambda i: mod(*sets[i], None, None), len(sets), min(warmup, 10), max(3, steps // 5))
+        out[label] = {"ms": ms, "stages_ms": stage_breakdown(torch, mod, sets, 3), "note": "forward only; " + note}
+        del mod, sets
+    # the first module and shape in training: forward operator by operator (each with its HIP backward kernels; the two
     # matrix products, the softmax and the dropout are torch's) and backward to q, k, v and the four weights
     mod, sets = build_general(torch, mta, O, device, train=True)
     params = [p for p in mod.parameters()]

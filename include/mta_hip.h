@@ -50,8 +50,15 @@ enum mta_error {
  * causal with the output above the diagonal written (+0.0 / fill).  The other entry points read `causal` as a flag. */
 #define MTA_CAUSAL_LOWER_ONLY 2
 
-#define MTA_MAX_KERNEL_R 32
-#define MTA_MAX_KERNEL_S 63
+/* Largest conv kernel (rows x keys) of the conv operator and its gradients (mta_conv2d_*): beyond the sizes with a
+ * matrix-core or unrolled instance they run on the general fp32-FMA kernels, whose staged tile must fit the LDS.  The
+ * reference's published rows go up to 77 x 77 (benchmark_seq_len_results.jsonl:140-180). */
+#define MTA_MAX_KERNEL_R 80
+#define MTA_MAX_KERNEL_S 95
+/* ... and of the kernels that keep score tiles in LDS next to K and V blocks (mta_conv_attn_fwd*, mta_qk_conv_fwd,
+ * mta_conv2d_headmix_fwd) */
+#define MTA_MAX_FUSED_KERNEL_R 32
+#define MTA_MAX_FUSED_KERNEL_S 63
 
 int mta_abi_version(void);
 const char *mta_strerror(int code);

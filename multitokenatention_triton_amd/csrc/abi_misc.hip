@@ -10,7 +10,9 @@ extern "C" const char *mta_strerror(int code)
     case MTA_ERR_NULL: return "null pointer argument";
     case MTA_ERR_DTYPE: return "unsupported dtype code";
     case MTA_ERR_SHAPE: return "size is not positive or exceeds the kernel's index range";
-    case MTA_ERR_KERNEL_SIZE: return "conv kernel size outside the supported range";
+    case MTA_ERR_KERNEL_SIZE:
+        return "conv kernel size outside the supported range (conv operator and its gradients: 1x1 to 80x95 rows x keys; "
+               "fused conv-attention, scores and conv + head-mixing kernels: up to 32x63)";
     case MTA_ERR_GROUP: return "group size does not divide the number of heads";
     case MTA_ERR_ALIGN: return "pointer not aligned to its element size";
     case MTA_ERR_HEAD_DIM: return "head dimension not supported by the fused kernel";

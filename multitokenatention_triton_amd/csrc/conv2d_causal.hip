@@ -147,6 +147,11 @@ int launch_valu(const void *x, const void *w, void *y, int64_t N, int64_t C, int
     const int tiles_m = (int)((H + V_TM - 1) / V_TM), tiles_n = (int)((W + V_TN - 1) / V_TN);
     const size_t lds = sizeof(float) * (((R * S + 3) & ~3) + (size_t)(V_TM + R - 1) * (V_TN + S));
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)(N * C));
+    if (lds > 160 * 1024) return MTA_ERR_KERNEL_SIZE;
+    if (lds > 48 * 1024) {  // per device, so set on every such launch (a cheap host-side call)
+        hipError_t e = hipFuncSetAttribute((const void *)conv2d_valu<T, R_T, S_T, BWD>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+    }
     hipLaunchKernelGGL((conv2d_valu<T, R_T, S_T, BWD>), grid, dim3(NT), lds, st, (const T *)x, w, (T *)y, (int)C,
                        (int)H, (int)W, R, S, causal, in_scale, use_scale, w_dtype, tiles_n);
     return launch_status();

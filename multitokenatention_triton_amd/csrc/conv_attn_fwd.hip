@@ -311,8 +311,11 @@ typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
 // The scores-only kernel pins its conv phase by hand instead (reads issued from assembly, see below).
 constexpr int F_BK = 64;   // keys per iteration
 constexpr int QK_OCC = 3;     // wavefronts per SIMD the scores-only kernel is compiled for (three workgroups per CU)
-constexpr int QK_CHUNK = 32;  // key blocks per work item of the scores-only kernel (24..128 measured at S = 4096,
-                              // with the items started longest first)
+constexpr int QK_CHUNK = 32;  // key blocks per work item of the scores-only kernel when no item table is built
+// with an item table: long and short items (key blocks), and the share of a query block's key range that goes into short
+// ones (MTA_QK_CHUNK_LONG / MTA_QK_CHUNK_SHORT / MTA_QK_SHORT_PERCENT in the environment override them, for comparisons)
+// (measured at B2 H16 S4096 D128: 32/32/0 237 us, 16/16/0 231, 64/16/50 238, 48/24/50 228, 52/26/50 227, 48/24/35 243)
+constexpr int QK_CHUNK_LONG = 48, QK_CHUNK_SHORT = 24, QK_SHORT_PERCENT = 50;
 constexpr int F_SLD = 80;  // score-tile row stride (elements): exactly the retained columns + one key block.  A wider
                            // row costs the scores-only kernel its third workgroup per CU, and with this one a fragment
                            // read (16 consecutive rows x 64 bytes) is free of bank conflicts as it is: the LDS serves
@@ -426,14 +429,17 @@ template <int R, int SK, int NW> struct fused_geom {
     static constexpr int WZ_OFF = SHIFT + 16, WZ_LD = WZ_OFF + 32;
 };
 
-// A head's work items (query block, key chunk) in the order they are to be started: longest first, so that the long
-// items all start early and the short ones fill the end of the grid.  Built on the host for every launch (a counting
-// sort over at most ITEM_TABLE_MAX items) and passed by value as a kernel argument; n = 0: no table, the kernel
-// walks the query blocks from the last to the first instead.
-constexpr int ITEM_TABLE_MAX = 1024;
+// A head's work items (query block, range of key blocks) in the order they are to be started: longest first, so that the
+// long items all start early and the short ones fill the end of the grid.  Built on the host for every launch (a
+// counting sort over at most ITEM_TABLE_MAX items) and passed by value as a kernel argument; n = 0: no table, the kernel
+// cuts every query block's key range into chunks of jc_len blocks and walks the query blocks from the last to the first.
+// The chunks need not be equal: the first part of a query block's key range goes into long items (one extra key block
+// per item rebuilds the retained score columns, and an item costs a few microseconds to set up), the rest into short
+// ones, which are started last and even out the end of the grid.
+constexpr int ITEM_TABLE_MAX = 768;
 struct item_table {
     int n;
-    uint16_t e[ITEM_TABLE_MAX];  // query block (11 bits) | key chunk << 11
+    uint32_t e[ITEM_TABLE_MAX];  // query block (11 bits) | first key block << 11 (11 bits) | key blocks << 22
 };
 
 // SCORES_ONLY: stop after the conv and write  conv(mask0(scale * Q K^T))  as an (S,S) plane per (batch, head)
@@ -497,10 +503,12 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? (R > 7 ? 2 : QK_OCC) : 2) vo
     // the attention kernel accumulates over all keys and gets jc_len = all of them.
     const int64_t bh = lid / items_per_bh;
     int item = (int)(lid % items_per_bh), qb = nqb - 1, jc = 0;
+    int tbl_lo = -1, tbl_len = 0;
     if (tbl.n > 0) {
         const unsigned e = tbl.e[item];
         qb = (int)(e & 2047u);
-        jc = (int)(e >> 11);
+        tbl_lo = (int)((e >> 11) & 2047u);
+        tbl_len = (int)(e >> 22);
     } else {
         for (; qb > 0; --qb) {  // longest query blocks first
             const int ql = (qb * G::BQ + G::BQ - 1 < S - 1) ? qb * G::BQ + G::BQ - 1 : S - 1;
@@ -562,8 +570,9 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? (R > 7 ? 2 : QK_OCC) : 2) vo
 
     const int q_last = (q0 + G::BQ - 1 < S - 1) ? q0 + G::BQ - 1 : S - 1;
     const int j_last = causal ? q_last / F_BK : (S - 1) / F_BK;  // last key block of the query block
-    const int j_lo = jc * jc_len;                                 // first key block whose outputs this item produces
-    const int j_end = (j_lo + jc_len - 1 < j_last) ? j_lo + jc_len - 1 : j_last;
+    const int j_lo = tbl_lo >= 0 ? tbl_lo : jc * jc_len;          // first key block whose outputs this item produces
+    const int j_len = tbl_lo >= 0 ? tbl_len : jc_len;
+    const int j_end = (j_lo + j_len - 1 < j_last) ? j_lo + j_len - 1 : j_last;
     // one key block earlier only fills the retained score columns (before the first one: the right pad, if any)
     const int j_start = j_lo > 0 ? j_lo - 1 : (G::PWR > 0 ? -1 : 0);
     issue_k(j_start, B0);
@@ -989,50 +998,50 @@ int launch_mfma(const void *q, const void *k, const void *v, const void *w, void
         const int64_t ql = std::min<int64_t>((int64_t)qb * G::BQ + G::BQ - 1, S - 1);
         items_per_bh += ((causal ? ql / F_BK : (S - 1) / F_BK) + jc_len) / jc_len;
     }
-    const int64_t total_wg = B * H * items_per_bh, per_xcd = (total_wg + 7) / 8;
-    if (per_xcd * 8 > 0x7fffffffLL || items_per_bh > 0x7fffffffLL) return MTA_ERR_SHAPE;
     // the items of a head, longest first (the number of key blocks an item visits, as the kernel computes it)
     item_table tbl;
     tbl.n = 0;
-    if (SCORES_ONLY && items_per_bh <= ITEM_TABLE_MAX && nqb <= 2047 && items_per_bh > 1) {
-        constexpr int MAXLEN = 4096;
+    if (SCORES_ONLY && nqb <= 2047 && (S + F_BK - 1) / F_BK <= 2047) {
+        constexpr int MAXLEN = 1023;
         static thread_local int count[MAXLEN + 2];
-        bool ok = true;
-        auto length = [&](int qb, int jc) {
-            const int64_t ql = std::min<int64_t>((int64_t)qb * G::BQ + G::BQ - 1, S - 1);
-            const int j_last = (int)(causal ? ql / F_BK : (S - 1) / F_BK);
-            const int j_lo = jc * jc_len, j_end = std::min(j_lo + jc_len - 1, j_last);
-            const int j_start = j_lo > 0 ? j_lo - 1 : (G::PWR > 0 ? -1 : 0);
-            return j_end - j_start + 1;
-        };
-        auto chunks = [&](int qb) {
-            const int64_t ql = std::min<int64_t>((int64_t)qb * G::BQ + G::BQ - 1, S - 1);
-            return (int)(((causal ? ql / F_BK : (S - 1) / F_BK) + jc_len) / jc_len);
-        };
-        std::fill(count, count + MAXLEN + 2, 0);
+        static thread_local uint32_t items[ITEM_TABLE_MAX];
+        static thread_local int lens[ITEM_TABLE_MAX];
+        // long chunks for the first part of a query block's key range, short ones for the last QK_SHORT_SHARE of it
+        static const int big = [] { const char *e = getenv("MTA_QK_CHUNK_LONG"); return e ? atoi(e) : QK_CHUNK_LONG; }();
+        static const int small = [] { const char *e = getenv("MTA_QK_CHUNK_SHORT"); return e ? atoi(e) : QK_CHUNK_SHORT; }();
+        static const int share = [] { const char *e = getenv("MTA_QK_SHORT_PERCENT"); return e ? atoi(e) : QK_SHORT_PERCENT; }();
+        int n = 0;
+        bool ok = big >= 1 && small >= 1 && big <= MAXLEN && small <= MAXLEN && share >= 0 && share <= 100;
         for (int qb = 0; qb < nqb && ok; ++qb) {
-            const int nch = chunks(qb);
-            if (nch > 31) ok = false;
-            for (int jc = 0; jc < nch && ok; ++jc) {
-                const int len = length(qb, jc);
-                if (len < 0 || len > MAXLEN) ok = false;
-                else ++count[len];
+            const int64_t ql = std::min<int64_t>((int64_t)qb * G::BQ + G::BQ - 1, S - 1);
+            const int nk = (int)(causal ? ql / F_BK : (S - 1) / F_BK) + 1;  // key blocks 0 .. j_last
+            const int nshort = std::min(nk, (nk * share / 100 + small / 2) / small * small);
+            const int nlong = nk - nshort;
+            for (int j0 = 0; j0 < nk && ok;) {
+                const int len = j0 < nlong ? std::min(big, nlong - j0) : std::min(small, nk - j0);
+                if (n >= ITEM_TABLE_MAX) { ok = false; break; }
+                // what the kernel visits: one key block earlier rebuilds the retained columns (ahead of the first: the right pad)
+                lens[n] = len + ((j0 > 0 || G::PWR > 0) ? 1 : 0);
+                items[n++] = (uint32_t)qb | ((uint32_t)j0 << 11) | ((uint32_t)len << 22);
+                j0 += len;
             }
         }
-        if (ok) {
-            // positions: longer items first; among equal lengths later query blocks first
+        if (ok && n > 1) {
+            std::fill(count, count + MAXLEN + 2, 0);
+            for (int i = 0; i < n; ++i) ++count[lens[i]];
             int pos = 0;
-            for (int len = MAXLEN; len >= 0; --len) {
+            for (int len = MAXLEN + 1; len >= 0; --len) {  // positions: longer items first
                 const int c = count[len];
                 count[len] = pos;
                 pos += c;
             }
-            for (int qb = nqb - 1; qb >= 0; --qb)
-                for (int jc = 0, nch = chunks(qb); jc < nch; ++jc)
-                    tbl.e[count[length(qb, jc)]++] = (uint16_t)(qb | (jc << 11));
-            tbl.n = (int)items_per_bh;
+            for (int i = n - 1; i >= 0; --i) tbl.e[count[lens[i]]++] = items[i];  // among equal lengths later query blocks first
+            tbl.n = n;
+            items_per_bh = n;
         }
     }
+    const int64_t total_wg = B * H * items_per_bh, per_xcd = (total_wg + 7) / 8;
+    if (per_xcd * 8 > 0x7fffffffLL || items_per_bh > 0x7fffffffLL) return MTA_ERR_SHAPE;
     dim3 grid((unsigned)(per_xcd * 8));
     hipLaunchKernelGGL(kern, grid, dim3(F_NT), 0, st, (const T *)q, (const T *)k, (const T *)v, (const T *)w, (T *)o,
                        lse, (int)S, causal, scale, (int)H, nqb, fill_upper, total_wg, per_xcd, jc_len, (int)items_per_bh,
@@ -1093,7 +1102,7 @@ extern "C" int mta_conv_attn_fwd_lse(const void *q, const void *k, const void *v
     if (lse && !aligned_to(lse, 4)) return MTA_ERR_ALIGN;
     if (!dtype_size(io_dtype) || !dtype_size(w_dtype)) return MTA_ERR_DTYPE;
     if (B <= 0 || H <= 0 || S <= 0 || S > (1 << 24) || B * H > 65535) return MTA_ERR_SHAPE;
-    if (R < 1 || Sk < 1 || R > MTA_MAX_KERNEL_R || Sk > MTA_MAX_KERNEL_S) return MTA_ERR_KERNEL_SIZE;
+    if (R < 1 || Sk < 1 || R > MTA_MAX_FUSED_KERNEL_R || Sk > MTA_MAX_FUSED_KERNEL_S) return MTA_ERR_KERNEL_SIZE;
     if (D != 64 && D != 128) return MTA_ERR_HEAD_DIM;
     if (!aligned_to(q, 16) || !aligned_to(k, 16) || !aligned_to(v, 16) || !aligned_to(o, 16) ||
         !aligned_to(w, dtype_size(w_dtype)))
@@ -1143,7 +1152,7 @@ extern "C" int mta_qk_conv_fwd(const void *q, const void *k, const void *w, void
     if (!q || !k || !w || !s_out) return MTA_ERR_NULL;
     if (!dtype_size(io_dtype) || !dtype_size(w_dtype)) return MTA_ERR_DTYPE;
     if (B <= 0 || H <= 0 || S <= 0 || S > (1 << 24) || B * H > 65535) return MTA_ERR_SHAPE;
-    if (R < 1 || Sk < 1 || R > MTA_MAX_KERNEL_R || Sk > MTA_MAX_KERNEL_S) return MTA_ERR_KERNEL_SIZE;
+    if (R < 1 || Sk < 1 || R > MTA_MAX_FUSED_KERNEL_R || Sk > MTA_MAX_FUSED_KERNEL_S) return MTA_ERR_KERNEL_SIZE;
     if (D != 64 && D != 128) return MTA_ERR_HEAD_DIM;
     if (!aligned_to(q, 16) || !aligned_to(k, 16) || !aligned_to(s_out, 16) || !aligned_to(w, dtype_size(w_dtype)))
         return MTA_ERR_ALIGN;

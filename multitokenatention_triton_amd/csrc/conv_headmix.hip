@@ -330,7 +330,7 @@ extern "C" int mta_conv2d_headmix_fwd(const void *x, const void *w_conv, const v
     if (!x || !w_conv || !w_mix || !y) return MTA_ERR_NULL;
     if (!dtype_size(io_dtype) || !dtype_size(wconv_dtype) || !dtype_size(wmix_dtype)) return MTA_ERR_DTYPE;
     if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || H > (1 << 24) || W > (1 << 24) || C > 4096) return MTA_ERR_SHAPE;
-    if (R < 1 || S < 1 || R > MTA_MAX_KERNEL_R || S > MTA_MAX_KERNEL_S) return MTA_ERR_KERNEL_SIZE;
+    if (R < 1 || S < 1 || R > MTA_MAX_FUSED_KERNEL_R || S > MTA_MAX_FUSED_KERNEL_S) return MTA_ERR_KERNEL_SIZE;
     if (group_size < 0 || (group_size > 0 && C % group_size != 0)) return MTA_ERR_GROUP;
     if (!aligned_to(x, dtype_size(io_dtype)) || !aligned_to(y, dtype_size(io_dtype)) ||
         !aligned_to(w_conv, dtype_size(wconv_dtype)) || !aligned_to(w_mix, dtype_size(wmix_dtype)))

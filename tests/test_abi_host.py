@@ -64,9 +64,14 @@ def test_argument_validation_needs_no_gpu():
     assert lib.mta_headmix_fwd(p, p, p, 1, 2, 0, 8, 0, 1, 0.0, 0, 0, None) == -3
     assert lib.mta_conv_attn_fwd(p, p, p, p, p, 1, 1, 0, 64, 3, 3, 1, 0.1, 0, 0, None) == -3
     # kernel size
-    assert lib.mta_conv2d_fwd(p, p, p, 1, 1, 8, 8, 33, 3, 1, 0, 0, None) == -4
-    assert lib.mta_conv2d_fwd(p, p, p, 1, 1, 8, 8, 3, 64, 1, 0, 0, None) == -4
+    # (the conv operator takes up to 80 x 95 - the reference publishes rows for 77 x 77 -, the fused kernels up to 32 x 63)
+    assert lib.mta_conv2d_fwd(p, p, p, 1, 1, 8, 8, 81, 3, 1, 0, 0, None) == -4
+    assert lib.mta_conv2d_fwd(p, p, p, 1, 1, 8, 8, 3, 96, 1, 0, 0, None) == -4
+    assert lib.mta_conv2d_bwd_input(p, p, p, 1, 1, 8, 8, 3, 96, 1, 0, 0, None) == -4
     assert lib.mta_conv_attn_fwd(p, p, p, p, p, 1, 1, 8, 64, 0, 3, 1, 0.1, 0, 0, None) == -4
+    assert lib.mta_conv_attn_fwd(p, p, p, p, p, 1, 1, 8, 64, 33, 3, 1, 0.1, 0, 0, None) == -4
+    assert lib.mta_qk_conv_fwd(p, p, p, p, 1, 1, 8, 64, 3, 64, 1, 0.1, 1, 1, 1, None) == -4
+    assert b"80x95" in lib.mta_strerror(-4) and b"32x63" in lib.mta_strerror(-4)
     # group
     assert lib.mta_headmix_fwd(p, p, p, 1, 6, 8, 8, 4, 1, 0.0, 0, 0, None) == -5
     assert lib.mta_headmix_softmax_fwd(p, p, p, p, 1, 6, 8, 8, 4, 1, 1, 0, 0, None) == -5

@@ -96,6 +96,7 @@ CONV_CASES = [
     (1, 2, 96, 40, 3, 5, True),        # causal rule on a tall plane: keys beyond the row index never take part
     (1, 1, 1040, 1040, 7, 7, True),    # key range cut into segments, many steps per item
     (3, 5, 136, 136, 5, 7, True),
+    (1, 1, 80, 80, 77, 77, True),      # the largest kernel of the reference's published rows
 ]
 
 

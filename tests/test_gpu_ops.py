@@ -47,6 +47,9 @@ CONV_CASES = [
     (1, 3, 8, 6, 11), (1, 1, 392, 7, 7), (1, 2, 200, 5, 5),
     # several 256-key strips per row strip, ragged last one; 11x15 on the matrix cores
     (1, 2, 776, 6, 11), (1, 1, 128, 11, 15), (1, 2, 520, 11, 15), (3, 1, 264, 6, 11),
+    # the largest kernel of the reference's published rows (77 x 77, benchmark_seq_len_results.jsonl:140-180) and the
+    # largest the operator takes: general fp32-FMA kernel, staged tile beyond 64 KB of LDS
+    (1, 1, 96, 77, 77), (1, 1, 40, 80, 95),
 ]
 
 
@@ -399,7 +402,7 @@ def test_conv_headmix_unsupported_group(ops):
 def test_error_codes(ops):
     x = torch.zeros(1, 2, 8, 8, device="cuda")
     with pytest.raises(ValueError, match="kernel size"):
-        ops.conv2d_causal(x, torch.zeros(2, 40, 3, device="cuda"), True)
+        ops.conv2d_causal(x, torch.zeros(2, 81, 3, device="cuda"), True)     # (up to 80 x 95)
     with pytest.raises(ValueError, match="group"):
         ops.headmix(torch.zeros(1, 6, 8, 8, device="cuda"), torch.eye(6).cuda(), True, 0.0, group_size=4)
     with pytest.raises(AssertionError):

@@ -16,6 +16,9 @@ GROUPS = [
     ({"MTA_HEADMIX_NO_MFMA": "1", "MTA_SOFTMAX_NO_PACKED": "1", "MTA_FUSED_FORCE_GENERAL": "1"},
      ["tests/test_gpu_ops.py", "tests/test_gpu_attention.py"],
      "test_headmix_parity or test_mix_softmax_mix_parity or test_conv_attention_parity or test_mta_general"),
+    # another cut of the scores kernel's work items (long / short items of 20 / 7 key blocks, 30 % of a key range short)
+    ({"MTA_QK_CHUNK_LONG": "20", "MTA_QK_CHUNK_SHORT": "7", "MTA_QK_SHORT_PERCENT": "30"},
+     ["tests/test_gpu_attention.py"], "test_qk_conv_parity or test_mta_headline_route_long_sequence"),
     # fp32-FMA conv kernels (forward, input gradient, weight gradient) for 16-bit data
     ({"MTA_CONV_FORCE_VALU": "1"},
      ["tests/test_gpu_ops.py", "tests/test_gpu_backward.py"],
