@@ -190,9 +190,10 @@ constexpr int M_TM = 32;           // strip rows
 constexpr int M_TN = 256;          // strip cols: two halves of 8 column blocks of 16
 constexpr int M_HALF = M_TN / 2;   // keys per wavefront
 constexpr int M_RPB = M_TN / M_TM;  // row strips per M_TN x M_TN block of the lower triangle
-// persistent workgroups per CU (two 24 KB strip buffers each); kernels of more than 7 rows keep that many more Toeplitz
-// fragments in registers and are compiled for two
-template <int R> constexpr int wg_per_cu() { return R > 7 ? 2 : 3; }
+// persistent workgroups per CU: four where two strip buffers take a quarter of the LDS (kernels of up to 6 rows: 37 staged
+// rows of 544 bytes are 1258 slots, five copy rounds, 20 KB), else three; kernels of more than 7 rows keep that many more
+// Toeplitz fragments in registers and are compiled for two
+template <int R> constexpr int wg_per_cu() { return R > 7 ? 2 : (R > 6 ? 3 : 4); }
 static_assert(M_NW == 4 && M_TM == 32 && M_TN % M_TM == 0 && M_RPB % 2 == 0, "strip geometry");
 
 // 16 outputs + S-1 taps (+ alignment shift) must fit the 32-key contraction of one 16x16x32 MFMA
@@ -202,7 +203,12 @@ template <int R, int S> struct mfma_geom {
     static constexpr int SHIFT = HL - PADW;                // first tap's offset inside a block's 32-key window
     static constexpr bool fits = SHIFT + 16 + S - 1 <= 32;
     static constexpr int TW = M_TN - 16 + 32;              // staged columns
-    static constexpr int LD = TW + ((24 - TW % 16) % 16);  // row stride = 8 (mod 16) elements: conflict-free b128 reads
+    // Row stride in LDS.  A fragment read takes 16 bytes per lane from 16 consecutive rows (lane group kg at byte offset
+    // 16 kg); the LDS serves lanes 0-7 together with lanes 24-31 (8-15 with 16-23, ...), i.e. rows 0-7 at one offset with
+    // rows 8-15 at the next: with a stride of 2 (mod 8) 16-byte slots those sixteen accesses fall on sixteen different
+    // slots of the 256-byte bank line (3 (mod 8), one padding slot after the 34 of data, put rows 3 and 8 on the same one).
+    static constexpr int LD = TW;
+    static_assert((LD / 8) % 8 == 2, "row stride of the staged strip");
     static constexpr int ROWS = M_TM + R - 1;
     // results of the wavefronts that own key half `h` go back to LDS columns h * RES_OFF .. + M_HALF - 1, which no
     // wavefront of the other half reads as input (half 0 reads columns 0 .. M_HALF+15, half 1 columns M_HALF ..)
@@ -369,13 +375,15 @@ __global__ __launch_bounds__(M_WT, wg_per_cu<R>()) void conv2d_mfma(
     constexpr int SPR = LD / VEC;                           // 16-byte slots per LDS row (35)
     constexpr int SLOTS = G::ROWS * SPR;
     constexpr int STAGE_IT = (SLOTS + M_WT - 1) / M_WT;     // copies per strip and lane (the last round may be partial)
-    static_assert(SPR == VPR + 1, "one padding slot per row");
-    constexpr int BUF = STAGE_IT * M_WT * VEC;               // elements per LDS strip buffer
-    __shared__ __align__(16) T tiles[2 * BUF];               // double buffer: strip n is computed while strip n+1 lands
-    // the channel's kernel as it lies in memory (see above), by strip parity
+    static_assert(SPR == VPR, "no padding slots");
+    // the channel's kernel as it lies in memory (see above) travels with its strip: behind the strip's last slot
     constexpr int WRAW_DW = (R * S + 2) / 2;                 // dwords that cover R*S taps starting in either half of the first
     constexpr int WRAW_IT = (WRAW_DW + 63) / 64;
-    __shared__ __align__(16) unsigned wraw[2][WRAW_IT * 64];
+    constexpr int WRAW_SLOT = (SLOTS + 3) & ~3;              // (64-byte aligned)
+    constexpr int NEED_SLOTS = WRAW_SLOT + WRAW_IT * 16;     // (a copy instruction of the kernel rows covers 16 slots)
+    constexpr int BUF_SLOTS = NEED_SLOTS > STAGE_IT * M_WT ? (NEED_SLOTS + 3) / 4 * 4 : STAGE_IT * M_WT;
+    constexpr int BUF = BUF_SLOTS * VEC;                     // elements per LDS strip buffer
+    __shared__ __align__(16) T tiles[2 * BUF];               // double buffer: strip n is computed while strip n+1 lands
     using V16 = pack16<T>;
 
     // XCD-aware split: workgroup ids are dealt round-robin to the 8 XCDs; each XCD gets one
@@ -451,13 +459,13 @@ __global__ __launch_bounds__(M_WT, wg_per_cu<R>()) void conv2d_mfma(
                 if (slot_valid(slot, h0_, k0_))
                     __builtin_amdgcn_global_load_lds((glb_void_t *)(base + goff[it]),
                                                      (lds_void_t *)(buf + (it * M_WT + wave * 64) * VEC), 16, 0, 0);
-                else
+                else if (slot < SLOTS)
                     lds_store16(buf_lds + (unsigned)slot * 16u, zero4);
             }
         }
     };
-    // asynchronous copy of a channel's kernel into wraw[par] (first wavefront); returns nothing: the taps start
-    // wshift(channel) 16-bit elements into the buffer
+    // asynchronous copy of a channel's kernel into the spare slots of strip buffer `par` (first wavefront); the taps start
+    // wshift(channel) 16-bit elements into them
     auto wshift = [&](int channel_) { return (int)((reinterpret_cast<uintptr_t>(w + (int64_t)channel_ * (R * S)) >> 1) & 1u); };
     auto fetch_weights = [&](int channel_, int par) {
         if (wave != 0) return;
@@ -467,7 +475,8 @@ __global__ __launch_bounds__(M_WT, wg_per_cu<R>()) void conv2d_mfma(
 #pragma unroll
         for (int k = 0; k < WRAW_IT; ++k)
             if (k * 64 + lane < ndw)
-                __builtin_amdgcn_global_load_lds((glb_void_t *)(base + (k * 64 + lane) * 4), (lds_void_t *)(&wraw[par][k * 64]), 4, 0, 0);
+                __builtin_amdgcn_global_load_lds((glb_void_t *)(base + (k * 64 + lane) * 4),
+                                                 (lds_void_t *)(tiles + par * BUF + (WRAW_SLOT + k * 16) * VEC), 4, 0, 0);
     };
     // current and next work item: position inside the plane, plane (as element offset, and its parity) and channel
     int t_nx;
@@ -573,7 +582,7 @@ __global__ __launch_bounds__(M_WT, wg_per_cu<R>()) void conv2d_mfma(
                     for (int u = 0; u < VEC; ++u)
                         if (col + u > h) v.v[u] = from_float<T>(0.0f);
                 }
-                lds_store16(tile_lds + (unsigned)slot * 16u, __builtin_bit_cast(u32x4, v));
+                if (slot < SLOTS) lds_store16(tile_lds + (unsigned)slot * 16u, __builtin_bit_cast(u32x4, v));
             }
         }
         lds_wait();    // this wavefront's LDS stores above are complete
@@ -583,7 +592,7 @@ __global__ __launch_bounds__(M_WT, wg_per_cu<R>()) void conv2d_mfma(
             cur_channel = channel;
             const int lane_ = opaque(lane);
             const int ln_ = lane_ & 15, kg_ = lane_ >> 4;
-            const unsigned wa = (unsigned)(uintptr_t)(lds_void_t *)&wraw[parity][0] + 2u * (unsigned)wshift(channel);
+            const unsigned wa = tile_lds + (unsigned)(WRAW_SLOT * 16) + 2u * (unsigned)wshift(channel);
 #pragma unroll
             for (int i = 0; i < R; ++i) {  // row m = ln, slots k = 8*kg + t, tap j = k-SHIFT-m
                 unsigned tap[8];
@@ -651,7 +660,9 @@ __global__ __launch_bounds__(M_WT, wg_per_cu<R>()) void conv2d_mfma(
             // into a ring of registers, and a product waits only for its own operand (LDS operations complete in order:
             // exactly the reads issued after it may be outstanding).  Source order is pinned (the scheduler would regroup
             // reads and products).  Blocks above the diagonal are computed like the others and masked below.
-            constexpr int NPROD = NCB * R, NLD = 2 * R < 12 ? 2 * R : 12, NSLOT = NLD + 1;
+            // (operands in flight: 12, or 6 where four workgroups per CU leave a wavefront 128 registers)
+            constexpr int NLD_MAX = wg_per_cu<R>() >= 4 ? 6 : 12;
+            constexpr int NPROD = NCB * R, NLD = 2 * R < NLD_MAX ? 2 * R : NLD_MAX, NSLOT = NLD + 1;
             static_assert(NLD <= 15 && NPROD > NLD, "lgkmcnt field; pipeline deeper than the work");
             u32x4 ring[NSLOT];
             // product n: column block 2*(n / 2R) + n % 2, kernel row (n % 2R) / 2
@@ -687,20 +698,25 @@ __global__ __launch_bounds__(M_WT, wg_per_cu<R>()) void conv2d_mfma(
                 lds_store8_at(ra, (int)(cb * 16 * sizeof(T)), lo, hi);
             }
         }
-        // ---- coalesced stores of this wavefront's 16 rows: 16 lanes cover one 256-byte output row (the LDS writes
-        // above precede these reads in the wavefront's LDS queue) ----
+        // ---- coalesced stores.  The four wavefronts' results lie in LDS; after a barrier wavefront w stores rows 8w .. 8w+7
+        // of the strip in full, two 512-byte rows per instruction (the halves of a row come from two wavefronts' results):
+        // whole rows in one instruction move a few percent faster through memory than 256-byte pieces of four rows ----
+        lds_wait();
+        wg_barrier();
         {
             // (uniform row base + one 32-bit per-lane byte offset: no 64-bit address arithmetic per store)
-            char *ybase = reinterpret_cast<char *>(yp + (int64_t)(p0 + rb0) * W + qw);
+            const int sr0 = wave * 8;                                   // first strip row this wavefront stores
+            const int sres = sr0 < 16 ? sr0 : sr0 + R - 1;              // ... and where its results lie (see res0)
+            char *ybase = reinterpret_cast<char *>(yp + (int64_t)(p0 + sr0) * W + q0);
             const int lane_o = opaque(lane);  // (row offsets formed here, not kept in registers across the loop)
-            const int r_l = lane_o >> 4, cv = (lane_o & 15) * VEC;
-            const unsigned yoff = (unsigned)(r_l * W + cv) * (unsigned)sizeof(T);
-            const int64_t ystep = (int64_t)4 * W * (int64_t)sizeof(T);
-            static_assert(ST == 4, "four row groups per wavefront");
+            const int r_l = lane_o >> 5, hf = (lane_o >> 4) & 1, cv = (lane_o & 15) * VEC;
+            const unsigned yoff = (unsigned)(r_l * W + hf * M_HALF + cv) * (unsigned)sizeof(T);
+            const int64_t ystep = (int64_t)2 * W * (int64_t)sizeof(T);
+            static_assert(ST == 4, "four row pairs per wavefront");
             u32x4 v[4];
-            const unsigned va = tile_lds + (unsigned)((res0 + r_l) * LD + ch * G::RES_OFF + cv) * sizeof(T);
+            const unsigned va = tile_lds + (unsigned)((sres + r_l) * LD + hf * G::RES_OFF + cv) * sizeof(T);
 #pragma unroll
-            for (int k = 0; k < 4; ++k) v[k] = lds_load16_at(va, (int)(k * 4 * LD * sizeof(T)));
+            for (int k = 0; k < 4; ++k) v[k] = lds_load16_at(va, (int)(k * 2 * LD * sizeof(T)));
             asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : : "memory");
             if (full_out) {  // unconditional: exactly ST vector-memory instructions
 #pragma unroll
@@ -708,8 +724,8 @@ __global__ __launch_bounds__(M_WT, wg_per_cu<R>()) void conv2d_mfma(
             } else {
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    const int r = k * 4 + r_l;
-                    if (p0 + rb0 + r < H && qw + cv < W) MTA_CONV_STORE(reinterpret_cast<u32x4 *>(ybase + k * ystep + yoff), v[k]);
+                    const int r = k * 2 + r_l;
+                    if (p0 + sr0 + r < H && q0 + hf * M_HALF + cv < W) MTA_CONV_STORE(reinterpret_cast<u32x4 *>(ybase + k * ystep + yoff), v[k]);
                 }
             }
             younger = full_out ? ST : -1;
@@ -744,7 +760,10 @@ int launch_mfma(const void *x, const void *w, void *y, int64_t N, int64_t C, int
     const int ipp = (int)ipp64;
     const int64_t total = N * C * ipp64;
     const int64_t per_xcd = (total + 7) / 8;
-    int nw = device_cu_count() * wg_per_cu<R>() / 8;  // persistent workgroups per XCD
+    // persistent workgroups per XCD: as many as fit when only the strips of the lower triangle are walked; with the zero
+    // strips in the list three per CU move the tensor fastest (measured at (2,16,2048,2048): 84 us against 85.5 with four)
+    const int wgs = tri ? wg_per_cu<R>() : (wg_per_cu<R>() < 3 ? wg_per_cu<R>() : 3);
+    int nw = device_cu_count() * wgs / 8;
     if (nw < 1) nw = 1;
     if (per_xcd < nw) nw = (int)per_xcd;
     dim3 grid((unsigned)(nw * 8));
