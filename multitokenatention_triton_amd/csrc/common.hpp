@@ -93,4 +93,8 @@ inline int launch_status()
         else { using io_t = mta::f16_t; __VA_ARGS__; }                \
     } while (0)
 
+// conv_mix16.hip: depthwise conv + dense mixing of groups of 16 heads on the matrix cores; MTA_ERR_UNSUPPORTED when no
+// instance covers the arguments
+int conv_mix16_dispatch(const void *x, const void *wc, const void *wm, void *y, int64_t N, int64_t C, int64_t H, int64_t W, int R,
+                        int S, int causal, int fill_upper, int io_dtype, hipStream_t st);
 }  // namespace mta

@@ -336,9 +336,14 @@ extern "C" int mta_conv2d_headmix_fwd(const void *x, const void *w_conv, const v
         !aligned_to(w_conv, dtype_size(wconv_dtype)) || !aligned_to(w_mix, dtype_size(wmix_dtype)))
         return MTA_ERR_ALIGN;
     const int G = group_size > 0 ? group_size : (int)C;
+    hipStream_t st = (hipStream_t)stream;
+    // groups of 16 heads, 16-bit data and weights of the same dtype: conv and mixing both on the matrix cores
+    if (G == 16 && io_dtype != MTA_F32 && wconv_dtype == io_dtype && wmix_dtype == io_dtype) {
+        const int rc = conv_mix16_dispatch(x, w_conv, w_mix, y, N, C, H, W, R, S, causal, causal ? fill_upper : 1, io_dtype, st);
+        if (rc != MTA_ERR_UNSUPPORTED) return rc;
+    }
     const int64_t tiles = ((H + CH_TM - 1) / CH_TM) * ((W + CH_TN - 1) / CH_TN);
     if (tiles > 0x7fffffffLL || N * (C / G) > 65535) return MTA_ERR_SHAPE;
-    hipStream_t st = (hipStream_t)stream;
     MTA_DISPATCH_IO(io_dtype, return dispatch<io_t>(x, w_conv, w_mix, y, N, C, H, W, R, S, G, causal, causal ? fill_upper : 1,
                                                     wconv_dtype, wmix_dtype, st));
     return MTA_ERR_DTYPE;

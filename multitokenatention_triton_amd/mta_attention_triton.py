@@ -73,6 +73,8 @@ def _one_pass_group(group: int, scores_dtype, n_keys: int, *weights) -> bool:
 # where the one-pass post-softmax conv + head mixing kernel is used (see forward)
 _CONV_MIX_MAX_GROUP = 4
 _CONV_MIX_SIZES = ((3, 3), (7, 7))
+# ... and for dense groups of 16 heads at 16-bit dtypes (conv and mixing both on the matrix cores)
+_CONV_MIX16_SIZES = ((3, 3), (5, 5), (7, 7))
 
 
 _IDENTITY_KERNELS = {}
@@ -354,7 +356,11 @@ class MTAAttentionTriton(nn.Module):
             # conv and mix in one pass, the conv result never written: taken where it measures at least as fast as the
             # two kernels (mixing groups of up to 4 heads, kernel sizes with a vector-staged instance: 3x3, 7x7)
             ks = tuple(self.mta_conv_after_sm_triton.weight.shape[1:])
-            if not post_conv_identity and w2 is not None and g_post <= _CONV_MIX_MAX_GROUP and ks in _CONV_MIX_SIZES:
+            conv_w = self.mta_conv_after_sm_triton.weight
+            mix16 = (g_post == 16 and ks in _CONV_MIX16_SIZES and scores.dtype in (torch.bfloat16, torch.float16)
+                     and conv_w.dtype == scores.dtype and w_post.dtype == scores.dtype and n_keys % 8 == 0)
+            if not post_conv_identity and w2 is not None and (
+                    (g_post <= _CONV_MIX_MAX_GROUP and ks in _CONV_MIX_SIZES) or mix16):
                 self._mark("conv_mix_post")
                 done = ops.conv2d_headmix(scores, self.mta_conv_after_sm_triton.weight, w_post, self.causal,
                                           group_size=g_post, fill_upper=not own_pv)
