@@ -94,7 +94,7 @@ __device__ __forceinline__ void decode_tile(int t, int tiles_n, int tri, int &tm
 }
 
 template <typename T, int R, int S>
-__global__ __launch_bounds__(X_WT, X_OCC) void conv_mix16_mfma(const T *__restrict__ x, const T *__restrict__ wc,
+__global__ __launch_bounds__(X_WT, R <= 3 ? 3 : X_OCC) void conv_mix16_mfma(const T *__restrict__ x, const T *__restrict__ wc,
                                                                const T *__restrict__ wm, T *__restrict__ y, int C, int H,
                                                                int W, int causal, int fill_upper, int tiles_n, int ipp,
                                                                int64_t total, int64_t per_xcd, int tri)
@@ -105,14 +105,15 @@ __global__ __launch_bounds__(X_WT, X_OCC) void conv_mix16_mfma(const T *__restri
     constexpr int SLOTS = G::ROWS * SPR;
     constexpr int STAGE_IT = (SLOTS + X_WT - 1) / X_WT;
     constexpr int BUF = ((SLOTS + 63) & ~63) * VEC;              // elements per window buffer (whole copy instructions)
-    constexpr int NBUF = 4;                                      // window buffers: head h + NBUF - 1 is copied during head h
+    // window buffers: head h + NBUF - 1 is copied during head h (seven where that leaves room for three workgroups per CU)
+    constexpr int NBUF = R <= 3 ? 7 : 8;
     constexpr int TAB_VECS = X_HG * R * G::NVEC;                 // 16-byte vectors of the fragment table
     constexpr int STG_BYTES = 4 * X_TM * X_TN * (int)sizeof(T);  // output staging: 4 heads x 32 rows x 128 bytes
     constexpr int RAW_BYTES = (X_HG * R * S * (int)sizeof(T) + 15) & ~15;
-    static_assert(RAW_BYTES <= STG_BYTES, "the raw kernels lie in the staging area until the table is built");
+    static_assert(STG_BYTES <= NBUF * BUF * (int)sizeof(T), "the outputs are staged in the window buffers, which are free by then");
     __shared__ __align__(16) T tiles[NBUF * BUF];
     __shared__ __align__(16) u32x4 table[TAB_VECS + 1];          // (+ one vector of zeros)
-    __shared__ __align__(16) unsigned char stage[STG_BYTES];
+    __shared__ __align__(16) unsigned char rawk[RAW_BYTES];      // the group's kernels as they lie in memory
 
     // XCD-aware: workgroup ids are dealt round-robin to the 8 XCDs; each XCD takes a contiguous run of the item list
     const int64_t idx = (int64_t)(blockIdx.x & 7) * per_xcd + (int64_t)(blockIdx.x >> 3);
@@ -188,6 +189,11 @@ __global__ __launch_bounds__(X_WT, X_OCC) void conv_mix16_mfma(const T *__restri
         }
     };
 
+    // the group's kernels as they lie in memory: one 16-byte load per thread, issued ahead of the window copies
+    constexpr int NRAW = RAW_BYTES / 16;
+    static_assert(X_HG * R * S * (int)sizeof(T) % 16 == 0 && NRAW <= X_WT, "the kernels of a group are whole 16-byte vectors");
+    u32x4 rawv = {0u, 0u, 0u, 0u};
+    if (tid < NRAW) rawv = *reinterpret_cast<const u32x4 *>(wc + (int64_t)g * X_HG * (R * S) + tid * VEC);
 #pragma unroll
     for (int b = 0; b < NBUF - 1; ++b) prefetch(b, tiles + b * BUF);
     // copy instructions of this wavefront per window (interior tiles)
@@ -196,14 +202,11 @@ __global__ __launch_bounds__(X_WT, X_OCC) void conv_mix16_mfma(const T *__restri
     for (int it = 0; it < STAGE_IT; ++it) n_copy += (it * X_WT + wave * 64 < SLOTS) ? 1 : 0;
 
     // ---- the group's kernels as they lie in memory -> LDS (staging area), then the table of Toeplitz vectors ----
-    const unsigned stage_lds = (unsigned)(uintptr_t)(lds_void_t *)stage;
+    const unsigned stage_lds = (unsigned)(uintptr_t)(lds_void_t *)tiles;
+    const unsigned raw_lds = (unsigned)(uintptr_t)(lds_void_t *)rawk;
     const unsigned table_lds = (unsigned)(uintptr_t)(lds_void_t *)table;
     {
-        const T *wg = wc + (int64_t)g * X_HG * (R * S);
-        for (int t = tid; t < X_HG * R * S; t += X_WT) {
-            const unsigned short raw = __builtin_bit_cast(unsigned short, wg[t]);
-            lds_store2(stage_lds + 2u * (unsigned)t, (unsigned)raw);
-        }
+        if (tid < NRAW) lds_store16(raw_lds + 16u * (unsigned)tid, rawv);
         lds_wait();
         wg_barrier();
         // vector (h, i, ve): taps j = ve + t - 7, t = 0..7, of kernel row i of head h (0 outside the row)
@@ -213,7 +216,7 @@ __global__ __launch_bounds__(X_WT, X_OCC) void conv_mix16_mfma(const T *__restri
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
                 const int j = ve + t - 7;
-                tap[t] = lds_load_u16(stage_lds + 2u * (unsigned)(hi * S + ((j >= 0 && j < S) ? j : 0)));
+                tap[t] = lds_load_u16(raw_lds + 2u * (unsigned)(hi * S + ((j >= 0 && j < S) ? j : 0)));
             }
             asm volatile("s_waitcnt lgkmcnt(0)"
                          : "+v"(tap[0]), "+v"(tap[1]), "+v"(tap[2]), "+v"(tap[3]), "+v"(tap[4]), "+v"(tap[5]), "+v"(tap[6]), "+v"(tap[7])
@@ -230,7 +233,7 @@ __global__ __launch_bounds__(X_WT, X_OCC) void conv_mix16_mfma(const T *__restri
         }
         if (tid == 0) lds_store16(table_lds + 16u * (unsigned)TAB_VECS, u32x4{0u, 0u, 0u, 0u});
         lds_wait();
-        wg_barrier();  // the table is complete; the staging area is free
+        wg_barrier();  // the table is complete
     }
 
     // this lane's Toeplitz vector: e = 8kg - ln; lanes outside the band read the vector of zeros
@@ -253,7 +256,7 @@ __global__ __launch_bounds__(X_WT, X_OCC) void conv_mix16_mfma(const T *__restri
         // h+1 .. h+NBUF-2 may stay in flight when their number of instructions is known (interior tiles).
         {
             constexpr int ahead = (h + NBUF - 2 < X_HG - 1 ? h + NBUF - 2 : X_HG - 1) - h;
-            static_assert(STAGE_IT * (NBUF - 2) <= 15, "vmcnt field");
+            static_assert(STAGE_IT * (NBUF - 2) <= 63, "vmcnt field");
             if (!interior || ahead == 0) asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
             else if (n_copy == STAGE_IT) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(ahead * STAGE_IT) : "memory");
             else if (n_copy == STAGE_IT - 1) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(ahead * (STAGE_IT - 1)) : "memory");
@@ -369,6 +372,7 @@ __global__ __launch_bounds__(X_WT, X_OCC) void conv_mix16_mfma(const T *__restri
     }
 
     // ---- stores through LDS: round v carries output head 4*og + v of every lane group og ----
+    wg_barrier();  // every wavefront is done with the last window: the buffers now stage the outputs
     // staging: [og][row 0..31][8 slots of 16 bytes], slot index XOR ((row >> 1) & 7)
     const int srow = rb0 + ln;
     const unsigned wbase = stage_lds + (unsigned)((kg * X_TM + srow) * (X_TN * (int)sizeof(T)));
@@ -432,7 +436,7 @@ int conv_mix16_dispatch(const void *x, const void *wc, const void *wm, void *y, 
     // MTA_CONV_MIX16_OFF=1 in the environment keeps groups of 16 heads on the other kernels (for comparisons)
     static const bool off = [] { const char *e = getenv("MTA_CONV_MIX16_OFF"); return e && e[0] == '1'; }();
     if (off || io_dtype == MTA_F32 || C % X_HG != 0 || W % 8 != 0 || !aligned_to(x, 16) || !aligned_to(y, 16) ||
-        !aligned_to(wm, 8) || !aligned_to(wc, 2))
+        !aligned_to(wm, 8) || !aligned_to(wc, 16))
         return MTA_ERR_UNSUPPORTED;
 #define MTA_XM_CASE(r, s)                                                                                            \
     static_assert(xgeom<r, s>::fits, "window exceeds 32 keys");                                                        \
