@@ -34,6 +34,14 @@ __device__ __forceinline__ u32x4 lds_load16(unsigned addr)
     asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
     return v;
 }
+// read and wait in one statement: the value is defined when the statement ends (for values that live across code the
+// compiler arranges freely)
+__device__ __forceinline__ u32x4 lds_load16_sync(unsigned addr)
+{
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+}
 // the same with a compile-time byte offset in the instruction (no address arithmetic per access)
 // (`off` must fold to a constant below 65536: it goes into the instruction's offset field)
 __device__ __forceinline__ u32x4 lds_load16_at(unsigned addr, int off)
