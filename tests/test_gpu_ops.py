@@ -358,6 +358,8 @@ CH_CASES = [
     # N, C, H(=W), R, S, group (None = dense)
     (1, 4, 64, 3, 3, 2), (2, 4, 100, 3, 3, 4), (1, 8, 264, 3, 3, 4), (1, 16, 136, 3, 3, None), (1, 16, 200, 7, 7, None),
     (1, 8, 72, 5, 7, 8), (1, 2, 33, 3, 5, 1), (1, 6, 50, 2, 2, 2), (1, 32, 96, 3, 3, 16),
+    # dense groups of 16 heads at 16-bit dtypes: conv and mixing on the matrix cores, several items per workgroup
+    (2, 32, 328, 7, 7, 16), (1, 16, 520, 5, 5, None), (1, 16, 776, 3, 3, None),
 ]
 
 
@@ -390,6 +392,33 @@ def test_conv_headmix_parity(ops, case, causal, dt):
     if dtype != torch.float32:
         got = ops.conv2d_headmix(x.cuda(), wc.cuda(), wm.float().cuda(), causal, group_size=group).cpu()
         torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("ks", [(3, 3), (7, 7)])
+def test_conv_headmix_dense16_equals_the_two_operators(ops, ks, dt):
+    """Dense groups of 16 heads at a benchmark-sized plane (B1 H16 S2048): the one-pass kernel against conv followed by
+    head mixing - the same products in the same order, so bit for bit on and below the diagonal - with the input above
+    the diagonal poisoned (it must never be read), in both fill modes and without the causal rule."""
+    dtype = DT[dt]
+    s, c = 2048, 16
+    print(f"conv_headmix dense16 ks={ks} dt={dt}", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.softmax(torch.randn(1, c, s, s, device="cuda", generator=g) * 2 +
+                      torch.triu(torch.full((s, s), float("-inf"), device="cuda"), 1), -1).to(dtype)
+    wc = (torch.randn(c, *ks, device="cuda", generator=g) * 0.3).to(dtype)
+    wm = (torch.randn(c, c, device="cuda", generator=g) * 0.3).to(dtype)
+    want = ops.headmix(ops.conv2d_causal(x, wc, True), wm, True, 0.0)
+    poisoned = x.masked_fill(torch.triu(torch.ones(s, s, dtype=torch.bool, device="cuda"), 1), float("nan"))
+    for fill in (True, False):
+        got = ops.conv2d_headmix(poisoned, wc, wm, True, fill_upper=fill)
+        assert got is not None
+        if fill:
+            assert torch.equal(got, want)
+        else:
+            assert torch.equal(torch.tril(got), torch.tril(want))
+    want = ops.headmix(ops.conv2d_causal(x, wc, False), wm, False, 0.0)
+    assert torch.equal(ops.conv2d_headmix(x, wc, wm, False), want)
 
 
 def test_conv_headmix_unsupported_group(ops):
