@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTA_ABI_VERSION 7
+#define MTA_ABI_VERSION 8
 
 enum mta_dtype { MTA_F32 = 0, MTA_BF16 = 1, MTA_F16 = 2 };
 
@@ -142,6 +142,15 @@ int mta_headmix_softmax_bias_fwd(const void *x, const void *w1, const void *w2, 
                                  int64_t N, int64_t C, int64_t P, int64_t Q, int group_size, int causal,
                                  int fill_upper, int io_dtype, int w_dtype, void *stream);
 
+/* The same under a band mask: first_visible is int32, (N,P); key q of query row p of batch entry n is hidden (its
+ * mixed score becomes -inf ahead of the softmax) when q < first_visible[n, p]; NULL = no band (identical to the entry
+ * point above).  With the causal rule this is the `scores + mask` of mta_attention_triton.py:77-78 for every mask of
+ * the form "row p sees the keys first_visible[p] .. p" - sliding windows, packed documents - without the (B,H,S,S)
+ * mask tensor.  key_bias may be given as well.  A row without a visible key comes out as NaN. */
+int mta_headmix_softmax_band_fwd(const void *x, const void *w1, const void *w2, const void *key_bias,
+                                 const void *first_visible, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
+                                 int group_size, int causal, int fill_upper, int io_dtype, int w_dtype, void *stream);
+
 /* Depthwise causal conv followed by head mixing, the conv result never written:
  *   t[h] = round(conv2d(x[h], w_conv[h]))                     as mta_conv2d_fwd
  *   y[o] = round(sum_h w_mix[o,h] t[h])                        as mta_headmix_fwd with fill 0
@@ -193,6 +202,14 @@ int mta_qk_conv_fwd(const void *q, const void *k, const void *w, void *s_out, in
  * caller choose between the one-kernel stage and matmul -> conv (mta_attention_triton.py:69-73) before it launches
  * anything.  Host-side only; needs no GPU. */
 int mta_qk_conv_supported(int64_t S, int64_t D, int R, int Sk, int io_dtype, int w_dtype);
+
+/* mta_qk_conv_fwd under a band mask (causal by construction): first_visible is int32, (B,S); the score of key k of
+ * query row p enters the conv as 0 unless first_visible[b, p] <= k <= p - the `scores.masked_fill(mask == -inf, 0)`
+ * ahead of the conv of mta_attention_triton.py:70-73 for masks of that form.  Same conditions and return codes as
+ * mta_qk_conv_fwd (mta_qk_conv_supported answers for both). */
+int mta_qk_conv_band_fwd(const void *q, const void *k, const void *w, const void *first_visible, void *s_out, int64_t B,
+                         int64_t H, int64_t S, int64_t D, int R, int Sk, float scale, int fill_upper, int io_dtype,
+                         int w_dtype, void *stream);
 
 /* O = P V with P (B,H,S,S), V (B,H,S,D), O (B,H,S,D).  When causal only keys q <= p of P are read
  * (what lies above the diagonal may be uninitialised).  Replaces torch.matmul(scores, xv) of

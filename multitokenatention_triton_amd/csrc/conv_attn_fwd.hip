@@ -445,14 +445,18 @@ struct item_table {
 // SCORES_ONLY: stop after the conv and write  conv(mask0(scale * Q K^T))  as an (S,S) plane per (batch, head)
 // (`O` is then the score tensor, V is unused).  Only q <= p is written when causal, plus +0 above the
 // diagonal when `fill_upper` is set.
-template <typename T, int D, int R, int SK, bool SCORES_ONLY, int NW>
-__global__ __launch_bounds__(64 * NW, SCORES_ONLY ? (R > 7 ? 2 : QK_OCC) : 2) void conv_attn_fwd_mfma(const T *__restrict__ Q, const T *__restrict__ K,
+// BAND (scores-only kernel): a mask of the form "key k of query row p is visible iff band_lo[b, p] <= k <= p" - the
+// scores of the hidden keys enter the conv as 0, as the reference's masked_fill ahead of its conv leaves them
+// (mta_attention_triton.py:70-73).
+template <typename T, int D, int R, int SK, bool SCORES_ONLY, int NW, bool BAND = false>
+__global__ __launch_bounds__(64 * NW, SCORES_ONLY ? ((R > 7 || (BAND && R >= 7)) ? 2 : QK_OCC) : 2) void conv_attn_fwd_mfma(const T *__restrict__ Q, const T *__restrict__ K,
                                                              const T *__restrict__ V, const T *__restrict__ Wt,
                                                              T *__restrict__ O, float *__restrict__ Lse, int S, int causal,
                                                              float scale, int H, int nqb, int fill_upper, int64_t total_wg,
                                                              int64_t per_xcd, int jc_len, int items_per_bh, int hpx,
-                                                             item_table tbl)
+                                                             item_table tbl, const int *__restrict__ band_lo)
 {
+    static_assert(!BAND || SCORES_ONLY, "the band mask belongs to the scores-only kernel");
     using G = fused_geom<R, SK, NW>;
     constexpr int F_NT = 64 * NW, F_SR = 32 * NW;
     constexpr int CPR = D / 8;                     // 16-byte chunks per K/V row
@@ -606,6 +610,21 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? (R > 7 ? 2 : QK_OCC) : 2) vo
             if (prow[rb] < 0 || prow[rb] >= S) qf[rb][ks] = zero_frag<T>();  // rows outside the sequence are conv padding
         }
     }
+    // band mask: first visible key of this lane's two rows, and the largest of them over the wavefront's 32 rows (a key
+    // block that starts at or beyond it is visible to all of them)
+    int flo[2] = {0, 0}, fmax_w = 0;
+    if constexpr (BAND) {
+        const int64_t brow = (bh / H) * (int64_t)S;
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) flo[rb] = (prow[rb] >= 0 && prow[rb] < S) ? band_lo[brow + prow[rb]] : 0;
+        int m = flo[0] > flo[1] ? flo[0] : flo[1];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const int o = __shfl_xor(m, off);
+            m = o > m ? o : m;
+        }
+        fmax_w = __builtin_amdgcn_readfirstlane(m);
+    }
     __syncthreads();
 
     // Toeplitz fragments T_i^T: accumulator row m = ln, slots k = 8*kg + t, tap = k - SHIFT - m
@@ -693,7 +712,8 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? (R > 7 ? 2 : QK_OCC) : 2) vo
             auto epilogue = [&](auto cbc) __attribute__((always_inline)) {
                 constexpr int cb = decltype(cbc)::value;
                 // key block wholly inside the sequence and on or below the diagonal for all 32 rows: no masks
-                const bool s_plain = PLAIN || (cbase + cb * 16 >= 0 && cbase + cb * 16 + 16 <= S && (!causal || cbase + cb * 16 + 15 <= pmin));
+                const bool s_plain = PLAIN || (cbase + cb * 16 >= 0 && cbase + cb * 16 + 16 <= S && (!causal || cbase + cb * 16 + 15 <= pmin) &&
+                                               (!BAND || cbase + cb * 16 >= fmax_w));
 #pragma unroll
                 for (int rb = 0; rb < 2; ++rb) {
                     const f32x4 a = sacc[cb & 1][rb];
@@ -709,10 +729,11 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? (R > 7 ? 2 : QK_OCC) : 2) vo
                         MTA_KEEP_BRANCH();
                         const int col = cbase + cb * 16 + kg * 4;
                         const int lim = causal ? (prow[rb] < S - 1 ? prow[rb] : S - 1) : S - 1;  // last key kept
-                        if (col < 0 || col > lim) lo &= 0xffff0000u;
-                        if (col + 1 < 0 || col + 1 > lim) lo &= 0x0000ffffu;
-                        if (col + 2 < 0 || col + 2 > lim) hi &= 0xffff0000u;
-                        if (col + 3 < 0 || col + 3 > lim) hi &= 0x0000ffffu;
+                        const int first = BAND ? (flo[rb] > 0 ? flo[rb] : 0) : 0;  // first key kept
+                        if (col < first || col > lim) lo &= 0xffff0000u;
+                        if (col + 1 < first || col + 1 > lim) lo &= 0x0000ffffu;
+                        if (col + 2 < first || col + 2 > lim) hi &= 0xffff0000u;
+                        if (col + 3 < first || col + 3 > lim) hi &= 0x0000ffffu;
                     }
                     // Two 16-key blocks go to the tile together.  A lane holds keys 4kg..4kg+3 of each; after the
                     // exchange between neighbouring lane groups (even groups give their second block's part and take
@@ -918,7 +939,7 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? (R > 7 ? 2 : QK_OCC) : 2) vo
     };
     auto plain = [&](int j) {  // (scores-only kernel: a second body per buffer rotation makes the attention kernel spill)
         const int cbase = j * F_BK + G::PWR;
-        return SCORES_ONLY && j >= 0 && cbase + F_BK <= S && (!causal || cbase + F_BK - 1 <= pmin);
+        return SCORES_ONLY && j >= 0 && cbase + F_BK <= S && (!causal || cbase + F_BK - 1 <= pmin) && (!BAND || cbase >= fmax_w);
     };
     if constexpr (SCORES_ONLY) {
         for (int j = j_start;;) {  // block(tag, j, K(j), V(j), where K(j+1) goes, where V(j+1) goes)
@@ -981,16 +1002,16 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? (R > 7 ? 2 : QK_OCC) : 2) vo
     }
 }
 
-template <typename T, int D, int R, int SK, bool SCORES_ONLY>
+template <typename T, int D, int R, int SK, bool SCORES_ONLY, bool BAND = false>
 int launch_mfma(const void *q, const void *k, const void *v, const void *w, void *o, float *lse, int64_t B, int64_t H,
-                int64_t S, int causal, float scale, int fill_upper, hipStream_t st)
+                int64_t S, int causal, float scale, int fill_upper, hipStream_t st, const int *band_lo = nullptr)
 {
     constexpr int NW = 4;
     constexpr int F_NT = 64 * NW;
     using G = fused_geom<R, SK, NW>;
     static_assert(G::fits, "conv window exceeds the 32-key MFMA contraction");
     const int nqb = (int)((S + G::BQ - 1) / G::BQ);
-    auto kern = conv_attn_fwd_mfma<T, D, R, SK, SCORES_ONLY, NW>;
+    auto kern = conv_attn_fwd_mfma<T, D, R, SK, SCORES_ONLY, NW, BAND>;
     // key blocks per work item: all of them for the attention kernel; QK_CHUNK for the scores-only kernel
     const int jc_len = SCORES_ONLY ? QK_CHUNK : (int)((S + F_BK - 1) / F_BK) + 1;
     int64_t items_per_bh = 0;
@@ -1045,18 +1066,18 @@ int launch_mfma(const void *q, const void *k, const void *v, const void *w, void
     dim3 grid((unsigned)(per_xcd * 8));
     hipLaunchKernelGGL(kern, grid, dim3(F_NT), 0, st, (const T *)q, (const T *)k, (const T *)v, (const T *)w, (T *)o,
                        lse, (int)S, causal, scale, (int)H, nqb, fill_upper, total_wg, per_xcd, jc_len, (int)items_per_bh,
-                       (B * H) % 8 == 0 ? (int)(B * H / 8) : 0, tbl);
+                       (B * H) % 8 == 0 ? (int)(B * H / 8) : 0, tbl, band_lo);
     return launch_status();
 }
 
 // returns 1 when no instantiation covers the kernel size (the caller then uses the general kernel)
-template <typename T, int D, bool SCORES_ONLY>
+template <typename T, int D, bool SCORES_ONLY, bool BAND = false>
 int dispatch_mfma(const void *q, const void *k, const void *v, const void *w, void *o, float *lse, int64_t B, int64_t H,
-                  int64_t S, int R, int Sk, int causal, float scale, int fill_upper, hipStream_t st)
+                  int64_t S, int R, int Sk, int causal, float scale, int fill_upper, hipStream_t st, const int *band_lo = nullptr)
 {
     if constexpr (sizeof(T) == 2) {
 #define MTA_FUSED_CASE(r, s) \
-    if (R == r && Sk == s) return launch_mfma<T, D, r, s, SCORES_ONLY>(q, k, v, w, o, lse, B, H, S, causal, scale, fill_upper, st);
+    if (R == r && Sk == s) return launch_mfma<T, D, r, s, SCORES_ONLY, BAND>(q, k, v, w, o, lse, B, H, S, causal, scale, fill_upper, st, band_lo);
         MTA_FUSED_CASE(3, 3)
         MTA_FUSED_CASE(5, 5)
         MTA_FUSED_CASE(5, 7)
@@ -1164,6 +1185,32 @@ extern "C" int mta_qk_conv_fwd(const void *q, const void *k, const void *w, void
                      : dispatch_mfma<io_t, 128, true>(q, k, nullptr, w, s_out, nullptr, B, H, S, R, Sk, causal, scale, fill_upper, st);
     });
     // (mta_qk_conv_supported must agree with the dispatch: a kernel size it names always has an instance)
+    if (rc == 1 && scores_instance(R, Sk)) return MTA_ERR_KERNEL_SIZE;
+    return rc == 1 ? MTA_ERR_UNSUPPORTED : rc;
+}
+
+// mta_qk_conv_fwd under a band mask: key k of query row p of batch entry b is visible iff first_visible[b, p] <= k <= p
+// (int32, (B, S)); the scores of hidden keys enter the conv as 0.  Causal by construction.
+extern "C" int mta_qk_conv_band_fwd(const void *q, const void *k, const void *w, const void *first_visible, void *s_out,
+                                    int64_t B, int64_t H, int64_t S, int64_t D, int R, int Sk, float scale, int fill_upper,
+                                    int io_dtype, int w_dtype, void *stream)
+{
+    if (!q || !k || !w || !s_out || !first_visible) return MTA_ERR_NULL;
+    if (!dtype_size(io_dtype) || !dtype_size(w_dtype)) return MTA_ERR_DTYPE;
+    if (B <= 0 || H <= 0 || S <= 0 || S > (1 << 24) || B * H > 65535) return MTA_ERR_SHAPE;
+    if (R < 1 || Sk < 1 || R > MTA_MAX_FUSED_KERNEL_R || Sk > MTA_MAX_FUSED_KERNEL_S) return MTA_ERR_KERNEL_SIZE;
+    if (D != 64 && D != 128) return MTA_ERR_HEAD_DIM;
+    if (!aligned_to(q, 16) || !aligned_to(k, 16) || !aligned_to(s_out, 16) || !aligned_to(w, dtype_size(w_dtype)) ||
+        !aligned_to(first_visible, 4))
+        return MTA_ERR_ALIGN;
+    if (io_dtype == MTA_F32 || w_dtype != io_dtype || S % 8 != 0) return MTA_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    const int *lo = (const int *)first_visible;
+    int rc = 1;
+    MTA_DISPATCH_IO(io_dtype, {
+        rc = D == 64 ? dispatch_mfma<io_t, 64, true, true>(q, k, nullptr, w, s_out, nullptr, B, H, S, R, Sk, 1, scale, fill_upper, st, lo)
+                     : dispatch_mfma<io_t, 128, true, true>(q, k, nullptr, w, s_out, nullptr, B, H, S, R, Sk, 1, scale, fill_upper, st, lo);
+    });
     if (rc == 1 && scores_instance(R, Sk)) return MTA_ERR_KERNEL_SIZE;
     return rc == 1 ? MTA_ERR_UNSUPPORTED : rc;
 }

@@ -113,13 +113,13 @@ template <int NT> __device__ __forceinline__ float block_sum(float v, float *red
 }
 
 // Register-resident row: Q <= NT*VEC*NV.
-// (KB: with a key bias.  An instantiation of its own, compiled without the occupancy target: the bias vector costs the
-// registers that target leaves none of.)
+// (KB: with a key bias and / or a first visible key per query row.  An instantiation of its own, compiled without the
+// occupancy target: the bias vector costs the registers that target leaves none of.)
 template <typename T, int G, int NV, int VEC, int NT, bool KB>
 __global__ __launch_bounds__(NT, (!KB && NT == 256 && G * NV == 8) ? RS_OCC : 1) void mix_softmax_mix(const T *__restrict__ x, const void *__restrict__ w1,
                                                       const void *__restrict__ w2, const float *__restrict__ kb,
                                                       T *__restrict__ y, int C, int P, int Q, int causal,
-                                                      int w_dtype, int fill_upper)
+                                                      int w_dtype, int fill_upper, const int *__restrict__ row_lo)
 {
     __shared__ float w1s[G * G];
     __shared__ float w2s[G * G];
@@ -201,21 +201,33 @@ __global__ __launch_bounds__(NT, (!KB && NT == 256 && G * NV == 8) ? RS_OCC : 1)
                 }
             }
         }
-        if constexpr (KB) {  // additive key bias of this batch entry (0 / -inf for a key mask), added in the I/O dtype
-            const int qs = (q <= last) ? q : 0;
-            float kbv[VEC];
+        if constexpr (KB) {
+            if (kb) {  // additive key bias of this batch entry (0 / -inf for a key mask), added in the I/O dtype
+                const int qs = (q <= last) ? q : 0;
+                float kbv[VEC];
 #pragma unroll
-            for (int u = 0; u < VEC; ++u) kbv[u] = kb[n * Q + qs + u];
+                for (int u = 0; u < VEC; ++u) kbv[u] = kb[n * Q + qs + u];
 #pragma unroll
-            for (int o = 0; o < G; ++o) {
+                for (int o = 0; o < G; ++o) {
 #pragma unroll
-                for (int u = 0; u < VEC; ++u) s[o][k][u] += kbv[u];
-                if constexpr (VEC % 2 == 0) {
+                    for (int u = 0; u < VEC; ++u) s[o][k][u] += kbv[u];
+                    if constexpr (VEC % 2 == 0) {
 #pragma unroll
-                    for (int u = 0; u < VEC; u += 2) round_pair<T>(s[o][k][u], s[o][k][u + 1]);
-                } else {
+                        for (int u = 0; u < VEC; u += 2) round_pair<T>(s[o][k][u], s[o][k][u + 1]);
+                    } else {
 #pragma unroll
-                    for (int u = 0; u < VEC; ++u) s[o][k][u] = round_to<T>(s[o][k][u]);
+                        for (int u = 0; u < VEC; ++u) s[o][k][u] = round_to<T>(s[o][k][u]);
+                    }
+                }
+            }
+            if (row_lo) {  // band mask: the keys ahead of the row's first visible one are hidden
+                const int lo = row_lo[n * P + p];
+                if (q < lo) {
+#pragma unroll
+                    for (int o = 0; o < G; ++o)
+#pragma unroll
+                        for (int u = 0; u < VEC; ++u)
+                            if (q + u < lo) s[o][k][u] = -INFINITY;
                 }
             }
         }
@@ -709,7 +721,7 @@ template <typename T, int NT>
 __global__ __launch_bounds__(NT) void mix_softmax_mix_any(const T *__restrict__ x, const void *__restrict__ w1,
                                                           const void *__restrict__ w2, const float *__restrict__ kb,
                                                           T *__restrict__ y, int C, int G, int P, int Q, int causal,
-                                                          int w_dtype, int fill_upper)
+                                                          int w_dtype, int fill_upper, const int *__restrict__ row_lo)
 {
     __shared__ float red[NT / 64];
     extern __shared__ float stats[];  // [G] max, [G] 1/sum
@@ -723,7 +735,9 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix_any(const T *__restrict__ 
     const int64_t base = (n * C + (int64_t)g * G) * plane + (int64_t)p * Q;
     const int last = causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;
 
+    const int lo = row_lo ? row_lo[n * P + p] : 0;  // first visible key of the row (band mask)
     auto mixed = [&](int o, int q) -> float {
+        if (q < lo) return -INFINITY;
         float acc;
         if (!w1) {
             acc = to_float(x[base + o * plane + q]);
@@ -765,24 +779,27 @@ __global__ __launch_bounds__(NT) void mix_softmax_mix_any(const T *__restrict__ 
 }
 
 template <typename T, int G, int NV, int NT = 256>
-int launch_fixed(const void *x, const void *w1, const void *w2, const float *kb, void *y, int64_t N, int64_t C, int64_t P,
-                 int64_t Q, int causal, int w_dtype, int fill_upper, hipStream_t st)
+int launch_fixed(const void *x, const void *w1, const void *w2, const float *kb, const int *row_lo, void *y, int64_t N, int64_t C,
+                 int64_t P, int64_t Q, int causal, int w_dtype, int fill_upper, hipStream_t st)
 {
     constexpr int VEC = vec_of<T>::n;
     const int64_t blocks = N * (C / G) * P;
-    if (kb)
+    if (kb || row_lo)
         hipLaunchKernelGGL((mix_softmax_mix<T, G, NV, VEC, NT, true>), dim3((unsigned)blocks), dim3(NT), 0, st, (const T *)x,
-                           w1, w2, kb, (T *)y, (int)C, (int)P, (int)Q, causal, w_dtype, fill_upper);
+                           w1, w2, kb, (T *)y, (int)C, (int)P, (int)Q, causal, w_dtype, fill_upper, row_lo);
     else
         hipLaunchKernelGGL((mix_softmax_mix<T, G, NV, VEC, NT, false>), dim3((unsigned)blocks), dim3(NT), 0, st, (const T *)x,
-                           w1, w2, kb, (T *)y, (int)C, (int)P, (int)Q, causal, w_dtype, fill_upper);
+                           w1, w2, kb, (T *)y, (int)C, (int)P, (int)Q, causal, w_dtype, fill_upper, row_lo);
     return launch_status();
 }
 
 template <typename T>
-int dispatch(const void *x, const void *w1, const void *w2, const float *kb, void *y, int64_t N, int64_t C, int64_t P,
-             int64_t Q, int G, int causal, int w_dtype, int fill_upper, hipStream_t st)
+int dispatch(const void *x, const void *w1, const void *w2, const float *kb_in, const int *row_lo, void *y, int64_t N, int64_t C,
+             int64_t P, int64_t Q, int G, int causal, int w_dtype, int fill_upper, hipStream_t st)
 {
+    // (the kernels without a key bias are the ones without a band mask too: `kb` below stands for "either")
+    const float *kb = kb_in;
+    const bool plain = !kb_in && !row_lo;
     constexpr int VEC = vec_of<T>::n;
     const bool vec_ok = (Q % VEC == 0) && aligned_to(x, 16) && aligned_to(y, 16);
     const int64_t nv = (Q + 256 * VEC - 1) / (256 * VEC);
@@ -791,11 +808,11 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb, voi
         // the general one, for comparisons)
         static const bool no_packed = [] { const char *e_ = getenv("MTA_SOFTMAX_NO_PACKED"); return e_ && e_[0] == '1'; }();
         const int io_code = std::is_same<T, bf16_t>::value ? MTA_BF16 : MTA_F16;
-        if (G == 16 && !kb && !no_packed) {
+        if (G == 16 && plain && !no_packed) {
             const int rc = mix16_softmax_launch(x, w1, w2, y, N, C, P, Q, causal, fill_upper, io_code, w_dtype, st);
             if (rc != MTA_ERR_UNSUPPORTED) return rc;
         }
-        if (vec_ok && !kb && !no_packed && w_dtype == io_code && (w1 || w2) && (!w1 || aligned_to(w1, 4)) &&
+        if (vec_ok && plain && !no_packed && w_dtype == io_code && (w1 || w2) && (!w1 || aligned_to(w1, 4)) &&
             (!w2 || aligned_to(w2, 4)) && C % 2 == 0 && Q <= 256 * VEC * 4) {
 #define MTA_RSP_LAUNCH(g, v, h1, h2, nt, occ)                                                                          \
     {                                                                                                                  \
@@ -821,7 +838,7 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb, voi
     }
     if (vec_ok) {
 #define MTA_RS_CASE(g, v)                                                                   \
-    if (G == g && nv <= v) return launch_fixed<T, g, v>(x, w1, w2, kb, y, N, C, P, Q, causal, w_dtype, fill_upper, st);
+    if (G == g && nv <= v) return launch_fixed<T, g, v>(x, w1, w2, kb, row_lo, y, N, C, P, Q, causal, w_dtype, fill_upper, st);
         MTA_RS_CASE(1, 1) MTA_RS_CASE(1, 2) MTA_RS_CASE(1, 4) MTA_RS_CASE(1, 8)
         MTA_RS_CASE(2, 1) MTA_RS_CASE(2, 2) MTA_RS_CASE(2, 4)
         MTA_RS_CASE(4, 1) MTA_RS_CASE(4, 2) MTA_RS_CASE(4, 4)
@@ -831,17 +848,17 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb, voi
     constexpr int NT = 256;
     const int64_t blocks = N * (C / G) * P;
     hipLaunchKernelGGL((mix_softmax_mix_any<T, NT>), dim3((unsigned)blocks), dim3(NT), sizeof(float) * 2 * G, st,
-                       (const T *)x, w1, w2, kb, (T *)y, (int)C, G, (int)P, (int)Q, causal, w_dtype, fill_upper);
+                       (const T *)x, w1, w2, kb, (T *)y, (int)C, G, (int)P, (int)Q, causal, w_dtype, fill_upper, row_lo);
     return launch_status();
 }
 }  // namespace
 
-extern "C" int mta_headmix_softmax_bias_fwd(const void *x, const void *w1, const void *w2, const void *key_bias,
-                                            void *y, int64_t N, int64_t C, int64_t P, int64_t Q, int group_size,
-                                            int causal, int fill_upper, int io_dtype, int w_dtype, void *stream)
+extern "C" int mta_headmix_softmax_band_fwd(const void *x, const void *w1, const void *w2, const void *key_bias,
+                                            const void *first_visible, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
+                                            int group_size, int causal, int fill_upper, int io_dtype, int w_dtype, void *stream)
 {
     if (!x || !y) return MTA_ERR_NULL;
-    if (key_bias && !aligned_to(key_bias, 4)) return MTA_ERR_ALIGN;
+    if ((key_bias && !aligned_to(key_bias, 4)) || (first_visible && !aligned_to(first_visible, 4))) return MTA_ERR_ALIGN;
     if (!dtype_size(io_dtype) || !dtype_size(w_dtype)) return MTA_ERR_DTYPE;
     if (N <= 0 || C <= 0 || P <= 0 || Q <= 0 || P > (1 << 24) || Q > (1 << 24) || C > 4096) return MTA_ERR_SHAPE;
     if (group_size < 0 || (group_size > 0 && C % group_size != 0)) return MTA_ERR_GROUP;
@@ -852,9 +869,17 @@ extern "C" int mta_headmix_softmax_bias_fwd(const void *x, const void *w1, const
     if (!w1 && !w2) G = 1;
     if (N * (C / G) * P > 0x7fffffffLL) return MTA_ERR_SHAPE;
     hipStream_t st = (hipStream_t)stream;
-    MTA_DISPATCH_IO(io_dtype, return dispatch<io_t>(x, w1, w2, (const float *)key_bias, y, N, C, P, Q, G, causal, w_dtype,
-                                                    fill_upper || !causal, st));
+    MTA_DISPATCH_IO(io_dtype, return dispatch<io_t>(x, w1, w2, (const float *)key_bias, (const int *)first_visible, y, N, C, P, Q,
+                                                    G, causal, w_dtype, fill_upper || !causal, st));
     return MTA_ERR_DTYPE;
+}
+
+extern "C" int mta_headmix_softmax_bias_fwd(const void *x, const void *w1, const void *w2, const void *key_bias,
+                                            void *y, int64_t N, int64_t C, int64_t P, int64_t Q, int group_size,
+                                            int causal, int fill_upper, int io_dtype, int w_dtype, void *stream)
+{
+    return mta_headmix_softmax_band_fwd(x, w1, w2, key_bias, nullptr, y, N, C, P, Q, group_size, causal, fill_upper, io_dtype,
+                                        w_dtype, stream);
 }
 
 extern "C" int mta_headmix_softmax_fwd(const void *x, const void *w1, const void *w2, void *y, int64_t N,

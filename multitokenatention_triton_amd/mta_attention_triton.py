@@ -298,9 +298,12 @@ class MTAAttentionTriton(nn.Module):
             return self._forward_stagewise(xq, xk, xv)
         return self._forward_fused(xq, xk, xv)
 
-    def _forward_fused(self, xq, xk, xv, key_bias=None):
+    def _forward_fused(self, xq, xk, xv, key_bias=None, first_visible=None):
         """Inference route (module docstring).  ``key_bias``: fp32 (B,Sk), added to the mixed scores ahead of the
-        softmax -- the caller has zeroed the K and V rows of the keys it hides."""
+        softmax -- the caller has zeroed the K and V rows of the keys it hides.  ``first_visible``: int32 (B,S), a band
+        mask (row p sees the keys first_visible[p] .. p): applied to the scores inside the first kernel and as -inf
+        inside the softmax kernel; the caller has checked that the first kernel exists and that the post-softmax conv
+        is the identity."""
         head_dim = xq.size(-1)
         # the reference multiplies by rsqrt(tensor(head_dim)), an fp32 scalar (mta_attention_triton.py:69-71)
         scale = float(torch.rsqrt(torch.tensor(float(head_dim))))
@@ -317,9 +320,10 @@ class MTAAttentionTriton(nn.Module):
         post_conv_identity = st.post_conv_identity
         n_keys = xk.size(-2)
         g_both = _lcm(g_pre, g_post)
-        # (the matrix-core variant for groups of 16 takes no key bias)
+        # (the matrix-core variant for groups of 16 takes neither a key bias nor a band mask)
+        row_plain = key_bias is None and first_visible is None
         one_pass = (post_conv_identity and _one_pass_group(g_both, xq.dtype, n_keys, w1, w2)
-                    and (key_bias is None or g_both <= _FUSED_MAX_GROUP))
+                    and (row_plain or g_both <= _FUSED_MAX_GROUP))
         # the last stage may leave the upper triangle unwritten only if our own P V kernel consumes it
         own_pv = (xq.size(-2) == xk.size(-2) and xq.dtype == xv.dtype
                   and ops.causal_pv_supported(xq.dtype, xq.size(-2), xv.size(-1)))
@@ -328,8 +332,10 @@ class MTAAttentionTriton(nn.Module):
         scores = None
         if ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight):
             self._mark("qk_conv")
-            scores = ops.qk_conv(xq, xk, self.mta_conv_triton.weight, self.causal, scale, fill_upper=False)
+            scores = ops.qk_conv(xq, xk, self.mta_conv_triton.weight, self.causal, scale, fill_upper=False,
+                                 first_visible=first_visible)
         if scores is None:
+            assert first_visible is None, "the band mask needs the one-kernel first stage"
             self._mark("qk")
             scores = torch.matmul(xq, xk.transpose(2, 3))
             self._mark("conv_pre")
@@ -338,11 +344,12 @@ class MTAAttentionTriton(nn.Module):
         if one_pass:
             self._mark("mix_softmax_mix")
             scores = ops.headmix_softmax(scores, w1, w2, self.causal, group_size=g_both,
-                                         fill_upper=not own_pv, key_bias=key_bias)
+                                         fill_upper=not own_pv, key_bias=key_bias, first_visible=first_visible)
         else:
-            if _one_pass_group(g_pre, xq.dtype, n_keys, w1) and (key_bias is None or g_pre <= _FUSED_MAX_GROUP):
+            if _one_pass_group(g_pre, xq.dtype, n_keys, w1) and (row_plain or g_pre <= _FUSED_MAX_GROUP):
                 self._mark("mix_softmax")
                 scores = ops.headmix_softmax(scores, w1, None, self.causal, group_size=g_pre, key_bias=key_bias,
+                                             first_visible=first_visible,
                                              fill_upper=post_conv_identity and w2 is None and not own_pv)
             else:
                 self._mark("mix_pre")
@@ -351,6 +358,7 @@ class MTAAttentionTriton(nn.Module):
                 scores = ops.headmix(scores, w_pre, self.causal, fill, group_size=g_pre, fill_upper=False)
                 self._mark("softmax")
                 scores = ops.headmix_softmax(scores, None, None, self.causal, key_bias=key_bias,
+                                             first_visible=first_visible,
                                              fill_upper=post_conv_identity and w2 is None and not own_pv)
             done = None
             # conv and mix in one pass, the conv result never written: taken where it measures at least as fast as the
@@ -489,6 +497,13 @@ class MTAAttentionTriton(nn.Module):
                 hidden = (bias == float("-inf"))[:, None, :, None]
                 return self._forward_fused(xq, xk.masked_fill(hidden, 0), xv.masked_fill(hidden, 0),
                                            key_bias=bias.contiguous())
+            # a band mask - the same for all heads, row p seeing the keys first[p] .. p (sliding windows, packed
+            # documents) - goes into the kernels as one int32 per (batch entry, row)
+            if (mask.dim() == 4 and self._current_structure().post_conv_identity
+                    and ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight)):
+                first = self._band_of_mask(mask, xq.size(0), xq.size(-2))
+                if first is not None:
+                    return self._forward_fused(xq, xk, xv, first_visible=first)
         mask = self._update_mask(mask=mask, bsz=xq.size(0), xq=xq, xk_size=xk.size(-2))
         scale = float(torch.rsqrt(torch.tensor(float(xq.size(-1)))))  # a host scalar: the product stays one vectorised pass
         scores = torch.matmul(xq, xk.transpose(2, 3)) * scale
@@ -502,6 +517,33 @@ class MTAAttentionTriton(nn.Module):
         scores = self.wposm_triton(scores)
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         return torch.matmul(scores, xv).transpose(1, 2)
+
+    def _band_of_mask(self, mask, bsz: int, s: int):
+        """int32 (B,S) first visible key per query row when ``mask`` (4-D, bool with True = attend, or additive with
+        0 / -inf) together with the causal rule has the form "row p sees the keys first[p] .. p" for every row, the same
+        for all heads; else None.  The answer for the last mask seen is kept (same storage, same version)."""
+        if mask.size(1) != 1 or mask.size(0) not in (1, bsz) or mask.size(-2) != s or mask.size(-1) != s:
+            return None
+        key = (mask._version, bsz)
+        cached = getattr(self, "_band_cache", None)   # (the mask object itself is kept: its identity cannot be reused)
+        if cached is not None and cached[0] is mask and cached[1] == key:
+            return cached[2]
+        if mask.dtype == torch.bool:
+            visible = mask[:, 0]
+        else:
+            visible = mask[:, 0] == 0
+            if not bool(((mask[:, 0] == float("-inf")) | visible).all()):
+                visible = None   # other finite values: not a 0 / -inf mask
+        first = None
+        if visible is not None:
+            rows = torch.arange(s, device=mask.device)
+            visible = visible & (rows[None, :] <= rows[:, None])
+            count = visible.sum(-1)
+            lead = visible.int().argmax(-1)
+            if bool(((count >= 1) & (count == rows[None, :] - lead + 1)).all()):
+                first = lead.to(torch.int32).expand(bsz, s).contiguous()
+        self._band_cache = (mask, key, first)
+        return first
 
     def _update_mask(self, mask, bsz: int, xq: torch.Tensor, xk_size: int):
         """Additive (B,H,Sq,Sk) mask, 0 = attend, -inf = blocked (mta_attention_triton.py:106-127)."""

@@ -190,8 +190,12 @@ def headmix_bwd_weight(x: torch.Tensor, dy: torch.Tensor, causal: bool = True) -
 
 def headmix_softmax(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optional[torch.Tensor], causal: bool = True,
                     group_size: Optional[int] = None, out: Optional[torch.Tensor] = None,
-                    fill_upper: bool = True, key_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    fill_upper: bool = True, key_bias: Optional[torch.Tensor] = None,
+                    first_visible: Optional[torch.Tensor] = None) -> torch.Tensor:
     """mix(w1) -> causal row softmax -> mix(w2) in one pass; see mta_headmix_softmax_fwd.
+
+    ``first_visible``: int32 (N,P), the first visible key of every query row (band mask); see
+    mta_headmix_softmax_band_fwd.
 
     ``fill_upper=False`` leaves everything above the diagonal unwritten (for consumers that never read it).
     ``key_bias``: fp32 (N,Q), added to the mixed scores ahead of the softmax (0 = keep, -inf = key hidden); see
@@ -214,14 +218,20 @@ def headmix_softmax(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optional[to
         key_bias = _device_tensor(key_bias, "key_bias")
         if key_bias.dtype != torch.float32 or tuple(key_bias.shape) != (n, q):
             raise ValueError(f"key_bias must be fp32 of shape ({n},{q}), got {key_bias.dtype} {tuple(key_bias.shape)}")
+    if first_visible is not None:
+        first_visible = _device_tensor(first_visible, "first_visible")
+        if first_visible.dtype != torch.int32 or tuple(first_visible.shape) != (n, p):
+            raise ValueError(f"first_visible must be int32 of shape ({n},{p}), got {first_visible.dtype} "
+                             f"{tuple(first_visible.shape)}")
     y = _out_like(x, out)
     with torch.cuda.device(x.device):
-        rc = _lib.load().mta_headmix_softmax_bias_fwd(
+        rc = _lib.load().mta_headmix_softmax_band_fwd(
             x.data_ptr(), ws[0].data_ptr() if ws[0] is not None else None,
             ws[1].data_ptr() if ws[1] is not None else None, key_bias.data_ptr() if key_bias is not None else None,
+            first_visible.data_ptr() if first_visible is not None else None,
             y.data_ptr(), n, c, p, q, int(group_size or 0), int(bool(causal)), int(bool(fill_upper)), _code(x, "input"),
             wcode, _stream(x))
-    _lib.check(rc, "mta_headmix_softmax_bias_fwd")
+    _lib.check(rc, "mta_headmix_softmax_band_fwd")
     return y
 
 
@@ -297,8 +307,12 @@ def conv_attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, weight: tor
 
 
 def qk_conv(q: torch.Tensor, k: torch.Tensor, weight: torch.Tensor, causal: bool, scale: float,
-            fill_upper: bool = True, out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+            fill_upper: bool = True, out: Optional[torch.Tensor] = None,
+            first_visible: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """scale * conv(mask0(Q K^T)) as a (B,H,S,S) tensor without materialising Q K^T; see mta_qk_conv_fwd.
+
+    ``first_visible``: int32 (B,S), band mask (requires ``causal``): key k of row p counts only when
+    first_visible[b,p] <= k <= p; see mta_qk_conv_band_fwd.
 
     Returns ``None`` when the library has no kernel for this dtype / size combination (the caller then
     takes matmul + conv2d_causal).  With ``fill_upper=False`` entries above the diagonal are left unwritten."""
@@ -313,10 +327,22 @@ def qk_conv(q: torch.Tensor, k: torch.Tensor, weight: torch.Tensor, causal: bool
         out = torch.empty((b, h, s, s), dtype=q.dtype, device=q.device)
     elif out.shape != (b, h, s, s) or out.dtype != q.dtype or out.device != q.device or not out.is_contiguous():
         raise ValueError("out must be a contiguous (B,H,S,S) tensor of the inputs' dtype and device")
+    if first_visible is not None:
+        if not causal:
+            raise ValueError("a band mask implies the causal rule")
+        first_visible = _device_tensor(first_visible, "first_visible")
+        if first_visible.dtype != torch.int32 or tuple(first_visible.shape) != (b, s):
+            raise ValueError(f"first_visible must be int32 of shape ({b},{s}), got {first_visible.dtype} "
+                             f"{tuple(first_visible.shape)}")
     with torch.cuda.device(q.device):
-        rc = _lib.load().mta_qk_conv_fwd(q.data_ptr(), k.data_ptr(), weight.data_ptr(), out.data_ptr(), b, h, s, d,
-                                         weight.shape[1], weight.shape[2], int(bool(causal)), float(scale),
-                                         int(bool(fill_upper)), _code(q, "Q"), _code(weight, "W"), _stream(q))
+        if first_visible is not None:
+            rc = _lib.load().mta_qk_conv_band_fwd(q.data_ptr(), k.data_ptr(), weight.data_ptr(), first_visible.data_ptr(),
+                                                  out.data_ptr(), b, h, s, d, weight.shape[1], weight.shape[2], float(scale),
+                                                  int(bool(fill_upper)), _code(q, "Q"), _code(weight, "W"), _stream(q))
+        else:
+            rc = _lib.load().mta_qk_conv_fwd(q.data_ptr(), k.data_ptr(), weight.data_ptr(), out.data_ptr(), b, h, s, d,
+                                             weight.shape[1], weight.shape[2], int(bool(causal)), float(scale),
+                                             int(bool(fill_upper)), _code(q, "Q"), _code(weight, "W"), _stream(q))
     if rc in (_lib.MTA_ERR_UNSUPPORTED, -7):
         return None
     _lib.check(rc, "mta_qk_conv_fwd")

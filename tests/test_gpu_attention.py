@@ -250,6 +250,125 @@ def test_qk_conv_parity(pkg, case, fill):
             assert (got[..., 0, s - 64:].float() == torch.tensor(sentinel).to(dtype).float()).all()
 
 
+def _band_first(kind, b, s, seed=3):
+    """int32 (B,S) first visible key per row: a sliding window, packed documents (per batch entry), or ragged."""
+    rows = torch.arange(s)
+    if kind == "window":
+        return (rows - 99).clamp(min=0).to(torch.int32).expand(b, s).contiguous()
+    g = torch.Generator().manual_seed(seed)
+    if kind == "documents":   # a document starts where the random cut points fall; a row sees its own document
+        out = torch.zeros(b, s, dtype=torch.int32)
+        for i in range(b):
+            cuts = torch.sort(torch.randint(1, s, (5,), generator=g)).values
+            start = torch.zeros(s, dtype=torch.int64)
+            for c in cuts.tolist():
+                start[c:] = c
+            out[i] = start.to(torch.int32)
+        return out
+    lo = (torch.rand(b, s, generator=g) * (rows + 1)[None, :]).floor().to(torch.int32)   # any value in 0 .. row
+    return torch.minimum(lo, rows.to(torch.int32)[None, :]).contiguous()
+
+
+BAND_CASES = [
+    # B, H, S, D, R, Sk, dtype, kind
+    (1, 2, 520, 64, 3, 3, torch.bfloat16, "window"), (2, 2, 776, 128, 6, 11, torch.bfloat16, "documents"),
+    (1, 2, 264, 128, 7, 7, torch.float16, "ragged"), (2, 1, 2048, 128, 6, 11, torch.bfloat16, "window"),
+    (1, 2, 520, 64, 11, 15, torch.float16, "documents"), (1, 1, 1160, 64, 5, 5, torch.bfloat16, "ragged"),
+]
+
+
+@pytest.mark.parametrize("case", BAND_CASES)
+def test_qk_conv_band_parity(pkg, case):
+    """The first stage under a band mask: the scores of the keys a row does not see are 0 on the way into the conv
+    (mta_attention_pytorch.py:63-67 with a mask tensor), here from one int32 per (batch entry, row)."""
+    b, h, s, d, r, sk, dtype, kind = case
+    print(f"qk_conv band case={case}", flush=True)
+    q, k, _ = O.seeded_qkv(b, h, s, d, dtype, seed=8)
+    w = O.seeded_conv_weight(h, r, sk, 0.05, dtype)
+    first = _band_first(kind, b, s)
+    keys = torch.arange(s)
+    visible = (keys[None, None, :] >= first[:, :, None]) & (keys[None, None, :] <= keys[None, :, None])   # (B,S,S)
+    scale = float(torch.rsqrt(torch.tensor(float(d))))
+    s0 = torch.matmul(q, k.transpose(2, 3)) * torch.rsqrt(torch.tensor(d))
+    want = O.depthwise_conv(s0.masked_fill(~visible[:, None], 0), w, True)
+    got = pkg.ops.qk_conv(q.cuda(), k.cuda(), w.cuda(), True, scale, fill_upper=True, first_visible=first.cuda()).cpu()
+    low = torch.tril(torch.ones(s, s, dtype=torch.bool))
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    torch.testing.assert_close(got[..., low].float(), want[..., low].float(), rtol=2 * ulp, atol=2e-2)
+    assert (got[..., ~low] == 0).all()
+    # no band at all is the plain kernel, bit for bit
+    zero = torch.zeros(b, s, dtype=torch.int32, device="cuda")
+    plain = pkg.ops.qk_conv(q.cuda(), k.cuda(), w.cuda(), True, scale, fill_upper=True)
+    assert torch.equal(pkg.ops.qk_conv(q.cuda(), k.cuda(), w.cuda(), True, scale, fill_upper=True, first_visible=zero), plain)
+    with pytest.raises(ValueError):
+        pkg.ops.qk_conv(q.cuda(), k.cuda(), w.cuda(), False, scale, first_visible=zero)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("group,s", [(4, 520), (2, 2304), (8, 264), (1, 1000), (16, 136)])
+def test_headmix_softmax_band_parity(pkg, group, s, dtype):
+    """mix -> `scores + mask` -> softmax -> mix (mta_attention_triton.py:75-85) for a band mask given as the first
+    visible key of every row."""
+    print(f"headmix_softmax band group={group} s={s} {dtype}", flush=True)
+    n, c = 2, 16
+    g = torch.Generator().manual_seed(13)
+    x = (torch.randn(n, c, s, s, generator=g) * 2).to(dtype)
+    w1 = O.block_diag_head_weight(c, group, 0.1, g, dtype)
+    w2 = O.block_diag_head_weight(c, group, 0.1, g, dtype)
+    first = _band_first("ragged", n, s, seed=5)
+    keys = torch.arange(s)
+    hidden = keys[None, None, :] < first[:, :, None]                                     # (N,S,S)
+    s2 = O.head_linear(x, w1, True, float("-inf")).masked_fill(hidden[:, None], float("-inf"))
+    p0 = torch.softmax(s2.float(), -1).to(dtype)
+    want = O.head_linear(p0, w2, True, 0.0)
+    got = pkg.ops.headmix_softmax(x.cuda(), w1.cuda(), w2.cuda(), True, group_size=group, first_visible=first.cuda()).cpu()
+    up = torch.triu(torch.ones(s, s, dtype=torch.bool), 1)
+    assert (got[..., up] == 0).all()
+    t = tol(dtype)
+    torch.testing.assert_close(got.float(), want.float(), rtol=t["rtol"] * 2, atol=2e-3 if dtype != torch.float32 else 1e-6)
+    # a band that hides nothing is the entry point without one
+    zero = torch.zeros(n, s, dtype=torch.int32, device="cuda")
+    a = pkg.ops.headmix_softmax(x.cuda(), w1.cuda(), w2.cuda(), True, group_size=group, first_visible=zero)
+    torch.testing.assert_close(a.float().cpu(), pkg.ops.headmix_softmax(x.cuda(), w1.cuda(), w2.cuda(), True, group_size=group).float().cpu(),
+                               rtol=t["rtol"] * 2, atol=2e-3 if dtype != torch.float32 else 1e-6)
+
+
+@pytest.mark.parametrize("kind", ["window", "documents"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mta_use_mask_band_masks_run_through_the_kernels(pkg, kind, dtype):
+    """use_mask=True with a (B,1,S,S) mask of the form "row p sees the keys first[p] .. p" (sliding window, packed
+    documents), bool and additive: the mask becomes one int32 per (batch entry, row) and the forward stays on the
+    three-kernel route; against the oracle given the mask tensor (mta_attention_triton.py:63-64, 77-83, 96-127)."""
+    print(f"mta use_mask band {kind} {dtype}", flush=True)
+    b, h, s, d = 2, 4, 1032, 64
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=96)
+    params = _config_like(h, 2, 6, 11, 0.05, dtype, post="identity")
+    first = _band_first(kind, b, s)
+    keys = torch.arange(s)
+    visible = ((keys[None, None, :] >= first[:, :, None]) & (keys[None, None, :] <= keys[None, :, None]))[:, None]   # (B,1,S,S)
+    additive = torch.where(visible, 0.0, float("-inf")).to(dtype)
+    want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3],
+                         mask=additive.expand(b, h, s, s).contiguous())
+    assert torch.isfinite(want.float()).all()
+    mod = _mta_module(pkg, h, 6, 11, 3, 3, *params, dtype, use_mask=True, structure="infer")
+    for mask in (visible, additive):
+        stages = []
+        mod._stage_hook = stages.append
+        got = mod(q.cuda(), k.cuda(), v.cuda(), mask.cuda(), None).cpu()
+        assert stages == ["qk_conv", "mix_softmax_mix", "pv", "end"]
+        torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+    # a mask with a hole in a row is no band: the elementwise route (no stage marks), same values as the oracle's
+    holed = visible.clone()
+    holed[0, 0, 700:, 650] = False
+    want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3],
+                         mask=torch.where(holed, 0.0, float("-inf")).to(dtype).expand(b, h, s, s).contiguous())
+    stages = []
+    mod._stage_hook = stages.append
+    got = mod(q.cuda(), k.cuda(), v.cuda(), holed.cuda(), None).cpu()
+    assert "qk_conv" not in stages
+    torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+
+
 def test_qk_conv_reports_unsupported(pkg):
     q = torch.zeros(1, 2, 64, 64, device="cuda")
     assert pkg.ops.qk_conv(q, q, torch.zeros(2, 3, 3, device="cuda"), True, 0.1) is None          # fp32
@@ -554,8 +673,9 @@ def test_mta_use_mask_tensor_masks(pkg, name, dtype):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("group", [4, 16])
 def test_mta_general_route_is_four_stages(pkg, group, dtype):
-    """All four MTA weights non-trivial (what training produces).  Mixing groups of 4: QK^T+conv, mix+softmax, conv+mix,
-    P V -- four kernels, the score tensor written three times and read three times.  Dense 16x16 weights: five kernels."""
+    """All four MTA weights non-trivial (what training produces): QK^T+conv, mix+softmax, conv+mix, P V -- four
+    kernels, the score tensor written three times and read three times -- for mixing groups of 4 and for dense 16x16
+    weights."""
     print(f"mta general route group={group} {dtype}", flush=True)
     h, s, d = 16, 520, 64
     q, k, v = O.seeded_qkv(1, h, s, d, dtype, seed=97)
@@ -566,10 +686,9 @@ def test_mta_general_route_is_four_stages(pkg, group, dtype):
         stages = []
         mod._stage_hook = stages.append
         got = mod(q.cuda(), k.cuda(), v.cuda(), None, None).cpu()
-        if group <= 4 and structure == "infer":
-            assert stages == ["qk_conv", "mix_softmax", "conv_mix_post", "pv", "end"]
-        else:   # 16-head mixing groups (16-bit data): mix + softmax in one pass on the matrix cores; conv, then mix
-            assert stages == ["qk_conv", "mix_softmax", "conv_post", "mix_post", "pv", "end"]
+        # mixing groups of up to 4 heads, and dense groups of 16 at 16-bit dtypes (both halves on the matrix cores): the
+        # post-softmax conv and the head mixing are one kernel
+        assert stages == ["qk_conv", "mix_softmax", "conv_mix_post", "pv", "end"]
         torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
 
 
