@@ -307,6 +307,22 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
         ms = time_steps(torch, lambda i: mod(*sets[i], None, None), len(sets), min(warmup, 10), max(3, steps // 5))
         out[label] = {"ms": ms, "stages_ms": stage_breakdown(torch, mod, sets, 3), "note": "forward only; " + note}
         del mod, sets
+    # the headline forward under a sliding-window mask (each row sees its last 1024 keys), given to the module as a
+    # (1,1,S,S) boolean mask tensor: it travels to the kernels as one int32 per (batch entry, row)
+    mod, sets = build_c4(torch, mta, O, device)
+    mod.use_mask = True
+    s_len = sets[0][0].size(2)
+    pos = torch.arange(s_len, device=device)
+    window = ((pos[None, :] <= pos[:, None]) & (pos[None, :] > pos[:, None] - 1024))[None, None]
+    ms = time_steps(torch, lambda i: mod(*sets[i], window, None), len(sets), min(warmup, 30), max(3, steps // 2))
+    stages = []
+    mod._stage_hook = stages.append
+    mod(*sets[0], window, None)
+    mod._stage_hook = None
+    out["mta_forward_bf16_2x16x4096x128_window1024_mask"] = {
+        "ms": ms, "stages": stages,
+        "note": "the headline configuration with use_mask=True and a sliding-window mask tensor; not a row of the reference's"}
+    del mod, sets, window
     # the first module and shape in training: forward operator by operator (each with its HIP backward kernels; the two
     # matrix products, the softmax and the dropout are torch's) and backward to q, k, v and the four weights
     mod, sets = build_general(torch, mta, O, device, train=True)

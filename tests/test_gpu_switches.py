@@ -23,6 +23,8 @@ GROUPS = [
     ({"MTA_CONV_FORCE_VALU": "1"},
      ["tests/test_gpu_ops.py", "tests/test_gpu_backward.py"],
      "test_conv_parity or test_conv_identity_tap or test_conv_backward_parity"),
+    # dense groups of 16 heads in the one-pass conv + mixing entry point on the vector-ALU kernel
+    ({"MTA_CONV_MIX16_OFF": "1"}, ["tests/test_gpu_ops.py"], "test_conv_headmix_parity"),
 ]
 
 
