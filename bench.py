@@ -302,6 +302,12 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
             ("mta_forward_general_fp16_1x128x2048x64_7x7_pre_post_dense",
              dict(b=1, h=128, s=2048, d=64, dtype=torch.float16, ks=(7, 7)),
              "the reference's published row for this shape (Triton 22.579 ms, PyTorch 115.382 ms, hardware unstated) is "
+             "context, not a baseline"),
+            # fp32, the dtype of most of the reference's published rows: no one-kernel scores stage and no triangle-only
+            # P V (library GEMMs), fp32-FMA conv kernels (benchmark_seq_len_results.jsonl:1)
+            ("mta_forward_general_fp32_1x16x1024x64_11x15_pre_post_dense",
+             dict(b=1, h=16, s=1024, d=64, dtype=torch.float32, ks=(11, 15)),
+             "the reference's published row for this shape (Triton 1.887 ms, PyTorch 4.203 ms, hardware unstated) is "
              "context, not a baseline")):
         mod, sets = build_general(torch, mta, O, device, **kw)
         ms = time_steps(torch, lambda i: mod(*sets[i], None, None), len(sets), min(warmup, 10), max(3, steps // 5))

@@ -205,8 +205,10 @@ int mta_qk_conv_supported(int64_t S, int64_t D, int R, int Sk, int io_dtype, int
 
 /* mta_qk_conv_fwd under a band mask (causal by construction): first_visible is int32, (B,S); the score of key k of
  * query row p enters the conv as 0 unless first_visible[b, p] <= k <= p - the `scores.masked_fill(mask == -inf, 0)`
- * ahead of the conv of mta_attention_triton.py:70-73 for masks of that form.  Same conditions and return codes as
- * mta_qk_conv_fwd (mta_qk_conv_supported answers for both). */
+ * ahead of the conv of mta_attention_triton.py:70-73 for masks of that form.  What is defined are the outputs at visible
+ * positions; elsewhere below the diagonal the output is unspecified (key blocks ahead of the first key any row of a query
+ * block sees are not even visited).  Same conditions and return codes as mta_qk_conv_fwd (mta_qk_conv_supported answers
+ * for both). */
 int mta_qk_conv_band_fwd(const void *q, const void *k, const void *w, const void *first_visible, void *s_out, int64_t B,
                          int64_t H, int64_t S, int64_t D, int R, int Sk, float scale, int fill_upper, int io_dtype,
                          int w_dtype, void *stream);
@@ -217,6 +219,12 @@ int mta_qk_conv_band_fwd(const void *q, const void *k, const void *w, const void
  * else returns MTA_ERR_UNSUPPORTED. */
 int mta_causal_pv_fwd(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int64_t D,
                       int causal, int io_dtype, void *stream);
+
+/* The same under a band mask: first_visible is int32, (B,S), or NULL; P[b,h,p,k] must be 0 for k < first_visible[b,p]
+ * (what mta_headmix_softmax_band_fwd leaves there), and the key blocks ahead of the first key any row of a block of 128
+ * query rows sees are not read.  Requires causal when first_visible is given. */
+int mta_causal_pv_band_fwd(const void *p, const void *v, const void *first_visible, void *o, int64_t B, int64_t H,
+                           int64_t S, int64_t D, int causal, int io_dtype, void *stream);
 
 /* The transposed product, O[k,:] = sum_p P[p,k] X[p,:] with P (B,H,S,S), X and O (B,H,S,D); when causal only query rows
  * p >= k take part and nothing of P above the diagonal is read.  These are the gradients the two matrix products of the

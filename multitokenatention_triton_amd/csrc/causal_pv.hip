@@ -35,7 +35,7 @@ constexpr int P_KS = P_BK / 32;  // 32-key contraction steps per iteration
 template <typename T, int D>
 __global__ __launch_bounds__(P_NT, P_OCC) void causal_pv_kernel(const T *__restrict__ P, const T *__restrict__ V,
                                                            T *__restrict__ O, int S, int causal, int nqb, int64_t total_wg,
-                                                           int64_t per_xcd)
+                                                           int64_t per_xcd, const int *__restrict__ band_lo, int H)
 {
     constexpr int CPR = D / 8;               // 16-byte chunks per V row
     constexpr int TILE = P_BK * D;           // elements per V block
@@ -107,10 +107,31 @@ __global__ __launch_bounds__(P_NT, P_OCC) void causal_pv_kernel(const T *__restr
 
     const int q_last = (q0 + P_BQ - 1 < S - 1) ? q0 + P_BQ - 1 : S - 1;
     const int j_end = causal ? q_last / P_BK : (S - 1) / P_BK;
-    issue_v(0, v_a);
+    // band mask (band_lo[b, p]: first key row p sees, P is 0 ahead of it): the key blocks ahead of the first key any row
+    // of this query block sees are not visited (every wavefront reduces all the rows: the same answer in each)
+    int j0 = 0;
+    if (band_lo) {
+        const int64_t brow = (bh / H) * (int64_t)S;
+        int fmin = S;
+        for (int r = lane; r < P_BQ; r += 64) {
+            if (q0 + r < S) {
+                const int f = band_lo[brow + q0 + r];
+                fmin = f < fmin ? f : fmin;
+            }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const int o = __shfl_xor(fmin, off);
+            fmin = o < fmin ? o : fmin;
+        }
+        fmin = __builtin_amdgcn_readfirstlane(fmin);
+        j0 = (fmin > 0 ? fmin : 0) / P_BK;
+        if (j0 > j_end) j0 = j_end;
+    }
+    issue_v(j0, v_a);
     // P fragments are fetched one key block ahead, alternately into two register sets
     frag8<T> p_a[2][P_KS], p_b[2][P_KS];
-    load_p(0, p_a);
+    load_p(j0, p_a);
 
     f32x4 oacc[2][DB];
 #pragma unroll
@@ -166,7 +187,7 @@ __global__ __launch_bounds__(P_NT, P_OCC) void causal_pv_kernel(const T *__restr
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    for (int j = 0;;) {
+    for (int j = j0;;) {
         step(j, v_a, v_b, p_a, p_b);
         if (++j > j_end) break;
         step(j, v_b, v_a, p_b, p_a);
@@ -354,7 +375,8 @@ int launch_t(const void *p, const void *x, void *o, int64_t B, int64_t H, int64_
 }
 
 template <typename T, int D>
-int launch(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int causal, hipStream_t st)
+int launch(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int causal, hipStream_t st,
+           const int *band_lo = nullptr)
 {
     const int nqb = (int)((S + P_BQ - 1) / P_BQ);
     const int64_t total_wg = B * H * ((nqb + 1) / 2), per_xcd = (total_wg + 7) / 8;
@@ -362,24 +384,34 @@ int launch(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t 
     dim3 grid((unsigned)(per_xcd * 8));
     auto kern = causal_pv_kernel<T, D>;
     hipLaunchKernelGGL(kern, grid, dim3(P_NT), 0, st, (const T *)p, (const T *)v, (T *)o, (int)S, causal, nqb, total_wg,
-                       per_xcd);
+                       per_xcd, band_lo, (int)H);
     return launch_status();
 }
 }  // namespace
 
-extern "C" int mta_causal_pv_fwd(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int64_t D,
-                                 int causal, int io_dtype, void *stream)
+// first_visible (int32, (B,S); NULL = none): P[b,h,p,k] is 0 for k < first_visible[b,p] (what the softmax stage leaves
+// under a band mask); the key blocks ahead of a query block's first visible key are not read.  Implies causal.
+extern "C" int mta_causal_pv_band_fwd(const void *p, const void *v, const void *first_visible, void *o, int64_t B, int64_t H,
+                                      int64_t S, int64_t D, int causal, int io_dtype, void *stream)
 {
     if (!p || !v || !o) return MTA_ERR_NULL;
     if (!dtype_size(io_dtype)) return MTA_ERR_DTYPE;
     if (B <= 0 || H <= 0 || S <= 0 || S > (1 << 24) || B * H > 65535) return MTA_ERR_SHAPE;
     if (D != 64 && D != 128) return MTA_ERR_HEAD_DIM;
-    if (!aligned_to(p, 16) || !aligned_to(v, 16) || !aligned_to(o, 16)) return MTA_ERR_ALIGN;
-    if (io_dtype == MTA_F32 || S % 8 != 0) return MTA_ERR_UNSUPPORTED;
+    if (!aligned_to(p, 16) || !aligned_to(v, 16) || !aligned_to(o, 16) || (first_visible && !aligned_to(first_visible, 4)))
+        return MTA_ERR_ALIGN;
+    if (io_dtype == MTA_F32 || S % 8 != 0 || (first_visible && !causal)) return MTA_ERR_UNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
+    const int *lo = (const int *)first_visible;
     if (io_dtype == MTA_BF16)
-        return D == 64 ? launch<bf16_t, 64>(p, v, o, B, H, S, causal, st) : launch<bf16_t, 128>(p, v, o, B, H, S, causal, st);
-    return D == 64 ? launch<f16_t, 64>(p, v, o, B, H, S, causal, st) : launch<f16_t, 128>(p, v, o, B, H, S, causal, st);
+        return D == 64 ? launch<bf16_t, 64>(p, v, o, B, H, S, causal, st, lo) : launch<bf16_t, 128>(p, v, o, B, H, S, causal, st, lo);
+    return D == 64 ? launch<f16_t, 64>(p, v, o, B, H, S, causal, st, lo) : launch<f16_t, 128>(p, v, o, B, H, S, causal, st, lo);
+}
+
+extern "C" int mta_causal_pv_fwd(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int64_t D,
+                                 int causal, int io_dtype, void *stream)
+{
+    return mta_causal_pv_band_fwd(p, v, nullptr, o, B, H, S, D, causal, io_dtype, stream);
 }
 
 extern "C" int mta_causal_ptx_fwd(const void *p, const void *x, void *o, int64_t B, int64_t H, int64_t S, int64_t D,

@@ -574,9 +574,32 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? ((R > 7 || (BAND && R >= 7))
 
     const int q_last = (q0 + G::BQ - 1 < S - 1) ? q0 + G::BQ - 1 : S - 1;
     const int j_last = causal ? q_last / F_BK : (S - 1) / F_BK;  // last key block of the query block
-    const int j_lo = tbl_lo >= 0 ? tbl_lo : jc * jc_len;          // first key block whose outputs this item produces
+    int j_lo = tbl_lo >= 0 ? tbl_lo : jc * jc_len;                // first key block whose outputs this item produces
     const int j_len = tbl_lo >= 0 ? tbl_len : jc_len;
     const int j_end = (j_lo + j_len - 1 < j_last) ? j_lo + j_len - 1 : j_last;
+    if constexpr (BAND) {
+        // Key blocks that lie wholly ahead of the first key any row of this query block sees are skipped: no visible
+        // position takes a tap from them, and what they would hold is hidden from every row (left unwritten).  Every
+        // wavefront reduces all the rows (the same answer in each: no exchange).
+        const int64_t brow = (bh / H) * (int64_t)S;
+        int fmin = S;
+        for (int r = lane; r < G::BQ + G::HR; r += 64) {
+            const int p = q0 - G::HR + r;
+            if (p >= 0 && p < S) {
+                const int f = band_lo[brow + p];
+                fmin = f < fmin ? f : fmin;
+            }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const int o = __shfl_xor(fmin, off);
+            fmin = o < fmin ? o : fmin;
+        }
+        fmin = __builtin_amdgcn_readfirstlane(fmin);
+        const int j_first = (fmin > 0 ? fmin : 0) / F_BK;
+        if (j_first > j_lo) j_lo = j_first;
+        if (j_lo > j_end) return;
+    }
     // one key block earlier only fills the retained score columns (before the first one: the right pad, if any)
     const int j_start = j_lo > 0 ? j_lo - 1 : (G::PWR > 0 ? -1 : 0);
     issue_k(j_start, B0);

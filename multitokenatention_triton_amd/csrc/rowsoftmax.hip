@@ -142,10 +142,18 @@ __global__ __launch_bounds__(NT, (!KB && NT == 256 && G * NV == 8) ? RS_OCC : 1)
     // skipped everywhere below: the arithmetic follows the triangle, not the square.
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     auto dead = [&](int k) { return (k * NT + wave * 64) * VEC > last; };
+    // band mask: the keys ahead of the row's first visible one are hidden; a pass wholly ahead of it is neither read nor
+    // computed (its outputs are +0)
+    int lo = 0;
+    if constexpr (KB) {
+        if (row_lo) lo = row_lo[n * P + p];
+    }
+    auto hid = [&](int k) { return KB && (k * NT + wave * 64 + 64) * VEC <= lo; };
+    auto gone = [&](int k) { return dead(k) || hid(k); };
     V xin[NV][G];
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
-        if (dead(k)) continue;
+        if (gone(k)) continue;
         const int q = (k * NT + tid) * VEC;
         const int qs = (q <= last) ? q : 0;
 #pragma unroll
@@ -175,7 +183,7 @@ __global__ __launch_bounds__(NT, (!KB && NT == 256 && G * NV == 8) ? RS_OCC : 1)
     float s[G][NV][VEC];
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
-        if (dead(k)) continue;
+        if (gone(k)) continue;
         const int q = (k * NT + tid) * VEC;
 #pragma unroll
         for (int o = 0; o < G; ++o) {
@@ -221,7 +229,6 @@ __global__ __launch_bounds__(NT, (!KB && NT == 256 && G * NV == 8) ? RS_OCC : 1)
                 }
             }
             if (row_lo) {  // band mask: the keys ahead of the row's first visible one are hidden
-                const int lo = row_lo[n * P + p];
                 if (q < lo) {
 #pragma unroll
                     for (int o = 0; o < G; ++o)
@@ -248,7 +255,7 @@ __global__ __launch_bounds__(NT, (!KB && NT == 256 && G * NV == 8) ? RS_OCC : 1)
         float v = -INFINITY;
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
-            if (dead(k)) continue;
+            if (gone(k)) continue;
 #pragma unroll
             for (int u = 0; u < VEC; ++u) v = fmaxf(v, s[o][k][u]);
         }
@@ -274,7 +281,7 @@ __global__ __launch_bounds__(NT, (!KB && NT == 256 && G * NV == 8) ? RS_OCC : 1)
         const float mneg = -m[o] * LOG2E;
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
-            if (dead(k)) continue;
+            if (gone(k)) continue;
 #pragma unroll
             for (int u = 0; u < VEC; ++u) {
                 const float e = __builtin_amdgcn_exp2f(fmaf(s[o][k][u], LOG2E, mneg));
@@ -298,7 +305,7 @@ __global__ __launch_bounds__(NT, (!KB && NT == 256 && G * NV == 8) ? RS_OCC : 1)
     for (int o = 0; o < G; ++o)
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
-            if (dead(k)) continue;
+            if (gone(k)) continue;
 #pragma unroll
             for (int u = 0; u < VEC; ++u) s[o][k][u] *= inv[o];
             if (use_dot) continue;  // rounded below, when the heads are packed in pairs
@@ -314,6 +321,16 @@ __global__ __launch_bounds__(NT, (!KB && NT == 256 && G * NV == 8) ? RS_OCC : 1)
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
         const int q = (k * NT + tid) * VEC;
+        if (hid(k) && !dead(k)) {  // pass wholly ahead of the row's first visible key: +0
+            if (q < Q) {
+                V z;
+#pragma unroll
+                for (int u = 0; u < VEC; ++u) z.v[u] = from_float<T>(0.0f);
+#pragma unroll
+                for (int o = 0; o < G; ++o) store_stream(reinterpret_cast<V *>(y + base + o * plane + q), z);
+            }
+            continue;
+        }
         if (dead(k)) {  // pass wholly above the diagonal: +0 only on request
             if (fill_upper && q < Q) {
                 V z;

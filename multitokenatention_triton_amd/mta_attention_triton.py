@@ -386,7 +386,7 @@ class MTAAttentionTriton(nn.Module):
 
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         self._mark("pv")
-        output = ops.causal_pv(scores, xv, self.causal) if own_pv else None
+        output = ops.causal_pv(scores, xv, self.causal, first_visible=first_visible) if own_pv else None
         if output is None:
             output = torch.matmul(scores, xv)
         self._mark("end")

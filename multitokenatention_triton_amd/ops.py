@@ -359,9 +359,12 @@ def qk_conv_supported(q: torch.Tensor, k: torch.Tensor, weight: torch.Tensor) ->
                                                   _DTYPE_CODE[q.dtype], _DTYPE_CODE[weight.dtype]))
 
 
-def causal_pv(p: torch.Tensor, v: torch.Tensor, causal: bool) -> Optional[torch.Tensor]:
+def causal_pv(p: torch.Tensor, v: torch.Tensor, causal: bool,
+              first_visible: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """P V for P (B,H,S,S), V (B,H,S,D), reading only the lower triangle of P when causal; see mta_causal_pv_fwd.
 
+    ``first_visible``: int32 (B,S), band mask (P is 0 ahead of a row's first visible key): the key blocks no row of a
+    query block sees are not read; see mta_causal_pv_band_fwd.
     Returns ``None`` when unsupported (the caller then uses torch.matmul on a fully defined P)."""
     p = _device_tensor(p, "P")
     v = _device_tensor(v, "V")
@@ -369,9 +372,15 @@ def causal_pv(p: torch.Tensor, v: torch.Tensor, causal: bool) -> Optional[torch.
         return None
     b, h, s, d = v.shape
     out = torch.empty_like(v)
+    if first_visible is not None:
+        first_visible = _device_tensor(first_visible, "first_visible")
+        if first_visible.dtype != torch.int32 or tuple(first_visible.shape) != (b, s):
+            raise ValueError(f"first_visible must be int32 of shape ({b},{s}), got {first_visible.dtype} "
+                             f"{tuple(first_visible.shape)}")
     with torch.cuda.device(p.device):
-        rc = _lib.load().mta_causal_pv_fwd(p.data_ptr(), v.data_ptr(), out.data_ptr(), b, h, s, d, int(bool(causal)),
-                                           _code(p, "P"), _stream(p))
+        rc = _lib.load().mta_causal_pv_band_fwd(p.data_ptr(), v.data_ptr(),
+                                                first_visible.data_ptr() if first_visible is not None else None,
+                                                out.data_ptr(), b, h, s, d, int(bool(causal)), _code(p, "P"), _stream(p))
     if rc in (_lib.MTA_ERR_UNSUPPORTED, -7):
         return None
     _lib.check(rc, "mta_causal_pv_fwd")

@@ -294,7 +294,9 @@ def test_qk_conv_band_parity(pkg, case):
     got = pkg.ops.qk_conv(q.cuda(), k.cuda(), w.cuda(), True, scale, fill_upper=True, first_visible=first.cuda()).cpu()
     low = torch.tril(torch.ones(s, s, dtype=torch.bool))
     ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
-    torch.testing.assert_close(got[..., low].float(), want[..., low].float(), rtol=2 * ulp, atol=2e-2)
+    # (defined where a row sees the key; key blocks that no row of a query block sees are not even visited)
+    seen = visible[:, None].expand(b, h, s, s)
+    torch.testing.assert_close(got[seen].float(), want[seen].float(), rtol=2 * ulp, atol=2e-2)
     assert (got[..., ~low] == 0).all()
     # no band at all is the plain kernel, bit for bit
     zero = torch.zeros(b, s, dtype=torch.int32, device="cuda")
@@ -331,6 +333,61 @@ def test_headmix_softmax_band_parity(pkg, group, s, dtype):
     a = pkg.ops.headmix_softmax(x.cuda(), w1.cuda(), w2.cuda(), True, group_size=group, first_visible=zero)
     torch.testing.assert_close(a.float().cpu(), pkg.ops.headmix_softmax(x.cuda(), w1.cuda(), w2.cuda(), True, group_size=group).float().cpu(),
                                rtol=t["rtol"] * 2, atol=2e-3 if dtype != torch.float32 else 1e-6)
+
+
+@pytest.mark.parametrize("case", [(2, 2, 776, 64, torch.bfloat16, "documents"), (1, 3, 2048, 128, torch.float16, "window"),
+                                  (2, 1, 520, 128, torch.bfloat16, "ragged")])
+def test_causal_pv_band_skips_only_zeros(pkg, case):
+    """P V under a band mask: P is 0 ahead of a row's first visible key, and the key blocks no row of a query block sees
+    are not read -- the same sums as the product over the whole triangle, bit for bit; poisoning what is skipped
+    (NaN in the blocks no row sees) changes nothing."""
+    b, h, s, d, dtype, kind = case
+    print(f"causal_pv band case={case}", flush=True)
+    g = torch.Generator().manual_seed(17)
+    first = _band_first(kind, b, s)
+    keys = torch.arange(s)
+    visible = (keys[None, None, :] >= first[:, :, None]) & (keys[None, None, :] <= keys[None, :, None])
+    logits = (torch.randn(b, h, s, s, generator=g) * 2).masked_fill(~visible[:, None], float("-inf"))
+    p = torch.softmax(logits, -1).to(dtype).cuda()
+    v = torch.randn(b, h, s, d, generator=g).to(dtype).cuda()
+    want = pkg.ops.causal_pv(p, v, True)
+    got = pkg.ops.causal_pv(p, v, True, first_visible=first.cuda())
+    assert torch.equal(got, want)
+    # blocks of 64 keys wholly ahead of the first key any row of a block of 128 query rows sees: never read
+    poisoned = p.clone()
+    for bi in range(b):
+        for q0 in range(0, s, 128):
+            k_first = int(first[bi, q0:q0 + 128].min()) // 64 * 64
+            poisoned[bi, :, q0:q0 + 128, :k_first] = float("nan")
+    assert torch.equal(pkg.ops.causal_pv(poisoned, v, True, first_visible=first.cuda()), want)
+
+
+def test_band_route_never_reads_what_it_skips(pkg):
+    """The three kernels of the band route chained by hand, each writing into a NaN-filled buffer: what the scores kernel
+    leaves unwritten (blocks no row sees, everything above the diagonal) must not reach the output."""
+    print("band route poisoned buffers", flush=True)
+    dtype = torch.bfloat16
+    b, h, s, d = 2, 4, 1032, 64
+    ops = pkg.ops
+    q, k, v = (t.cuda() for t in O.seeded_qkv(b, h, s, d, dtype, seed=98))
+    w = O.seeded_conv_weight(h, 6, 11, 0.05, dtype).cuda()
+    g = torch.Generator().manual_seed(3)
+    w1 = O.block_diag_head_weight(h, 2, 0.1, g, dtype).cuda()
+    w2 = O.block_diag_head_weight(h, 2, 0.1, g, dtype).cuda()
+    first = _band_first("window", b, s).cuda()
+    scale = float(torch.rsqrt(torch.tensor(float(d))))
+
+    def run(poison):
+        fill = float("nan") if poison else 0.0
+        s1 = ops.qk_conv(q, k, w, True, scale, fill_upper=False, first_visible=first,
+                         out=torch.full((b, h, s, s), fill, dtype=dtype, device="cuda"))
+        p1 = ops.headmix_softmax(s1, w1, w2, True, group_size=2, fill_upper=False, first_visible=first,
+                                 out=torch.full((b, h, s, s), fill, dtype=dtype, device="cuda"))
+        return ops.causal_pv(p1, v, True, first_visible=first)
+
+    clean, poisoned = run(False), run(True)
+    assert torch.isfinite(poisoned.float()).all()
+    assert torch.equal(clean, poisoned)
 
 
 @pytest.mark.parametrize("kind", ["window", "documents"])
