@@ -261,10 +261,10 @@ __device__ __forceinline__ void zero_fill_strip(T *yp, int H, int W, int p0, int
 
 // Persistent four-wavefront workgroups: each walks a run of M_TM x M_TN strips dealt round-robin within its XCD's share
 // of the item list.  Wavefront w owns row block w & 1 (16 rows) and key half w >> 1 (128 keys) of the strip: it issues a
-// quarter of the staging copies, computes its 16 x 128 outputs and stores them.  The wavefronts meet at one barrier per
-// strip (the strip has landed; the previous strip's buffer may be overwritten); latency is hidden by the other
-// workgroups resident on the CU, each in its own phase (loading / matrix cores / storing) with its own two 24 KB LDS
-// strip buffers.
+// quarter of the staging copies and computes its 16 x 128 outputs.  The wavefronts meet at two barriers per strip (the
+// strip has landed and the previous strip's buffer may be overwritten; the results are in LDS); latency is hidden by the
+// other workgroups resident on the CU, each in its own phase (loading / matrix cores / storing) with its own two LDS
+// strip buffers of (M_TM + R - 1) rows x 272 keys.
 //
 // Item order.  Strips are taken row strip by row strip, each from the left, so that an XCD's workgroups sweep whole
 // rows of the output together, zero strips included: under the causal rule a strip wholly above the diagonal is an
@@ -280,16 +280,16 @@ __device__ __forceinline__ void zero_fill_strip(T *yp, int H, int W, int p0, int
 // Toeplitz fragment (4 VGPRs per kernel row, kept while the channel is unchanged), B operand = 16 contiguous
 // bytes of one staged row per lane.  A wavefront sustains about one such 1 KB LDS operand per 35 cycles whatever the
 // addresses, against 16 cycles for the product: the products of a strip are therefore split over four wavefronts (on
-// four SIMDs).  Results go back through LDS rows and columns that only the owning wavefront reads (row block 0: the
-// strip's first 16 staged rows; row block 1: the last 16 staged rows of its window; see mfma_geom::RES_OFF for the
-// columns) so that the global stores are whole 256-byte row segments.
+// four SIMDs).  Results go back through LDS rows that are no longer needed as input (row block 0: the strip's first 16
+// staged rows; row block 1: the last 16 staged rows of its window; see mfma_geom::RES_OFF for the columns); after a
+// barrier wavefront w stores strip rows 8w .. 8w+7 whole, two 512-byte rows per instruction.
 //
-// Staging.  A strip whose halo lies wholly inside the tensor and on or below the diagonal (the
-// common case, decided per workgroup) is copied global -> LDS by global_load_lds_dwordx4: no
-// registers, no masks, no LDS store instructions.  The LDS row stride is 35 16-byte slots (34 of
-// data + 1 of padding), so thread t of copy `it` simply owns slot it*256+t.  Diagonal and border strips
-// are copied the same way and fixed up in LDS; the rare strips whose copy could leave the tensor go
-// through registers, where bounds and the causal col<=row rule are applied.
+// Staging.  A strip whose halo lies wholly inside the tensor and on or below the diagonal (the common case, decided per
+// workgroup) is copied global -> LDS by global_load_lds_dwordx4: no registers, no masks, no LDS store instructions.
+// The LDS row stride is 34 16-byte slots (see mfma_geom::LD), and thread t of copy round `it` owns slot it*256+t.  Any
+// other strip is copied slot by slot under a predicate - a slot inside the plane and on or below the diagonal is
+// copied, any other is written as zeros while the buffer waits for its data - and after landing only the one vector
+// per row that straddles the diagonal is masked in LDS.  Nothing is read from outside the tensor.
 //
 // Kernel rows.  The channel's R*S taps are copied global -> LDS the same way, one strip ahead, as the dwords that hold
 // them (from the 4-byte aligned address at or below the first tap: such a dword holds at least one tap, so it lies in
