@@ -478,14 +478,14 @@ template <bool IS_MAX, int G, int NW> __device__ __forceinline__ void heads_redu
     }
 }
 
-// What the first `nlw` wavefronts left in src[head*NW + wave], combined per head, the same in every lane: lane l takes
+// What the wavefronts flw .. nlw-1 left in src[head*NW + wave], combined per head, the same in every lane: lane l takes
 // entry l, NW neighbouring lanes fold with DPP steps, and one lane per head is read out as a wavefront-uniform value.
-template <bool IS_MAX, int G, int NW> __device__ __forceinline__ void heads_combine(const float *src, int nlw, int lane, float (&out)[G])
+template <bool IS_MAX, int G, int NW> __device__ __forceinline__ void heads_combine(const float *src, int nlw, int lane, float (&out)[G], int flw = 0)
 {
     static_assert(NW * G <= 64 && (NW == 4 || NW == 8), "one entry per lane");
     const float neutral = IS_MAX ? -INFINITY : 0.0f;
     const float got = src[lane & (NW * G - 1)];
-    float v = (lane & (NW - 1)) < nlw ? got : neutral, r;
+    float v = ((lane & (NW - 1)) < nlw && (lane & (NW - 1)) >= flw) ? got : neutral, r;
     if constexpr (IS_MAX) {
         MTA_RS_DPP_STEP("v_max_f32", "quad_perm:[1,0,3,2]")
         MTA_RS_DPP_STEP("v_max_f32", "quad_perm:[2,3,0,1]")
@@ -500,13 +500,16 @@ template <bool IS_MAX, int G, int NW> __device__ __forceinline__ void heads_comb
 }
 #undef MTA_RS_DPP_STEP
 
-template <typename T, int G, int NV, bool HAS1, bool HAS2, int NT, int OCC>
+// BAND (one pass per wavefront only): row_lo[n, p] is the first key row p sees; a wavefront whose slice lies wholly ahead
+// of it stores +0 and ends, like those above the diagonal, and the slice that holds it masks the keys ahead of it.
+template <typename T, int G, int NV, bool HAS1, bool HAS2, int NT, int OCC, bool BAND = false>
 __global__ __launch_bounds__(NT, OCC) void mix_softmax_mix_packed(
     const T *__restrict__ x, const T *__restrict__ w1, const T *__restrict__ w2, T *__restrict__ y, int C, int P, int Q,
-    int causal, int fill_upper)
+    int causal, int fill_upper, const int *__restrict__ row_lo)
 {
     constexpr int VEC = 8, NW = NT / 64, H2 = G / 2;
     static_assert(sizeof(T) == 2 && G % 2 == 0, "packed pairs of a 16-bit type");
+    static_assert(!BAND || NV == 1, "the band mask is built for one pass per wavefront");
     __shared__ float red[2][NW * G];  // [0] maxima, [1] sums
     const int lane = threadIdx.x & 63;
     const unsigned groups = (unsigned)(C / G);
@@ -528,6 +531,19 @@ __global__ __launch_bounds__(NT, OCC) void mix_softmax_mix_packed(
     // the workgroup barriers (a barrier waits for the surviving wavefronts only), and free their registers for the next
     // workgroup; the others reduce over the first `nlw` slices.
     const int nlw = last / (64 * VEC) + 1 < NW ? last / (64 * VEC) + 1 : NW;
+    int lo = 0, flw = 0;  // band mask: first visible key, and the wavefront whose slice holds it
+    if constexpr (BAND) {
+        lo = row_lo[n * P + p];
+        lo = lo < 0 ? 0 : lo;
+        flw = lo / (64 * VEC) < nlw - 1 ? lo / (64 * VEC) : nlw - 1;  // (a row that sees no key: NaN from the last slice)
+        if (wave < flw) {  // slice wholly ahead of the first visible key (and below the diagonal): +0
+            const int q = tid * VEC;
+            const rs_u4 z = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int o = 0; o < G; ++o) __builtin_nontemporal_store(z, reinterpret_cast<rs_u4 *>(y + base + o * plane + q));
+            return;
+        }
+    }
     if (nlive == 0) {
         if (fill_upper) {
 #pragma unroll
@@ -610,17 +626,24 @@ __global__ __launch_bounds__(NT, OCC) void mix_softmax_mix_packed(
                             if (q + 2 * d + 1 > last) a[o][1] = -INFINITY;
                         }
                     }
+                    if constexpr (BAND) {
+#pragma unroll
+                        for (int o = 0; o < G; ++o) {
+                            if (q + 2 * d < lo) a[o][0] = -INFINITY;
+                            if (q + 2 * d + 1 < lo) a[o][1] = -INFINITY;
+                        }
+                    }
 #pragma unroll
                     for (int o = 0; o < G; ++o) {
                         m[o] = HAS1 ? max3_after_dot(m[o], a[o][0], a[o][1]) : max3(m[o], a[o][0], a[o][1]);
-                        sp[o][k][d] = (HAS1 || (EDGE && k == L - 1)) ? pack2<T>(a[o][0], a[o][1]) : xin[k][o][d];
+                        sp[o][k][d] = (HAS1 || BAND || (EDGE && k == L - 1)) ? pack2<T>(a[o][0], a[o][1]) : xin[k][o][d];
                     }
                 }
             }
         }
         heads_reduce_store<true, G, NW>(m, red[0], wave, lane);
         __syncthreads();
-        heads_combine<true, G, NW>(red[0], nlw, lane, m);
+        heads_combine<true, G, NW>(red[0], nlw, lane, m, flw);
         if constexpr (HAS1) {
             // the maximum of the rounded scores is the rounded maximum (the row's first key is always attended: finite)
 #pragma unroll
@@ -649,7 +672,7 @@ __global__ __launch_bounds__(NT, OCC) void mix_softmax_mix_packed(
         }
         heads_reduce_store<false, G, NW>(inv, red[1], wave, lane);
         __syncthreads();
-        heads_combine<false, G, NW>(red[1], nlw, lane, inv);
+        heads_combine<false, G, NW>(red[1], nlw, lane, inv, flw);
 #pragma unroll
         for (int o = 0; o < G; ++o) {  // 1/sum: the hardware reciprocal and one Newton step (within an ulp of the quotient)
             const float r = __builtin_amdgcn_rcpf(inv[o]);
@@ -829,13 +852,33 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb_in, 
             const int rc = mix16_softmax_launch(x, w1, w2, y, N, C, P, Q, causal, fill_upper, io_code, w_dtype, st);
             if (rc != MTA_ERR_UNSUPPORTED) return rc;
         }
-        if (vec_ok && plain && !no_packed && w_dtype == io_code && (w1 || w2) && (!w1 || aligned_to(w1, 4)) &&
-            (!w2 || aligned_to(w2, 4)) && C % 2 == 0 && Q <= 256 * VEC * 4) {
+        const bool packed_ok = vec_ok && !no_packed && w_dtype == io_code && (w1 || w2) && (!w1 || aligned_to(w1, 4)) &&
+                               (!w2 || aligned_to(w2, 4)) && C % 2 == 0 && Q <= 256 * VEC * 4;
+        // band mask without a key bias, one weight, rows that one pass per wavefront covers: the packed kernel's BAND
+        // instances (causal by construction)
+        if (packed_ok && row_lo && !kb && causal && !(w1 && w2)) {
+#define MTA_RSB_LAUNCH(g, h1, h2, nt, occ)                                                                             \
+    {                                                                                                                  \
+        hipLaunchKernelGGL((mix_softmax_mix_packed<T, g, 1, h1, h2, nt, occ, true>), dim3((unsigned)(N * (C / g) * P)), \
+                           dim3(nt), 0, st, (const T *)x, (const T *)w1, (const T *)w2, (T *)y, (int)C, (int)P,        \
+                           (int)Q, causal, fill_upper, row_lo);                                                        \
+        return launch_status();                                                                                        \
+    }
+#define MTA_RSB_CASE(g, nt, occ)                                                                                       \
+    if (G == g && Q <= (int64_t)(nt) * VEC) {                                                                          \
+        if (w1) MTA_RSB_LAUNCH(g, true, false, nt, occ)                                                                \
+        MTA_RSB_LAUNCH(g, false, true, nt, occ)                                                                        \
+    }
+            MTA_RSB_CASE(2, 256, 1) MTA_RSB_CASE(4, 256, 1) MTA_RSB_CASE(4, 512, 8) MTA_RSB_CASE(8, 256, RS_OCC)
+#undef MTA_RSB_CASE
+#undef MTA_RSB_LAUNCH
+        }
+        if (packed_ok && plain) {
 #define MTA_RSP_LAUNCH(g, v, h1, h2, nt, occ)                                                                          \
     {                                                                                                                  \
         hipLaunchKernelGGL((mix_softmax_mix_packed<T, g, v, h1, h2, nt, occ>), dim3((unsigned)(N * (C / g) * P)),      \
                            dim3(nt), 0, st, (const T *)x, (const T *)w1, (const T *)w2, (T *)y, (int)C, (int)P,        \
-                           (int)Q, causal, fill_upper);                                                                \
+                           (int)Q, causal, fill_upper, nullptr);                                                       \
         return launch_status();                                                                                        \
     }
 #define MTA_RSP_CASE(g, v, nt, occ)                                                                                    \
