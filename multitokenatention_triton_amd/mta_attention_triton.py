@@ -479,9 +479,10 @@ class MTAAttentionTriton(nn.Module):
         """use_mask=True: an explicit additive mask tensor drives the masking (mta_attention_triton.py:63-64,
         77-83, 96-98); the kernels still apply their own causal rule when ``causal`` is set.
 
-        Two kinds of mask never become a (B,H,S,S) tensor here (inference, causal module): no mask at all, which the
-        reference turns into the causal rule the kernels apply anyway, and a 2-D key mask, which the reference turns
-        into "causal rule + one value per key" (mta_attention_triton.py:118-122).  A hidden key's scores enter the
+        These masks never become a (B,H,S,S) tensor here (inference, causal module): no mask at all, which the
+        reference turns into the causal rule the kernels apply anyway; a 2-D key mask, which the reference turns into
+        "causal rule + one value per key" (mta_attention_triton.py:118-122); a 4-D mask that says the same per batch
+        entry (key padding for B > 1, which the reference's 2-D form cannot express); and a 4-D band mask.  A hidden key's scores enter the
         pre-softmax conv as 0 -- which is what a zero K row produces -- its mixed score gets -inf ahead of the softmax
         (the kernel's per-key bias), its probability is 0, and whatever the post-softmax conv writes into its column,
         which the reference zeroes, meets a zero V row."""
@@ -497,13 +498,18 @@ class MTAAttentionTriton(nn.Module):
                 hidden = (bias == float("-inf"))[:, None, :, None]
                 return self._forward_fused(xq, xk.masked_fill(hidden, 0), xv.masked_fill(hidden, 0),
                                            key_bias=bias.contiguous())
-            # a band mask - the same for all heads, row p seeing the keys first[p] .. p (sliding windows, packed
-            # documents) - goes into the kernels as one int32 per (batch entry, row)
-            if (mask.dim() == 4 and self._current_structure().post_conv_identity
-                    and ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight)):
-                first = self._band_of_mask(mask, xq.size(0), xq.size(-2))
-                if first is not None:
-                    return self._forward_fused(xq, xk, xv, first_visible=first)
+            # a 4-D mask, the same for all heads, of one of two forms goes into the kernels without a (B,H,S,S) tensor:
+            # "causal rule + hidden keys" per batch entry (key padding: a key bias and zeroed K and V rows, as for the
+            # 2-D mask above) and "row p sees the keys first[p] .. p" (sliding windows, packed documents: one int32 per
+            # batch entry and row)
+            if mask.dim() == 4:
+                kind, what = self._structured_mask(mask, xq.size(0), xq.size(-2))
+                if kind == "keys":
+                    hidden = (what == float("-inf"))[:, None, :, None]
+                    return self._forward_fused(xq, xk.masked_fill(hidden, 0), xv.masked_fill(hidden, 0), key_bias=what)
+                if (kind == "band" and self._current_structure().post_conv_identity
+                        and ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight)):
+                    return self._forward_fused(xq, xk, xv, first_visible=what)
         mask = self._update_mask(mask=mask, bsz=xq.size(0), xq=xq, xk_size=xk.size(-2))
         scale = float(torch.rsqrt(torch.tensor(float(xq.size(-1)))))  # a host scalar: the product stays one vectorised pass
         scores = torch.matmul(xq, xk.transpose(2, 3)) * scale
@@ -518,32 +524,45 @@ class MTAAttentionTriton(nn.Module):
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         return torch.matmul(scores, xv).transpose(1, 2)
 
-    def _band_of_mask(self, mask, bsz: int, s: int):
-        """int32 (B,S) first visible key per query row when ``mask`` (4-D, bool with True = attend, or additive with
-        0 / -inf) together with the causal rule has the form "row p sees the keys first[p] .. p" for every row, the same
-        for all heads; else None.  The answer for the last mask seen is kept (same storage, same version)."""
-        if mask.size(1) != 1 or mask.size(0) not in (1, bsz) or mask.size(-2) != s or mask.size(-1) != s:
-            return None
+    def _structured_mask(self, mask, bsz: int, s: int):
+        """What a 4-D ``mask`` (bool with True = attend, or additive with 0 / -inf; one plane for all heads) amounts to
+        together with the causal rule:
+          ("keys", bias)   every row sees the kept keys up to itself and key 0 is kept: fp32 (B,S), 0 / -inf per key;
+          ("band", first)  row p sees exactly the keys first[p] .. p: int32 (B,S);
+          (None, None)     anything else (per-head planes, holes that differ between rows, other finite values, a row
+                           that sees nothing).
+        A few reductions over the mask and one read back; the answer for the last mask object seen is kept while its
+        version does not change."""
+        if mask.size(0) not in (1, bsz) or mask.size(-2) != s or mask.size(-1) != s or mask.size(1) not in (1, self.n_heads):
+            return None, None
         key = (mask._version, bsz)
-        cached = getattr(self, "_band_cache", None)   # (the mask object itself is kept: its identity cannot be reused)
+        cached = getattr(self, "_mask_cache", None)   # (the mask object itself is kept: its identity cannot be reused)
         if cached is not None and cached[0] is mask and cached[1] == key:
             return cached[2]
+        answer = (None, None)
+        plane = mask[:, 0]
+        same_heads = mask.size(1) == 1 or bool((mask == mask[:, :1]).all())
         if mask.dtype == torch.bool:
-            visible = mask[:, 0]
+            visible = plane
         else:
-            visible = mask[:, 0] == 0
-            if not bool(((mask[:, 0] == float("-inf")) | visible).all()):
+            visible = plane == 0
+            if not bool(((plane == float("-inf")) | visible).all()):
                 visible = None   # other finite values: not a 0 / -inf mask
-        first = None
-        if visible is not None:
+        if same_heads and visible is not None:
             rows = torch.arange(s, device=mask.device)
-            visible = visible & (rows[None, :] <= rows[:, None])
-            count = visible.sum(-1)
-            lead = visible.int().argmax(-1)
-            if bool(((count >= 1) & (count == rows[None, :] - lead + 1)).all()):
-                first = lead.to(torch.int32).expand(bsz, s).contiguous()
-        self._band_cache = (mask, key, first)
-        return first
+            lower = rows[None, :] <= rows[:, None]
+            visible = visible & lower
+            keep = visible[:, -1, :]                       # what the last row sees: every kept key
+            if bool((visible == (keep[:, None, :] & lower)).all()) and bool(keep[:, 0].all()):
+                bias = torch.where(keep, 0.0, float("-inf")).to(torch.float32).expand(bsz, s).contiguous()
+                answer = ("keys", bias)
+            else:
+                count = visible.sum(-1)
+                lead = visible.int().argmax(-1)
+                if bool(((count >= 1) & (count == rows[None, :] - lead + 1)).all()):
+                    answer = ("band", lead.to(torch.int32).expand(bsz, s).contiguous())
+        self._mask_cache = (mask, key, answer)
+        return answer
 
     def _update_mask(self, mask, bsz: int, xq: torch.Tensor, xk_size: int):
         """Additive (B,H,Sq,Sk) mask, 0 = attend, -inf = blocked (mta_attention_triton.py:106-127)."""

@@ -797,7 +797,35 @@ def test_mta_use_mask_key_mask_batched_additive_4d(pkg):
     mask = torch.where(visible, 0.0, float("-inf")).to(dtype).contiguous()
     want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3], mask=mask)
     mod = _mta_module(pkg, h, 3, 3, 3, 3, *params, dtype, use_mask=True)
+    stages = []
+    mod._stage_hook = stages.append
     got = mod(q.cuda(), k.cuda(), v.cuda(), mask.cuda(), None).cpu()
+    torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+    # "causal rule + hidden keys" per batch entry is recognised: the kernels run, with a key bias per batch entry
+    assert "qk_conv" in stages and "pv" in stages
+
+
+@pytest.mark.parametrize("post", ["identity", "random"])
+def test_mta_use_mask_right_padded_batch(pkg, post):
+    """Key padding for B > 1 (sequences of different lengths, padded on the right), given as a (B,1,S,S) boolean mask:
+    recognised as "causal rule + hidden keys" and run through the kernels; the rows of real tokens against the oracle
+    given the mask tensor (the padding rows see their own batch entry's kept keys only, like everybody else)."""
+    print(f"mta use_mask right padding post={post}", flush=True)
+    dtype = torch.bfloat16
+    b, h, s, d = 3, 4, 520, 64
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=94)
+    params = _config_like(h, 2, 6, 11, 0.05, dtype, post=post)
+    lengths = torch.tensor([520, 333, 97])
+    keep = torch.arange(s)[None, :] < lengths[:, None]                                  # (B,S)
+    causal = torch.tril(torch.ones(s, s, dtype=torch.bool))
+    visible = (keep[:, None, None, :] & causal[None, None])                            # (B,1,S,S)
+    want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3],
+                         mask=torch.where(visible, 0.0, float("-inf")).to(dtype).expand(b, h, s, s).contiguous())
+    mod = _mta_module(pkg, h, 6, 11, 3, 3, *params, dtype, use_mask=True, structure="infer")
+    stages = []
+    mod._stage_hook = stages.append
+    got = mod(q.cuda(), k.cuda(), v.cuda(), visible.cuda(), None).cpu()
+    assert "qk_conv" in stages and "pv" in stages
     torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
 
 
