@@ -13,14 +13,15 @@
 // receives head-dim value i of 4 consecutive keys.
 #include <type_traits>
 
+#include <cstdlib>
+
 #include "common.hpp"
 #include "mfma.hpp"
+#include "strip_common.hpp"
 
 namespace {
 using namespace mta;
 
-typedef __attribute__((address_space(3))) void lds_void_t;
-typedef const __attribute__((address_space(1))) void glb_void_t;
 typedef short v4s_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4s_t lds_v4s_t;
 
@@ -32,22 +33,29 @@ constexpr int P_BK = 64;  // keys per iteration (128 measured no faster): each l
                                  // iteration, back to back, so that DRAM pages are used in long runs
 constexpr int P_KS = P_BK / 32;  // 32-key contraction steps per iteration
 
-template <typename T, int D>
-__global__ __launch_bounds__(P_NT, P_OCC) void causal_pv_kernel(const T *__restrict__ P, const T *__restrict__ V,
-                                                           T *__restrict__ O, int S, int causal, int nqb, int64_t total_wg,
-                                                           int64_t per_xcd, const int *__restrict__ band_lo, int H)
+// SPLIT = 2: two such groups of wavefronts in a workgroup share the query rows and take the even and the odd key
+// blocks; the second group's sums reach the first through LDS at the end.  For grids that put one workgroup on a CU
+// (few heads): twice the loads in flight for the same bytes.
+template <typename T, int D, int SPLIT>
+__global__ __launch_bounds__(P_NT * SPLIT, SPLIT == 2 ? 1 : P_OCC) void causal_pv_kernel(
+    const T *__restrict__ P, const T *__restrict__ V, T *__restrict__ O, int S, int causal, int nqb, int64_t total_wg,
+    int64_t per_xcd, const int *__restrict__ band_lo, int H)
 {
     constexpr int CPR = D / 8;               // 16-byte chunks per V row
     constexpr int TILE = P_BK * D;           // elements per V block
     constexpr int ROUNDS = (TILE / 8 + P_NT - 1) / P_NT;
     constexpr int DB = D / 16;
+    static_assert(SPLIT == 1 || (size_t)SPLIT * TILE * sizeof(T) == (size_t)DB * P_NT * 16, "the sums of one row block fit one V buffer pair");
     // Double buffer as two separate arrays, and a loop body instantiated once per array: the compiler then sees that
     // the LDS reads of one block never touch the asynchronous copy in flight into the other.  With one array it
     // cannot, and waits for the copy (and for every load issued before it) ahead of the first LDS read.
-    __shared__ __align__(16) T v_a[TILE];
-    __shared__ __align__(16) T v_b[TILE];
+    __shared__ __align__(16) T v_a_all[SPLIT * TILE];
+    __shared__ __align__(16) T v_b_all[SPLIT * TILE];
 
-    const int tid = threadIdx.x;
+    const int grp = SPLIT == 2 ? (int)(threadIdx.x >> 8) : 0;  // which key blocks: j % SPLIT == grp
+    T *const v_a = v_a_all + grp * TILE;
+    T *const v_b = v_b_all + grp * TILE;
+    const int tid = threadIdx.x & (P_NT - 1);
     const int wave = tid >> 6, lane = tid & 63, ln = lane & 15, kg = lane >> 4;
     // XCD-aware order: XCD x (workgroup id % 8) takes the x-th eighth of the (batch*head, query block) list, so
     // the workgroups that share one head's V run on one L2; within a head the longest query blocks come first
@@ -128,10 +136,14 @@ __global__ __launch_bounds__(P_NT, P_OCC) void causal_pv_kernel(const T *__restr
         j0 = (fmin > 0 ? fmin : 0) / P_BK;
         if (j0 > j_end) j0 = j_end;
     }
-    issue_v(j0, v_a);
+    // this group's key blocks: jg, jg + SPLIT, ... (by the block's own parity, whatever the first block is: a band mask
+    // that skips blocks of zeros leaves every sum as it is, bit for bit)
+    const int jg = SPLIT == 2 ? j0 + ((j0 & 1) != grp) : j0;
+    const int nsteps = (j_end - j0) / SPLIT + 1;  // of the group that starts at j0: the other one idles in its last step
+    if (jg <= j_end) issue_v(jg, v_a);
     // P fragments are fetched one key block ahead, alternately into two register sets
     frag8<T> p_a[2][P_KS], p_b[2][P_KS];
-    load_p(j0, p_a);
+    load_p(jg, p_a);
 
     f32x4 oacc[2][DB];
 #pragma unroll
@@ -142,9 +154,10 @@ __global__ __launch_bounds__(P_NT, P_OCC) void causal_pv_kernel(const T *__restr
     auto step = [&](int j, const T *Vb, T *Vn, frag8<T> (&pcur)[2][P_KS], frag8<T> (&pnext)[2][P_KS]) __attribute__((always_inline)) {
         __builtin_amdgcn_s_waitcnt(0);  // V block j and the P fragments have arrived
         __syncthreads();                // for every wavefront; reads of the other buffer are finished
-        if (j < j_end) {
-            issue_v(j + 1, Vn);
-            load_p(j + 1, pnext);
+        if (SPLIT == 2 && j > j_end) return;  // (the other group's last block: this one only meets it at the barrier)
+        if (j + SPLIT <= j_end) {
+            issue_v(j + SPLIT, Vn);
+            load_p(j + SPLIT, pnext);
         }
         // mask the fragments of this block: keys beyond the row (causal) or the sequence count as 0
         frag8<T> pf[2][P_KS];
@@ -187,13 +200,33 @@ __global__ __launch_bounds__(P_NT, P_OCC) void causal_pv_kernel(const T *__restr
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    for (int j = j0;;) {
+    for (int i = 0, j = jg;; j += SPLIT) {
         step(j, v_a, v_b, p_a, p_b);
-        if (++j > j_end) break;
+        if (++i >= nsteps) break;
+        j += SPLIT;
         step(j, v_b, v_a, p_b, p_a);
-        if (++j > j_end) break;
+        if (++i >= nsteps) break;
     }
 
+    if constexpr (SPLIT == 2) {
+        // the second group's sums travel through the V buffers (rows' first block in one, second in the other)
+        typedef __attribute__((address_space(3))) f32x4 lds_f4;
+        __syncthreads();  // nobody reads V any more
+        if (grp == 1) {
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                reinterpret_cast<f32x4 *>(v_a_all)[db * P_NT + tid] = oacc[0][db];
+                reinterpret_cast<f32x4 *>(v_b_all)[db * P_NT + tid] = oacc[1][db];
+            }
+        }
+        __syncthreads();
+        if (grp == 1) continue;  // (the barrier ahead of the second row block is met at the top of the loop)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            oacc[0][db] += reinterpret_cast<const f32x4 *>(v_a_all)[db * P_NT + tid];
+            oacc[1][db] += reinterpret_cast<const f32x4 *>(v_b_all)[db * P_NT + tid];
+        }
+    }
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb) {
         if (prow[rb] >= S) continue;
@@ -382,9 +415,18 @@ int launch(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t 
     const int64_t total_wg = B * H * ((nqb + 1) / 2), per_xcd = (total_wg + 7) / 8;
     if (per_xcd * 8 > 0x7fffffffLL) return MTA_ERR_SHAPE;
     dim3 grid((unsigned)(per_xcd * 8));
-    auto kern = causal_pv_kernel<T, D>;
-    hipLaunchKernelGGL(kern, grid, dim3(P_NT), 0, st, (const T *)p, (const T *)v, (T *)o, (int)S, causal, nqb, total_wg,
-                       per_xcd, band_lo, (int)H);
+    // a grid of at most one workgroup per CU runs the two-group instance (key blocks split between them)
+    static const int force = [] { const char *e = getenv("MTA_PV_SPLIT"); return e ? atoi(e) : 0; }();  // 1 / 2: test switch
+    const bool split = force ? force == 2 : total_wg <= device_cu_count();
+    if (split) {
+        auto kern = causal_pv_kernel<T, D, 2>;
+        hipLaunchKernelGGL(kern, grid, dim3(P_NT * 2), 0, st, (const T *)p, (const T *)v, (T *)o, (int)S, causal, nqb,
+                           total_wg, per_xcd, band_lo, (int)H);
+    } else {
+        auto kern = causal_pv_kernel<T, D, 1>;
+        hipLaunchKernelGGL(kern, grid, dim3(P_NT), 0, st, (const T *)p, (const T *)v, (T *)o, (int)S, causal, nqb,
+                           total_wg, per_xcd, band_lo, (int)H);
+    }
     return launch_status();
 }
 }  // namespace

@@ -25,6 +25,9 @@ GROUPS = [
      "test_conv_parity or test_conv_identity_tap or test_conv_backward_parity"),
     # dense groups of 16 heads in the one-pass conv + mixing entry point on the vector-ALU kernel
     ({"MTA_CONV_MIX16_OFF": "1"}, ["tests/test_gpu_ops.py"], "test_conv_headmix_parity"),
+    # P V of small grids on the one-group kernel that large grids run (by default they split the key blocks between two
+    # groups of wavefronts)
+    ({"MTA_PV_SPLIT": "1"}, ["tests/test_gpu_attention.py"], "test_causal_pv"),
 ]
 
 
