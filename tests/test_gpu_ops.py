@@ -291,6 +291,9 @@ MS_CASES = [
     # inside a tile of 128 keys / on its boundary, the longest row the kernel takes
     (1, 16, 200, 16, True, False), (2, 16, 264, 16, True, True), (1, 32, 136, 16, False, True), (1, 16, 2048, 16, True, True),
     (1, 16, 4096, 16, True, False),
+    # lists of rows per workgroup with several steps each: two batch entries and two groups, rows of all three kinds
+    # (4, 8, 16 wavefronts); rows that end inside a tile with the second weight only
+    (2, 32, 2304, 16, True, True), (1, 16, 3000, 16, False, True),
 ]
 
 
@@ -318,6 +321,29 @@ def test_mix_softmax_mix_parity(ops, case, causal, dt):
         assert (got[..., up] == 0).all() and not torch.signbit(got[..., up]).any()
     t = tol(dtype)
     torch.testing.assert_close(got.float(), want.float(), rtol=t["rtol"] * 2, atol=2e-3 if dtype != torch.float32 else 1e-6)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("case", [(1, 16, 2560, True, True), (2, 16, 1160, True, False), (1, 32, 4096, False, True)])
+def test_mix_softmax_mix_dense16_leaves_the_upper_triangle_alone(ops, case, dt):
+    """Groups of 16 heads with fill_upper=False: on and below the diagonal bit for bit the filling call's result, above it
+    the buffer's old content (or +0 inside the tile the diagonal crosses); NaN above the diagonal of the input is
+    never read."""
+    n, c, s, use1, use2 = case
+    dtype = DT[dt]
+    print(f"mix_softmax_mix dense16 lower-only case={case} dt={dt}", flush=True)
+    x = _gpu_randn((n, c, s, s), 41, dtype, 2.0)
+    g = torch.Generator().manual_seed(42)
+    w1 = O.block_diag_head_weight(c, 16, 0.1, g, dtype).cuda() if use1 else None
+    w2 = O.block_diag_head_weight(c, 16, 0.1, g, dtype).cuda() if use2 else None
+    full = ops.headmix_softmax(x, w1, w2, True, group_size=16)
+    up = _upper(s, s).cuda()
+    got = ops.headmix_softmax(x.masked_fill(up, float("nan")), w1, w2, True, group_size=16, out=torch.full_like(x, 7.0),
+                              fill_upper=False)
+    assert torch.equal(got[..., ~up], full[..., ~up])
+    above = got[..., up].float()
+    assert ((above == 7.0) | (above == 0)).all()
+    assert (got[..., 0, 128:].float() == 7.0).all()
 
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])

@@ -28,6 +28,8 @@ GROUPS = [
     # P V of small grids on the one-group kernel that large grids run (by default they split the key blocks between two
     # groups of wavefronts)
     ({"MTA_PV_SPLIT": "1"}, ["tests/test_gpu_attention.py"], "test_causal_pv"),
+    # mix -> softmax -> mix for groups of 16 heads with a workgroup per row (by default workgroups take lists of rows)
+    ({"MTA_MIX16_NO_ROW_LISTS": "1"}, ["tests/test_gpu_ops.py"], "(test_mix_softmax_mix_parity and not f32) or test_mix_softmax_mix_dense16"),
 ]
 
 
