@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTA_ABI_VERSION 8
+#define MTA_ABI_VERSION 9
 
 enum mta_dtype { MTA_F32 = 0, MTA_BF16 = 1, MTA_F16 = 2 };
 
@@ -225,6 +225,33 @@ int mta_causal_pv_fwd(const void *p, const void *v, void *o, int64_t B, int64_t 
  * query rows sees are not read.  Requires causal when first_visible is given. */
 int mta_causal_pv_band_fwd(const void *p, const void *v, const void *first_visible, void *o, int64_t B, int64_t H,
                            int64_t S, int64_t D, int causal, int io_dtype, void *stream);
+
+/* ---- The three stages of the causal forward (mta_attention_triton.py:68-89 with an identity post-softmax conv) over
+ * score tensors in a TRIANGULAR LAYOUT.  The (B,H,S,S) tensors between the three kernels never leave the library's
+ * caller, so their layout is free; this one stores what lies on and below the diagonal only and puts the rows that one
+ * workgroup of the softmax stage reads side by side:
+ *   row p holds len(p) = 64*(p/64 + 1) elements (keys 0..p, then padding of unspecified content);
+ *   off(p) = 2048*a*(a+1) + (p%64)*64*(a+1), a = p/64, elements of one head lie ahead of row p;  T = off(S);
+ *   the heads are taken in groups of `group` consecutive heads (H % group == 0) and a group's rows are interleaved:
+ *   element (b, h, p, q <= p) sits at  ((b*H + h)/group)*group*T + group*off(p) + (h%group)*len(p) + q.
+ * The tensor has B*H*T elements (about half of B*H*S*S).  Same values as the entry points they mirror; they have no
+ * counterpart in the reference, whose kernels exchange full (B,H,S,S) tensors.  16-bit I/O only.
+ *   mta_qk_conv_tri_fwd:         mta_qk_conv_fwd (causal) / mta_qk_conv_band_fwd (first_visible not NULL), output layout;
+ *                                group*T must stay below 2^31.
+ *   mta_headmix_softmax_tri_fwd: mta_headmix_softmax_fwd (causal, fill_upper = 0) / mta_headmix_softmax_band_fwd, input
+ *                                and output layout, the layout's group = group_size (2, 4 or 8), weights of the I/O dtype.
+ *   mta_causal_pv_tri_fwd:       mta_causal_pv_band_fwd (causal), layout of P. */
+int mta_qk_conv_tri_fwd(const void *q, const void *k, const void *w, const void *first_visible, void *s_out, int64_t B,
+                        int64_t H, int64_t S, int64_t D, int R, int Sk, float scale, int group, int io_dtype, int w_dtype,
+                        void *stream);
+int mta_headmix_softmax_tri_fwd(const void *x, const void *w1, const void *w2, const void *first_visible, void *y, int64_t N,
+                                int64_t C, int64_t S, int group_size, int io_dtype, int w_dtype, void *stream);
+int mta_causal_pv_tri_fwd(const void *p, const void *v, const void *first_visible, void *o, int64_t B, int64_t H, int64_t S,
+                          int64_t D, int group, int io_dtype, void *stream);
+/* 1 when mta_headmix_softmax_tri_fwd has a kernel for these sizes and dtypes (has_w1 / has_w2: which weights are given;
+ * band: with first_visible), else 0.  A host-side question: nothing is launched. */
+int mta_headmix_softmax_tri_supported(int64_t C, int64_t S, int group_size, int io_dtype, int w_dtype, int has_w1, int has_w2,
+                                      int band);
 
 /* The transposed product, O[k,:] = sum_p P[p,k] X[p,:] with P (B,H,S,S), X and O (B,H,S,D); when causal only query rows
  * p >= k take part and nothing of P above the diagonal is read.  These are the gradients the two matrix products of the

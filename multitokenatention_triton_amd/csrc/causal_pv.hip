@@ -39,7 +39,7 @@ constexpr int P_KS = P_BK / 32;  // 32-key contraction steps per iteration
 template <typename T, int D, int SPLIT>
 __global__ __launch_bounds__(P_NT * SPLIT, SPLIT == 2 ? 1 : P_OCC) void causal_pv_kernel(
     const T *__restrict__ P, const T *__restrict__ V, T *__restrict__ O, int S, int causal, int nqb, int64_t total_wg,
-    int64_t per_xcd, const int *__restrict__ band_lo, int H)
+    int64_t per_xcd, const int *__restrict__ band_lo, int H, int tri_gl)
 {
     constexpr int CPR = D / 8;               // 16-byte chunks per V row
     constexpr int TILE = P_BK * D;           // elements per V block
@@ -67,7 +67,8 @@ __global__ __launch_bounds__(P_NT * SPLIT, SPLIT == 2 ? 1 : P_OCC) void causal_p
     const int npairs = (nqb + 1) / 2;
     const int pi = (int)(lid % npairs);
     const int64_t bh = lid / npairs;
-    const T *Pp = P + bh * (int64_t)S * S;
+    // (tri_gl > 0: P in the triangular layout, groups of tri_gl heads interleaved by rows)
+    const T *Pp = tri_gl > 0 ? P + (bh / tri_gl) * (tri_gl * tri_rowoff(S)) : P + bh * (int64_t)S * S;
     const T *Vp = V + bh * (int64_t)S * D;
     T *Op = O + bh * (int64_t)S * D;
   for (int half = 0; half < 2; ++half) {
@@ -95,7 +96,8 @@ __global__ __launch_bounds__(P_NT * SPLIT, SPLIT == 2 ? 1 : P_OCC) void causal_p
     for (int rb = 0; rb < 2; ++rb) {
         prow[rb] = q0 + wave * 32 + rb * 16 + ln;
         const int pc = prow[rb] < S ? prow[rb] : S - 1;
-        prow_ptr[rb] = Pp + (int64_t)pc * S + kg * 8;
+        prow_ptr[rb] = tri_gl > 0 ? Pp + tri_gl * tri_rowoff(pc) + (int)(bh % tri_gl) * tri_rowlen(pc) + kg * 8
+                                  : Pp + (int64_t)pc * S + kg * 8;
     }
     // P^T fragments of key block j: slots t = 0..7 of k-step ks are keys j*64 + 32ks + 8kg + t; out-of-range
     // vectors re-read the row start, the values are masked when used
@@ -409,7 +411,7 @@ int launch_t(const void *p, const void *x, void *o, int64_t B, int64_t H, int64_
 
 template <typename T, int D>
 int launch(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int causal, hipStream_t st,
-           const int *band_lo = nullptr)
+           const int *band_lo = nullptr, int tri_gl = 0)
 {
     const int nqb = (int)((S + P_BQ - 1) / P_BQ);
     const int64_t total_wg = B * H * ((nqb + 1) / 2), per_xcd = (total_wg + 7) / 8;
@@ -421,11 +423,11 @@ int launch(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t 
     if (split) {
         auto kern = causal_pv_kernel<T, D, 2>;
         hipLaunchKernelGGL(kern, grid, dim3(P_NT * 2), 0, st, (const T *)p, (const T *)v, (T *)o, (int)S, causal, nqb,
-                           total_wg, per_xcd, band_lo, (int)H);
+                           total_wg, per_xcd, band_lo, (int)H, tri_gl);
     } else {
         auto kern = causal_pv_kernel<T, D, 1>;
         hipLaunchKernelGGL(kern, grid, dim3(P_NT), 0, st, (const T *)p, (const T *)v, (T *)o, (int)S, causal, nqb,
-                           total_wg, per_xcd, band_lo, (int)H);
+                           total_wg, per_xcd, band_lo, (int)H, tri_gl);
     }
     return launch_status();
 }
@@ -448,6 +450,25 @@ extern "C" int mta_causal_pv_band_fwd(const void *p, const void *v, const void *
     if (io_dtype == MTA_BF16)
         return D == 64 ? launch<bf16_t, 64>(p, v, o, B, H, S, causal, st, lo) : launch<bf16_t, 128>(p, v, o, B, H, S, causal, st, lo);
     return D == 64 ? launch<f16_t, 64>(p, v, o, B, H, S, causal, st, lo) : launch<f16_t, 128>(p, v, o, B, H, S, causal, st, lo);
+}
+
+// P in the triangular layout (see tri_rowoff in common.hpp), groups of `group` heads interleaved by rows; causal.
+extern "C" int mta_causal_pv_tri_fwd(const void *p, const void *v, const void *first_visible, void *o, int64_t B, int64_t H,
+                                     int64_t S, int64_t D, int group, int io_dtype, void *stream)
+{
+    if (!p || !v || !o) return MTA_ERR_NULL;
+    if (!dtype_size(io_dtype)) return MTA_ERR_DTYPE;
+    if (B <= 0 || H <= 0 || S <= 0 || S > (1 << 24) || B * H > 65535) return MTA_ERR_SHAPE;
+    if (group <= 0 || H % group != 0) return MTA_ERR_GROUP;
+    if (D != 64 && D != 128) return MTA_ERR_HEAD_DIM;
+    if (!aligned_to(p, 16) || !aligned_to(v, 16) || !aligned_to(o, 16) || (first_visible && !aligned_to(first_visible, 4)))
+        return MTA_ERR_ALIGN;
+    if (io_dtype == MTA_F32 || S % 8 != 0) return MTA_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    const int *lo = (const int *)first_visible;
+    if (io_dtype == MTA_BF16)
+        return D == 64 ? launch<bf16_t, 64>(p, v, o, B, H, S, 1, st, lo, group) : launch<bf16_t, 128>(p, v, o, B, H, S, 1, st, lo, group);
+    return D == 64 ? launch<f16_t, 64>(p, v, o, B, H, S, 1, st, lo, group) : launch<f16_t, 128>(p, v, o, B, H, S, 1, st, lo, group);
 }
 
 extern "C" int mta_causal_pv_fwd(const void *p, const void *v, void *o, int64_t B, int64_t H, int64_t S, int64_t D,

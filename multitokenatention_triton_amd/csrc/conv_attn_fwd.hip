@@ -454,7 +454,7 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? ((R > 7 || (BAND && R >= 7))
                                                              T *__restrict__ O, float *__restrict__ Lse, int S, int causal,
                                                              float scale, int H, int nqb, int fill_upper, int64_t total_wg,
                                                              int64_t per_xcd, int jc_len, int items_per_bh, int hpx,
-                                                             item_table tbl, const int *__restrict__ band_lo)
+                                                             item_table tbl, const int *__restrict__ band_lo, int tri_gl)
 {
     static_assert(!BAND || SCORES_ONLY, "the band mask belongs to the scores-only kernel");
     using G = fused_geom<R, SK, NW>;
@@ -527,7 +527,11 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? ((R > 7 || (BAND && R >= 7))
     const T *Qp = Q + bh * (int64_t)S * D;
     const T *Kp = K + bh * (int64_t)S * D;
     const T *Vp = SCORES_ONLY ? Kp : V + bh * (int64_t)S * D;
-    T *Op = O + bh * (int64_t)S * (SCORES_ONLY ? S : D);
+    // (scores only, tri_gl > 0: the scores go out in the triangular layout, groups of tri_gl heads interleaved by rows;
+    // nothing above the diagonal is stored then)
+    const bool tri = SCORES_ONLY && tri_gl > 0;
+    T *Op = tri ? O + (bh / (tri ? tri_gl : 1)) * ((tri ? tri_gl : 1) * tri_rowoff(S)) : O + bh * (int64_t)S * (SCORES_ONLY ? S : D);
+    const int tri_i = tri ? (int)(bh % tri_gl) : 0;
 
     // asynchronous copy of key block j into buffer `buf`: K rows cb.., V rows j*BK..; out-of-range keys
     // re-read a valid row (their scores are zeroed / their probabilities are 0 later)
@@ -856,8 +860,11 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? ((R > 7 || (BAND && R >= 7))
                     // of being kept in registers across the key-block loop - the kernel is at its register limit)
                     const int kg_o = opaque_lane(kg);
                     const int col = j * F_BK + (cb - 1 + (kg_o & 1)) * 16 + (kg_o >> 1) * 8;
-                    if (row_stored[rb] && (PLAIN || (col < S && (!causal || fill_upper || col <= p_))))
-                        *reinterpret_cast<u32x4_t *>(Op + (int64_t)p_ * S + col) = u32x4_t{s0[0], s1[0], s0[1], s1[1]};
+                    if (row_stored[rb] && (PLAIN || (col < S && (!causal || fill_upper || col <= p_)))) {
+                        // (triangular layout: the row's start from a laundered row number, for the same reason)
+                        T *dst = tri ? Op + (tri_row_start(opaque_lane(p_), tri_gl, tri_i) + (unsigned)col) : Op + (int64_t)p_ * S + col;
+                        *reinterpret_cast<u32x4_t *>(dst) = u32x4_t{s0[0], s1[0], s0[1], s1[1]};
+                    }
                 }
             } else {
                 // conv output and scaled logits are rounded to the I/O dtype, as the unfused pipeline stores them
@@ -1027,7 +1034,7 @@ __global__ __launch_bounds__(64 * NW, SCORES_ONLY ? ((R > 7 || (BAND && R >= 7))
 
 template <typename T, int D, int R, int SK, bool SCORES_ONLY, bool BAND = false>
 int launch_mfma(const void *q, const void *k, const void *v, const void *w, void *o, float *lse, int64_t B, int64_t H,
-                int64_t S, int causal, float scale, int fill_upper, hipStream_t st, const int *band_lo = nullptr)
+                int64_t S, int causal, float scale, int fill_upper, hipStream_t st, const int *band_lo = nullptr, int tri_gl = 0)
 {
     constexpr int NW = 4;
     constexpr int F_NT = 64 * NW;
@@ -1089,18 +1096,19 @@ int launch_mfma(const void *q, const void *k, const void *v, const void *w, void
     dim3 grid((unsigned)(per_xcd * 8));
     hipLaunchKernelGGL(kern, grid, dim3(F_NT), 0, st, (const T *)q, (const T *)k, (const T *)v, (const T *)w, (T *)o,
                        lse, (int)S, causal, scale, (int)H, nqb, fill_upper, total_wg, per_xcd, jc_len, (int)items_per_bh,
-                       (B * H) % 8 == 0 ? (int)(B * H / 8) : 0, tbl, band_lo);
+                       (B * H) % 8 == 0 ? (int)(B * H / 8) : 0, tbl, band_lo, tri_gl);
     return launch_status();
 }
 
 // returns 1 when no instantiation covers the kernel size (the caller then uses the general kernel)
 template <typename T, int D, bool SCORES_ONLY, bool BAND = false>
 int dispatch_mfma(const void *q, const void *k, const void *v, const void *w, void *o, float *lse, int64_t B, int64_t H,
-                  int64_t S, int R, int Sk, int causal, float scale, int fill_upper, hipStream_t st, const int *band_lo = nullptr)
+                  int64_t S, int R, int Sk, int causal, float scale, int fill_upper, hipStream_t st, const int *band_lo = nullptr,
+                  int tri_gl = 0)
 {
     if constexpr (sizeof(T) == 2) {
 #define MTA_FUSED_CASE(r, s) \
-    if (R == r && Sk == s) return launch_mfma<T, D, r, s, SCORES_ONLY, BAND>(q, k, v, w, o, lse, B, H, S, causal, scale, fill_upper, st, band_lo);
+    if (R == r && Sk == s) return launch_mfma<T, D, r, s, SCORES_ONLY, BAND>(q, k, v, w, o, lse, B, H, S, causal, scale, fill_upper, st, band_lo, tri_gl);
         MTA_FUSED_CASE(3, 3)
         MTA_FUSED_CASE(5, 5)
         MTA_FUSED_CASE(5, 7)
@@ -1208,6 +1216,39 @@ extern "C" int mta_qk_conv_fwd(const void *q, const void *k, const void *w, void
                      : dispatch_mfma<io_t, 128, true>(q, k, nullptr, w, s_out, nullptr, B, H, S, R, Sk, causal, scale, fill_upper, st);
     });
     // (mta_qk_conv_supported must agree with the dispatch: a kernel size it names always has an instance)
+    if (rc == 1 && scores_instance(R, Sk)) return MTA_ERR_KERNEL_SIZE;
+    return rc == 1 ? MTA_ERR_UNSUPPORTED : rc;
+}
+
+// mta_qk_conv_fwd (causal) / mta_qk_conv_band_fwd (first_visible not NULL) with the scores stored in the triangular
+// layout (see tri_rowoff in common.hpp), groups of `group` heads interleaved by rows: B*H*tri_rowoff(S) elements, nothing
+// above the diagonal.
+extern "C" int mta_qk_conv_tri_fwd(const void *q, const void *k, const void *w, const void *first_visible, void *s_out,
+                                   int64_t B, int64_t H, int64_t S, int64_t D, int R, int Sk, float scale, int group,
+                                   int io_dtype, int w_dtype, void *stream)
+{
+    if (!q || !k || !w || !s_out) return MTA_ERR_NULL;
+    if (!dtype_size(io_dtype) || !dtype_size(w_dtype)) return MTA_ERR_DTYPE;
+    if (B <= 0 || H <= 0 || S <= 0 || S > (1 << 24) || B * H > 65535) return MTA_ERR_SHAPE;
+    if (group <= 0 || H % group != 0) return MTA_ERR_GROUP;
+    if (R < 1 || Sk < 1 || R > MTA_MAX_FUSED_KERNEL_R || Sk > MTA_MAX_FUSED_KERNEL_S) return MTA_ERR_KERNEL_SIZE;
+    if (D != 64 && D != 128) return MTA_ERR_HEAD_DIM;
+    if (!aligned_to(q, 16) || !aligned_to(k, 16) || !aligned_to(s_out, 16) || !aligned_to(w, dtype_size(w_dtype)) ||
+        (first_visible && !aligned_to(first_visible, 4)))
+        return MTA_ERR_ALIGN;
+    if (io_dtype == MTA_F32 || w_dtype != io_dtype || S % 8 != 0) return MTA_ERR_UNSUPPORTED;
+    if ((int64_t)group * tri_rowoff((int)S) > 0x7fffffffLL) return MTA_ERR_UNSUPPORTED;  // (32-bit offsets inside a group)
+    hipStream_t st = (hipStream_t)stream;
+    const int *lo = (const int *)first_visible;
+    int rc = 1;
+    MTA_DISPATCH_IO(io_dtype, {
+        if (lo)
+            rc = D == 64 ? dispatch_mfma<io_t, 64, true, true>(q, k, nullptr, w, s_out, nullptr, B, H, S, R, Sk, 1, scale, 0, st, lo, group)
+                         : dispatch_mfma<io_t, 128, true, true>(q, k, nullptr, w, s_out, nullptr, B, H, S, R, Sk, 1, scale, 0, st, lo, group);
+        else
+            rc = D == 64 ? dispatch_mfma<io_t, 64, true>(q, k, nullptr, w, s_out, nullptr, B, H, S, R, Sk, 1, scale, 0, st, nullptr, group)
+                         : dispatch_mfma<io_t, 128, true>(q, k, nullptr, w, s_out, nullptr, B, H, S, R, Sk, 1, scale, 0, st, nullptr, group);
+    });
     if (rc == 1 && scores_instance(R, Sk)) return MTA_ERR_KERNEL_SIZE;
     return rc == 1 ? MTA_ERR_UNSUPPORTED : rc;
 }

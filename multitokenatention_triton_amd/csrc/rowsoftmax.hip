@@ -505,7 +505,7 @@ template <bool IS_MAX, int G, int NW> __device__ __forceinline__ void heads_comb
 template <typename T, int G, int NV, bool HAS1, bool HAS2, int NT, int OCC, bool BAND = false>
 __global__ __launch_bounds__(NT, OCC) void mix_softmax_mix_packed(
     const T *__restrict__ x, const T *__restrict__ w1, const T *__restrict__ w2, T *__restrict__ y, int C, int P, int Q,
-    int causal, int fill_upper, const int *__restrict__ row_lo)
+    int causal, int fill_upper, const int *__restrict__ row_lo, int tri)
 {
     constexpr int VEC = 8, NW = NT / 64, H2 = G / 2;
     static_assert(sizeof(T) == 2 && G % 2 == 0, "packed pairs of a 16-bit type");
@@ -519,8 +519,12 @@ __global__ __launch_bounds__(NT, OCC) void mix_softmax_mix_packed(
     const int tid = threadIdx.x;
     const int g = (int)(b % groups);
     const int64_t n = b / groups;
-    const int64_t plane = (int64_t)P * Q;
-    const int64_t base = (n * C + (int64_t)g * G) * plane + (int64_t)p * Q;
+    int64_t plane = (int64_t)P * Q;
+    int64_t base = (n * C + (int64_t)g * G) * plane + (int64_t)p * Q;
+    if (tri) {  // triangular layout (square, causal, nothing stored above the diagonal): the group's rows p lie side by side
+        plane = tri_rowlen(p);
+        base = (n * groups + g) * (G * tri_rowoff(P)) + G * tri_rowoff(p);
+    }
     const int last = causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;  // last attended key
 
     // live passes of this wavefront: pass k covers keys [(k*NT + 64*wave)*VEC, +64*VEC)
@@ -835,7 +839,7 @@ int launch_fixed(const void *x, const void *w1, const void *w2, const float *kb,
 
 template <typename T>
 int dispatch(const void *x, const void *w1, const void *w2, const float *kb_in, const int *row_lo, void *y, int64_t N, int64_t C,
-             int64_t P, int64_t Q, int G, int causal, int w_dtype, int fill_upper, hipStream_t st)
+             int64_t P, int64_t Q, int G, int causal, int w_dtype, int fill_upper, hipStream_t st, int tri = 0)
 {
     // (the kernels without a key bias are the ones without a band mask too: `kb` below stands for "either")
     const float *kb = kb_in;
@@ -848,7 +852,7 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb_in, 
         // the general one, for comparisons)
         static const bool no_packed = [] { const char *e_ = getenv("MTA_SOFTMAX_NO_PACKED"); return e_ && e_[0] == '1'; }();
         const int io_code = std::is_same<T, bf16_t>::value ? MTA_BF16 : MTA_F16;
-        if (G == 16 && plain && !no_packed) {
+        if (G == 16 && plain && !no_packed && !tri) {
             const int rc = mix16_softmax_launch(x, w1, w2, y, N, C, P, Q, causal, fill_upper, io_code, w_dtype, st);
             if (rc != MTA_ERR_UNSUPPORTED) return rc;
         }
@@ -861,7 +865,7 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb_in, 
     {                                                                                                                  \
         hipLaunchKernelGGL((mix_softmax_mix_packed<T, g, 1, h1, h2, nt, occ, true>), dim3((unsigned)(N * (C / g) * P)), \
                            dim3(nt), 0, st, (const T *)x, (const T *)w1, (const T *)w2, (T *)y, (int)C, (int)P,        \
-                           (int)Q, causal, fill_upper, row_lo);                                                        \
+                           (int)Q, causal, fill_upper, row_lo, tri);                                                   \
         return launch_status();                                                                                        \
     }
 #define MTA_RSB_CASE(g, nt, occ)                                                                                       \
@@ -878,7 +882,7 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb_in, 
     {                                                                                                                  \
         hipLaunchKernelGGL((mix_softmax_mix_packed<T, g, v, h1, h2, nt, occ>), dim3((unsigned)(N * (C / g) * P)),      \
                            dim3(nt), 0, st, (const T *)x, (const T *)w1, (const T *)w2, (T *)y, (int)C, (int)P,        \
-                           (int)Q, causal, fill_upper, nullptr);                                                       \
+                           (int)Q, causal, fill_upper, nullptr, tri);                                                  \
         return launch_status();                                                                                        \
     }
 #define MTA_RSP_CASE(g, v, nt, occ)                                                                                    \
@@ -896,6 +900,7 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb_in, 
 #undef MTA_RSP_LAUNCH
         }
     }
+    if (tri) return MTA_ERR_UNSUPPORTED;  // (only the kernels above know the triangular layout)
     if (vec_ok) {
 #define MTA_RS_CASE(g, v)                                                                   \
     if (G == g && nv <= v) return launch_fixed<T, g, v>(x, w1, w2, kb, row_lo, y, N, C, P, Q, causal, w_dtype, fill_upper, st);
@@ -932,6 +937,43 @@ extern "C" int mta_headmix_softmax_band_fwd(const void *x, const void *w1, const
     MTA_DISPATCH_IO(io_dtype, return dispatch<io_t>(x, w1, w2, (const float *)key_bias, (const int *)first_visible, y, N, C, P, Q,
                                                     G, causal, w_dtype, fill_upper || !causal, st));
     return MTA_ERR_DTYPE;
+}
+
+// The same pass over a causal square score tensor in the triangular layout (see tri_rowoff in common.hpp), groups of
+// `group_size` heads interleaved by rows, input and output alike; nothing above the diagonal exists.  16-bit data with
+// weights of the same dtype and groups of 2, 4 or 8 heads only (MTA_ERR_UNSUPPORTED otherwise).
+extern "C" int mta_headmix_softmax_tri_fwd(const void *x, const void *w1, const void *w2, const void *first_visible, void *y,
+                                           int64_t N, int64_t C, int64_t S, int group_size, int io_dtype, int w_dtype,
+                                           void *stream)
+{
+    if (!x || !y) return MTA_ERR_NULL;
+    if (first_visible && !aligned_to(first_visible, 4)) return MTA_ERR_ALIGN;
+    if (!dtype_size(io_dtype) || !dtype_size(w_dtype)) return MTA_ERR_DTYPE;
+    if (N <= 0 || C <= 0 || S <= 0 || S > (1 << 24) || C > 4096) return MTA_ERR_SHAPE;
+    if (group_size <= 0 || C % group_size != 0) return MTA_ERR_GROUP;
+    if (!aligned_to(x, 16) || !aligned_to(y, 16)) return MTA_ERR_ALIGN;
+    if (N * (C / group_size) * S > 0x7fffffffLL) return MTA_ERR_SHAPE;
+    if (io_dtype == MTA_F32 || (!w1 && !w2)) return MTA_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    if (io_dtype == MTA_BF16)
+        return dispatch<bf16_t>(x, w1, w2, nullptr, (const int *)first_visible, y, N, C, S, S, group_size, 1, w_dtype, 0, st, 1);
+    return dispatch<f16_t>(x, w1, w2, nullptr, (const int *)first_visible, y, N, C, S, S, group_size, 1, w_dtype, 0, st, 1);
+}
+
+// Whether mta_headmix_softmax_tri_fwd has a kernel for these sizes (the cases of `dispatch` that know the layout: the
+// packed kernel's instances, with a band mask those for one weight and one pass per wavefront).  Nothing is launched.
+extern "C" int mta_headmix_softmax_tri_supported(int64_t C, int64_t S, int group_size, int io_dtype, int w_dtype,
+                                                 int has_w1, int has_w2, int band)
+{
+    if (io_dtype != MTA_BF16 && io_dtype != MTA_F16) return 0;
+    if (w_dtype != io_dtype || (!has_w1 && !has_w2) || group_size <= 0 || C <= 0 || C % group_size != 0 || S <= 0 || S % 8 != 0)
+        return 0;
+    const char *e = getenv("MTA_SOFTMAX_NO_PACKED");
+    if (e && e[0] == '1') return 0;
+    if (band && has_w1 && has_w2) return 0;
+    const int g = group_size;
+    const int64_t cap = band ? (g == 4 ? 4096 : (g == 2 || g == 8) ? 2048 : 0) : (g == 2 ? 8192 : g == 4 ? 4096 : g == 8 ? 2048 : 0);
+    return S <= cap ? 1 : 0;
 }
 
 extern "C" int mta_headmix_softmax_bias_fwd(const void *x, const void *w1, const void *w2, const void *key_bias,

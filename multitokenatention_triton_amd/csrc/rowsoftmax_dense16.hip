@@ -231,20 +231,6 @@ __global__ __launch_bounds__(64 * NW, 4) void mix16_softmax_kernel(const T *__re
     }
 }
 
-// Four 16-byte LDS reads (1 KB apart) and the wait for them in one statement: the values are defined when it ends.
-template <int OFF>
-__device__ __forceinline__ void lds_load4x16_sync(unsigned addr, u32x4_t &a, u32x4_t &b, u32x4_t &c, u32x4_t &d)
-{
-    asm volatile("ds_read_b128 %0, %4 offset:%5\n\t"
-                 "ds_read_b128 %1, %4 offset:%6\n\t"
-                 "ds_read_b128 %2, %4 offset:%7\n\t"
-                 "ds_read_b128 %3, %4 offset:%8\n\t"
-                 "s_waitcnt lgkmcnt(0)"
-                 : "=&v"(a), "=&v"(b), "=&v"(c), "=&v"(d)
-                 : "v"(addr), "n"(OFF), "n"(OFF + 1024), "n"(OFF + 2048), "n"(OFF + 3072)
-                 : "memory");
-}
-
 // Lists of rows per workgroup.  A workgroup that walks "load, reduce, barrier, exponentials, reduce, barrier, store"
 // alone on its CU leaves the memory pipe idle while it computes and the vector units idle while it loads, so here a
 // workgroup of 16 wavefronts takes a list of steps of one (batch, group) - a step is one row of more than 2048 attended
@@ -350,7 +336,7 @@ __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(cons
             const int key = q0 + ln * 8;
             if (q0 > last) return;  // (wavefront-uniform) wholly beyond the attended keys: s[i] stays unused
             u32x4_t xv[4];
-            lds_load4x16_sync<i * 4096>(stage_lds, xv[0], xv[1], xv[2], xv[3]);
+            lds_load4x16_sync(stage_lds, i * 4096, xv[0], xv[1], xv[2], xv[3]);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 if constexpr (HAS1) {

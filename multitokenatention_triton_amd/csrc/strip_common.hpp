@@ -42,6 +42,18 @@ __device__ __forceinline__ u32x4 lds_load16_sync(unsigned addr)
     asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
     return v;
 }
+// four such reads (1 KB apart, from byte offset `off`: a compile-time constant below 62464) and the wait, one statement
+__device__ __forceinline__ void lds_load4x16_sync(unsigned addr, int off, u32x4 &a, u32x4 &b, u32x4 &c, u32x4 &d)
+{
+    asm volatile("ds_read_b128 %0, %4 offset:%5\n\t"
+                 "ds_read_b128 %1, %4 offset:%6\n\t"
+                 "ds_read_b128 %2, %4 offset:%7\n\t"
+                 "ds_read_b128 %3, %4 offset:%8\n\t"
+                 "s_waitcnt lgkmcnt(0)"
+                 : "=&v"(a), "=&v"(b), "=&v"(c), "=&v"(d)
+                 : "v"(addr), "n"(off), "n"(off + 1024), "n"(off + 2048), "n"(off + 3072)
+                 : "memory");
+}
 // the same with a compile-time byte offset in the instruction (no address arithmetic per access)
 // (`off` must fold to a constant below 65536: it goes into the instruction's offset field)
 __device__ __forceinline__ u32x4 lds_load16_at(unsigned addr, int off)

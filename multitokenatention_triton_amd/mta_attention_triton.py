@@ -48,6 +48,8 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Optional
 
+import os
+
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
@@ -277,6 +279,10 @@ class MTAAttentionTriton(nn.Module):
         self.wposm_triton = TritonLinearHead(n_heads, causal=causal)
         # optional observer: called as hook(stage_name) right before each stage is enqueued
         self._stage_hook = None
+        # layout of the score tensors between the kernels of the inference route: "auto" = triangular where all three
+        # kernels know it, "planes" = (B,H,S,S) always (MTA_SCORE_LAYOUT=planes in the environment: the same, for
+        # comparisons)
+        self.score_layout = "planes" if os.environ.get("MTA_SCORE_LAYOUT") == "planes" else "auto"
         # "dense": assume nothing; "declared": use self._declared; "probe": look at the weights on every call
         self.weight_structure = "dense"
         self._declared = WeightStructure()
@@ -327,6 +333,22 @@ class MTAAttentionTriton(nn.Module):
         # the last stage may leave the upper triangle unwritten only if our own P V kernel consumes it
         own_pv = (xq.size(-2) == xk.size(-2) and xq.dtype == xv.dtype
                   and ops.causal_pv_supported(xq.dtype, xq.size(-2), xv.size(-1)))
+
+        # Three kernels with nothing elementwise between them: the two score tensors are nobody else's business, and they
+        # travel in the triangular layout (what lies on and below the diagonal only, the rows a workgroup of the softmax
+        # stage reads side by side): half the footprint, and every stage streams memory in longer runs.
+        if (self.score_layout != "planes" and self.causal and one_pass and key_bias is None and own_pv
+                and not (self.training and self.dropout > 0) and g_both in (2, 4, 8)
+                and ops.tri_route_supported(xq, xk, self.mta_conv_triton.weight, g_both, w1, w2, first_visible is not None)):
+            self._mark("qk_conv")
+            scores = ops.qk_conv_tri(xq, xk, self.mta_conv_triton.weight, scale, g_both, first_visible=first_visible)
+            self._mark("mix_softmax_mix")
+            scores = ops.headmix_softmax_tri(scores, w1, w2, xq.size(0), self.n_heads, n_keys, g_both,
+                                             first_visible=first_visible)
+            self._mark("pv")
+            output = ops.causal_pv_tri(scores, xv, g_both, first_visible=first_visible)
+            self._mark("end")
+            return output.transpose(1, 2)
 
         # QK^T -> *1/sqrt(d) -> conv: one kernel when it exists for this dtype / size, else GEMM + conv
         scores = None

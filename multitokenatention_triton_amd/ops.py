@@ -387,6 +387,138 @@ def causal_pv(p: torch.Tensor, v: torch.Tensor, causal: bool,
     return out
 
 
+# ---------------------------------------------------------------------------------------
+# the causal forward's three stages over score tensors in the triangular layout (include/mta_hip.h): what lies on and
+# below the diagonal only, rows padded to 64 keys, the heads of a mixing group interleaved by rows
+# ---------------------------------------------------------------------------------------
+def tri_row_offset(p: int) -> int:
+    """Elements of one head ahead of row p in the triangular layout; tri_row_offset(S) is a head's size."""
+    a = p >> 6
+    return 2048 * a * (a + 1) + (p & 63) * 64 * (a + 1)
+
+
+def _band_arg(first_visible, b, s):
+    if first_visible is None:
+        return None
+    first_visible = _device_tensor(first_visible, "first_visible")
+    if first_visible.dtype != torch.int32 or tuple(first_visible.shape) != (b, s):
+        raise ValueError(f"first_visible must be int32 of shape ({b},{s}), got {first_visible.dtype} "
+                         f"{tuple(first_visible.shape)}")
+    return first_visible
+
+
+def tri_route_supported(q: torch.Tensor, k: torch.Tensor, conv_weight: torch.Tensor, group: int, w1, w2, band: bool) -> bool:
+    """Whether the three triangular-layout kernels exist for these tensors (host-side questions to the library)."""
+    if not qk_conv_supported(q, k, conv_weight) or q.dtype not in (torch.bfloat16, torch.float16):
+        return False
+    b, h, s, d = q.shape
+    ws = [w for w in (w1, w2) if w is not None]
+    if not ws or any(w.dtype != q.dtype or w.data_ptr() % 4 for w in ws) or h % group != 0:
+        return False
+    if group * tri_row_offset(s) >= 2 ** 31 or not causal_pv_supported(q.dtype, s, d):
+        return False
+    return bool(_lib.load().mta_headmix_softmax_tri_supported(h, s, group, _DTYPE_CODE[q.dtype], _DTYPE_CODE[ws[0].dtype],
+                                                              int(w1 is not None), int(w2 is not None), int(band)))
+
+
+def qk_conv_tri(q: torch.Tensor, k: torch.Tensor, weight: torch.Tensor, scale: float, group: int,
+                first_visible: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal scale * conv(mask0(Q K^T)) in the triangular layout with groups of ``group`` heads: a flat tensor of
+    B*H*tri_row_offset(S) elements; see mta_qk_conv_tri_fwd."""
+    q = _device_tensor(q, "Q")
+    k = _device_tensor(k, "K")
+    weight = _device_tensor(weight.detach(), "W")
+    if q.dim() != 4 or q.shape != k.shape or q.dtype != k.dtype:
+        raise ValueError(f"Q and K must share a (B,H,S,D) shape and dtype, got {tuple(q.shape)}, {tuple(k.shape)}")
+    b, h, s, d = q.shape
+    assert weight.dim() == 3 and weight.shape[0] == h, "conv weight must be (H,R,S)"
+    first_visible = _band_arg(first_visible, b, s)
+    out = torch.empty((b * h * tri_row_offset(s),), dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = _lib.load().mta_qk_conv_tri_fwd(q.data_ptr(), k.data_ptr(), weight.data_ptr(),
+                                             first_visible.data_ptr() if first_visible is not None else None,
+                                             out.data_ptr(), b, h, s, d, weight.shape[1], weight.shape[2], float(scale),
+                                             int(group), _code(q, "Q"), _code(weight, "W"), _stream(q))
+    _lib.check(rc, "mta_qk_conv_tri_fwd")
+    return out
+
+
+def headmix_softmax_tri(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optional[torch.Tensor], n: int, c: int, s: int,
+                        group: int, first_visible: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """mix(w1) -> causal row softmax -> mix(w2) over a flat tensor in the triangular layout (mixing groups = the layout's
+    groups); see mta_headmix_softmax_tri_fwd."""
+    x = _device_tensor(x, "input")
+    if x.dim() != 1 or x.numel() != n * c * tri_row_offset(s):
+        raise ValueError(f"expected a flat tensor of {n * c * tri_row_offset(s)} elements, got {tuple(x.shape)}")
+    ws = []
+    for w in (w1, w2):
+        if w is not None:
+            w = _device_tensor(w.detach(), "weight")
+            assert tuple(w.shape) == (c, c), f"Weight must be ({c},{c}), got {tuple(w.shape)}"
+        ws.append(w)
+    present = [w for w in ws if w is not None]
+    if not present or any(w.dtype != present[0].dtype for w in present):
+        raise TypeError("one or two weights of one dtype")
+    first_visible = _band_arg(first_visible, n, s)
+    y = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().mta_headmix_softmax_tri_fwd(
+            x.data_ptr(), ws[0].data_ptr() if ws[0] is not None else None, ws[1].data_ptr() if ws[1] is not None else None,
+            first_visible.data_ptr() if first_visible is not None else None, y.data_ptr(), n, c, s, int(group),
+            _code(x, "input"), _code(present[0], "weight"), _stream(x))
+    _lib.check(rc, "mta_headmix_softmax_tri_fwd")
+    return y
+
+
+def causal_pv_tri(p: torch.Tensor, v: torch.Tensor, group: int, first_visible: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """P V with P a flat tensor in the triangular layout and V (B,H,S,D); see mta_causal_pv_tri_fwd."""
+    p = _device_tensor(p, "P")
+    v = _device_tensor(v, "V")
+    b, h, s, d = v.shape
+    if p.dim() != 1 or p.numel() != b * h * tri_row_offset(s) or p.dtype != v.dtype:
+        raise ValueError(f"expected a flat tensor of {b * h * tri_row_offset(s)} elements of V's dtype")
+    first_visible = _band_arg(first_visible, b, s)
+    out = torch.empty_like(v)
+    with torch.cuda.device(p.device):
+        rc = _lib.load().mta_causal_pv_tri_fwd(p.data_ptr(), v.data_ptr(),
+                                               first_visible.data_ptr() if first_visible is not None else None,
+                                               out.data_ptr(), b, h, s, d, int(group), _code(p, "P"), _stream(p))
+    _lib.check(rc, "mta_causal_pv_tri_fwd")
+    return out
+
+
+def _tri_index(b: int, h: int, s: int, group: int, device) -> torch.Tensor:
+    """Flat positions of the elements (b, h, p, q <= p) of the triangular layout, as a (B,H,S,S) int64 tensor (-1 above the
+    diagonal)."""
+    rows = torch.arange(s, device=device)
+    a = rows >> 6
+    off = 2048 * a * (a + 1) + (rows & 63) * 64 * (a + 1)            # (S,)
+    length = (a + 1) * 64
+    bh = torch.arange(b * h, device=device)
+    gbase = (bh // group) * (group * tri_row_offset(s))              # (B*H,)
+    idx = (gbase[:, None, None] + (group * off)[None, :, None] + ((bh % group)[:, None, None] * length[None, :, None])
+           + rows[None, None, :])
+    idx = idx.masked_fill(rows[None, None, :] > rows[None, :, None], -1)
+    return idx.view(b, h, s, s)
+
+
+def tri_unpack(x: torch.Tensor, b: int, h: int, s: int, group: int) -> torch.Tensor:
+    """(B,H,S,S) tensor (zero above the diagonal) from a flat tensor in the triangular layout; for tests and inspection."""
+    idx = _tri_index(b, h, s, group, x.device)
+    out = x[idx.clamp_min(0)]
+    return out.masked_fill(idx < 0, 0)
+
+
+def tri_pack(x: torch.Tensor, group: int, pad_value: float = float("nan")) -> torch.Tensor:
+    """The inverse of tri_unpack (padding and nothing else filled with ``pad_value``); for tests and inspection."""
+    b, h, s, _ = x.shape
+    idx = _tri_index(b, h, s, group, x.device)
+    out = torch.full((b * h * tri_row_offset(s),), pad_value, dtype=x.dtype, device=x.device)
+    keep = idx >= 0
+    out[idx[keep]] = x[keep]
+    return out
+
+
 def causal_ptx(p: torch.Tensor, x: torch.Tensor, causal: bool) -> Optional[torch.Tensor]:
     """P^T X for P (B,H,S,S), X (B,H,S,D): out[k] = sum_p P[p,k] X[p], over p >= k only when causal (nothing of P above
     the diagonal is read); see mta_causal_ptx_fwd.  Returns ``None`` when unsupported (the caller then uses

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/mta_hip.h but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes signatures out of sync with the header"
-    assert lib.mta_abi_version() == 8
+    assert lib.mta_abi_version() == 9
 
 
 def test_no_torch_symbols_in_the_library():

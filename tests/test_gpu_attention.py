@@ -435,6 +435,81 @@ def test_mta_use_mask_band_masks_run_through_the_kernels(pkg, kind, dtype):
     torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
 
 
+TRI_CASES = [
+    # B, H, S, D, R, Sk, group, dtype, band kind, weights
+    (2, 8, 520, 64, 6, 11, 4, torch.bfloat16, None, "both"), (1, 4, 1160, 128, 3, 3, 2, torch.float16, None, "first"),
+    (1, 8, 264, 128, 7, 7, 8, torch.bfloat16, None, "second"), (1, 8, 2304, 64, 6, 11, 4, torch.bfloat16, None, "both"),
+    (2, 4, 776, 128, 6, 11, 4, torch.bfloat16, "documents", "first"), (1, 4, 2048, 64, 5, 5, 2, torch.float16, "window", "second"),
+    (1, 8, 520, 64, 11, 15, 8, torch.bfloat16, "ragged", "first"), (1, 4, 4096, 128, 6, 11, 4, torch.bfloat16, None, "both"),
+]
+
+
+@pytest.mark.parametrize("case", TRI_CASES)
+def test_triangular_layout_stages_equal_the_plane_layout(pkg, case):
+    """The three kernels of the causal forward over score tensors in the triangular layout (lower triangle only, rows
+    padded to 64 keys, the heads of a group interleaved by rows): the same values, bit for bit, as over (B,H,S,S)
+    tensors, stage by stage; padding and whatever lies ahead of a band is never read (NaN there changes nothing)."""
+    b, h, s, d, r, sk, group, dtype, kind, weights = case
+    print(f"triangular layout case={case}", flush=True)
+    ops = pkg.ops
+    q, k, v = (t.cuda() for t in O.seeded_qkv(b, h, s, d, dtype, seed=61))
+    g = torch.Generator().manual_seed(62)
+    w = (torch.randn(h, r, sk, generator=g) * 0.2).to(dtype).cuda()
+    w1 = O.block_diag_head_weight(h, group, 0.1, g, dtype).cuda() if weights in ("both", "first") else None
+    w2 = O.block_diag_head_weight(h, group, 0.1, g, dtype).cuda() if weights in ("both", "second") else None
+    first = _band_first(kind, b, s).cuda() if kind else None
+    assert ops.tri_route_supported(q, k, w, group, w1, w2, kind is not None)
+    scale = d ** -0.5
+    rows = torch.arange(s, device="cuda")
+    visible = rows[None, :] <= rows[:, None]                                                   # (S,S)
+    visible = visible[None].expand(b, s, s) if first is None else visible[None] & (rows[None, None, :] >= first[:, :, None])
+    visible = visible[:, None].expand(b, h, s, s)
+
+    s_plane = ops.qk_conv(q, k, w, True, scale, fill_upper=False, first_visible=first)
+    s_tri = ops.qk_conv_tri(q, k, w, scale, group, first_visible=first)
+    assert s_tri.numel() == b * h * ops.tri_row_offset(s)
+    assert torch.equal(ops.tri_unpack(s_tri, b, h, s, group)[visible], s_plane[visible])
+
+    p_plane = ops.headmix_softmax(s_plane, w1, w2, True, group_size=group, fill_upper=False, first_visible=first)
+    p_tri = ops.headmix_softmax_tri(s_tri, w1, w2, b, h, s, group, first_visible=first)
+    lower = (rows[None, :] <= rows[:, None])[None, None].expand(b, h, s, s)
+    assert torch.equal(ops.tri_unpack(p_tri, b, h, s, group)[lower], p_plane[lower])
+    # the same from an input whose padding, and whatever a band hides, is NaN
+    poisoned = ops.tri_pack(s_plane.masked_fill(~visible, float("nan")), group)
+    assert torch.equal(ops.headmix_softmax_tri(poisoned, w1, w2, b, h, s, group, first_visible=first)[ops.tri_pack(lower.to(dtype), group, 0.0) > 0],
+                       p_tri[ops.tri_pack(lower.to(dtype), group, 0.0) > 0])
+
+    o_plane = ops.causal_pv(p_plane, v, True, first_visible=first)
+    assert torch.equal(ops.causal_pv_tri(p_tri, v, group, first_visible=first), o_plane)
+    assert torch.equal(ops.causal_pv_tri(ops.tri_pack(p_plane.masked_fill(~lower, float("nan")), group), v, group,
+                                         first_visible=first), o_plane)
+
+
+@pytest.mark.parametrize("masked", [False, True])
+def test_mta_score_layouts_agree(pkg, masked):
+    """The module's inference route with the score tensors in the triangular layout (the default where the three kernels
+    know it) and in planes: the same stages, the same output bit for bit."""
+    print(f"mta score layouts masked={masked}", flush=True)
+    dtype = torch.bfloat16
+    b, h, s, d = 2, 8, 1160, 128
+    q, k, v = (t.cuda() for t in O.seeded_qkv(b, h, s, d, dtype, seed=71))
+    params = _config_like(h, 4, 6, 11, 0.05, dtype)
+    mod = _mta_module(pkg, h, 6, 11, 3, 3, *params, dtype, use_mask=masked, structure="infer")
+    mask = None
+    if masked:
+        rows = torch.arange(s)
+        mask = ((rows[None, :] <= rows[:, None]) & (rows[None, :] > rows[:, None] - 300))[None, None].cuda()
+    outs, stages = {}, {}
+    for layout in ("auto", "planes"):
+        mod.score_layout = layout
+        seen = []
+        mod._stage_hook = seen.append
+        outs[layout] = mod(q, k, v, mask, None)
+        stages[layout] = seen
+    assert stages["auto"] == stages["planes"] == ["qk_conv", "mix_softmax_mix", "pv", "end"]
+    assert torch.equal(outs["auto"], outs["planes"])
+
+
 def test_qk_conv_reports_unsupported(pkg):
     q = torch.zeros(1, 2, 64, 64, device="cuda")
     assert pkg.ops.qk_conv(q, q, torch.zeros(2, 3, 3, device="cuda"), True, 0.1) is None          # fp32

@@ -29,6 +29,9 @@ GROUPS = [
     # groups of wavefronts)
     ({"MTA_PV_SPLIT": "1"}, ["tests/test_gpu_attention.py"], "test_causal_pv"),
     # mix -> softmax -> mix for groups of 16 heads with a workgroup per row (by default workgroups take lists of rows)
+    # the inference route with its score tensors as (B,H,S,S) planes (by default: the triangular layout)
+    ({"MTA_SCORE_LAYOUT": "planes"}, ["tests/test_gpu_attention.py"],
+     "test_mta_headline or test_mta_use_mask or test_mta_fused_route or test_mta_module"),
     ({"MTA_MIX16_NO_ROW_LISTS": "1"}, ["tests/test_gpu_ops.py"], "(test_mix_softmax_mix_parity and not f32) or test_mix_softmax_mix_dense16"),
 ]
 
