@@ -21,7 +21,7 @@ constexpr int RS_OCC = 5;  // wavefronts per SIMD the G*NV = 8 instances (e.g. 4
 namespace mta {
 // rowsoftmax_dense16.hip: the same pass for groups of 16 heads, both mixes on the matrix cores
 int mix16_softmax_launch(const void *x, const void *w1, const void *w2, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
-                         int causal, int fill_upper, int io_dtype, int w_dtype, hipStream_t st);
+                         int causal, int fill_upper, int io_dtype, int w_dtype, hipStream_t st, int tri_in = 0, int tri_out = 0);
 }  // namespace mta
 
 namespace {
@@ -839,8 +839,9 @@ int launch_fixed(const void *x, const void *w1, const void *w2, const float *kb,
 
 template <typename T>
 int dispatch(const void *x, const void *w1, const void *w2, const float *kb_in, const int *row_lo, void *y, int64_t N, int64_t C,
-             int64_t P, int64_t Q, int G, int causal, int w_dtype, int fill_upper, hipStream_t st, int tri = 0)
+             int64_t P, int64_t Q, int G, int causal, int w_dtype, int fill_upper, hipStream_t st, int tri_in = 0, int tri_out = 0)
 {
+    const int tri = tri_in && tri_out;  // (the packed kernels: both tensors in the triangular layout, or neither)
     // (the kernels without a key bias are the ones without a band mask too: `kb` below stands for "either")
     const float *kb = kb_in;
     const bool plain = !kb_in && !row_lo;
@@ -852,10 +853,11 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb_in, 
         // the general one, for comparisons)
         static const bool no_packed = [] { const char *e_ = getenv("MTA_SOFTMAX_NO_PACKED"); return e_ && e_[0] == '1'; }();
         const int io_code = std::is_same<T, bf16_t>::value ? MTA_BF16 : MTA_F16;
-        if (G == 16 && plain && !no_packed && !tri) {
-            const int rc = mix16_softmax_launch(x, w1, w2, y, N, C, P, Q, causal, fill_upper, io_code, w_dtype, st);
+        if (G == 16 && plain && !no_packed) {
+            const int rc = mix16_softmax_launch(x, w1, w2, y, N, C, P, Q, causal, fill_upper, io_code, w_dtype, st, tri_in, tri_out);
             if (rc != MTA_ERR_UNSUPPORTED) return rc;
         }
+        if (tri_in != tri_out) return MTA_ERR_UNSUPPORTED;
         const bool packed_ok = vec_ok && !no_packed && w_dtype == io_code && (w1 || w2) && (!w1 || aligned_to(w1, 4)) &&
                                (!w2 || aligned_to(w2, 4)) && C % 2 == 0 && Q <= 256 * VEC * 4;
         // band mask without a key bias, one weight, rows that one pass per wavefront covers: the packed kernel's BAND
@@ -900,7 +902,7 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb_in, 
 #undef MTA_RSP_LAUNCH
         }
     }
-    if (tri) return MTA_ERR_UNSUPPORTED;  // (only the kernels above know the triangular layout)
+    if (tri_in || tri_out) return MTA_ERR_UNSUPPORTED;  // (only the kernels above know the triangular layout)
     if (vec_ok) {
 #define MTA_RS_CASE(g, v)                                                                   \
     if (G == g && nv <= v) return launch_fixed<T, g, v>(x, w1, w2, kb, row_lo, y, N, C, P, Q, causal, w_dtype, fill_upper, st);
@@ -940,11 +942,12 @@ extern "C" int mta_headmix_softmax_band_fwd(const void *x, const void *w1, const
 }
 
 // The same pass over a causal square score tensor in the triangular layout (see tri_rowoff in common.hpp), groups of
-// `group_size` heads interleaved by rows, input and output alike; nothing above the diagonal exists.  16-bit data with
-// weights of the same dtype and groups of 2, 4 or 8 heads only (MTA_ERR_UNSUPPORTED otherwise).
+// `group_size` heads interleaved by rows; nothing above the diagonal exists.  out_planes = 0: the output in the same
+// layout (groups of 2, 4, 8 or 16 heads); 1: the output as (N,C,S,S) planes with nothing written above the diagonal
+// (groups of 16).  16-bit data with weights of the same dtype only (MTA_ERR_UNSUPPORTED otherwise).
 extern "C" int mta_headmix_softmax_tri_fwd(const void *x, const void *w1, const void *w2, const void *first_visible, void *y,
-                                           int64_t N, int64_t C, int64_t S, int group_size, int io_dtype, int w_dtype,
-                                           void *stream)
+                                           int64_t N, int64_t C, int64_t S, int group_size, int out_planes, int io_dtype,
+                                           int w_dtype, void *stream)
 {
     if (!x || !y) return MTA_ERR_NULL;
     if (first_visible && !aligned_to(first_visible, 4)) return MTA_ERR_ALIGN;
@@ -956,20 +959,25 @@ extern "C" int mta_headmix_softmax_tri_fwd(const void *x, const void *w1, const 
     if (io_dtype == MTA_F32 || (!w1 && !w2)) return MTA_ERR_UNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
     if (io_dtype == MTA_BF16)
-        return dispatch<bf16_t>(x, w1, w2, nullptr, (const int *)first_visible, y, N, C, S, S, group_size, 1, w_dtype, 0, st, 1);
-    return dispatch<f16_t>(x, w1, w2, nullptr, (const int *)first_visible, y, N, C, S, S, group_size, 1, w_dtype, 0, st, 1);
+        return dispatch<bf16_t>(x, w1, w2, nullptr, (const int *)first_visible, y, N, C, S, S, group_size, 1, w_dtype, 0, st, 1, !out_planes);
+    return dispatch<f16_t>(x, w1, w2, nullptr, (const int *)first_visible, y, N, C, S, S, group_size, 1, w_dtype, 0, st, 1, !out_planes);
 }
 
 // Whether mta_headmix_softmax_tri_fwd has a kernel for these sizes (the cases of `dispatch` that know the layout: the
 // packed kernel's instances, with a band mask those for one weight and one pass per wavefront).  Nothing is launched.
-extern "C" int mta_headmix_softmax_tri_supported(int64_t C, int64_t S, int group_size, int io_dtype, int w_dtype,
-                                                 int has_w1, int has_w2, int band)
+extern "C" int mta_headmix_softmax_tri_supported(int64_t C, int64_t S, int group_size, int out_planes, int io_dtype,
+                                                 int w_dtype, int has_w1, int has_w2, int band)
 {
     if (io_dtype != MTA_BF16 && io_dtype != MTA_F16) return 0;
     if (w_dtype != io_dtype || (!has_w1 && !has_w2) || group_size <= 0 || C <= 0 || C % group_size != 0 || S <= 0 || S % 8 != 0)
         return 0;
     const char *e = getenv("MTA_SOFTMAX_NO_PACKED");
     if (e && e[0] == '1') return 0;
+    if (group_size == 16) {  // the matrix-core kernel's row lists (rowsoftmax_dense16.hip)
+        const char *e2 = getenv("MTA_MIX16_NO_ROW_LISTS");
+        return !band && S <= 4096 && S * S <= (1LL << 27) && !(e2 && e2[0] == '1');
+    }
+    if (out_planes) return 0;
     if (band && has_w1 && has_w2) return 0;
     const int g = group_size;
     const int64_t cap = band ? (g == 4 ? 4096 : (g == 2 || g == 8) ? 2048 : 0) : (g == 2 ? 8192 : g == 4 ? 4096 : g == 8 ? 2048 : 0);

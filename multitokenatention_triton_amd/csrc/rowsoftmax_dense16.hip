@@ -244,7 +244,7 @@ template <typename T, bool HAS1, bool HAS2>
 __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(const T *__restrict__ x, const T *__restrict__ w1,
                                                                            const T *__restrict__ w2, T *__restrict__ y, int C,
                                                                            int P, int Q, int causal, int fill_upper, int r4,
-                                                                           int r8, int wpg)
+                                                                           int r8, int wpg, int tri_in, int tri_out)
 {
     constexpr int NW = M16_NW, TPW = M16_TPW, HG = M16_HG;
     __shared__ __align__(16) u32x4_t stage[NW * TPW * 4 * 64];  // [wavefront][tile][head of the lane's four][lane]
@@ -258,6 +258,9 @@ __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(cons
     const int64_t n = ng / groups;
     const unsigned plane = (unsigned)P * (unsigned)Q;  // (16 planes of 16-bit values within 4 GB: checked by the launch)
     const int64_t base0 = (n * C + (int64_t)g * HG) * (int64_t)plane;  // head 16g, row 0, key 0
+    // (tri_in / tri_out: that tensor is in the triangular layout - causal, square, groups of 16 heads interleaved by rows,
+    // nothing above the diagonal: row p of the group starts 16*tri_rowoff(p) elements into the group, head i a row length on)
+    const int64_t tbase0 = (n * groups + g) * (HG * tri_rowoff(P));
     // the steps of a (batch, group), longest rows first, and the k-th of this workgroup: its workgroups take the steps in
     // turn, back and forth, so that each gets short and long rows alike
     const int n16 = P - r8, n8 = (r8 - r4 + 1) >> 1, nsteps = n16 + n8 + ((r4 + 3) >> 2);
@@ -287,17 +290,19 @@ __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(cons
     auto issue = [&](int p, int lg, int ln, int kg) {
         const int wr = wave & ((1 << lg) - 1);
         const int last = causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;
-        const char *xrow = reinterpret_cast<const char *>(x + base0 + (int64_t)p * Q);  // (uniform base + 32-bit lane offset)
+        // (uniform base + 32-bit lane offset)
+        const char *xrow = reinterpret_cast<const char *>(tri_in ? x + tbase0 + HG * tri_rowoff(p) : x + base0 + (int64_t)p * Q);
+        const unsigned xplane = tri_in ? (unsigned)tri_rowlen(p) : plane;
 #pragma unroll
         for (int i = 0; i < TPW; ++i) {
             const int q0 = ((i << lg) + wr) * M16_TK;
             if (q0 > last) continue;  // (wavefront-uniform)
             const int key = q0 + ln * 8;
             // beyond the attended keys a lane re-reads the row start; its values are masked
-            const unsigned off = ((unsigned)(kg * 4) * plane + (unsigned)(key <= last ? key : 0)) * (unsigned)sizeof(T);
+            const unsigned off = ((unsigned)(kg * 4) * xplane + (unsigned)(key <= last ? key : 0)) * (unsigned)sizeof(T);
 #pragma unroll
             for (int t = 0; t < 4; ++t)
-                __builtin_amdgcn_global_load_lds((glb_void_t *)(xrow + (off + (unsigned)t * plane * (unsigned)sizeof(T))),
+                __builtin_amdgcn_global_load_lds((glb_void_t *)(xrow + (off + (unsigned)t * xplane * (unsigned)sizeof(T))),
                                                  (lds_void_t *)(stage + ((wave * TPW + i) * 4 + t) * 64), 16, 0, 0);
         }
     };
@@ -318,7 +323,8 @@ __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(cons
         const int lane_o = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, (unsigned)opaque(0)));  // (the lane number)
         const int ln = lane_o & 15, kg = lane_o >> 4;
         const unsigned stage_lds = stage_wave + (unsigned)lane_o * 16u;
-        char *const yrow = reinterpret_cast<char *>(y + base0 + (int64_t)p * Q);
+        char *const yrow = reinterpret_cast<char *>(tri_out ? y + tbase0 + HG * tri_rowoff(p > 0 ? p : 0) : y + base0 + (int64_t)p * Q);
+        const unsigned yplane = tri_out ? (unsigned)tri_rowlen(p > 0 ? p : 0) : plane;
         const int last = !active ? -1 : causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;
         if (nst == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
         else if (nst == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
@@ -449,7 +455,7 @@ __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(cons
                     const u32x4_t z = {0u, 0u, 0u, 0u};
 #pragma unroll
                     for (int v = 0; v < 4; ++v)
-                        __builtin_nontemporal_store(z, reinterpret_cast<u32x4_t *>(yrow + ((unsigned)(kg * 4 + v) * plane + (unsigned)key) * (unsigned)sizeof(T)));
+                        __builtin_nontemporal_store(z, reinterpret_cast<u32x4_t *>(yrow + ((unsigned)(kg * 4 + v) * yplane + (unsigned)key) * (unsigned)sizeof(T)));
                 }
                 continue;
             }
@@ -479,7 +485,7 @@ __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(cons
             if (key < Q && (fill_upper || key <= last)) {
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
-                    __builtin_nontemporal_store(out[v], reinterpret_cast<u32x4_t *>(yrow + ((unsigned)(kg * 4 + v) * plane + (unsigned)key) * (unsigned)sizeof(T)));
+                    __builtin_nontemporal_store(out[v], reinterpret_cast<u32x4_t *>(yrow + ((unsigned)(kg * 4 + v) * yplane + (unsigned)key) * (unsigned)sizeof(T)));
             }
         }
         // keys beyond the tiles of this instance lie wholly above the diagonal: +0 on request (plain vector stores; the
@@ -489,7 +495,7 @@ __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(cons
             for (int key = (TPW * nwr + wr) * M16_TK + ln * 8; key < Q; key += nwr * M16_TK) {
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
-                    __builtin_nontemporal_store(z, reinterpret_cast<u32x4_t *>(yrow + ((unsigned)(kg * 4 + v) * plane + (unsigned)key) * (unsigned)sizeof(T)));
+                    __builtin_nontemporal_store(z, reinterpret_cast<u32x4_t *>(yrow + ((unsigned)(kg * 4 + v) * yplane + (unsigned)key) * (unsigned)sizeof(T)));
             }
         }
         p = pn;
@@ -505,7 +511,7 @@ namespace mta {
 // Launches the kernel when it applies (16-bit I/O, weights of the same dtype, groups of 16 heads, Q % 8 == 0,
 // Q <= 4096, 16-byte aligned tensors, 8-byte aligned weights); returns MTA_ERR_UNSUPPORTED otherwise.
 int mix16_softmax_launch(const void *x, const void *w1, const void *w2, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
-                         int causal, int fill_upper, int io_dtype, int w_dtype, hipStream_t st)
+                         int causal, int fill_upper, int io_dtype, int w_dtype, hipStream_t st, int tri_in, int tri_out)
 {
     if (io_dtype == MTA_F32 || w_dtype != io_dtype || (!w1 && !w2) || C % M16_HG != 0 || Q % 8 != 0 ||
         Q > (int64_t)M16_NW * M16_TPW * M16_TK)
@@ -527,6 +533,7 @@ int mix16_softmax_launch(const void *x, const void *w1, const void *w2, void *y,
     // one launch of row lists, about one workgroup per CU; or a launch per kind of row, a workgroup per row
 #define MTA_M16_ALL(T, h1, h2)                                                                                          \
     if (no_rows || !small_planes) {                                                                                     \
+        if (tri_in || tri_out) return MTA_ERR_UNSUPPORTED;                                                              \
         MTA_M16_LAUNCH(T, h1, h2, 4, 0, r4);                                                                            \
         MTA_M16_LAUNCH(T, h1, h2, 8, r4, r8 - r4);                                                                      \
         MTA_M16_LAUNCH(T, h1, h2, 16, r8, P - r8);                                                                      \
@@ -536,7 +543,7 @@ int mix16_softmax_launch(const void *x, const void *w1, const void *w2, void *y,
         wpg = wpg < 1 ? 1 : (wpg > steps ? steps : wpg);                                                                \
         hipLaunchKernelGGL((mix16_softmax_rows_kernel<T, h1, h2>), dim3((unsigned)(N * (C / M16_HG) * wpg)),            \
                            dim3(64 * M16_NW), 0, st, (const T *)x, (const T *)w1, (const T *)w2, (T *)y, (int)C, (int)P, \
-                           (int)Q, causal, fill_upper, (int)r4, (int)r8, (int)wpg);                                     \
+                           (int)Q, causal, fill_upper, (int)r4, (int)r8, (int)wpg, tri_in, tri_out);                    \
     }
 #define MTA_M16_CASES(T)                                          \
     if (w1 && w2) { MTA_M16_ALL(T, true, true) }                  \

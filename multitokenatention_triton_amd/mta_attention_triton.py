@@ -338,7 +338,7 @@ class MTAAttentionTriton(nn.Module):
         # travel in the triangular layout (what lies on and below the diagonal only, the rows a workgroup of the softmax
         # stage reads side by side): half the footprint, and every stage streams memory in longer runs.
         if (self.score_layout != "planes" and self.causal and one_pass and key_bias is None and own_pv
-                and not (self.training and self.dropout > 0) and g_both in (2, 4, 8)
+                and not (self.training and self.dropout > 0) and g_both in (2, 4, 8, 16)
                 and ops.tri_route_supported(xq, xk, self.mta_conv_triton.weight, g_both, w1, w2, first_visible is not None)):
             self._mark("qk_conv")
             scores = ops.qk_conv_tri(xq, xk, self.mta_conv_triton.weight, scale, g_both, first_visible=first_visible)
@@ -352,7 +352,15 @@ class MTAAttentionTriton(nn.Module):
 
         # QK^T -> *1/sqrt(d) -> conv: one kernel when it exists for this dtype / size, else GEMM + conv
         scores = None
-        if ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight):
+        # (dense groups of 16 heads ahead of a post-softmax conv: the first score tensor still travels in the triangular
+        # layout, the softmax stage hands the conv (B,H,S,S) planes)
+        tri_first = (self.score_layout != "planes" and self.causal and not one_pass and row_plain and g_pre == 16
+                     and w1 is not None and not (post_conv_identity and w2 is None and not own_pv)
+                     and ops.tri_route_supported(xq, xk, self.mta_conv_triton.weight, 16, w1, None, False, out_planes=True))
+        if tri_first:
+            self._mark("qk_conv")
+            scores = ops.qk_conv_tri(xq, xk, self.mta_conv_triton.weight, scale, 16)
+        elif ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight):
             self._mark("qk_conv")
             scores = ops.qk_conv(xq, xk, self.mta_conv_triton.weight, self.causal, scale, fill_upper=False,
                                  first_visible=first_visible)
@@ -368,7 +376,10 @@ class MTAAttentionTriton(nn.Module):
             scores = ops.headmix_softmax(scores, w1, w2, self.causal, group_size=g_both,
                                          fill_upper=not own_pv, key_bias=key_bias, first_visible=first_visible)
         else:
-            if _one_pass_group(g_pre, xq.dtype, n_keys, w1) and (row_plain or g_pre <= _FUSED_MAX_GROUP):
+            if tri_first:
+                self._mark("mix_softmax")
+                scores = ops.headmix_softmax_tri(scores, w1, None, xq.size(0), self.n_heads, n_keys, g_pre, out_planes=True)
+            elif _one_pass_group(g_pre, xq.dtype, n_keys, w1) and (row_plain or g_pre <= _FUSED_MAX_GROUP):
                 self._mark("mix_softmax")
                 scores = ops.headmix_softmax(scores, w1, None, self.causal, group_size=g_pre, key_bias=key_bias,
                                              first_visible=first_visible,

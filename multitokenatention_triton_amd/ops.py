@@ -407,8 +407,10 @@ def _band_arg(first_visible, b, s):
     return first_visible
 
 
-def tri_route_supported(q: torch.Tensor, k: torch.Tensor, conv_weight: torch.Tensor, group: int, w1, w2, band: bool) -> bool:
-    """Whether the three triangular-layout kernels exist for these tensors (host-side questions to the library)."""
+def tri_route_supported(q: torch.Tensor, k: torch.Tensor, conv_weight: torch.Tensor, group: int, w1, w2, band: bool,
+                        out_planes: bool = False) -> bool:
+    """Whether the triangular-layout kernels exist for these tensors (host-side questions to the library);
+    ``out_planes``: the softmax stage hands on (B,H,S,S) planes (then only the first two kernels are asked for)."""
     if not qk_conv_supported(q, k, conv_weight) or q.dtype not in (torch.bfloat16, torch.float16):
         return False
     b, h, s, d = q.shape
@@ -417,8 +419,9 @@ def tri_route_supported(q: torch.Tensor, k: torch.Tensor, conv_weight: torch.Ten
         return False
     if group * tri_row_offset(s) >= 2 ** 31 or not causal_pv_supported(q.dtype, s, d):
         return False
-    return bool(_lib.load().mta_headmix_softmax_tri_supported(h, s, group, _DTYPE_CODE[q.dtype], _DTYPE_CODE[ws[0].dtype],
-                                                              int(w1 is not None), int(w2 is not None), int(band)))
+    return bool(_lib.load().mta_headmix_softmax_tri_supported(h, s, group, int(out_planes), _DTYPE_CODE[q.dtype],
+                                                              _DTYPE_CODE[ws[0].dtype], int(w1 is not None),
+                                                              int(w2 is not None), int(band)))
 
 
 def qk_conv_tri(q: torch.Tensor, k: torch.Tensor, weight: torch.Tensor, scale: float, group: int,
@@ -444,9 +447,10 @@ def qk_conv_tri(q: torch.Tensor, k: torch.Tensor, weight: torch.Tensor, scale: f
 
 
 def headmix_softmax_tri(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optional[torch.Tensor], n: int, c: int, s: int,
-                        group: int, first_visible: Optional[torch.Tensor] = None) -> torch.Tensor:
+                        group: int, first_visible: Optional[torch.Tensor] = None, out_planes: bool = False) -> torch.Tensor:
     """mix(w1) -> causal row softmax -> mix(w2) over a flat tensor in the triangular layout (mixing groups = the layout's
-    groups); see mta_headmix_softmax_tri_fwd."""
+    groups); the result in the same layout or, with ``out_planes``, as an (N,C,S,S) tensor with nothing written above the
+    diagonal; see mta_headmix_softmax_tri_fwd."""
     x = _device_tensor(x, "input")
     if x.dim() != 1 or x.numel() != n * c * tri_row_offset(s):
         raise ValueError(f"expected a flat tensor of {n * c * tri_row_offset(s)} elements, got {tuple(x.shape)}")
@@ -460,12 +464,12 @@ def headmix_softmax_tri(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optiona
     if not present or any(w.dtype != present[0].dtype for w in present):
         raise TypeError("one or two weights of one dtype")
     first_visible = _band_arg(first_visible, n, s)
-    y = torch.empty_like(x)
+    y = torch.empty((n, c, s, s), dtype=x.dtype, device=x.device) if out_planes else torch.empty_like(x)
     with torch.cuda.device(x.device):
         rc = _lib.load().mta_headmix_softmax_tri_fwd(
             x.data_ptr(), ws[0].data_ptr() if ws[0] is not None else None, ws[1].data_ptr() if ws[1] is not None else None,
             first_visible.data_ptr() if first_visible is not None else None, y.data_ptr(), n, c, s, int(group),
-            _code(x, "input"), _code(present[0], "weight"), _stream(x))
+            int(bool(out_planes)), _code(x, "input"), _code(present[0], "weight"), _stream(x))
     _lib.check(rc, "mta_headmix_softmax_tri_fwd")
     return y
 

@@ -441,6 +441,8 @@ TRI_CASES = [
     (1, 8, 264, 128, 7, 7, 8, torch.bfloat16, None, "second"), (1, 8, 2304, 64, 6, 11, 4, torch.bfloat16, None, "both"),
     (2, 4, 776, 128, 6, 11, 4, torch.bfloat16, "documents", "first"), (1, 4, 2048, 64, 5, 5, 2, torch.float16, "window", "second"),
     (1, 8, 520, 64, 11, 15, 8, torch.bfloat16, "ragged", "first"), (1, 4, 4096, 128, 6, 11, 4, torch.bfloat16, None, "both"),
+    # groups of 16 heads (the matrix-core softmax kernel's row lists): rows of all three kinds, two groups
+    (1, 16, 2304, 64, 7, 7, 16, torch.float16, None, "first"), (2, 32, 1160, 64, 3, 3, 16, torch.bfloat16, None, "both"),
 ]
 
 
@@ -479,10 +481,36 @@ def test_triangular_layout_stages_equal_the_plane_layout(pkg, case):
     assert torch.equal(ops.headmix_softmax_tri(poisoned, w1, w2, b, h, s, group, first_visible=first)[ops.tri_pack(lower.to(dtype), group, 0.0) > 0],
                        p_tri[ops.tri_pack(lower.to(dtype), group, 0.0) > 0])
 
+    if group == 16:   # the same stage from the triangular layout into planes (what a post-softmax conv takes)
+        mixed = ops.headmix_softmax_tri(s_tri, w1, w2, b, h, s, group, out_planes=True)
+        assert torch.equal(mixed[lower], p_plane[lower])
+
     o_plane = ops.causal_pv(p_plane, v, True, first_visible=first)
     assert torch.equal(ops.causal_pv_tri(p_tri, v, group, first_visible=first), o_plane)
     assert torch.equal(ops.causal_pv_tri(ops.tri_pack(p_plane.masked_fill(~lower, float("nan")), group), v, group,
                                          first_visible=first), o_plane)
+
+
+def test_mta_score_layouts_agree_general_route(pkg):
+    """Dense 16-head weights and a post-softmax conv: the first score tensor in the triangular layout (the default) or in
+    planes, the same stages and the same output bit for bit."""
+    print("mta score layouts, general route", flush=True)
+    dtype = torch.float16
+    b, h, s, d = 1, 16, 1160, 128
+    q, k, v = (t.cuda() for t in O.seeded_qkv(b, h, s, d, dtype, seed=73))
+    g = torch.Generator().manual_seed(74)
+    dense = lambda: (torch.eye(h) + 0.05 * torch.randn(h, h, generator=g)).to(dtype)
+    conv = lambda: (torch.randn(h, 7, 7, generator=g) * 0.05).to(dtype)
+    mod = _mta_module(pkg, h, 7, 7, 7, 7, conv(), dense(), conv(), dense(), dtype, structure="dense")
+    outs, stages = {}, {}
+    for layout in ("auto", "planes"):
+        mod.score_layout = layout
+        seen = []
+        mod._stage_hook = seen.append
+        outs[layout] = mod(q, k, v, None, None)
+        stages[layout] = seen
+    assert stages["auto"] == stages["planes"] == ["qk_conv", "mix_softmax", "conv_mix_post", "pv", "end"]
+    assert torch.equal(outs["auto"], outs["planes"])
 
 
 @pytest.mark.parametrize("masked", [False, True])

@@ -31,7 +31,7 @@ GROUPS = [
     # mix -> softmax -> mix for groups of 16 heads with a workgroup per row (by default workgroups take lists of rows)
     # the inference route with its score tensors as (B,H,S,S) planes (by default: the triangular layout)
     ({"MTA_SCORE_LAYOUT": "planes"}, ["tests/test_gpu_attention.py"],
-     "test_mta_headline or test_mta_use_mask or test_mta_fused_route or test_mta_module"),
+     "test_mta_headline or test_mta_use_mask or test_mta_general"),
     ({"MTA_MIX16_NO_ROW_LISTS": "1"}, ["tests/test_gpu_ops.py"], "(test_mix_softmax_mix_parity and not f32) or test_mix_softmax_mix_dense16"),
 ]
 
