@@ -68,8 +68,9 @@ def stage_model(name, b, h, s, d, r=6, sk=11, esize=2):
 
 
 # Which kernel runs a stage of the headline forward, as rocprofv3 names it in profiles/mta_forward_c4_hbm_traffic.txt
-STAGE_KERNEL = {"qk_conv": "conv_attn_fwd_mfma<bf16_t, 128, 6, 11, true, 4>", "mix_softmax_mix": "mix_softmax_mix_packed<",
-                "pv": "causal_pv_kernel<"}
+STAGE_KERNEL = {"qk_conv": "conv_attn_fwd_mfma<bf16_t, 128, 6, 11, true, 4, false>",
+                "mix_softmax_mix": "mix_softmax_mix_packed<bf16_t, 4, 1, false, true, 512, 8, false>",
+                "pv": "causal_pv_kernel<bf16_t, 128, 1>"}
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "mta_forward_c4_hbm_traffic.txt")
 
 
