@@ -443,6 +443,9 @@ TRI_CASES = [
     (1, 8, 520, 64, 11, 15, 8, torch.bfloat16, "ragged", "first"), (1, 4, 4096, 128, 6, 11, 4, torch.bfloat16, None, "both"),
     # groups of 16 heads (the matrix-core softmax kernel's row lists): rows of all three kinds, two groups
     (1, 16, 2304, 64, 7, 7, 16, torch.float16, None, "first"), (2, 32, 1160, 64, 3, 3, 16, torch.bfloat16, None, "both"),
+    # a sequence shorter than one padded row; the longest rows the 8-head kernel takes; a band with groups of 8
+    (1, 2, 8, 128, 3, 3, 2, torch.bfloat16, None, "both"), (1, 8, 2048, 128, 5, 7, 8, torch.float16, None, "both"),
+    (1, 16, 72, 64, 3, 3, 16, torch.bfloat16, None, "second"), (2, 8, 1032, 64, 7, 7, 8, torch.bfloat16, "window", "second"),
 ]
 
 
