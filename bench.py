@@ -329,7 +329,19 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
     out["mta_forward_bf16_2x16x4096x128_window1024_mask"] = {
         "ms": ms, "stages": stages,
         "note": "the headline configuration with use_mask=True and a sliding-window mask tensor; not a row of the reference's"}
-    del mod, sets, window
+    # ... and under a key-padding mask of the batch (the second sequence is 3000 tokens long), given as a (B,1,S,S) boolean
+    # mask tensor: it travels to the kernels as one fp32 value per (batch entry, key)
+    lengths = torch.tensor([s_len, 3000], device=device)
+    padded = ((pos[None, :] < lengths[:, None])[:, None, None, :] & (pos[None, :] <= pos[:, None])[None, None])
+    ms = time_steps(torch, lambda i: mod(*sets[i], padded, None), len(sets), min(warmup, 30), max(3, steps // 2))
+    stages = []
+    mod._stage_hook = stages.append
+    mod(*sets[0], padded, None)
+    mod._stage_hook = None
+    out["mta_forward_bf16_2x16x4096x128_key_padding_mask"] = {
+        "ms": ms, "stages": stages,
+        "note": "the headline configuration with use_mask=True and a key-padding mask tensor (lengths 4096 and 3000); not a row of the reference's"}
+    del mod, sets, window, padded
     # the first module and shape in training: forward operator by operator (each with its HIP backward kernels; the two
     # matrix products, the softmax and the dropout are torch's) and backward to q, k, v and the four weights
     mod, sets = build_general(torch, mta, O, device, train=True)

@@ -238,7 +238,8 @@ int mta_causal_pv_band_fwd(const void *p, const void *v, const void *first_visib
  * counterpart in the reference, whose kernels exchange full (B,H,S,S) tensors.  16-bit I/O only.
  *   mta_qk_conv_tri_fwd:         mta_qk_conv_fwd (causal) / mta_qk_conv_band_fwd (first_visible not NULL), output layout;
  *                                group*T must stay below 2^31.
- *   mta_headmix_softmax_tri_fwd: mta_headmix_softmax_fwd (causal, fill_upper = 0) / mta_headmix_softmax_band_fwd, layout of
+ *   mta_headmix_softmax_tri_fwd: mta_headmix_softmax_fwd (causal, fill_upper = 0) / mta_headmix_softmax_bias_fwd (key_bias
+ *                                not NULL; fp32 (N,S), 16-byte aligned) / mta_headmix_softmax_band_fwd, layout of
  *                                the input and, with out_planes = 0, of the output; the layout's group = group_size
  *                                (2, 4, 8; 16 without a band mask); out_planes = 1 (groups of 16 only): the output as
  *                                (N,C,S,S) planes, nothing written above the diagonal; weights of the I/O dtype.
@@ -246,14 +247,15 @@ int mta_causal_pv_band_fwd(const void *p, const void *v, const void *first_visib
 int mta_qk_conv_tri_fwd(const void *q, const void *k, const void *w, const void *first_visible, void *s_out, int64_t B,
                         int64_t H, int64_t S, int64_t D, int R, int Sk, float scale, int group, int io_dtype, int w_dtype,
                         void *stream);
-int mta_headmix_softmax_tri_fwd(const void *x, const void *w1, const void *w2, const void *first_visible, void *y, int64_t N,
-                                int64_t C, int64_t S, int group_size, int out_planes, int io_dtype, int w_dtype, void *stream);
+int mta_headmix_softmax_tri_fwd(const void *x, const void *w1, const void *w2, const void *key_bias, const void *first_visible,
+                                void *y, int64_t N, int64_t C, int64_t S, int group_size, int out_planes, int io_dtype,
+                                int w_dtype, void *stream);
 int mta_causal_pv_tri_fwd(const void *p, const void *v, const void *first_visible, void *o, int64_t B, int64_t H, int64_t S,
                           int64_t D, int group, int io_dtype, void *stream);
 /* 1 when mta_headmix_softmax_tri_fwd has a kernel for these sizes and dtypes (has_w1 / has_w2: which weights are given;
- * band: with first_visible), else 0.  A host-side question: nothing is launched. */
+ * band: with first_visible; key_bias: with a key bias), else 0.  A host-side question: nothing is launched. */
 int mta_headmix_softmax_tri_supported(int64_t C, int64_t S, int group_size, int out_planes, int io_dtype, int w_dtype,
-                                      int has_w1, int has_w2, int band);
+                                      int has_w1, int has_w2, int band, int key_bias);
 
 /* The transposed product, O[k,:] = sum_p P[p,k] X[p,:] with P (B,H,S,S), X and O (B,H,S,D); when causal only query rows
  * p >= k take part and nothing of P above the diagonal is read.  These are the gradients the two matrix products of the

@@ -502,10 +502,12 @@ template <bool IS_MAX, int G, int NW> __device__ __forceinline__ void heads_comb
 
 // BAND (one pass per wavefront only): row_lo[n, p] is the first key row p sees; a wavefront whose slice lies wholly ahead
 // of it stores +0 and ends, like those above the diagonal, and the slice that holds it masks the keys ahead of it.
-template <typename T, int G, int NV, bool HAS1, bool HAS2, int NT, int OCC, bool BAND = false>
+// KBIAS: key_bias[n, q] (fp32, a value of the I/O dtype) is added to the mixed, rounded scores and the sum rounded again:
+// the reference's `scores + mask` for a mask that is one value per (batch entry, key).
+template <typename T, int G, int NV, bool HAS1, bool HAS2, int NT, int OCC, bool BAND = false, bool KBIAS = false>
 __global__ __launch_bounds__(NT, OCC) void mix_softmax_mix_packed(
     const T *__restrict__ x, const T *__restrict__ w1, const T *__restrict__ w2, T *__restrict__ y, int C, int P, int Q,
-    int causal, int fill_upper, const int *__restrict__ row_lo, int tri)
+    int causal, int fill_upper, const int *__restrict__ row_lo, int tri, const float *__restrict__ key_bias)
 {
     constexpr int VEC = 8, NW = NT / 64, H2 = G / 2;
     static_assert(sizeof(T) == 2 && G % 2 == 0, "packed pairs of a 16-bit type");
@@ -599,6 +601,15 @@ __global__ __launch_bounds__(NT, OCC) void mix_softmax_mix_packed(
 #pragma unroll
             for (int k = 0; k < L; ++k) {
                 const int q = (k * NT + tid) * VEC;
+                float kbv[KBIAS ? VEC : 1];
+                if constexpr (KBIAS) {
+                    typedef float rs_f4 __attribute__((ext_vector_type(4)));
+                    const int qs = (!EDGE || k < L - 1 || q <= last) ? q : 0;  // (as for x: beyond the attended keys, the row start)
+                    const rs_f4 b0 = *reinterpret_cast<const rs_f4 *>(key_bias + n * Q + qs);
+                    const rs_f4 b1 = *reinterpret_cast<const rs_f4 *>(key_bias + n * Q + qs + 4);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) { kbv[u] = b0[u]; kbv[4 + u] = b1[u]; }
+                }
 #pragma unroll
                 for (int d = 0; d < VEC / 2; ++d) {
                     float a[G][2];
@@ -623,6 +634,14 @@ __global__ __launch_bounds__(NT, OCC) void mix_softmax_mix_packed(
 #pragma unroll
                         for (int o = 0; o < G; ++o) unpack2<T>(xin[k][o][d], a[o][0], a[o][1]);
                     }
+                    if constexpr (KBIAS) {
+#pragma unroll
+                        for (int o = 0; o < G; ++o) {
+                            if constexpr (HAS1) round_pair<T>(a[o][0], a[o][1]);  // (the mixed scores as the unfused chain stores them)
+                            a[o][0] += kbv[2 * d];
+                            a[o][1] += kbv[2 * d + 1];
+                        }
+                    }
                     if (EDGE && k == L - 1) {
 #pragma unroll
                         for (int o = 0; o < G; ++o) {
@@ -639,8 +658,8 @@ __global__ __launch_bounds__(NT, OCC) void mix_softmax_mix_packed(
                     }
 #pragma unroll
                     for (int o = 0; o < G; ++o) {
-                        m[o] = HAS1 ? max3_after_dot(m[o], a[o][0], a[o][1]) : max3(m[o], a[o][0], a[o][1]);
-                        sp[o][k][d] = (HAS1 || BAND || (EDGE && k == L - 1)) ? pack2<T>(a[o][0], a[o][1]) : xin[k][o][d];
+                        m[o] = (HAS1 && !KBIAS) ? max3_after_dot(m[o], a[o][0], a[o][1]) : max3(m[o], a[o][0], a[o][1]);
+                        sp[o][k][d] = (HAS1 || BAND || KBIAS || (EDGE && k == L - 1)) ? pack2<T>(a[o][0], a[o][1]) : xin[k][o][d];
                     }
                 }
             }
@@ -648,7 +667,7 @@ __global__ __launch_bounds__(NT, OCC) void mix_softmax_mix_packed(
         heads_reduce_store<true, G, NW>(m, red[0], wave, lane);
         __syncthreads();
         heads_combine<true, G, NW>(red[0], nlw, lane, m, flw);
-        if constexpr (HAS1) {
+        if constexpr (HAS1 || KBIAS) {
             // the maximum of the rounded scores is the rounded maximum (the row's first key is always attended: finite)
 #pragma unroll
             for (int o = 0; o < G; o += 2) round_pair<T>(m[o], m[o + 1]);
@@ -860,6 +879,28 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb_in, 
         if (tri_in != tri_out) return MTA_ERR_UNSUPPORTED;
         const bool packed_ok = vec_ok && !no_packed && w_dtype == io_code && (w1 || w2) && (!w1 || aligned_to(w1, 4)) &&
                                (!w2 || aligned_to(w2, 4)) && C % 2 == 0 && Q <= 256 * VEC * 4;
+        // key bias without a band mask: the packed kernel's KBIAS instances, one per group size (the one for the longest
+        // rows; with 4 heads and one weight the 512-thread shape)
+        if (packed_ok && kb && !row_lo && aligned_to(kb, 16)) {
+#define MTA_RSK_LAUNCH(g, v, h1, h2, nt, occ)                                                                          \
+    {                                                                                                                  \
+        hipLaunchKernelGGL((mix_softmax_mix_packed<T, g, v, h1, h2, nt, occ, false, true>),                            \
+                           dim3((unsigned)(N * (C / g) * P)), dim3(nt), 0, st, (const T *)x, (const T *)w1,            \
+                           (const T *)w2, (T *)y, (int)C, (int)P, (int)Q, causal, fill_upper, nullptr, tri, kb);      \
+        return launch_status();                                                                                        \
+    }
+#define MTA_RSK_CASE(g, v, nt, occ)                                                                                    \
+    if (G == g && Q <= (int64_t)(nt) * VEC * (v)) {                                                                    \
+        if (w1 && w2) MTA_RSK_LAUNCH(g, v, true, true, nt, occ)                                                        \
+        if (w1) MTA_RSK_LAUNCH(g, v, true, false, nt, occ)                                                             \
+        MTA_RSK_LAUNCH(g, v, false, true, nt, occ)                                                                     \
+    }
+            MTA_RSK_CASE(2, 4, 256, RS_OCC)
+            if (!(w1 && w2)) MTA_RSK_CASE(4, 1, 512, 8)
+            MTA_RSK_CASE(4, 2, 256, RS_OCC) MTA_RSK_CASE(8, 1, 256, 4)  // (8 heads: a register budget without spills)
+#undef MTA_RSK_CASE
+#undef MTA_RSK_LAUNCH
+        }
         // band mask without a key bias, one weight, rows that one pass per wavefront covers: the packed kernel's BAND
         // instances (causal by construction)
         if (packed_ok && row_lo && !kb && causal && !(w1 && w2)) {
@@ -867,7 +908,7 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb_in, 
     {                                                                                                                  \
         hipLaunchKernelGGL((mix_softmax_mix_packed<T, g, 1, h1, h2, nt, occ, true>), dim3((unsigned)(N * (C / g) * P)), \
                            dim3(nt), 0, st, (const T *)x, (const T *)w1, (const T *)w2, (T *)y, (int)C, (int)P,        \
-                           (int)Q, causal, fill_upper, row_lo, tri);                                                   \
+                           (int)Q, causal, fill_upper, row_lo, tri, nullptr);                                          \
         return launch_status();                                                                                        \
     }
 #define MTA_RSB_CASE(g, nt, occ)                                                                                       \
@@ -884,7 +925,7 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb_in, 
     {                                                                                                                  \
         hipLaunchKernelGGL((mix_softmax_mix_packed<T, g, v, h1, h2, nt, occ>), dim3((unsigned)(N * (C / g) * P)),      \
                            dim3(nt), 0, st, (const T *)x, (const T *)w1, (const T *)w2, (T *)y, (int)C, (int)P,        \
-                           (int)Q, causal, fill_upper, nullptr, tri);                                                  \
+                           (int)Q, causal, fill_upper, nullptr, tri, nullptr);                                         \
         return launch_status();                                                                                        \
     }
 #define MTA_RSP_CASE(g, v, nt, occ)                                                                                    \
@@ -945,12 +986,12 @@ extern "C" int mta_headmix_softmax_band_fwd(const void *x, const void *w1, const
 // `group_size` heads interleaved by rows; nothing above the diagonal exists.  out_planes = 0: the output in the same
 // layout (groups of 2, 4, 8 or 16 heads); 1: the output as (N,C,S,S) planes with nothing written above the diagonal
 // (groups of 16).  16-bit data with weights of the same dtype only (MTA_ERR_UNSUPPORTED otherwise).
-extern "C" int mta_headmix_softmax_tri_fwd(const void *x, const void *w1, const void *w2, const void *first_visible, void *y,
-                                           int64_t N, int64_t C, int64_t S, int group_size, int out_planes, int io_dtype,
-                                           int w_dtype, void *stream)
+extern "C" int mta_headmix_softmax_tri_fwd(const void *x, const void *w1, const void *w2, const void *key_bias,
+                                           const void *first_visible, void *y, int64_t N, int64_t C, int64_t S,
+                                           int group_size, int out_planes, int io_dtype, int w_dtype, void *stream)
 {
     if (!x || !y) return MTA_ERR_NULL;
-    if (first_visible && !aligned_to(first_visible, 4)) return MTA_ERR_ALIGN;
+    if ((first_visible && !aligned_to(first_visible, 4)) || (key_bias && !aligned_to(key_bias, 4))) return MTA_ERR_ALIGN;
     if (!dtype_size(io_dtype) || !dtype_size(w_dtype)) return MTA_ERR_DTYPE;
     if (N <= 0 || C <= 0 || S <= 0 || S > (1 << 24) || C > 4096) return MTA_ERR_SHAPE;
     if (group_size <= 0 || C % group_size != 0) return MTA_ERR_GROUP;
@@ -959,14 +1000,14 @@ extern "C" int mta_headmix_softmax_tri_fwd(const void *x, const void *w1, const 
     if (io_dtype == MTA_F32 || (!w1 && !w2)) return MTA_ERR_UNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
     if (io_dtype == MTA_BF16)
-        return dispatch<bf16_t>(x, w1, w2, nullptr, (const int *)first_visible, y, N, C, S, S, group_size, 1, w_dtype, 0, st, 1, !out_planes);
-    return dispatch<f16_t>(x, w1, w2, nullptr, (const int *)first_visible, y, N, C, S, S, group_size, 1, w_dtype, 0, st, 1, !out_planes);
+        return dispatch<bf16_t>(x, w1, w2, (const float *)key_bias, (const int *)first_visible, y, N, C, S, S, group_size, 1, w_dtype, 0, st, 1, !out_planes);
+    return dispatch<f16_t>(x, w1, w2, (const float *)key_bias, (const int *)first_visible, y, N, C, S, S, group_size, 1, w_dtype, 0, st, 1, !out_planes);
 }
 
 // Whether mta_headmix_softmax_tri_fwd has a kernel for these sizes (the cases of `dispatch` that know the layout: the
 // packed kernel's instances, with a band mask those for one weight and one pass per wavefront).  Nothing is launched.
 extern "C" int mta_headmix_softmax_tri_supported(int64_t C, int64_t S, int group_size, int out_planes, int io_dtype,
-                                                 int w_dtype, int has_w1, int has_w2, int band)
+                                                 int w_dtype, int has_w1, int has_w2, int band, int key_bias)
 {
     if (io_dtype != MTA_BF16 && io_dtype != MTA_F16) return 0;
     if (w_dtype != io_dtype || (!has_w1 && !has_w2) || group_size <= 0 || C <= 0 || C % group_size != 0 || S <= 0 || S % 8 != 0)
@@ -975,9 +1016,9 @@ extern "C" int mta_headmix_softmax_tri_supported(int64_t C, int64_t S, int group
     if (e && e[0] == '1') return 0;
     if (group_size == 16) {  // the matrix-core kernel's row lists (rowsoftmax_dense16.hip)
         const char *e2 = getenv("MTA_MIX16_NO_ROW_LISTS");
-        return !band && S <= 4096 && S * S <= (1LL << 27) && !(e2 && e2[0] == '1');
+        return !band && !key_bias && S <= 4096 && S * S <= (1LL << 27) && !(e2 && e2[0] == '1');
     }
-    if (out_planes) return 0;
+    if (out_planes || (band && key_bias)) return 0;
     if (band && has_w1 && has_w2) return 0;
     const int g = group_size;
     const int64_t cap = band ? (g == 4 ? 4096 : (g == 2 || g == 8) ? 2048 : 0) : (g == 2 ? 8192 : g == 4 ? 4096 : g == 8 ? 2048 : 0);

@@ -337,14 +337,16 @@ class MTAAttentionTriton(nn.Module):
         # Three kernels with nothing elementwise between them: the two score tensors are nobody else's business, and they
         # travel in the triangular layout (what lies on and below the diagonal only, the rows a workgroup of the softmax
         # stage reads side by side): half the footprint, and every stage streams memory in longer runs.
-        if (self.score_layout != "planes" and self.causal and one_pass and key_bias is None and own_pv
+        if (self.score_layout != "planes" and self.causal and one_pass and own_pv
                 and not (self.training and self.dropout > 0) and g_both in (2, 4, 8, 16)
-                and ops.tri_route_supported(xq, xk, self.mta_conv_triton.weight, g_both, w1, w2, first_visible is not None)):
+                and (key_bias is None or (key_bias.is_contiguous() and key_bias.data_ptr() % 16 == 0))
+                and ops.tri_route_supported(xq, xk, self.mta_conv_triton.weight, g_both, w1, w2, first_visible is not None,
+                                            key_bias=key_bias is not None)):
             self._mark("qk_conv")
             scores = ops.qk_conv_tri(xq, xk, self.mta_conv_triton.weight, scale, g_both, first_visible=first_visible)
             self._mark("mix_softmax_mix")
             scores = ops.headmix_softmax_tri(scores, w1, w2, xq.size(0), self.n_heads, n_keys, g_both,
-                                             first_visible=first_visible)
+                                             first_visible=first_visible, key_bias=key_bias)
             self._mark("pv")
             output = ops.causal_pv_tri(scores, xv, g_both, first_visible=first_visible)
             self._mark("end")
@@ -528,9 +530,7 @@ class MTAAttentionTriton(nn.Module):
                     bias = torch.where(mask, 0.0, float("-inf")).to(torch.float32)
                 else:
                     bias = mask.type(xq.dtype).to(torch.float32)   # the reference adds it in the I/O dtype
-                hidden = (bias == float("-inf"))[:, None, :, None]
-                return self._forward_fused(xq, xk.masked_fill(hidden, 0), xv.masked_fill(hidden, 0),
-                                           key_bias=bias.contiguous())
+                return self._forward_hidden_keys(xq, xk, xv, bias.contiguous())
             # a 4-D mask, the same for all heads, of one of two forms goes into the kernels without a (B,H,S,S) tensor:
             # "causal rule + hidden keys" per batch entry (key padding: a key bias and zeroed K and V rows, as for the
             # 2-D mask above) and "row p sees the keys first[p] .. p" (sliding windows, packed documents: one int32 per
@@ -538,8 +538,7 @@ class MTAAttentionTriton(nn.Module):
             if mask.dim() == 4:
                 kind, what = self._structured_mask(mask, xq.size(0), xq.size(-2))
                 if kind == "keys":
-                    hidden = (what == float("-inf"))[:, None, :, None]
-                    return self._forward_fused(xq, xk.masked_fill(hidden, 0), xv.masked_fill(hidden, 0), key_bias=what)
+                    return self._forward_hidden_keys(xq, xk, xv, what)
                 if (kind == "band" and self._current_structure().post_conv_identity
                         and ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight)):
                     return self._forward_fused(xq, xk, xv, first_visible=what)
@@ -556,6 +555,16 @@ class MTAAttentionTriton(nn.Module):
         scores = self.wposm_triton(scores)
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         return torch.matmul(scores, xv).transpose(1, 2)
+
+    def _forward_hidden_keys(self, xq, xk, xv, bias):
+        """The fused route under "causal rule + one additive value per (batch entry, key)" (``bias``: fp32 (B,S)).  The K
+        rows of hidden keys (-inf) are zeroed: their scores then enter the pre-softmax conv as 0.  Their probabilities
+        are 0; a post-softmax conv that is not the identity writes into their columns all the same, which the reference
+        zeroes again - here those columns meet zeroed V rows instead."""
+        hidden = (bias == float("-inf"))[:, None, :, None]
+        if not self._current_structure().post_conv_identity:
+            xv = xv.masked_fill(hidden, 0)
+        return self._forward_fused(xq, xk.masked_fill(hidden, 0), xv, key_bias=bias)
 
     def _structured_mask(self, mask, bsz: int, s: int):
         """What a 4-D ``mask`` (bool with True = attend, or additive with 0 / -inf; one plane for all heads) amounts to

@@ -408,7 +408,7 @@ def _band_arg(first_visible, b, s):
 
 
 def tri_route_supported(q: torch.Tensor, k: torch.Tensor, conv_weight: torch.Tensor, group: int, w1, w2, band: bool,
-                        out_planes: bool = False) -> bool:
+                        out_planes: bool = False, key_bias: bool = False) -> bool:
     """Whether the triangular-layout kernels exist for these tensors (host-side questions to the library);
     ``out_planes``: the softmax stage hands on (B,H,S,S) planes (then only the first two kernels are asked for)."""
     if not qk_conv_supported(q, k, conv_weight) or q.dtype not in (torch.bfloat16, torch.float16):
@@ -421,7 +421,7 @@ def tri_route_supported(q: torch.Tensor, k: torch.Tensor, conv_weight: torch.Ten
         return False
     return bool(_lib.load().mta_headmix_softmax_tri_supported(h, s, group, int(out_planes), _DTYPE_CODE[q.dtype],
                                                               _DTYPE_CODE[ws[0].dtype], int(w1 is not None),
-                                                              int(w2 is not None), int(band)))
+                                                              int(w2 is not None), int(band), int(key_bias)))
 
 
 def qk_conv_tri(q: torch.Tensor, k: torch.Tensor, weight: torch.Tensor, scale: float, group: int,
@@ -447,7 +447,8 @@ def qk_conv_tri(q: torch.Tensor, k: torch.Tensor, weight: torch.Tensor, scale: f
 
 
 def headmix_softmax_tri(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optional[torch.Tensor], n: int, c: int, s: int,
-                        group: int, first_visible: Optional[torch.Tensor] = None, out_planes: bool = False) -> torch.Tensor:
+                        group: int, first_visible: Optional[torch.Tensor] = None, out_planes: bool = False,
+                        key_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """mix(w1) -> causal row softmax -> mix(w2) over a flat tensor in the triangular layout (mixing groups = the layout's
     groups); the result in the same layout or, with ``out_planes``, as an (N,C,S,S) tensor with nothing written above the
     diagonal; see mta_headmix_softmax_tri_fwd."""
@@ -464,10 +465,15 @@ def headmix_softmax_tri(x: torch.Tensor, w1: Optional[torch.Tensor], w2: Optiona
     if not present or any(w.dtype != present[0].dtype for w in present):
         raise TypeError("one or two weights of one dtype")
     first_visible = _band_arg(first_visible, n, s)
+    if key_bias is not None:
+        key_bias = _device_tensor(key_bias, "key_bias")
+        if key_bias.dtype != torch.float32 or tuple(key_bias.shape) != (n, s) or not key_bias.is_contiguous():
+            raise ValueError(f"key_bias must be a contiguous fp32 tensor of shape ({n},{s})")
     y = torch.empty((n, c, s, s), dtype=x.dtype, device=x.device) if out_planes else torch.empty_like(x)
     with torch.cuda.device(x.device):
         rc = _lib.load().mta_headmix_softmax_tri_fwd(
             x.data_ptr(), ws[0].data_ptr() if ws[0] is not None else None, ws[1].data_ptr() if ws[1] is not None else None,
+            key_bias.data_ptr() if key_bias is not None else None,
             first_visible.data_ptr() if first_visible is not None else None, y.data_ptr(), n, c, s, int(group),
             int(bool(out_planes)), _code(x, "input"), _code(present[0], "weight"), _stream(x))
     _lib.check(rc, "mta_headmix_softmax_tri_fwd")

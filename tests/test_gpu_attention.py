@@ -484,6 +484,15 @@ def test_triangular_layout_stages_equal_the_plane_layout(pkg, case):
     assert torch.equal(ops.headmix_softmax_tri(poisoned, w1, w2, b, h, s, group, first_visible=first)[ops.tri_pack(lower.to(dtype), group, 0.0) > 0],
                        p_tri[ops.tri_pack(lower.to(dtype), group, 0.0) > 0])
 
+    if kind is None and group != 16:   # with a key bias (key masks): a few keys hidden, a few finite values
+        kb = torch.zeros(b, s)
+        kb[:, 3::7] = float("-inf")
+        kb[:, 5::11] = -1.5
+        kb[:, 0] = 0
+        kb = kb.cuda()
+        biased = ops.headmix_softmax(s_plane, w1, w2, True, group_size=group, fill_upper=False, key_bias=kb)
+        assert torch.equal(ops.tri_unpack(ops.headmix_softmax_tri(s_tri, w1, w2, b, h, s, group, key_bias=kb), b, h, s, group)[lower],
+                           biased[lower])
     if group == 16:   # the same stage from the triangular layout into planes (what a post-softmax conv takes)
         mixed = ops.headmix_softmax_tri(s_tri, w1, w2, b, h, s, group, out_planes=True)
         assert torch.equal(mixed[lower], p_plane[lower])
@@ -516,20 +525,24 @@ def test_mta_score_layouts_agree_general_route(pkg):
     assert torch.equal(outs["auto"], outs["planes"])
 
 
-@pytest.mark.parametrize("masked", [False, True])
+@pytest.mark.parametrize("masked", [False, "band", "keys"])
 def test_mta_score_layouts_agree(pkg, masked):
     """The module's inference route with the score tensors in the triangular layout (the default where the three kernels
-    know it) and in planes: the same stages, the same output bit for bit."""
+    know it) and in planes: the same stages, the same output bit for bit - without a mask, under a sliding window and
+    under a key-padding mask of a batch."""
     print(f"mta score layouts masked={masked}", flush=True)
     dtype = torch.bfloat16
     b, h, s, d = 2, 8, 1160, 128
     q, k, v = (t.cuda() for t in O.seeded_qkv(b, h, s, d, dtype, seed=71))
     params = _config_like(h, 4, 6, 11, 0.05, dtype)
-    mod = _mta_module(pkg, h, 6, 11, 3, 3, *params, dtype, use_mask=masked, structure="infer")
+    mod = _mta_module(pkg, h, 6, 11, 3, 3, *params, dtype, use_mask=bool(masked), structure="infer")
     mask = None
-    if masked:
-        rows = torch.arange(s)
+    rows = torch.arange(s)
+    if masked == "band":
         mask = ((rows[None, :] <= rows[:, None]) & (rows[None, :] > rows[:, None] - 300))[None, None].cuda()
+    elif masked == "keys":
+        keep = rows[None, :] < torch.tensor([s, 700])[:, None]
+        mask = (keep[:, None, None, :] & (rows[None, :] <= rows[:, None])[None, None]).cuda()
     outs, stages = {}, {}
     for layout in ("auto", "planes"):
         mod.score_layout = layout
@@ -802,6 +815,38 @@ def test_mta_headline_full_size_all_groups(pkg):
         print(f"  slab {r0}:{r1}", flush=True)
         want = O.mta_forward_rows(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3], r0, r1)
         torch.testing.assert_close(got[:, r0:r1].float(), want.float(), **tol(dtype))
+
+
+def test_mta_headline_full_size_key_padding(pkg):
+    """BASELINE config 4 at full size under a key-padding mask of the batch (lengths 4096 and 3000, a (B,1,S,S) boolean
+    tensor; what bench.py times as its key-padding row).  Under the causal rule a row of a real token sees no padding
+    key, so those rows must come out as without a mask, bit for bit - both batch entries, every head; the padding rows
+    (whose own keys are hidden: they see the real tokens only) against the oracle on one mixing group."""
+    print("mta headline full size, key padding", flush=True)
+    dtype = torch.bfloat16
+    b, h, s, d, grp = 2, 16, 4096, 128, 4
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=300)
+    g = torch.Generator().manual_seed(127)
+    params = [O.seeded_conv_weight(h, 6, 11, 0.05, dtype), torch.eye(h, dtype=dtype),
+              O.identity_conv_kernel(h, 3, 3, dtype), O.block_diag_head_weight(h, grp, 0.1, g, dtype)]
+    mod = _mta_module(pkg, h, 6, 11, 3, 3, *params, dtype, use_mask=True)
+    plain = mod(q.cuda(), k.cuda(), v.cuda(), None, None)
+    rows = torch.arange(s)
+    lengths = torch.tensor([4096, 3000])
+    mask = ((rows[None, :] < lengths[:, None])[:, None, None, :] & (rows[None, :] <= rows[:, None])[None, None]).cuda()
+    stages = []
+    mod._stage_hook = stages.append
+    got = mod(q.cuda(), k.cuda(), v.cuda(), mask, None)
+    assert stages == ["qk_conv", "mix_softmax_mix", "pv", "end"]
+    assert torch.equal(got[0], plain[0]) and torch.equal(got[1, :3000], plain[1, :3000])
+    assert torch.isfinite(got.float()).all()
+    # the padding rows of batch entry 1, heads 4..7, against the oracle given the mask tensor (a slab of 64 rows)
+    bi, sl, r0, r1 = 1, slice(4, 8), 3500, 3564
+    sub = [params[0][sl], params[1][sl, sl], params[2][sl], params[3][sl, sl]]
+    additive = torch.where(mask[bi:bi + 1].cpu(), 0.0, float("-inf")).to(dtype).expand(1, grp, s, s).contiguous()
+    want = O.mta_forward(q[bi:bi + 1, sl], k[bi:bi + 1, sl], v[bi:bi + 1, sl], sub[0].unsqueeze(1), sub[1],
+                         sub[2].unsqueeze(1), sub[3], mask=additive)
+    torch.testing.assert_close(got[bi:bi + 1, r0:r1, sl].float().cpu(), want[:, r0:r1].float(), **tol(dtype))
 
 
 # ------------------------------------------------------------------------------------------------------
