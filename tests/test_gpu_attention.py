@@ -446,6 +446,8 @@ TRI_CASES = [
     # a sequence shorter than one padded row; the longest rows the 8-head kernel takes; a band with groups of 8
     (1, 2, 8, 128, 3, 3, 2, torch.bfloat16, None, "both"), (1, 8, 2048, 128, 5, 7, 8, torch.float16, None, "both"),
     (1, 16, 72, 64, 3, 3, 16, torch.bfloat16, None, "second"), (2, 8, 1032, 64, 7, 7, 8, torch.bfloat16, "window", "second"),
+    # the longest rows any of the kernels takes (pairs of heads, four passes per wavefront)
+    (1, 2, 8192, 64, 3, 3, 2, torch.bfloat16, None, "both"),
 ]
 
 
