@@ -226,6 +226,12 @@ int mta_causal_pv_fwd(const void *p, const void *v, void *o, int64_t B, int64_t 
 int mta_causal_pv_band_fwd(const void *p, const void *v, const void *first_visible, void *o, int64_t B, int64_t H,
                            int64_t S, int64_t D, int causal, int io_dtype, void *stream);
 
+/* x[n,c,p,q] = 0 for q < first_visible[n,p], in place; x is (N,C,S,S), first_visible int32 (N,S).  The reference's
+ * `scores = torch.where(mask == float("-inf"), 0.0, scores)` behind its post-softmax conv (mta_attention_triton.py:82-83)
+ * for a band mask, below the diagonal (above it nothing is touched: the causal kernels on either side neither read nor
+ * need it).  16-bit I/O, S % 8 == 0; MTA_ERR_UNSUPPORTED otherwise. */
+int mta_band_zero_fwd(void *x, const void *first_visible, int64_t N, int64_t C, int64_t S, int io_dtype, void *stream);
+
 /* ---- The three stages of the causal forward (mta_attention_triton.py:68-89 with an identity post-softmax conv) over
  * score tensors in a TRIANGULAR LAYOUT.  The (B,H,S,S) tensors between the three kernels never leave the library's
  * caller, so their layout is free; this one stores what lies on and below the diagonal only and puts the rows that one

@@ -21,7 +21,8 @@ constexpr int RS_OCC = 5;  // wavefronts per SIMD the G*NV = 8 instances (e.g. 4
 namespace mta {
 // rowsoftmax_dense16.hip: the same pass for groups of 16 heads, both mixes on the matrix cores
 int mix16_softmax_launch(const void *x, const void *w1, const void *w2, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
-                         int causal, int fill_upper, int io_dtype, int w_dtype, hipStream_t st, int tri_in = 0, int tri_out = 0);
+                         int causal, int fill_upper, int io_dtype, int w_dtype, hipStream_t st, int tri_in = 0, int tri_out = 0,
+                         const float *key_bias = nullptr, const int *row_lo = nullptr);
 }  // namespace mta
 
 namespace {
@@ -872,8 +873,9 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb_in, 
         // the general one, for comparisons)
         static const bool no_packed = [] { const char *e_ = getenv("MTA_SOFTMAX_NO_PACKED"); return e_ && e_[0] == '1'; }();
         const int io_code = std::is_same<T, bf16_t>::value ? MTA_BF16 : MTA_F16;
-        if (G == 16 && plain && !no_packed) {
-            const int rc = mix16_softmax_launch(x, w1, w2, y, N, C, P, Q, causal, fill_upper, io_code, w_dtype, st, tri_in, tri_out);
+        if (G == 16 && !no_packed && (!kb || aligned_to(kb, 4))) {
+            const int rc = mix16_softmax_launch(x, w1, w2, y, N, C, P, Q, causal, fill_upper, io_code, w_dtype, st, tri_in, tri_out,
+                                                kb, row_lo);
             if (rc != MTA_ERR_UNSUPPORTED) return rc;
         }
         if (tri_in != tri_out) return MTA_ERR_UNSUPPORTED;
@@ -1016,7 +1018,7 @@ extern "C" int mta_headmix_softmax_tri_supported(int64_t C, int64_t S, int group
     if (e && e[0] == '1') return 0;
     if (group_size == 16) {  // the matrix-core kernel's row lists (rowsoftmax_dense16.hip)
         const char *e2 = getenv("MTA_MIX16_NO_ROW_LISTS");
-        return !band && !key_bias && S <= 4096 && S * S <= (1LL << 27) && !(e2 && e2[0] == '1');
+        return S <= 4096 && S * S <= (1LL << 27) && !(e2 && e2[0] == '1');
     }
     if (out_planes || (band && key_bias)) return 0;
     if (band && has_w1 && has_w2) return 0;

@@ -240,13 +240,20 @@ __global__ __launch_bounds__(64 * NW, 4) void mix16_softmax_kernel(const T *__re
 // needs no barrier, only the wavefront's own count of outstanding memory instructions - the copies of a row are followed
 // by the stores of the row before it, 4 per tile that stores, which the wait leaves in flight.
 // Rows [0, r4) take 4 wavefronts, [r4, r8) take 8, [r8, P) take 16.
-template <typename T, bool HAS1, bool HAS2>
+// MASKED instances: key_bias (fp32 (N,Q), or NULL) is added to the mixed, rounded scores and the sum rounded again (the
+// reference's `scores + mask` for one value per key; the batch entry's bias row waits in LDS); row_lo (int32 (N,P), or
+// NULL) is the first key a row sees (band mask): the keys ahead of it count as -inf, and a tile that lies wholly ahead of
+// it is neither copied nor computed - it is stored as +0.
+template <typename T, bool HAS1, bool HAS2, bool MASKED = false>
 __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(const T *__restrict__ x, const T *__restrict__ w1,
                                                                            const T *__restrict__ w2, T *__restrict__ y, int C,
                                                                            int P, int Q, int causal, int fill_upper, int r4,
-                                                                           int r8, int wpg, int tri_in, int tri_out)
+                                                                           int r8, int wpg, int tri_in, int tri_out,
+                                                                           const float *__restrict__ key_bias,
+                                                                           const int *__restrict__ row_lo)
 {
     constexpr int NW = M16_NW, TPW = M16_TPW, HG = M16_HG;
+    __shared__ __align__(16) float kbias[MASKED ? NW * TPW * M16_TK : 4];  // (MASKED) the batch entry's key bias
     __shared__ __align__(16) u32x4_t stage[NW * TPW * 4 * 64];  // [wavefront][tile][head of the lane's four][lane]
     __shared__ __align__(16) float red[2][HG * NW];             // [0] maxima, [1] sums; entry (row*16 + head)*NWR + wavefront
     __shared__ __align__(8) u32x2_t wts[2][64];                 // the lanes' weight fragments
@@ -284,7 +291,19 @@ __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(cons
         if constexpr (HAS1) wts[0][lane] = *reinterpret_cast<const u32x2_t *>(w1 + wo);
         if constexpr (HAS2) wts[1][lane] = *reinterpret_cast<const u32x2_t *>(w2 + wo);
     }
+    if constexpr (MASKED) {
+        if (key_bias)
+            for (int q = (int)threadIdx.x; q < Q; q += 64 * NW) kbias[q] = key_bias[n * Q + q];
+    }
     __syncthreads();  // (also: nothing is in flight when the loop starts counting)
+    // first visible key of row p (0 without a band mask)
+    auto lo_of = [&](int p) {
+        int lo = 0;
+        if constexpr (MASKED) {
+            if (row_lo && p >= 0) lo = row_lo[n * P + p];
+        }
+        return lo < 0 ? 0 : lo;
+    };
 
     // (ln, kg: the lane's key octet and head quad, handed in by the loop: see there)
     auto issue = [&](int p, int lg, int ln, int kg) {
@@ -293,10 +312,11 @@ __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(cons
         // (uniform base + 32-bit lane offset)
         const char *xrow = reinterpret_cast<const char *>(tri_in ? x + tbase0 + HG * tri_rowoff(p) : x + base0 + (int64_t)p * Q);
         const unsigned xplane = tri_in ? (unsigned)tri_rowlen(p) : plane;
+        const int lo = lo_of(p);
 #pragma unroll
         for (int i = 0; i < TPW; ++i) {
             const int q0 = ((i << lg) + wr) * M16_TK;
-            if (q0 > last) continue;  // (wavefront-uniform)
+            if (q0 > last || q0 + M16_TK <= lo) continue;  // (wavefront-uniform) nothing attended / nothing visible in the tile
             const int key = q0 + ln * 8;
             // beyond the attended keys a lane re-reads the row start; its values are masked
             const unsigned off = ((unsigned)(kg * 4) * xplane + (unsigned)(key <= last ? key : 0)) * (unsigned)sizeof(T);
@@ -326,6 +346,7 @@ __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(cons
         char *const yrow = reinterpret_cast<char *>(tri_out ? y + tbase0 + HG * tri_rowoff(p > 0 ? p : 0) : y + base0 + (int64_t)p * Q);
         const unsigned yplane = tri_out ? (unsigned)tri_rowlen(p > 0 ? p : 0) : plane;
         const int last = !active ? -1 : causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;
+        const int lo = lo_of(p);
         if (nst == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
         else if (nst == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -340,7 +361,7 @@ __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(cons
             constexpr int i = decltype(ic)::value;
             const int q0 = ((i << lg) + wr) * M16_TK;
             const int key = q0 + ln * 8;
-            if (q0 > last) return;  // (wavefront-uniform) wholly beyond the attended keys: s[i] stays unused
+            if (q0 > last || q0 + M16_TK <= lo) return;  // (wavefront-uniform) no attended or no visible key: s[i] stays unused
             u32x4_t xv[4];
             lds_load4x16_sync(stage_lds, i * 4096, xv[0], xv[1], xv[2], xv[3]);
 #pragma unroll
@@ -361,6 +382,28 @@ __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(cons
                         unpack2<T>(xv[v][j >> 1], lo, hi);
                         s[i][j][v] = (j & 1) ? hi : lo;
                     }
+                }
+            }
+            if constexpr (MASKED) {
+                if (key_bias) {  // (wavefront-uniform) the sum in the I/O dtype, as the unfused chain stores it
+                    const int kq = key <= last ? key : 0;
+                    const f32x4 kb0 = *reinterpret_cast<const f32x4 *>(&kbias[kq]), kb1 = *reinterpret_cast<const f32x4 *>(&kbias[kq + 4]);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float kb = j < 4 ? kb0[j & 3] : kb1[j & 3];
+                        float r0 = s[i][j][0] + kb, r1 = s[i][j][1] + kb, r2 = s[i][j][2] + kb, r3 = s[i][j][3] + kb;
+                        unpack2<T>(pack2<T>(r0, r1), r0, r1);
+                        unpack2<T>(pack2<T>(r2, r3), r2, r3);
+                        s[i][j][0] = r0; s[i][j][1] = r1; s[i][j][2] = r2; s[i][j][3] = r3;
+                    }
+                }
+                if (q0 < lo) {  // (wavefront-uniform) the tile holds the row's first visible key
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (key + j < lo) {
+#pragma unroll
+                            for (int v = 0; v < 4; ++v) s[i][j][v] = -INFINITY;
+                        }
                 }
             }
             if (q0 + M16_TK - 1 > last) {  // (wavefront-uniform) the tile straddles the last attended key
@@ -409,7 +452,7 @@ __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(cons
             for (int v = 0; v < 4; ++v) m[v] = -m[v] * LOG2E;
 #pragma unroll
             for (int i = 0; i < TPW; ++i) {
-                if (((i << lg) + wr) * M16_TK > last) continue;  // (wavefront-uniform) no attended key in this tile
+                if (((i << lg) + wr) * M16_TK > last || ((i << lg) + wr + 1) * M16_TK <= lo) continue;  // (wavefront-uniform) no attended / visible key in this tile
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
 #pragma unroll
@@ -450,7 +493,7 @@ __global__ __launch_bounds__(64 * M16_NW, 1) void mix16_softmax_rows_kernel(cons
             const int key = q0 + ln * 8;
             if (!active || q0 >= Q || (q0 > last && !fill_upper)) continue;  // (wavefront-uniform; lane 0 of the others stores)
             nst += 4;
-            if (q0 > last) {  // (wavefront-uniform) wholly above the diagonal, stored on request: +0
+            if (q0 > last || q0 + M16_TK <= lo) {  // (wavefront-uniform) wholly above the diagonal, stored on request, or wholly hidden: +0
                 if (key < Q) {
                     const u32x4_t z = {0u, 0u, 0u, 0u};
 #pragma unroll
@@ -511,8 +554,11 @@ namespace mta {
 // Launches the kernel when it applies (16-bit I/O, weights of the same dtype, groups of 16 heads, Q % 8 == 0,
 // Q <= 4096, 16-byte aligned tensors, 8-byte aligned weights); returns MTA_ERR_UNSUPPORTED otherwise.
 int mix16_softmax_launch(const void *x, const void *w1, const void *w2, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
-                         int causal, int fill_upper, int io_dtype, int w_dtype, hipStream_t st, int tri_in, int tri_out)
+                         int causal, int fill_upper, int io_dtype, int w_dtype, hipStream_t st, int tri_in, int tri_out,
+                         const float *key_bias, const int *row_lo)
 {
+    const bool masked = key_bias || row_lo;
+    if (row_lo && !causal) return MTA_ERR_UNSUPPORTED;
     if (io_dtype == MTA_F32 || w_dtype != io_dtype || (!w1 && !w2) || C % M16_HG != 0 || Q % 8 != 0 ||
         Q > (int64_t)M16_NW * M16_TPW * M16_TK)
         return MTA_ERR_UNSUPPORTED;
@@ -533,7 +579,7 @@ int mix16_softmax_launch(const void *x, const void *w1, const void *w2, void *y,
     // one launch of row lists, about one workgroup per CU; or a launch per kind of row, a workgroup per row
 #define MTA_M16_ALL(T, h1, h2)                                                                                          \
     if (no_rows || !small_planes) {                                                                                     \
-        if (tri_in || tri_out) return MTA_ERR_UNSUPPORTED;                                                              \
+        if (tri_in || tri_out || masked) return MTA_ERR_UNSUPPORTED;                                                    \
         MTA_M16_LAUNCH(T, h1, h2, 4, 0, r4);                                                                            \
         MTA_M16_LAUNCH(T, h1, h2, 8, r4, r8 - r4);                                                                      \
         MTA_M16_LAUNCH(T, h1, h2, 16, r8, P - r8);                                                                      \
@@ -541,9 +587,16 @@ int mix16_softmax_launch(const void *x, const void *w1, const void *w2, void *y,
         const int64_t steps = (P - r8) + (r8 - r4 + 1) / 2 + (r4 + 3) / 4;                                              \
         int64_t wpg = device_cu_count() / (N * (C / M16_HG));                                                           \
         wpg = wpg < 1 ? 1 : (wpg > steps ? steps : wpg);                                                                \
-        hipLaunchKernelGGL((mix16_softmax_rows_kernel<T, h1, h2>), dim3((unsigned)(N * (C / M16_HG) * wpg)),            \
-                           dim3(64 * M16_NW), 0, st, (const T *)x, (const T *)w1, (const T *)w2, (T *)y, (int)C, (int)P, \
-                           (int)Q, causal, fill_upper, (int)r4, (int)r8, (int)wpg, tri_in, tri_out);                    \
+        if (masked)                                                                                                     \
+            hipLaunchKernelGGL((mix16_softmax_rows_kernel<T, h1, h2, true>), dim3((unsigned)(N * (C / M16_HG) * wpg)),  \
+                               dim3(64 * M16_NW), 0, st, (const T *)x, (const T *)w1, (const T *)w2, (T *)y, (int)C,    \
+                               (int)P, (int)Q, causal, fill_upper, (int)r4, (int)r8, (int)wpg, tri_in, tri_out,         \
+                               key_bias, row_lo);                                                                       \
+        else                                                                                                            \
+            hipLaunchKernelGGL((mix16_softmax_rows_kernel<T, h1, h2>), dim3((unsigned)(N * (C / M16_HG) * wpg)),        \
+                               dim3(64 * M16_NW), 0, st, (const T *)x, (const T *)w1, (const T *)w2, (T *)y, (int)C,    \
+                               (int)P, (int)Q, causal, fill_upper, (int)r4, (int)r8, (int)wpg, tri_in, tri_out,         \
+                               nullptr, nullptr);                                                                       \
     }
 #define MTA_M16_CASES(T)                                          \
     if (w1 && w2) { MTA_M16_ALL(T, true, true) }                  \

@@ -308,8 +308,8 @@ class MTAAttentionTriton(nn.Module):
         """Inference route (module docstring).  ``key_bias``: fp32 (B,Sk), added to the mixed scores ahead of the
         softmax -- the caller has zeroed the K and V rows of the keys it hides.  ``first_visible``: int32 (B,S), a band
         mask (row p sees the keys first_visible[p] .. p): applied to the scores inside the first kernel and as -inf
-        inside the softmax kernel; the caller has checked that the first kernel exists and that the post-softmax conv
-        is the identity."""
+        inside the softmax kernel, and behind a post-softmax conv that is not the identity the hidden stretch of every row
+        is zeroed again; the caller has checked that the first kernel exists."""
         head_dim = xq.size(-1)
         # the reference multiplies by rsqrt(tensor(head_dim)), an fp32 scalar (mta_attention_triton.py:69-71)
         scale = float(torch.rsqrt(torch.tensor(float(head_dim))))
@@ -326,10 +326,11 @@ class MTAAttentionTriton(nn.Module):
         post_conv_identity = st.post_conv_identity
         n_keys = xk.size(-2)
         g_both = _lcm(g_pre, g_post)
-        # (the matrix-core variant for groups of 16 takes neither a key bias nor a band mask)
+        # (the matrix-core variant for groups of 16 takes a key bias or a band mask in its row-list form only)
         row_plain = key_bias is None and first_visible is None
-        one_pass = (post_conv_identity and _one_pass_group(g_both, xq.dtype, n_keys, w1, w2)
-                    and (row_plain or g_both <= _FUSED_MAX_GROUP))
+        masks_ok = lambda group: row_plain or group <= _FUSED_MAX_GROUP or (
+            group == _FUSED_MFMA_GROUP and os.environ.get("MTA_MIX16_NO_ROW_LISTS") != "1")
+        one_pass = post_conv_identity and _one_pass_group(g_both, xq.dtype, n_keys, w1, w2) and masks_ok(g_both)
         # the last stage may leave the upper triangle unwritten only if our own P V kernel consumes it
         own_pv = (xq.size(-2) == xk.size(-2) and xq.dtype == xv.dtype
                   and ops.causal_pv_supported(xq.dtype, xq.size(-2), xv.size(-1)))
@@ -356,12 +357,14 @@ class MTAAttentionTriton(nn.Module):
         scores = None
         # (dense groups of 16 heads ahead of a post-softmax conv: the first score tensor still travels in the triangular
         # layout, the softmax stage hands the conv (B,H,S,S) planes)
-        tri_first = (self.score_layout != "planes" and self.causal and not one_pass and row_plain and g_pre == 16
+        tri_first = (self.score_layout != "planes" and self.causal and not one_pass and g_pre == 16 and masks_ok(16)
                      and w1 is not None and not (post_conv_identity and w2 is None and not own_pv)
-                     and ops.tri_route_supported(xq, xk, self.mta_conv_triton.weight, 16, w1, None, False, out_planes=True))
+                     and (key_bias is None or key_bias.is_contiguous())
+                     and ops.tri_route_supported(xq, xk, self.mta_conv_triton.weight, 16, w1, None, first_visible is not None,
+                                                 out_planes=True, key_bias=key_bias is not None))
         if tri_first:
             self._mark("qk_conv")
-            scores = ops.qk_conv_tri(xq, xk, self.mta_conv_triton.weight, scale, 16)
+            scores = ops.qk_conv_tri(xq, xk, self.mta_conv_triton.weight, scale, 16, first_visible=first_visible)
         elif ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight):
             self._mark("qk_conv")
             scores = ops.qk_conv(xq, xk, self.mta_conv_triton.weight, self.causal, scale, fill_upper=False,
@@ -380,8 +383,9 @@ class MTAAttentionTriton(nn.Module):
         else:
             if tri_first:
                 self._mark("mix_softmax")
-                scores = ops.headmix_softmax_tri(scores, w1, None, xq.size(0), self.n_heads, n_keys, g_pre, out_planes=True)
-            elif _one_pass_group(g_pre, xq.dtype, n_keys, w1) and (row_plain or g_pre <= _FUSED_MAX_GROUP):
+                scores = ops.headmix_softmax_tri(scores, w1, None, xq.size(0), self.n_heads, n_keys, g_pre, out_planes=True,
+                                                 first_visible=first_visible, key_bias=key_bias)
+            elif _one_pass_group(g_pre, xq.dtype, n_keys, w1) and masks_ok(g_pre):
                 self._mark("mix_softmax")
                 scores = ops.headmix_softmax(scores, w1, None, self.causal, group_size=g_pre, key_bias=key_bias,
                                              first_visible=first_visible,
@@ -402,7 +406,9 @@ class MTAAttentionTriton(nn.Module):
             conv_w = self.mta_conv_after_sm_triton.weight
             mix16 = (g_post == 16 and ks in _CONV_MIX16_SIZES and scores.dtype in (torch.bfloat16, torch.float16)
                      and conv_w.dtype == scores.dtype and w_post.dtype == scores.dtype and n_keys % 8 == 0)
-            if not post_conv_identity and w2 is not None and (
+            # (under a band mask the conv's result is zeroed at the hidden positions ahead of the mixing, as the reference
+            # does: two kernels with that step between them)
+            if first_visible is None and not post_conv_identity and w2 is not None and (
                     (g_post <= _CONV_MIX_MAX_GROUP and ks in _CONV_MIX_SIZES) or mix16):
                 self._mark("conv_mix_post")
                 done = ops.conv2d_headmix(scores, self.mta_conv_after_sm_triton.weight, w_post, self.causal,
@@ -415,6 +421,11 @@ class MTAAttentionTriton(nn.Module):
                     self._mark("conv_post")
                     scores = ops.conv2d_causal(scores, self.mta_conv_after_sm_triton.weight, self.causal,
                                                fill_upper=w2 is None and not own_pv)
+                    if first_visible is not None:
+                        # the conv has spread probability into columns the rows do not see
+                        # (mta_attention_triton.py:82-83: torch.where(mask == -inf, 0.0, scores))
+                        if ops.band_zero_(scores, first_visible) is None:
+                            raise RuntimeError("band masks need 16-bit scores of a length that is a multiple of 8")
                 if w2 is not None:
                     self._mark("mix_post")
                     scores = ops.headmix(scores, w_post, self.causal, 0.0, group_size=g_post, fill_upper=not own_pv)
@@ -539,8 +550,7 @@ class MTAAttentionTriton(nn.Module):
                 kind, what = self._structured_mask(mask, xq.size(0), xq.size(-2))
                 if kind == "keys":
                     return self._forward_hidden_keys(xq, xk, xv, what)
-                if (kind == "band" and self._current_structure().post_conv_identity
-                        and ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight)):
+                if kind == "band" and ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight):
                     return self._forward_fused(xq, xk, xv, first_visible=what)
         mask = self._update_mask(mask=mask, bsz=xq.size(0), xq=xq, xk_size=xk.size(-2))
         scale = float(torch.rsqrt(torch.tensor(float(xq.size(-1)))))  # a host scalar: the product stays one vectorised pass

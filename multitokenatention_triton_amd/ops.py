@@ -529,6 +529,22 @@ def tri_pack(x: torch.Tensor, group: int, pad_value: float = float("nan")) -> to
     return out
 
 
+def band_zero_(x: torch.Tensor, first_visible: torch.Tensor) -> Optional[torch.Tensor]:
+    """In place: x[n,c,p,q] = 0 for q < first_visible[n,p] (what the reference's ``torch.where(mask == -inf, 0, scores)``
+    behind the post-softmax conv does under a band mask); see mta_band_zero_fwd.  Returns ``None`` when unsupported."""
+    x = _device_tensor(x, "input")
+    if x.dim() != 4 or x.shape[2] != x.shape[3] or not x.is_contiguous():
+        raise ValueError(f"expected a contiguous (N,C,S,S) tensor, got {tuple(x.shape)}")
+    n, c, s, _ = x.shape
+    first_visible = _band_arg(first_visible, n, s)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().mta_band_zero_fwd(x.data_ptr(), first_visible.data_ptr(), n, c, s, _code(x, "input"), _stream(x))
+    if rc == _lib.MTA_ERR_UNSUPPORTED:
+        return None
+    _lib.check(rc, "mta_band_zero_fwd")
+    return x
+
+
 def causal_ptx(p: torch.Tensor, x: torch.Tensor, causal: bool) -> Optional[torch.Tensor]:
     """P^T X for P (B,H,S,S), X (B,H,S,D): out[k] = sum_p P[p,k] X[p], over p >= k only when causal (nothing of P above
     the diagonal is read); see mta_causal_ptx_fwd.  Returns ``None`` when unsupported (the caller then uses

@@ -101,6 +101,8 @@ def test_triangular_layout_entry_points_validate_and_answer_on_the_host():
     assert lib.mta_causal_pv_tri_fwd(p, p, None, None, 1, 4, 64, 64, 4, 1, None) == -1
     assert lib.mta_causal_pv_tri_fwd(p, p, None, p, 1, 6, 64, 64, 4, 1, None) == -5
     assert lib.mta_causal_pv_tri_fwd(p, p, None, p, 1, 4, 64, 48, 4, 1, None) == -7
+    assert lib.mta_band_zero_fwd(None, p, 1, 1, 8, 1, None) == -1 and lib.mta_band_zero_fwd(p, p, 1, 1, 8, 0, None) == -9
+    assert lib.mta_band_zero_fwd(p, p, 1, 1, 12, 1, None) == -9 and lib.mta_band_zero_fwd(p, p, 0, 1, 8, 1, None) == -3
     # which combinations the softmax stage has a kernel for: (C, S, group, out_planes, io, w, has_w1, has_w2, band, key_bias)
     q = lib.mta_headmix_softmax_tri_supported
     assert q(16, 4096, 4, 0, 1, 1, 1, 1, 0, 0) == 1 and q(16, 4104, 4, 0, 1, 1, 1, 1, 0, 0) == 0   # packed kernel: up to 4096 keys
@@ -108,8 +110,8 @@ def test_triangular_layout_entry_points_validate_and_answer_on_the_host():
     assert q(16, 4096, 4, 0, 1, 1, 1, 0, 1, 0) == 1 and q(16, 4096, 4, 0, 1, 1, 1, 1, 1, 0) == 0   # band: one weight only
     assert q(16, 4096, 4, 0, 0, 0, 1, 1, 0, 0) == 0 and q(16, 4096, 4, 0, 1, 0, 1, 1, 0, 0) == 0   # fp32 data / fp32 weights
     assert q(16, 4096, 4, 1, 1, 1, 1, 1, 0, 0) == 0 and q(16, 4096, 16, 1, 1, 1, 1, 0, 0, 0) == 1   # planes out: groups of 16 only
-    assert q(32, 4096, 16, 0, 2, 2, 1, 1, 0, 0) == 1 and q(32, 4096, 16, 0, 2, 2, 1, 1, 1, 0) == 0 and q(16, 4100, 16, 0, 1, 1, 1, 1, 0, 0) == 0
-    assert q(16, 4096, 4, 0, 1, 1, 1, 1, 0, 1) == 1 and q(16, 4096, 4, 0, 1, 1, 1, 0, 1, 1) == 0 and q(16, 4096, 16, 0, 1, 1, 1, 1, 0, 1) == 0  # key bias
+    assert q(32, 4096, 16, 0, 2, 2, 1, 1, 0, 0) == 1 and q(32, 4096, 16, 0, 2, 2, 1, 1, 1, 0) == 1 and q(16, 4100, 16, 0, 1, 1, 1, 1, 0, 0) == 0
+    assert q(16, 4096, 4, 0, 1, 1, 1, 1, 0, 1) == 1 and q(16, 4096, 4, 0, 1, 1, 1, 0, 1, 1) == 0 and q(16, 4096, 16, 0, 1, 1, 1, 1, 0, 1) == 1  # key bias
     # the layout's arithmetic: rows of 64*(p/64+1) elements, one after the other
     assert ops.tri_row_offset(0) == 0 and ops.tri_row_offset(1) == 64 and ops.tri_row_offset(64) == 4096
     assert ops.tri_row_offset(65) == 4096 + 128 and ops.tri_row_offset(4096) == sum(64 * (r // 64 + 1) for r in range(4096))

@@ -308,7 +308,8 @@ def test_qk_conv_band_parity(pkg, case):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("weights", ["both", "first", "second"])
-@pytest.mark.parametrize("group,s", [(4, 520), (2, 2304), (8, 264), (1, 1000), (16, 136), (4, 4096), (4, 1608), (8, 2048)])
+@pytest.mark.parametrize("group,s", [(4, 520), (2, 2304), (8, 264), (1, 1000), (16, 136), (4, 4096), (4, 1608), (8, 2048),
+                                     (16, 1160), (16, 2560)])
 def test_headmix_softmax_band_parity(pkg, group, s, weights, dtype):
     """mix -> `scores + mask` -> softmax -> mix (mta_attention_triton.py:75-85) for a band mask given as the first
     visible key of every row; with one weight and 16-bit data the packed kernel's band instances run."""
@@ -443,6 +444,8 @@ TRI_CASES = [
     (1, 8, 520, 64, 11, 15, 8, torch.bfloat16, "ragged", "first"), (1, 4, 4096, 128, 6, 11, 4, torch.bfloat16, None, "both"),
     # groups of 16 heads (the matrix-core softmax kernel's row lists): rows of all three kinds, two groups
     (1, 16, 2304, 64, 7, 7, 16, torch.float16, None, "first"), (2, 32, 1160, 64, 3, 3, 16, torch.bfloat16, None, "both"),
+    # groups of 16 heads under band masks
+    (1, 16, 1160, 64, 7, 7, 16, torch.bfloat16, "documents", "first"), (1, 32, 2304, 64, 3, 3, 16, torch.float16, "window", "both"),
     # a sequence shorter than one padded row; the longest rows the 8-head kernel takes; a band with groups of 8
     (1, 2, 8, 128, 3, 3, 2, torch.bfloat16, None, "both"), (1, 8, 2048, 128, 5, 7, 8, torch.float16, None, "both"),
     (1, 16, 72, 64, 3, 3, 16, torch.bfloat16, None, "second"), (2, 8, 1032, 64, 7, 7, 8, torch.bfloat16, "window", "second"),
@@ -486,7 +489,7 @@ def test_triangular_layout_stages_equal_the_plane_layout(pkg, case):
     assert torch.equal(ops.headmix_softmax_tri(poisoned, w1, w2, b, h, s, group, first_visible=first)[ops.tri_pack(lower.to(dtype), group, 0.0) > 0],
                        p_tri[ops.tri_pack(lower.to(dtype), group, 0.0) > 0])
 
-    if kind is None and group != 16:   # with a key bias (key masks): a few keys hidden, a few finite values
+    if kind is None:   # with a key bias (key masks): a few keys hidden, a few finite values
         kb = torch.zeros(b, s)
         kb[:, 3::7] = float("-inf")
         kb[:, 5::11] = -1.5
@@ -496,7 +499,7 @@ def test_triangular_layout_stages_equal_the_plane_layout(pkg, case):
         assert torch.equal(ops.tri_unpack(ops.headmix_softmax_tri(s_tri, w1, w2, b, h, s, group, key_bias=kb), b, h, s, group)[lower],
                            biased[lower])
     if group == 16:   # the same stage from the triangular layout into planes (what a post-softmax conv takes)
-        mixed = ops.headmix_softmax_tri(s_tri, w1, w2, b, h, s, group, out_planes=True)
+        mixed = ops.headmix_softmax_tri(s_tri, w1, w2, b, h, s, group, out_planes=True, first_visible=first)
         assert torch.equal(mixed[lower], p_plane[lower])
 
     o_plane = ops.causal_pv(p_plane, v, True, first_visible=first)
@@ -554,6 +557,71 @@ def test_mta_score_layouts_agree(pkg, masked):
         stages[layout] = seen
     assert stages["auto"] == stages["planes"] == ["qk_conv", "mix_softmax_mix", "pv", "end"]
     assert torch.equal(outs["auto"], outs["planes"])
+
+
+@pytest.mark.parametrize("case", [(2, 8, 776, 64, 4, "documents", torch.bfloat16), (1, 16, 1160, 128, 16, "window", torch.float16),
+                                  (1, 4, 520, 64, 2, "ragged", torch.bfloat16)])
+def test_mta_use_mask_band_masks_with_a_post_softmax_conv(pkg, case):
+    """Band masks with all four weights non-trivial (a 7x7 conv before and a 3x3 conv after the softmax, block-diagonal or
+    dense head weights): the kernels run - scores under the band, softmax under the band, post-softmax conv, the hidden stretch of
+    every row zeroed again (mta_attention_triton.py:82-83), head mixing, P V under the band - and the result is the
+    oracle's given the mask tensor."""
+    b, h, s, d, group, kind, dtype = case
+    print(f"mta use_mask band + post conv case={case}", flush=True)
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=95)
+    params = _config_like(h, group, 7, 7, 0.05, dtype, post="random")
+    first = _band_first(kind, b, s)
+    keys = torch.arange(s)
+    visible = ((keys[None, None, :] >= first[:, :, None]) & (keys[None, None, :] <= keys[None, :, None]))[:, None]   # (B,1,S,S)
+    want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3],
+                         mask=torch.where(visible, 0.0, float("-inf")).to(dtype).expand(b, h, s, s).contiguous())
+    mod = _mta_module(pkg, h, 7, 7, 3, 3, *params, dtype, use_mask=True, structure="infer")
+    stages = []
+    mod._stage_hook = stages.append
+    got = mod(q.cuda(), k.cuda(), v.cuda(), visible.cuda(), None).cpu()
+    assert stages[0] == "qk_conv" and "conv_post" in stages and stages[-2:] == ["pv", "end"], stages
+    torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+
+
+def test_mta_use_mask_key_padding_general_route(pkg):
+    """Dense 16-head weights, a conv before and after the softmax, a key-padding mask of a batch: the four-kernel route
+    (the matrix-core softmax kernel takes the key bias), against the oracle given the mask tensor."""
+    print("mta use_mask key padding, general route", flush=True)
+    dtype = torch.float16
+    b, h, s, d = 2, 16, 776, 64
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=96)
+    g = torch.Generator().manual_seed(97)
+    dense = lambda: (torch.eye(h) + 0.05 * torch.randn(h, h, generator=g)).to(dtype)
+    conv = lambda: (torch.randn(h, 7, 7, generator=g) * 0.05).to(dtype)
+    params = [conv(), dense(), conv(), dense()]
+    rows = torch.arange(s)
+    keep = rows[None, :] < torch.tensor([s, 500])[:, None]
+    visible = (keep[:, None, None, :] & (rows[None, :] <= rows[:, None])[None, None])
+    want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3],
+                         mask=torch.where(visible, 0.0, float("-inf")).to(dtype).expand(b, h, s, s).contiguous())
+    mod = _mta_module(pkg, h, 7, 7, 7, 7, *params, dtype, use_mask=True, structure="dense")
+    stages = []
+    mod._stage_hook = stages.append
+    got = mod(q.cuda(), k.cuda(), v.cuda(), visible.cuda(), None).cpu()
+    assert stages == ["qk_conv", "mix_softmax", "conv_mix_post", "pv", "end"], stages
+    torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+
+
+def test_band_zero_clears_exactly_the_hidden_stretch(pkg):
+    """mta_band_zero_fwd: x[n,c,p,q] = 0 for q < first[n,p], nothing else touched (not even NaN above the diagonal)."""
+    print("band_zero", flush=True)
+    for dtype, (n, c, s) in ((torch.bfloat16, (2, 3, 520)), (torch.float16, (1, 2, 72))):
+        first = _band_first("ragged", n, s).cuda()
+        first[:, 7] = 50                                     # beyond the diagonal: everything up to it is hidden
+        x = torch.randn(n, c, s, s).to(dtype).cuda()
+        x.masked_fill_(torch.triu(torch.ones(s, s, dtype=torch.bool, device="cuda"), 1), float("nan"))
+        want = x.clone()
+        keys = torch.arange(s, device="cuda")
+        hidden = (keys[None, None, :] < first[:, :, None]) & (keys[None, None, :] <= keys[None, :, None])
+        want.masked_fill_(hidden[:, None], 0)
+        got = pkg.ops.band_zero_(x, first)
+        assert got is x
+        assert torch.equal(torch.nan_to_num(got, nan=123.0), torch.nan_to_num(want, nan=123.0))
 
 
 def test_qk_conv_reports_unsupported(pkg):

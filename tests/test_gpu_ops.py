@@ -349,7 +349,9 @@ def test_mix_softmax_mix_dense16_leaves_the_upper_triangle_alone(ops, case, dt):
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 @pytest.mark.parametrize("case", [(1, 4, 64, 2, True, True), (2, 4, 100, 4, True, False), (1, 8, 257, 4, False, True),
                                   (2, 8, 2048, 4, True, True), (1, 8, 72, 8, True, True), (1, 2, 33, 1, False, False),
-                                  (1, 4, 4096, 4, False, True)])
+                                  (1, 4, 4096, 4, False, True),
+                                  # groups of 16 heads (the matrix-core kernel's row lists, the bias row in LDS)
+                                  (2, 16, 264, 16, True, True), (1, 32, 1160, 16, True, False), (1, 16, 2304, 16, False, True)])
 def test_mix_softmax_mix_key_bias(ops, case, dt):
     """`scores = scores + mask` of mta_attention_triton.py:77-78 for a mask that is the causal rule plus one value per
     key: hidden keys (-inf) get probability 0, finite values are added in the I/O dtype."""
