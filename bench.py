@@ -292,7 +292,20 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
         "ms": ms, "stages_ms": stages,
         "note": "forward only; the reference's published row for this shape (Triton 11.345 ms, PyTorch 43.795 ms, "
                 "hardware unstated) is context, not a baseline"}
-    del mod, sets
+    # the same module under a 1024-key sliding-window mask tensor: band masks behind a post-softmax conv
+    mod.use_mask = True
+    s_len = sets[0][0].size(2)
+    pos = torch.arange(s_len, device=device)
+    window = ((pos[None, :] <= pos[:, None]) & (pos[None, :] > pos[:, None] - 1024))[None, None]
+    ms = time_steps(torch, lambda i: mod(*sets[i], window, None), len(sets), min(warmup, 30), max(3, steps // 2))
+    stages = []
+    mod._stage_hook = stages.append
+    mod(*sets[0], window, None)
+    mod._stage_hook = None
+    out["mta_forward_general_fp16_1x16x4096x128_7x7_pre_post_dense_window1024_mask"] = {
+        "ms": ms, "stages": stages,
+        "note": "the general configuration with use_mask=True and a sliding-window mask tensor; not a row of the reference's"}
+    del mod, sets, window
     # two more of the reference's own benchmark shapes, forward only: its benchmark script's configuration (bf16, 11x15
     # kernels before and after the softmax, B1 H16 S4096 D64: benchmark_mta_attention.py:12-38) and the 128-head sweep's
     # first row (B1 H128 S2048 D64 fp16 7x7: benchmark_seq_len.py:22-30, benchmark_seq_len_results.jsonl:198)

@@ -1156,6 +1156,39 @@ def test_conv_attention_lse(pkg, case):
     assert torch.equal(o, o2)
 
 
+def test_mta_general_route_published_shape_under_a_window_mask(pkg):
+    """The published shape with all four weights non-trivial under a sliding-window mask tensor (what bench.py times as
+    its general window row): the kernels run with the band (stage marks), and two size-independent checks against the
+    unmasked forward of the same module - a window that hides nothing gives the same output (other kernels behind the
+    softmax: to the usual tolerance), and under a 1024-key window the first 1024 rows, whose window hides nothing, are
+    unchanged while later rows differ."""
+    print("mta general route, published shape, window mask", flush=True)
+    dtype = torch.float16
+    b, h, s, d = 1, 16, 4096, 128
+    q, k, v = (t.cuda() for t in O.seeded_qkv(b, h, s, d, dtype, seed=400))
+    g = torch.Generator().manual_seed(321)
+    params = [O.seeded_conv_weight(h, 7, 7, 0.05, dtype, seed=5), (torch.eye(h) + 0.1 * torch.randn(h, h, generator=g)).to(dtype),
+              O.seeded_conv_weight(h, 7, 7, 0.05, dtype, seed=6), (torch.eye(h) + 0.1 * torch.randn(h, h, generator=g)).to(dtype)]
+    mod = _mta_module(pkg, h, 7, 7, 7, 7, *params, dtype, use_mask=True, structure="dense")
+    plain = mod(q, k, v, None, None)
+    rows = torch.arange(s, device="cuda")
+    causal = rows[None, :] <= rows[:, None]
+    for width in (s, 1024):
+        window = (causal & (rows[None, :] > rows[:, None] - width))[None, None]
+        stages = []
+        mod._stage_hook = stages.append
+        got = mod(q, k, v, window, None)
+        mod._stage_hook = None
+        # (a window that hides nothing is "the causal rule and no hidden key": the route of key masks, with a zero bias)
+        behind = ["conv_mix_post"] if width == s else ["conv_post", "mix_post"]
+        assert stages == ["qk_conv", "mix_softmax", *behind, "pv", "end"], stages
+        assert torch.isfinite(got.float()).all()
+        same = slice(0, width)
+        torch.testing.assert_close(got[:, same].float(), plain[:, same].float(), **tol(dtype))
+        if width < s:
+            assert (got[:, 2048:].float() - plain[:, 2048:].float()).abs().max() > 1e-2
+
+
 @pytest.mark.parametrize("structure", ["infer", "dense"])
 def test_mta_general_route_published_shape(pkg, structure):
     """The reference's published shape (benchmark_seq_len_results.jsonl: B1 H16 S4096 D128 fp16, 7x7 kernels before and
