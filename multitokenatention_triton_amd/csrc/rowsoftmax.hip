@@ -779,6 +779,78 @@ __global__ __launch_bounds__(NT, OCC) void mix_softmax_mix_packed(
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// No weights, 16-bit data, rows of at most 2048 keys: a wavefront per row (up to 4 vectors of 8 keys per lane), no LDS
+// and no barrier; a workgroup of four wavefronts takes SR_ROWS consecutive rows of one plane.  With a workgroup per row,
+// a launch over 128 heads x 2048 rows starts 262144 workgroups that move 4 KB each, and that is what its time is.
+constexpr int SR_ROWS = 32, SR_NV = 4;
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_rows_wave(const T *__restrict__ x, T *__restrict__ y, int P, int Q, int causal,
+                                                         int fill_upper, int blocks_per_plane)
+{
+    constexpr int VEC = 8;
+    constexpr float LOG2E = 1.4426950408889634f;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t plane = blockIdx.x / (unsigned)blocks_per_plane;
+    const int p0 = (int)(blockIdx.x % (unsigned)blocks_per_plane) * SR_ROWS;
+    for (int p = p0 + wave; p < p0 + SR_ROWS && p < P; p += 4) {
+        const T *xr = x + (plane * P + p) * (int64_t)Q;
+        T *yr = y + (plane * P + p) * (int64_t)Q;
+        const int last = causal ? (p < Q - 1 ? p : Q - 1) : Q - 1;  // last attended key
+        rs_u4 xin[SR_NV];
+#pragma unroll
+        for (int k = 0; k < SR_NV; ++k) {
+            if (k * 64 * VEC > last) break;  // (wavefront-uniform) wholly beyond the attended keys
+            const int q = (k * 64 + lane) * VEC;
+            xin[k] = __builtin_nontemporal_load(reinterpret_cast<const rs_u4 *>(xr + (q <= last ? q : 0)));  // (beyond: the row start)
+        }
+        float sv[SR_NV][VEC];
+        float m = -INFINITY;
+#pragma unroll
+        for (int k = 0; k < SR_NV; ++k) {
+            if (k * 64 * VEC > last) break;
+            const int q = (k * 64 + lane) * VEC;
+#pragma unroll
+            for (int d = 0; d < VEC / 2; ++d) {
+                unpack2<T>(xin[k][d], sv[k][2 * d], sv[k][2 * d + 1]);
+                if (q + 2 * d > last) sv[k][2 * d] = -INFINITY;
+                if (q + 2 * d + 1 > last) sv[k][2 * d + 1] = -INFINITY;
+                m = fmaxf(m, fmaxf(sv[k][2 * d], sv[k][2 * d + 1]));
+            }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+        const float mneg = -m * LOG2E;
+        float sum = 0.0f;
+#pragma unroll
+        for (int k = 0; k < SR_NV; ++k) {
+            if (k * 64 * VEC > last) break;
+#pragma unroll
+            for (int u = 0; u < VEC; ++u) {
+                sv[k][u] = __builtin_amdgcn_exp2f(fmaf(sv[k][u], LOG2E, mneg));  // (-inf -> 0)
+                sum += sv[k][u];
+            }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+        const float rc = __builtin_amdgcn_rcpf(sum);  // 1/sum: the hardware reciprocal and one Newton step
+        const float inv = fmaf(fmaf(-sum, rc, 1.0f), rc, rc);
+#pragma unroll
+        for (int k = 0; k < SR_NV; ++k) {
+            const int q = (k * 64 + lane) * VEC;
+            if (q >= Q) break;
+            if (q > last) {  // wholly above the diagonal: +0 on request
+                if (fill_upper) __builtin_nontemporal_store(rs_u4{0u, 0u, 0u, 0u}, reinterpret_cast<rs_u4 *>(yr + q));
+                continue;
+            }
+            // (keys beyond the last attended one carry probability 0 and come out as +0)
+            const rs_u4 out = {pack2<T>(sv[k][0] * inv, sv[k][1] * inv), pack2<T>(sv[k][2] * inv, sv[k][3] * inv),
+                               pack2<T>(sv[k][4] * inv, sv[k][5] * inv), pack2<T>(sv[k][6] * inv, sv[k][7] * inv)};
+            __builtin_nontemporal_store(out, reinterpret_cast<rs_u4 *>(yr + q));
+        }
+    }
+}
+
 // Any row length / any group size: three sweeps over the row, inputs re-read (and re-mixed)
 // in each; scalar accesses.  Correctness fallback for ragged or very long rows.
 template <typename T, int NT>
@@ -946,6 +1018,18 @@ int dispatch(const void *x, const void *w1, const void *w2, const float *kb_in, 
         }
     }
     if (tri_in || tri_out) return MTA_ERR_UNSUPPORTED;  // (only the kernels above know the triangular layout)
+    if constexpr (sizeof(T) == 2) {
+        // no weights, short rows: a wavefront per row (MTA_SOFTMAX_NO_WAVE_ROWS=1 keeps a workgroup per row, for comparisons)
+        static const bool no_wave = [] { const char *e_ = getenv("MTA_SOFTMAX_NO_WAVE_ROWS"); return e_ && e_[0] == '1'; }();
+        if (G == 1 && !w1 && !w2 && plain && vec_ok && Q <= 64 * VEC * SR_NV && !no_wave) {
+            const int64_t bpp = (P + SR_ROWS - 1) / SR_ROWS;
+            if (N * C * bpp <= 0x7fffffffLL) {
+                hipLaunchKernelGGL((softmax_rows_wave<T>), dim3((unsigned)(N * C * bpp)), dim3(256), 0, st, (const T *)x,
+                                   (T *)y, (int)P, (int)Q, causal, fill_upper, (int)bpp);
+                return launch_status();
+            }
+        }
+    }
     if (vec_ok) {
 #define MTA_RS_CASE(g, v)                                                                   \
     if (G == g && nv <= v) return launch_fixed<T, g, v>(x, w1, w2, kb, row_lo, y, N, C, P, Q, causal, w_dtype, fill_upper, st);

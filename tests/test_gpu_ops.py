@@ -294,6 +294,9 @@ MS_CASES = [
     # lists of rows per workgroup with several steps each: two batch entries and two groups, rows of all three kinds
     # (4, 8, 16 wavefronts); rows that end inside a tile with the second weight only
     (2, 32, 2304, 16, True, True), (1, 16, 3000, 16, False, True),
+    # no weights, rows of up to 2048 keys (16-bit data: a wavefront per row): rows that end inside a lane's vector, the
+    # longest rows, several planes and batch entries; 2056 keys: back to a workgroup per row
+    (2, 3, 520, 1, False, False), (1, 2, 2048, 1, False, False), (1, 4, 72, 1, False, False), (1, 2, 2056, 1, False, False),
 ]
 
 

@@ -32,6 +32,8 @@ GROUPS = [
     # the inference route with its score tensors as (B,H,S,S) planes (by default: the triangular layout)
     ({"MTA_SCORE_LAYOUT": "planes"}, ["tests/test_gpu_attention.py"],
      "test_mta_headline or test_mta_use_mask or test_mta_general"),
+    # the softmax without weights with a workgroup per row (by default short rows take a wavefront per row)
+    ({"MTA_SOFTMAX_NO_WAVE_ROWS": "1"}, ["tests/test_gpu_ops.py"], "test_mix_softmax_mix_parity and not f32 and (case21 or case22 or case23)"),
     ({"MTA_MIX16_NO_ROW_LISTS": "1"}, ["tests/test_gpu_ops.py"], "(test_mix_softmax_mix_parity and not f32) or test_mix_softmax_mix_dense16"),
 ]
 
