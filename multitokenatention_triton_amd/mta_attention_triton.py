@@ -13,10 +13,18 @@ Inference (no input or parameter requires grad, or grad mode is off):
     post-softmax conv kernel is the identity tap -- the post-softmax head mixing run
     as one kernel (``mta_headmix_softmax_fwd``): one pass over the score tensor
     instead of four, and no fp32 copy of it;
-  * otherwise, for mixing groups of up to 4 heads and 3x3 or 7x7 kernels, the
-    post-softmax conv and head mixing run as one kernel (``mta_conv2d_headmix_fwd``):
-    the conv result never reaches HBM;
-  * P V reads only the lower triangle of P (``mta_causal_pv_fwd``).
+  * otherwise, for mixing groups of up to 4 heads and 3x3 or 7x7 kernels, and for dense
+    groups of 16 heads and 3x3, 5x5 or 7x7 kernels, the post-softmax conv and head mixing
+    run as one kernel (``mta_conv2d_headmix_fwd``): the conv result never reaches HBM;
+  * P V reads only the lower triangle of P (``mta_causal_pv_fwd``);
+  * where all of these kernels know it, the score tensors between them travel in a
+    triangular layout (``mta_qk_conv_tri_fwd`` and its two companions): the lower triangle
+    only, the rows one kernel reads side by side (``score_layout = "planes"`` keeps
+    (B,H,S,S) tensors);
+  * ``use_mask=True``: masks that amount to "the causal rule and hidden keys" (2-D key
+    masks, key padding of a batch) or to "row p sees the keys first[p] .. p" (sliding
+    windows, packed documents) go into the same kernels as one value per key or per row;
+    any other mask tensor takes the reference's elementwise steps around the kernels.
 
 Training (something requires grad): the stages run one by one through autograd
 Functions, as in the reference, so that ``backward()`` works: the two conv and the two
