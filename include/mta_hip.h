@@ -232,7 +232,7 @@ int mta_causal_pv_band_fwd(const void *p, const void *v, const void *first_visib
  * need it).  16-bit I/O, S % 8 == 0; MTA_ERR_UNSUPPORTED otherwise. */
 int mta_band_zero_fwd(void *x, const void *first_visible, int64_t N, int64_t C, int64_t S, int io_dtype, void *stream);
 
-/* ---- The three stages of the causal forward (mta_attention_triton.py:68-89 with an identity post-softmax conv) over
+/* ---- The three stages of the causal forward (mta_attention_triton.py:68-89 without a post-softmax conv) over
  * score tensors in a TRIANGULAR LAYOUT.  The (B,H,S,S) tensors between the three kernels never leave the library's
  * caller, so their layout is free; this one stores what lies on and below the diagonal only and puts the rows that one
  * workgroup of the softmax stage reads side by side:
@@ -247,7 +247,7 @@ int mta_band_zero_fwd(void *x, const void *first_visible, int64_t N, int64_t C, 
  *   mta_headmix_softmax_tri_fwd: mta_headmix_softmax_fwd (causal, fill_upper = 0) / mta_headmix_softmax_bias_fwd (key_bias
  *                                not NULL; fp32 (N,S), 16-byte aligned) / mta_headmix_softmax_band_fwd, layout of
  *                                the input and, with out_planes = 0, of the output; the layout's group = group_size
- *                                (2, 4, 8; 16 without a band mask); out_planes = 1 (groups of 16 only): the output as
+ *                                (2, 4, 8 or 16); out_planes = 1 (groups of 16 only): the output as
  *                                (N,C,S,S) planes, nothing written above the diagonal; weights of the I/O dtype.
  *   mta_causal_pv_tri_fwd:       mta_causal_pv_band_fwd (causal), layout of P. */
 int mta_qk_conv_tri_fwd(const void *q, const void *k, const void *w, const void *first_visible, void *s_out, int64_t B,
