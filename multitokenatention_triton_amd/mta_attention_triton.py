@@ -206,9 +206,11 @@ class _MixSoftmax(torch.autograd.Function):
     two gradient kernels."""
 
     @staticmethod
-    def forward(ctx, x, weight, causal, group_size, fill_upper=True, grad_fill_upper=True):
+    def forward(ctx, x, weight, causal, group_size, fill_upper=True, grad_fill_upper=True, key_bias=None):
+        # (key_bias: fp32 (B,Sk) added to the mixed scores, 0 or -inf per key - a constant: the gradient is the softmax's
+        # own, taken from the stored probabilities, which are 0 at the hidden keys)
         p = ops.headmix_softmax(x, weight, None, causal, group_size=group_size if weight is not None else None,
-                                fill_upper=fill_upper)
+                                fill_upper=fill_upper, key_bias=key_bias)
         ctx.save_for_backward(x if weight is not None else None, weight, p)
         ctx.causal, ctx.group_size, ctx.grad_fill_upper = causal, group_size, grad_fill_upper
         return p
@@ -220,7 +222,7 @@ class _MixSoftmax(torch.autograd.Function):
         ds = ops.softmax_bwd(p, grad_output.to(p.dtype), ctx.causal,
                              fill_upper=weight is None and ctx.grad_fill_upper)
         if weight is None:
-            return ds, None, None, None, None, None
+            return ds, None, None, None, None, None, None
         dx = dw = None
         if ctx.needs_input_grad[0]:
             dx = ops.headmix_bwd_input(ds, weight, ctx.causal, ctx.group_size, fill_upper=ctx.grad_fill_upper)
@@ -230,7 +232,7 @@ class _MixSoftmax(torch.autograd.Function):
                 blk = torch.arange(weight.shape[0], device=weight.device) // ctx.group_size
                 dw = dw * (blk[:, None] == blk[None, :])
             dw = dw.to(weight.dtype)
-        return dx, dw, None, None, None, None
+        return dx, dw, None, None, None, None, None
 
 
 @dataclass
@@ -446,10 +448,20 @@ class MTAAttentionTriton(nn.Module):
         self._mark("end")
         return output.transpose(1, 2)
 
-    def _forward_stagewise(self, xq, xk, xv):
+    def _forward_stagewise(self, xq, xk, xv, key_bias=None):
         """The reference's own sequence of operators (mta_attention_triton.py:68-92), each differentiable: taken
         whenever a gradient may be asked for.  No weight structure is assumed here, so every entry of the four
-        weights receives its gradient."""
+        weights receives its gradient.
+
+        ``key_bias`` (fp32 (B,Sk), 0 / -inf per key, or finite values of a 2-D additive mask): "causal rule + hidden
+        keys" under use_mask (mta_attention_triton.py:72-73, 77, 81-83).  The K and V rows of the hidden keys are zeroed
+        (differentiably: those rows receive no gradient, as in the reference, whose masked_fill / where cut it): the
+        scores of their columns then enter the pre-softmax conv as 0, the bias hides them from the softmax, and what the
+        post-softmax conv writes into their columns meets zero V rows - and receives a zero gradient from them."""
+        if key_bias is not None:
+            hidden = (key_bias == float("-inf"))[:, None, :, None]
+            xk = xk.masked_fill(hidden, 0)
+            xv = xv.masked_fill(hidden, 0)
         scale = float(torch.rsqrt(torch.tensor(float(xq.size(-1)))))
         scores = _ScaledScoresConv.apply(xq, xk, self.mta_conv_triton.weight, scale, self.causal, self._mark)
         group = self.wpsm_triton.group_size
@@ -458,15 +470,19 @@ class MTAAttentionTriton(nn.Module):
         # so nothing is written there: only the last stage's output, which torch's GEMM reads in full, and the score
         # gradient that goes into torch's GEMMs (inside _ScaledScoresConv) are filled.
         lower = not self.causal   # value of the fill flags: False (leave alone) when causal
-        if _one_pass_group(group or self.n_heads, scores.dtype, xk.size(-2), w_pre):
+        g_eff = group or self.n_heads
+        # (the matrix-core variant for groups of 16 takes a key bias in its row-list form only)
+        bias_ok = key_bias is None or g_eff <= _FUSED_MAX_GROUP or (
+            g_eff == _FUSED_MFMA_GROUP and os.environ.get("MTA_MIX16_NO_ROW_LISTS") != "1")
+        if _one_pass_group(g_eff, scores.dtype, xk.size(-2), w_pre) and bias_ok:
             self._mark("mix_softmax")
-            scores = _MixSoftmax.apply(scores, w_pre, self.causal, group, lower, lower)
+            scores = _MixSoftmax.apply(scores, w_pre, self.causal, group, lower, lower, key_bias)
         else:
             self._mark("mix_pre")
             scores = TritonLinearHeadFunction.apply(scores, w_pre, self.wpsm_triton.causal, self.wpsm_triton.output_value,
                                                     group, lower, lower)
             self._mark("softmax")
-            scores = _MixSoftmax.apply(scores, None, self.causal, None, lower, lower)
+            scores = _MixSoftmax.apply(scores, None, self.causal, None, lower, lower, key_bias)
         self._mark("conv_post")
         scores = Conv2dTritonFunction.apply(scores, self.mta_conv_after_sm_triton.weight, self.causal, lower, lower)
         self._mark("mix_post")
@@ -540,16 +556,19 @@ class MTAAttentionTriton(nn.Module):
         pre-softmax conv as 0 -- which is what a zero K row produces -- its mixed score gets -inf ahead of the softmax
         (the kernel's per-key bias), its probability is 0, and whatever the post-softmax conv writes into its column,
         which the reference zeroes, meets a zero V row."""
-        if self.causal and not wants_grad and xq.size(-2) == xk.size(-2):
+        if self.causal and xq.size(-2) == xk.size(-2):
+            # (with a gradient wanted: the same masks through the differentiable operators - "hidden keys" as a key bias
+            # and zeroed K and V rows there too; a band mask takes the composite below)
+            hidden_keys = self._forward_stagewise_hidden_keys if wants_grad else self._forward_hidden_keys
             if not isinstance(mask, torch.Tensor):
-                return self._forward_fused(xq, xk, xv)
+                return self._forward_stagewise(xq, xk, xv) if wants_grad else self._forward_fused(xq, xk, xv)
             if mask.dim() == 2 and xq.size(0) == 1:
                 assert mask.size(0) == xq.size(0)
                 if mask.dtype == torch.bool:
                     bias = torch.where(mask, 0.0, float("-inf")).to(torch.float32)
                 else:
                     bias = mask.type(xq.dtype).to(torch.float32)   # the reference adds it in the I/O dtype
-                return self._forward_hidden_keys(xq, xk, xv, bias.contiguous())
+                return hidden_keys(xq, xk, xv, bias.contiguous())
             # a 4-D mask, the same for all heads, of one of two forms goes into the kernels without a (B,H,S,S) tensor:
             # "causal rule + hidden keys" per batch entry (key padding: a key bias and zeroed K and V rows, as for the
             # 2-D mask above) and "row p sees the keys first[p] .. p" (sliding windows, packed documents: one int32 per
@@ -557,8 +576,8 @@ class MTAAttentionTriton(nn.Module):
             if mask.dim() == 4:
                 kind, what = self._structured_mask(mask, xq.size(0), xq.size(-2))
                 if kind == "keys":
-                    return self._forward_hidden_keys(xq, xk, xv, what)
-                if kind == "band" and ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight):
+                    return hidden_keys(xq, xk, xv, what)
+                if kind == "band" and not wants_grad and ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight):
                     return self._forward_fused(xq, xk, xv, first_visible=what)
         mask = self._update_mask(mask=mask, bsz=xq.size(0), xq=xq, xk_size=xk.size(-2))
         scale = float(torch.rsqrt(torch.tensor(float(xq.size(-1)))))  # a host scalar: the product stays one vectorised pass
@@ -573,6 +592,9 @@ class MTAAttentionTriton(nn.Module):
         scores = self.wposm_triton(scores)
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         return torch.matmul(scores, xv).transpose(1, 2)
+
+    def _forward_stagewise_hidden_keys(self, xq, xk, xv, bias):
+        return self._forward_stagewise(xq, xk, xv, key_bias=bias)
 
     def _forward_hidden_keys(self, xq, xk, xv, bias):
         """The fused route under "causal rule + one additive value per (batch entry, key)" (``bias``: fp32 (B,S)).  The K

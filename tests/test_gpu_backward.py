@@ -552,6 +552,55 @@ def test_mta_module_backward_key_mask_16bit(pkg):
     _check_all(dtype, out, want_out, gin + gw, want_in + want_w)
 
 
+@pytest.mark.parametrize("case", [(3, 4, 264, 64, 3, 5, torch.bfloat16), (2, 16, 520, 128, 6, 11, torch.float16),
+                                  (2, 8, 200, 64, 7, 7, torch.float32)])
+def test_mta_module_backward_right_padded_batch(pkg, case):
+    """Training under key padding for B > 1 (a (B,1,S,S) boolean mask: causal rule + hidden keys per batch entry): the mask
+    is recognised and the differentiable operators run with a key bias and zeroed K and V rows - the first stage is the
+    scores kernel, not a composite over (B,H,S,S) mask tensors.  All seven gradients against autograd through the oracle
+    given the mask tensor; the K and V rows of the padding receive exactly zero."""
+    b, h, s, d, r1, s1, dtype = case
+    print(f"mta module backward right padding {case}", flush=True)
+    mod, params = _mta_pair(pkg, h, r1, s1, dtype, seed=361)
+    mod.use_mask = True
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=362)
+    lengths = torch.tensor([s, s - s // 3, 41][:b])
+    keep = torch.arange(s)[None, :] < lengths[:, None]
+    visible = keep[:, None, None, :] & torch.tril(torch.ones(s, s, dtype=torch.bool))[None, None]
+    go = _rand((b, s, h, d), 363, dtype)
+    go = go * keep[:, :, None, None]   # (the padding rows' outputs are nobody's business)
+    want_out, want_in, want_w = _oracle_grads(q, k, v, params, go, mask=visible.expand(b, h, s, s))
+    stages = []
+    mod._stage_hook = stages.append
+    out, gin, gw = _module_grads(mod, q, k, v, go, mask=visible)
+    if (r1, s1, d) == (6, 11, 128):   # (a size the scores kernel is built for)
+        assert "qk_conv" in stages, stages
+    assert "pv" in stages and ("mix_softmax" in stages or "softmax" in stages), stages
+    real = keep[:, None, :, None]
+    _check_all(dtype, out.cpu() * keep[:, :, None, None], want_out * keep[:, :, None, None], [g.cpu() for g in gin + gw], want_in + want_w)
+    for name, g in (("xk", gin[1]), ("xv", gin[2])):
+        assert not (g.cpu() * ~real).any(), f"grad {name} of a hidden key is not zero"
+
+
+def test_mta_module_backward_key_mask_finite_values(pkg):
+    """A 2-D additive key mask with finite values besides -inf (B = 1), in training: the values are added ahead of the
+    softmax (mta_attention_triton.py:77), only -inf hides a key."""
+    print("mta module backward additive key mask", flush=True)
+    dtype = torch.bfloat16
+    b, h, s, d = 1, 8, 264, 64
+    mod, params = _mta_pair(pkg, h, 3, 5, dtype, seed=371)
+    mod.use_mask = True
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=372)
+    mask = torch.zeros(1, s)
+    mask[0, 10:14] = float("-inf")
+    mask[0, 100:120] = -1.5
+    mask[0, 200] = 0.75
+    go = _rand((b, s, h, d), 373, dtype)
+    want_out, want_in, want_w = _oracle_grads(q, k, v, params, go, mask=mask.to(dtype))
+    out, gin, gw = _module_grads(mod, q, k, v, go, mask=mask.to(dtype))
+    _check_all(dtype, out.cpu(), want_out, [g.cpu() for g in gin + gw], want_in + want_w)
+
+
 def test_mta_module_backward_with_dropout(pkg, monkeypatch):
     """Training mode with dropout 0.5 under a fixed seed.  The gradient with respect to the probabilities comes from the
     scores kernel, which writes nothing above the diagonal; the dropout's backward multiplies that buffer elementwise
