@@ -90,7 +90,7 @@ _CONV_MIX16_SIZES = ((3, 3), (5, 5), (7, 7))
 _IDENTITY_KERNELS = {}
 
 
-def _lower_scores(a: torch.Tensor, b: torch.Tensor) -> Optional[torch.Tensor]:
+def _lower_scores(a: torch.Tensor, b: torch.Tensor, first_visible: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """round(a b^T) on and below the diagonal of a (B,H,S,S) tensor, nothing written above it, for consumers that
     never read there: the scores kernel (``mta_qk_conv_fwd``) with factor 1 and a 3x3 kernel that is the pass-through
     tap, which copies its input exactly.  Half the output traffic of the library GEMM.  None where that kernel does not
@@ -104,7 +104,12 @@ def _lower_scores(a: torch.Tensor, b: torch.Tensor) -> Optional[torch.Tensor]:
         w = torch.zeros(h, 3, 3, dtype=a.dtype, device=a.device)
         w[:, 2, 1] = 1.0
         _IDENTITY_KERNELS[key] = w
-    return ops.qk_conv(a, b, w, True, 1.0, fill_upper=False)
+    out = ops.qk_conv(a, b, w, True, 1.0, fill_upper=False, first_visible=first_visible)
+    if out is not None and first_visible is not None:
+        # a band mask: the products ahead of a row's first visible key count as 0.  The kernel does not visit the key
+        # blocks that no row of a query block sees: the hidden stretch of every row is cleared afterwards.
+        out = ops.band_zero_(out, first_visible)
+    return out
 
 
 class _ProbsTimesValues(torch.autograd.Function):
@@ -115,25 +120,30 @@ class _ProbsTimesValues(torch.autograd.Function):
     head sizes) the caller has filled P and the library GEMMs run."""
 
     @staticmethod
-    def forward(ctx, p, v, lower):
-        ctx.save_for_backward(p, v)
+    def forward(ctx, p, v, lower, first_visible=None):
+        # (first_visible: a band mask, P is 0 ahead of every row's first visible key; needs ``lower``.  The gradient with
+        # respect to P is then formed inside the band only: 0 at the hidden positions, where the reference's
+        # ``torch.where(mask == -inf, 0.0, scores)`` cuts it)
+        assert first_visible is None or lower
+        ctx.save_for_backward(p, v, first_visible)
         ctx.lower = lower
-        out = ops.causal_pv(p, v, True) if lower else None
+        out = ops.causal_pv(p, v, True, first_visible=first_visible) if lower else None
         return out if out is not None else torch.matmul(p, v)
 
     @staticmethod
     def backward(ctx, grad_output):
-        p, v = ctx.saved_tensors
+        p, v, first_visible = ctx.saved_tensors
         dp = dv = None
         if ctx.needs_input_grad[0]:
-            dp = _lower_scores(grad_output, v) if ctx.lower else None
+            dp = _lower_scores(grad_output, v, first_visible) if ctx.lower else None
             if dp is None:
+                assert first_visible is None
                 dp = torch.matmul(grad_output, v.transpose(2, 3))
         if ctx.needs_input_grad[1]:
             dv = ops.causal_ptx(p, grad_output.contiguous(), True) if ctx.lower else None
             if dv is None:
                 dv = torch.matmul(p.transpose(2, 3), grad_output)
-        return dp, dv, None
+        return dp, dv, None, None
 
 
 def _lower_products_supported(x: torch.Tensor, s_keys: int) -> bool:
@@ -154,15 +164,24 @@ class _ScaledScoresConv(torch.autograd.Function):
     factor."""
 
     @staticmethod
-    def forward(ctx, xq, xk, weight, scale, causal, mark):
-        ctx.scale, ctx.causal = scale, causal
+    def forward(ctx, xq, xk, weight, scale, causal, mark, first_visible=None):
+        # (first_visible: a band mask, applied to the scores ahead of the conv (mta_attention_triton.py:72-73) inside the
+        # one kernel, which the caller has checked exists; backward: the conv's input gradient is zeroed at the hidden
+        # positions, the raw scores for the kernel gradient are recomputed inside the band)
+        ctx.scale, ctx.causal, ctx.first_visible = scale, causal, first_visible
         # (the stage that follows, head mixing or mixing + softmax, never reads above the diagonal)
         if ops.qk_conv_supported(xq, xk, weight):
             mark("qk_conv")
-            out = ops.qk_conv(xq, xk, weight, causal, scale, fill_upper=False)
+            out = ops.qk_conv(xq, xk, weight, causal, scale, fill_upper=False, first_visible=first_visible)
+            if out is not None and first_visible is not None:
+                # The kernel leaves the key blocks that no row of a query block sees unwritten.  The softmax stage does not
+                # read a row's hidden stretch, but its weight gradient multiplies what is stored there by a gradient that
+                # is 0: the stretch is cleared, so that the product is 0 too.
+                out = ops.band_zero_(out, first_visible)
             if out is not None:
                 ctx.save_for_backward(xq, xk, weight, None)
                 return out
+        assert first_visible is None, "the band mask needs the one-kernel first stage"
         mark("qk")
         raw = torch.matmul(xq, xk.transpose(2, 3))
         mark("conv_pre")
@@ -176,6 +195,10 @@ class _ScaledScoresConv(torch.autograd.Function):
         if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
             lower = ctx.causal and xq.shape == xk.shape and _lower_products_supported(xq, xk.size(-2))
             g = ops.conv2d_bwd_input(grad_output, weight, ctx.causal, fill_upper=not lower)
+            if ctx.first_visible is not None:
+                assert lower
+                if ops.band_zero_(g, ctx.first_visible) is None:
+                    raise RuntimeError("band masks need 16-bit scores of a length that is a multiple of 8")
             if ctx.needs_input_grad[0]:
                 dq = ops.causal_pv(g, xk, True) if lower else None
                 if dq is None:
@@ -190,12 +213,32 @@ class _ScaledScoresConv(torch.autograd.Function):
                 dk = dk * ctx.scale
         if ctx.needs_input_grad[2]:
             if raw is None:  # (the kernel gradient reads its first argument on and below the diagonal only)
-                raw = _lower_scores(xq, xk) if ctx.causal else None
+                raw = _lower_scores(xq, xk, ctx.first_visible) if ctx.causal else None
                 if raw is None:
+                    assert ctx.first_visible is None
                     raw = torch.matmul(xq, xk.transpose(2, 3))
             dw = ops.conv2d_bwd_weight(raw, grad_output.to(raw.dtype), tuple(weight.shape[1:]), ctx.causal)
             dw = (dw * ctx.scale).to(weight.dtype)
-        return dq, dk, dw, None, None, None
+        return dq, dk, dw, None, None, None, None
+
+
+class _BandZero(torch.autograd.Function):
+    """x[b,h,p,q] = 0 for q < first_visible[b,p], in place: what ``torch.where(mask == -inf, 0.0, scores)`` behind the
+    post-softmax conv does under a band mask (mta_attention_triton.py:82-83).  Its gradient would be the same zeroing;
+    here the gradient that arrives is zero at those positions already - the gradient with respect to the probabilities
+    is formed inside the band only (``_ProbsTimesValues``) and what lies between, dropout and head mixing, acts per
+    position - so it is handed on as it is."""
+
+    @staticmethod
+    def forward(ctx, x, first_visible):
+        if ops.band_zero_(x, first_visible) is None:
+            raise RuntimeError("band masks need 16-bit scores of a length that is a multiple of 8")
+        ctx.mark_dirty(x)
+        return x
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return grad_output, None
 
 
 class _MixSoftmax(torch.autograd.Function):
@@ -206,11 +249,12 @@ class _MixSoftmax(torch.autograd.Function):
     two gradient kernels."""
 
     @staticmethod
-    def forward(ctx, x, weight, causal, group_size, fill_upper=True, grad_fill_upper=True, key_bias=None):
-        # (key_bias: fp32 (B,Sk) added to the mixed scores, 0 or -inf per key - a constant: the gradient is the softmax's
-        # own, taken from the stored probabilities, which are 0 at the hidden keys)
+    def forward(ctx, x, weight, causal, group_size, fill_upper=True, grad_fill_upper=True, key_bias=None,
+                first_visible=None):
+        # (key_bias: fp32 (B,Sk) added to the mixed scores, 0 or -inf per key; first_visible: int32 (B,S), a band mask.
+        # Constants: the gradient is the softmax's own, taken from the stored probabilities, which are 0 at what is hidden)
         p = ops.headmix_softmax(x, weight, None, causal, group_size=group_size if weight is not None else None,
-                                fill_upper=fill_upper, key_bias=key_bias)
+                                fill_upper=fill_upper, key_bias=key_bias, first_visible=first_visible)
         ctx.save_for_backward(x if weight is not None else None, weight, p)
         ctx.causal, ctx.group_size, ctx.grad_fill_upper = causal, group_size, grad_fill_upper
         return p
@@ -222,7 +266,7 @@ class _MixSoftmax(torch.autograd.Function):
         ds = ops.softmax_bwd(p, grad_output.to(p.dtype), ctx.causal,
                              fill_upper=weight is None and ctx.grad_fill_upper)
         if weight is None:
-            return ds, None, None, None, None, None, None
+            return ds, None, None, None, None, None, None, None
         dx = dw = None
         if ctx.needs_input_grad[0]:
             dx = ops.headmix_bwd_input(ds, weight, ctx.causal, ctx.group_size, fill_upper=ctx.grad_fill_upper)
@@ -232,7 +276,7 @@ class _MixSoftmax(torch.autograd.Function):
                 blk = torch.arange(weight.shape[0], device=weight.device) // ctx.group_size
                 dw = dw * (blk[:, None] == blk[None, :])
             dw = dw.to(weight.dtype)
-        return dx, dw, None, None, None, None, None
+        return dx, dw, None, None, None, None, None, None
 
 
 @dataclass
@@ -448,7 +492,7 @@ class MTAAttentionTriton(nn.Module):
         self._mark("end")
         return output.transpose(1, 2)
 
-    def _forward_stagewise(self, xq, xk, xv, key_bias=None):
+    def _forward_stagewise(self, xq, xk, xv, key_bias=None, first_visible=None):
         """The reference's own sequence of operators (mta_attention_triton.py:68-92), each differentiable: taken
         whenever a gradient may be asked for.  No weight structure is assumed here, so every entry of the four
         weights receives its gradient.
@@ -457,13 +501,19 @@ class MTAAttentionTriton(nn.Module):
         keys" under use_mask (mta_attention_triton.py:72-73, 77, 81-83).  The K and V rows of the hidden keys are zeroed
         (differentiably: those rows receive no gradient, as in the reference, whose masked_fill / where cut it): the
         scores of their columns then enter the pre-softmax conv as 0, the bias hides them from the softmax, and what the
-        post-softmax conv writes into their columns meets zero V rows - and receives a zero gradient from them."""
+        post-softmax conv writes into their columns meets zero V rows - and receives a zero gradient from them.
+
+        ``first_visible`` (int32 (B,S)): a band mask, row p sees the keys first_visible[p] .. p.  Applied where the
+        reference applies the mask tensor: to the scores ahead of the pre-softmax conv (inside the scores kernel), as
+        -inf inside the softmax kernel, and as zeros behind the post-softmax conv; the caller has checked that the
+        kernels this needs exist (``_band_training_supported``)."""
         if key_bias is not None:
             hidden = (key_bias == float("-inf"))[:, None, :, None]
             xk = xk.masked_fill(hidden, 0)
             xv = xv.masked_fill(hidden, 0)
         scale = float(torch.rsqrt(torch.tensor(float(xq.size(-1)))))
-        scores = _ScaledScoresConv.apply(xq, xk, self.mta_conv_triton.weight, scale, self.causal, self._mark)
+        scores = _ScaledScoresConv.apply(xq, xk, self.mta_conv_triton.weight, scale, self.causal, self._mark,
+                                         first_visible)
         group = self.wpsm_triton.group_size
         w_pre = self.wpsm_triton.weight
         # Between two of these stages nothing reads above the diagonal (causal kernels never do, in either direction),
@@ -472,19 +522,21 @@ class MTAAttentionTriton(nn.Module):
         lower = not self.causal   # value of the fill flags: False (leave alone) when causal
         g_eff = group or self.n_heads
         # (the matrix-core variant for groups of 16 takes a key bias in its row-list form only)
-        bias_ok = key_bias is None or g_eff <= _FUSED_MAX_GROUP or (
+        bias_ok = (key_bias is None and first_visible is None) or g_eff <= _FUSED_MAX_GROUP or (
             g_eff == _FUSED_MFMA_GROUP and os.environ.get("MTA_MIX16_NO_ROW_LISTS") != "1")
         if _one_pass_group(g_eff, scores.dtype, xk.size(-2), w_pre) and bias_ok:
             self._mark("mix_softmax")
-            scores = _MixSoftmax.apply(scores, w_pre, self.causal, group, lower, lower, key_bias)
+            scores = _MixSoftmax.apply(scores, w_pre, self.causal, group, lower, lower, key_bias, first_visible)
         else:
             self._mark("mix_pre")
             scores = TritonLinearHeadFunction.apply(scores, w_pre, self.wpsm_triton.causal, self.wpsm_triton.output_value,
                                                     group, lower, lower)
             self._mark("softmax")
-            scores = _MixSoftmax.apply(scores, None, self.causal, None, lower, lower, key_bias)
+            scores = _MixSoftmax.apply(scores, None, self.causal, None, lower, lower, key_bias, first_visible)
         self._mark("conv_post")
         scores = Conv2dTritonFunction.apply(scores, self.mta_conv_after_sm_triton.weight, self.causal, lower, lower)
+        if first_visible is not None:
+            scores = _BandZero.apply(scores, first_visible)
         self._mark("mix_post")
         post = self.wposm_triton
         # the last stage's output is read by P V: in full by the library GEMM, on and below the diagonal by our kernels
@@ -496,7 +548,8 @@ class MTAAttentionTriton(nn.Module):
         self._mark("pv")
         # (the gradient with respect to the probabilities goes back into the head mixing's gradient kernels, through the
         # dropout's elementwise mask at most: nothing there reads above the diagonal when causal)
-        output = _ProbsTimesValues.apply(scores, xv, lower_pv)
+        assert first_visible is None or lower_pv
+        output = _ProbsTimesValues.apply(scores, xv, lower_pv, first_visible)
         self._mark("end")
         return output.transpose(1, 2)
 
@@ -557,8 +610,7 @@ class MTAAttentionTriton(nn.Module):
         (the kernel's per-key bias), its probability is 0, and whatever the post-softmax conv writes into its column,
         which the reference zeroes, meets a zero V row."""
         if self.causal and xq.size(-2) == xk.size(-2):
-            # (with a gradient wanted: the same masks through the differentiable operators - "hidden keys" as a key bias
-            # and zeroed K and V rows there too; a band mask takes the composite below)
+            # (with a gradient wanted: the same masks through the differentiable operators)
             hidden_keys = self._forward_stagewise_hidden_keys if wants_grad else self._forward_hidden_keys
             if not isinstance(mask, torch.Tensor):
                 return self._forward_stagewise(xq, xk, xv) if wants_grad else self._forward_fused(xq, xk, xv)
@@ -577,8 +629,11 @@ class MTAAttentionTriton(nn.Module):
                 kind, what = self._structured_mask(mask, xq.size(0), xq.size(-2))
                 if kind == "keys":
                     return hidden_keys(xq, xk, xv, what)
-                if kind == "band" and not wants_grad and ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight):
-                    return self._forward_fused(xq, xk, xv, first_visible=what)
+                if kind == "band" and ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight):
+                    if not wants_grad:
+                        return self._forward_fused(xq, xk, xv, first_visible=what)
+                    if self._band_training_supported(xq, xk, xv):
+                        return self._forward_stagewise(xq, xk, xv, first_visible=what)
         mask = self._update_mask(mask=mask, bsz=xq.size(0), xq=xq, xk_size=xk.size(-2))
         scale = float(torch.rsqrt(torch.tensor(float(xq.size(-1)))))  # a host scalar: the product stays one vectorised pass
         scores = torch.matmul(xq, xk.transpose(2, 3)) * scale
@@ -592,6 +647,16 @@ class MTAAttentionTriton(nn.Module):
         scores = self.wposm_triton(scores)
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         return torch.matmul(scores, xv).transpose(1, 2)
+
+    def _band_training_supported(self, xq, xk, xv) -> bool:
+        """Whether the differentiable route takes a band mask: 16-bit data of one dtype, a length the in-place zeroing
+        kernel takes, and the lower-triangle products (P V and its gradients, the recomputed raw scores) as kernels."""
+        s = xk.size(-2)
+        return (xq.dtype in (torch.bfloat16, torch.float16) and xq.dtype == xk.dtype == xv.dtype
+                and xq.shape == xk.shape and s % 8 == 0 and _lower_products_supported(xv, s)
+                and _lower_products_supported(xq, s)
+                and all(w.dtype == xq.dtype for w in (self.mta_conv_triton.weight, self.mta_conv_after_sm_triton.weight,
+                                                      self.wpsm_triton.weight, self.wposm_triton.weight)))
 
     def _forward_stagewise_hidden_keys(self, xq, xk, xv, bias):
         return self._forward_stagewise(xq, xk, xv, key_bias=bias)

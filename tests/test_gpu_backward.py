@@ -471,6 +471,16 @@ def test_lower_scores_is_the_rounded_product(pkg, d, dtype):
     out = pkg.ops.qk_conv(a.cuda(), c.cuda(), w.cuda(), True, 1.0, fill_upper=False, out=buf)
     assert out is buf and torch.equal(buf.cpu()[..., low], got[..., low])
 
+    # under a band mask: the same products inside the band, exact zeros ahead of it - also where the kernel skips whole
+    # key blocks (a window much shorter than the rows)
+    rows = torch.arange(s)
+    first = (rows - 70).clamp(min=0).to(torch.int32)
+    first[300:] = 290
+    got_band = _lower_scores(a.cuda(), c.cuda(), first[None].expand(b, s).contiguous().cuda()).cpu()
+    inside = low & (torch.arange(s)[None, :] >= first[:, None])
+    assert torch.equal(got_band[..., inside], got[..., inside])
+    assert not got_band[..., low & ~inside].any()
+
 
 def _oracle_grads(q, k, v, params, go, mask=None):
     leaves = [t.detach().clone().float().requires_grad_(True) for t in (q, k, v)]
@@ -582,6 +592,56 @@ def test_mta_module_backward_right_padded_batch(pkg, case):
         assert not (g.cpu() * ~real).any(), f"grad {name} of a hidden key is not zero"
 
 
+def _band_masks(s):
+    rows = torch.arange(s)
+    lower = rows[None, :] <= rows[:, None]
+    window = lower & (rows[:, None] - rows[None, :] < 37)
+    starts = torch.tensor([0, 50, 51, 130, s - 3])
+    doc = (rows[:, None] >= starts[None, :]).sum(-1) - 1          # document of every position
+    documents = lower & (doc[:, None] == doc[None, :])
+    return {"window": window, "documents": documents}
+
+
+@pytest.mark.parametrize("kind", ["window", "documents"])
+@pytest.mark.parametrize("case", [(2, 4, 264, 64, 3, 3, torch.bfloat16), (1, 16, 520, 128, 6, 11, torch.float16),
+                                  (2, 8, 200, 64, 7, 7, torch.bfloat16)])
+def test_mta_module_backward_band_masks(pkg, case, kind):
+    """Training under band masks (sliding window, packed documents; a (1,1,S,S) boolean mask): recognised as "row p
+    sees first[p] .. p" and run through the differentiable kernel operators - the mask inside the scores kernel and the
+    softmax kernel, zeros behind the post-softmax conv, the gradient with respect to the probabilities and the recomputed
+    raw scores formed inside the band, the conv's input gradient zeroed outside it.  All seven gradients against autograd
+    through the oracle given the mask tensor."""
+    b, h, s, d, r1, s1, dtype = case
+    print(f"mta module backward band mask {kind} {case}", flush=True)
+    mod, params = _mta_pair(pkg, h, r1, s1, dtype, seed=381)
+    mod.use_mask = True
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=382)
+    visible = _band_masks(s)[kind][None, None]
+    go = _rand((b, s, h, d), 383, dtype)
+    want_out, want_in, want_w = _oracle_grads(q, k, v, params, go, mask=visible)
+    stages = []
+    mod._stage_hook = stages.append
+    out, gin, gw = _module_grads(mod, q, k, v, go, mask=visible)
+    assert "qk_conv" in stages and "conv_post" in stages and "pv" in stages, stages
+    _check_all(dtype, out.cpu(), want_out, [g.cpu() for g in gin + gw], want_in + want_w)
+
+
+def test_mta_module_backward_band_mask_without_the_kernels_takes_the_composite(pkg):
+    """fp32 under a band mask in training: no in-place zeroing kernel, no lower-triangle products - the composite over the
+    mask tensor runs, with the same answers."""
+    print("mta module backward band mask fp32", flush=True)
+    dtype = torch.float32
+    b, h, s, d = 1, 4, 72, 64
+    mod, params = _mta_pair(pkg, h, 3, 3, dtype, seed=391)
+    mod.use_mask = True
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=392)
+    visible = _band_masks(s)["window"][None, None]
+    go = _rand((b, s, h, d), 393, dtype)
+    want_out, want_in, want_w = _oracle_grads(q, k, v, params, go, mask=visible)
+    out, gin, gw = _module_grads(mod, q, k, v, go, mask=visible)
+    _check_all(dtype, out.cpu(), want_out, [g.cpu() for g in gin + gw], want_in + want_w)
+
+
 def test_mta_module_backward_key_mask_finite_values(pkg):
     """A 2-D additive key mask with finite values besides -inf (B = 1), in training: the values are added ahead of the
     softmax (mta_attention_triton.py:77), only -inf hides a key."""
@@ -627,7 +687,7 @@ def test_mta_module_backward_with_dropout(pkg, monkeypatch):
     for t in [out1] + gin1 + gw1:
         assert torch.isfinite(t.float()).all()
     assert float((out1 == 0).float().mean()) < 0.5   # (dropout acts on the probabilities, not on the output)
-    monkeypatch.setattr(glue, "_lower_scores", lambda a, c: None)
+    monkeypatch.setattr(glue, "_lower_scores", lambda a, c, first_visible=None: None)
     out2, gin2, gw2 = run()
     assert torch.equal(out1, out2)                   # same seed, same dropout mask
     for name, a_, c_ in zip(_GRAD_NAMES, gin1 + gw1, gin2 + gw2):
