@@ -373,6 +373,24 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
         "ms": ms,
         "note": "forward + backward; the reference's published row for this shape (Triton 39.090 ms, PyTorch 253.350 ms, "
                 "hardware unstated) is context, not a baseline"}
+    # ... and the same training step under mask tensors (use_mask=True): a sliding window of 1024 keys and a key-padding
+    # mask, both recognised and run through the same differentiable kernel operators
+    mod.use_mask = True
+    s_len = sets[0][0].size(2)
+    pos = torch.arange(s_len, device=device)
+    lower = pos[None, :] <= pos[:, None]
+    masks = {"window1024_mask": (lower & (pos[None, :] > pos[:, None] - 1024))[None, None],
+             "key_padding_mask": ((pos < 3000)[None, :] & lower)[None, None]}
+    for name, mask in masks.items():
+        def masked_step(i, mask=mask):
+            for t in params + list(sets[i]):
+                t.grad = None
+            with torch.enable_grad():
+                mod(*sets[i], mask, None).backward(gout)
+
+        ms = time_steps(torch, masked_step, len(sets), min(warmup, 5), max(3, steps // 10))
+        out["mta_forward_backward_general_fp16_1x16x4096x128_7x7_pre_post_dense_" + name] = {
+            "ms": ms, "note": "forward + backward with use_mask=True and a mask tensor; not a row of the reference's"}
     return out
 
 

@@ -33,7 +33,13 @@ triton_linear_head); the 1/sqrt(D) factor folded into the pre-softmax conv and, 
 backward, into the (B,H,S,D) gradients of Q and K; pre-softmax head mixing and softmax as
 one forward kernel where the inference route has one, with the softmax gradient taken from
 the stored 16-bit probabilities (``mta_softmax_bwd``; no fp32 copy of the score tensor in
-either direction).  torch differentiates the two GEMMs and the dropout.
+either direction).  Under the causal rule the products around the score tensors (P V, the
+gradients it leaves, the recomputed raw scores) touch the lower triangle only; torch
+differentiates the dropout.  ``use_mask=True`` in training: the same two families of masks
+go through these operators -- hidden keys as a key bias inside the softmax kernel and
+zeroed K and V rows, band masks inside the scores and softmax kernels, with the gradients
+around them formed inside the band; any other mask tensor takes the reference's
+elementwise steps between the single operators.
 
 Weight structure.  By default nothing is assumed about the four weights: every stage runs
 with the dense weight it is given.  Skipping identity stages and applying block-diagonal

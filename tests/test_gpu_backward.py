@@ -642,6 +642,38 @@ def test_mta_module_backward_band_mask_without_the_kernels_takes_the_composite(p
     _check_all(dtype, out.cpu(), want_out, [g.cpu() for g in gin + gw], want_in + want_w)
 
 
+@pytest.mark.parametrize("kind", ["window1024", "key_padding"])
+def test_mta_module_backward_masks_benchmark_shape(pkg, kind):
+    """The training step under mask tensors at the shape the benchmark times it (B1 H16 S4096 D128 fp16, 7x7 kernels,
+    dense head weights), where the oracle on the host is out of reach: the route through the kernel operators against the
+    module's own composite over the (B,H,S,S) mask tensor (torch's operators and the single-stage kernels; the route
+    every mask took before it was recognised, pinned against the oracle at small sizes above), forward and all seven
+    gradients, to the 16-bit bars."""
+    print(f"mta module backward {kind} benchmark shape", flush=True)
+    dtype = torch.float16
+    b, h, s, d = 1, 16, 4096, 128
+    mod, params = _mta_pair(pkg, h, 7, 7, dtype, seed=401)
+    with torch.no_grad():   # a 7x7 post-softmax kernel as well
+        w = O.seeded_conv_weight(h, 7, 7, 0.05, torch.float32, seed=402).to(dtype)
+        mod.mta_conv_after_sm_triton = pkg.Conv2dTriton(h, (7, 7), causal=True).to(dtype).cuda()
+        mod.mta_conv_after_sm_triton.weight.copy_(w)
+    mod.use_mask = True
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=403)
+    pos = torch.arange(s)
+    lower = pos[None, :] <= pos[:, None]
+    visible = (lower & (pos[None, :] > pos[:, None] - 1024)) if kind == "window1024" else (lower & (pos < 3000)[None, :])
+    visible = visible[None, None]
+    go = _rand((b, s, h, d), 404, dtype)
+    stages = []
+    mod._stage_hook = stages.append
+    out, gin, gw = _module_grads(mod, q, k, v, go, mask=visible)
+    assert "qk_conv" in stages, stages
+    mod._stage_hook = None
+    mod._structured_mask = lambda *a: (None, None)     # nothing recognised: the composite
+    want_out, want_in, want_w = _module_grads(mod, q, k, v, go, mask=visible)
+    _check_all(dtype, out.cpu(), want_out.cpu(), [g.cpu() for g in gin + gw], [g.cpu() for g in want_in + want_w])
+
+
 def test_mta_module_backward_key_mask_finite_values(pkg):
     """A 2-D additive key mask with finite values besides -inf (B = 1), in training: the values are added ahead of the
     softmax (mta_attention_triton.py:77), only -inf hides a key."""
