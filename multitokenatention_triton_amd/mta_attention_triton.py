@@ -23,8 +23,10 @@ Inference (no input or parameter requires grad, or grad mode is off):
     (B,H,S,S) tensors);
   * ``use_mask=True``: masks that amount to "the causal rule and hidden keys" (2-D key
     masks, key padding of a batch) or to "row p sees the keys first[p] .. p" (sliding
-    windows, packed documents) go into the same kernels as one value per key or per row;
-    any other mask tensor takes the reference's elementwise steps around the kernels.
+    windows, packed documents) go into the same kernels as one value per key or per row
+    (a ``causal=False`` module: masks that hide the same keys from every row, the key
+    padding of an encoder batch); any other mask tensor takes the reference's elementwise
+    steps around the kernels.
 
 Training (something requires grad): the stages run one by one through autograd
 Functions, as in the reference, so that ``backward()`` works: the two conv and the two
@@ -640,6 +642,14 @@ class MTAAttentionTriton(nn.Module):
                         return self._forward_fused(xq, xk, xv, first_visible=what)
                     if self._band_training_supported(xq, xk, xv):
                         return self._forward_stagewise(xq, xk, xv, first_visible=what)
+        elif (not self.causal and isinstance(mask, torch.Tensor) and mask.dim() == 4 and xq.size(-2) == xk.size(-2)):
+            # no causal rule and a mask that hides the same keys from every row (key padding of an encoder batch): the same
+            # key bias and zeroed K and V rows, through the kernels' non-causal form
+            kind, what = self._structured_mask(mask, xq.size(0), xq.size(-2))
+            if kind == "keys":
+                if wants_grad:
+                    return self._forward_stagewise(xq, xk, xv, key_bias=what)
+                return self._forward_hidden_keys(xq, xk, xv, what)
         mask = self._update_mask(mask=mask, bsz=xq.size(0), xq=xq, xk_size=xk.size(-2))
         scale = float(torch.rsqrt(torch.tensor(float(xq.size(-1)))))  # a host scalar: the product stays one vectorised pass
         scores = torch.matmul(xq, xk.transpose(2, 3)) * scale
@@ -679,7 +689,7 @@ class MTAAttentionTriton(nn.Module):
 
     def _structured_mask(self, mask, bsz: int, s: int):
         """What a 4-D ``mask`` (bool with True = attend, or additive with 0 / -inf; one plane for all heads) amounts to
-        together with the causal rule:
+        together with the causal rule (a module with ``causal=False``: on its own, and only the first form):
           ("keys", bias)   every row sees the kept keys up to itself and key 0 is kept: fp32 (B,S), 0 / -inf per key;
           ("band", first)  row p sees exactly the keys first[p] .. p: int32 (B,S);
           (None, None)     anything else (per-head planes, holes that differ between rows, other finite values, a row
@@ -701,7 +711,13 @@ class MTAAttentionTriton(nn.Module):
             visible = plane == 0
             if not bool(((plane == float("-inf")) | visible).all()):
                 visible = None   # other finite values: not a 0 / -inf mask
-        if same_heads and visible is not None:
+        if same_heads and visible is not None and not self.causal:
+            # no causal rule: "hidden keys" means every row sees the same keys, and at least one
+            keep = visible[:, 0, :]
+            if bool((visible == keep[:, None, :]).all()) and bool(keep.any(-1).all()):
+                bias = torch.where(keep, 0.0, float("-inf")).to(torch.float32).expand(bsz, s).contiguous()
+                answer = ("keys", bias)
+        elif same_heads and visible is not None:
             rows = torch.arange(s, device=mask.device)
             lower = rows[None, :] <= rows[:, None]
             visible = visible & lower

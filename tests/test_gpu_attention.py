@@ -1050,6 +1050,34 @@ def test_mta_use_mask_right_padded_batch(pkg, post):
     torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("post", ["identity", "random"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_mta_non_causal_key_padding(pkg, dtype, post):
+    """MTAAttentionTriton(causal=False, use_mask=True) under key padding of a batch (a (B,1,S,S) boolean mask that hides
+    the same keys from every row): recognised and run through the kernels' non-causal form with a key bias and zeroed K
+    and V rows, no (B,H,S,S) mask tensor; against the oracle given the mask tensor.  A mask that is not of that form (a
+    band) takes the composite."""
+    print(f"mta causal=False key padding {dtype} post={post}", flush=True)
+    b, h, s, d = 3, 4, 264, 64
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=96)
+    params = _config_like(h, 2, 3, 5, 0.1, dtype, post=post)
+    lengths = torch.tensor([264, 200, 31])
+    keep = torch.arange(s)[None, :] < lengths[:, None]
+    visible = keep[:, None, None, :].expand(b, 1, s, s).contiguous()
+    want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3],
+                         mask=visible.expand(b, h, s, s))
+    for structure in ("dense", "infer"):
+        mod = _mta_module(pkg, h, 3, 5, 3, 3, *params, dtype, causal=False, use_mask=True, structure=structure)
+        seen = []
+        classify = mod._structured_mask
+        mod._structured_mask = lambda *a, f=classify: (seen.append(f(*a)) or seen[-1])
+        got = mod(q.cuda(), k.cuda(), v.cuda(), visible.cuda(), None).cpu()
+        assert seen and seen[-1][0] == "keys"
+        torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+    band = ((torch.arange(s)[:, None] - torch.arange(s)[None, :]).abs() <= 9)[None, None]
+    assert classify(band.cuda(), b, s)[0] is None
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_mta_non_causal_module(pkg, dtype):
     """MTAAttentionTriton(causal=False): no masking anywhere -- the oracle with an all-visible mask."""

@@ -674,6 +674,30 @@ def test_mta_module_backward_masks_benchmark_shape(pkg, kind):
     _check_all(dtype, out.cpu(), want_out.cpu(), [g.cpu() for g in gin + gw], [g.cpu() for g in want_in + want_w])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_mta_module_backward_non_causal_key_padding(pkg, dtype):
+    """causal=False, use_mask=True, key padding of a batch, in training: the differentiable operators in their non-causal
+    form with a key bias and zeroed K and V rows; all seven gradients against autograd through the oracle given the mask
+    tensor."""
+    print(f"mta module backward causal=False key padding {dtype}", flush=True)
+    b, h, s, d = 2, 4, 136, 64
+    mod, params = _mta_pair(pkg, h, 3, 5, dtype, seed=411, causal=False)
+    mod.use_mask = True
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=412)
+    keep = torch.arange(s)[None, :] < torch.tensor([136, 77])[:, None]
+    visible = keep[:, None, None, :].expand(b, 1, s, s).contiguous()
+    go = _rand((b, s, h, d), 413, dtype)
+    want_out, want_in, want_w = _oracle_grads(q, k, v, params, go, mask=visible.expand(b, h, s, s))
+    stages = []
+    mod._stage_hook = stages.append
+    out, gin, gw = _module_grads(mod, q, k, v, go, mask=visible)
+    assert "pv" in stages and ("mix_softmax" in stages or "softmax" in stages), stages   # (the operator route's marks)
+    _check_all(dtype, out.cpu(), want_out, [g.cpu() for g in gin + gw], want_in + want_w)
+    real = keep[:, None, :, None]
+    for name, g in (("xk", gin[1]), ("xv", gin[2])):
+        assert not (g.cpu() * ~real).any(), f"grad {name} of a hidden key is not zero"
+
+
 def test_mta_module_backward_key_mask_finite_values(pkg):
     """A 2-D additive key mask with finite values besides -inf (B = 1), in training: the values are added ahead of the
     softmax (mta_attention_triton.py:77), only -inf hides a key."""
