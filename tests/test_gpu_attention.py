@@ -1050,6 +1050,46 @@ def test_mta_use_mask_right_padded_batch(pkg, post):
     torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("kind", ["key_padding", "window"])
+def test_mta_use_mask_probe_mode_follows_a_weight_rewrite(pkg, kind):
+    """weight_structure = "probe" on the masked routes: the weights are looked at on every call, so a rewrite behind the
+    module's back (block-diagonal post weights and an identity post conv replaced by dense ones through ``.data``) moves
+    the next masked call from the three-kernel route to the general one, with the oracle's answer before and after."""
+    print(f"mta use_mask probe mode {kind}", flush=True)
+    dtype = torch.bfloat16
+    b, h, s, d = 2, 8, 264, 64
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=97)
+    g = torch.Generator().manual_seed(98)
+    first = [O.seeded_conv_weight(h, 6, 11, 0.05, dtype), torch.eye(h, dtype=dtype),
+             O.identity_conv_kernel(h, 3, 3, dtype), O.block_diag_head_weight(h, 4, 0.1, g, dtype)]
+    second = [O.seeded_conv_weight(h, 6, 11, 0.05, dtype, seed=7),
+              (torch.eye(h) + 0.1 * torch.randn(h, h, generator=g)).to(dtype),
+              O.seeded_conv_weight(h, 3, 3, 0.05, dtype, seed=8),
+              (torch.eye(h) + 0.1 * torch.randn(h, h, generator=g)).to(dtype)]
+    pos = torch.arange(s)
+    lower = pos[None, :] <= pos[:, None]
+    if kind == "key_padding":
+        keep = pos[None, :] < torch.tensor([264, 150])[:, None]
+        visible = keep[:, None, None, :] & lower[None, None]
+    else:
+        visible = (lower & (pos[None, :] > pos[:, None] - 40))[None, None].expand(b, 1, s, s)
+    full = visible.expand(b, h, s, s)
+    mod = _mta_module(pkg, h, 6, 11, 3, 3, *first, dtype, use_mask=True, structure="probe")
+    stages = []
+    mod._stage_hook = stages.append
+    got = mod(q.cuda(), k.cuda(), v.cuda(), visible.cuda(), None).cpu()
+    want = O.mta_forward(q, k, v, first[0].unsqueeze(1), first[1], first[2].unsqueeze(1), first[3], mask=full)
+    torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+    assert stages == ["qk_conv", "mix_softmax_mix", "pv", "end"], stages
+    for dst, src in zip((mod.mta_conv_triton, mod.wpsm_triton, mod.mta_conv_after_sm_triton, mod.wposm_triton), second):
+        dst.weight.data.copy_(src)
+    del stages[:]
+    got = mod(q.cuda(), k.cuda(), v.cuda(), visible.cuda(), None).cpu()
+    want = O.mta_forward(q, k, v, second[0].unsqueeze(1), second[1], second[2].unsqueeze(1), second[3], mask=full)
+    torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+    assert "conv_post" in stages or "conv_mix_post" in stages, stages
+
+
 @pytest.mark.parametrize("post", ["identity", "random"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_mta_non_causal_key_padding(pkg, dtype, post):
