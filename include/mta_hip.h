@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MTA_ABI_VERSION 9
+#define MTA_ABI_VERSION 10
 
 enum mta_dtype { MTA_F32 = 0, MTA_BF16 = 1, MTA_F16 = 2 };
 
@@ -231,6 +231,16 @@ int mta_causal_pv_band_fwd(const void *p, const void *v, const void *first_visib
  * for a band mask, below the diagonal (above it nothing is touched: the causal kernels on either side neither read nor
  * need it).  16-bit I/O, S % 8 == 0; MTA_ERR_UNSUPPORTED otherwise. */
 int mta_band_zero_fwd(void *x, const void *first_visible, int64_t N, int64_t C, int64_t S, int io_dtype, void *stream);
+
+/* y[n,c,p,q] = visible[n,c,p,q] ? x[n,c,p,q] : (neg_inf ? -inf : 0) for a mask tensor of arbitrary content: the
+ * reference's `scores_masked[mask == float("-inf")] = 0` ahead of its two convs, its `scores = scores + mask` ahead of the
+ * softmax for a 0 / -inf mask (neg_inf = 1) and its `torch.where(mask == float("-inf"), 0.0, scores)` behind the
+ * post-softmax conv (mta_attention_triton.py:72-73, 77-78, 81-83), one pass each.  x, y: (N,C,P,Q), y may be x;
+ * visible: uint8, non-zero = attend, (mask_batch, mask_heads, P, Q) with mask_batch 1 or N and mask_heads 1 or C
+ * (broadcast), 8-byte aligned.  causal != 0: only keys q <= p are read and written.  Q % 8 == 0; MTA_ERR_UNSUPPORTED
+ * otherwise. */
+int mta_mask_fill_fwd(const void *x, const void *visible, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
+                      int mask_batch, int mask_heads, int neg_inf, int causal, int io_dtype, void *stream);
 
 /* ---- The three stages of the causal forward (mta_attention_triton.py:68-89 without a post-softmax conv) over
  * score tensors in a TRIANGULAR LAYOUT.  The (B,H,S,S) tensors between the three kernels never leave the library's

@@ -172,11 +172,25 @@ class _ScaledScoresConv(torch.autograd.Function):
     factor."""
 
     @staticmethod
-    def forward(ctx, xq, xk, weight, scale, causal, mark, first_visible=None):
+    def forward(ctx, xq, xk, weight, scale, causal, mark, first_visible=None, mask_planes=None):
         # (first_visible: a band mask, applied to the scores ahead of the conv (mta_attention_triton.py:72-73) inside the
         # one kernel, which the caller has checked exists; backward: the conv's input gradient is zeroed at the hidden
         # positions, the raw scores for the kernel gradient are recomputed inside the band)
-        ctx.scale, ctx.causal, ctx.first_visible = scale, causal, first_visible
+        # (mask_planes: uint8 (1|B, 1|H, S, S), a mask of arbitrary content: the raw scores are written, the hidden ones
+        # zeroed in place, and kept for the kernel gradient; backward zeroes the conv's input gradient at the same positions)
+        ctx.scale, ctx.causal, ctx.first_visible, ctx.mask_planes = scale, causal, first_visible, mask_planes
+        if mask_planes is not None:
+            assert first_visible is None
+            mark("qk")
+            raw = _lower_scores(xq, xk) if causal else None
+            if raw is None:
+                raw = torch.matmul(xq, xk.transpose(2, 3))
+            mark("mask")
+            if ops.mask_fill(raw, mask_planes, False, causal, out=raw) is None:
+                raise RuntimeError("mask planes need a number of keys that is a multiple of 8")
+            mark("conv_pre")
+            ctx.save_for_backward(xq, xk, weight, raw)
+            return ops.conv2d_causal(raw, weight, causal, in_scale=scale, fill_upper=False)
         # (the stage that follows, head mixing or mixing + softmax, never reads above the diagonal)
         if ops.qk_conv_supported(xq, xk, weight):
             mark("qk_conv")
@@ -207,6 +221,8 @@ class _ScaledScoresConv(torch.autograd.Function):
                 assert lower
                 if ops.band_zero_(g, ctx.first_visible) is None:
                     raise RuntimeError("band masks need 16-bit scores of a length that is a multiple of 8")
+            if ctx.mask_planes is not None:
+                ops.mask_fill(g, ctx.mask_planes, False, lower, out=g)
             if ctx.needs_input_grad[0]:
                 dq = ops.causal_pv(g, xk, True) if lower else None
                 if dq is None:
@@ -227,7 +243,31 @@ class _ScaledScoresConv(torch.autograd.Function):
                     raw = torch.matmul(xq, xk.transpose(2, 3))
             dw = ops.conv2d_bwd_weight(raw, grad_output.to(raw.dtype), tuple(weight.shape[1:]), ctx.causal)
             dw = (dw * ctx.scale).to(weight.dtype)
-        return dq, dk, dw, None, None, None, None
+        return dq, dk, dw, None, None, None, None, None
+
+
+class _MaskFill(torch.autograd.Function):
+    """``visible ? x : fill`` in place for uint8 visibility planes (``mta_mask_fill_fwd``).  fill = -inf is the
+    reference's ``scores + mask`` ahead of the softmax (mta_attention_triton.py:77-78): the gradient is handed on as it
+    is, because the softmax that follows returns exactly 0 where its probabilities are 0.  fill = 0 is its
+    ``torch.where(mask == -inf, 0.0, scores)`` behind the post-softmax conv (:82-83): the gradient is zeroed at the same
+    positions, into a tensor of its own."""
+
+    @staticmethod
+    def forward(ctx, x, planes, neg_inf, causal):
+        if ops.mask_fill(x, planes, neg_inf, causal, out=x) is None:
+            raise RuntimeError("mask planes need a number of keys that is a multiple of 8")
+        ctx.mark_dirty(x)
+        ctx.neg_inf, ctx.causal = neg_inf, causal
+        ctx.save_for_backward(planes)
+        return x
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        if ctx.neg_inf:
+            return grad_output, None, None, None
+        planes, = ctx.saved_tensors
+        return ops.mask_fill(grad_output.contiguous(), planes, False, ctx.causal), None, None, None
 
 
 class _BandZero(torch.autograd.Function):
@@ -500,7 +540,7 @@ class MTAAttentionTriton(nn.Module):
         self._mark("end")
         return output.transpose(1, 2)
 
-    def _forward_stagewise(self, xq, xk, xv, key_bias=None, first_visible=None):
+    def _forward_stagewise(self, xq, xk, xv, key_bias=None, first_visible=None, mask_planes=None):
         """The reference's own sequence of operators (mta_attention_triton.py:68-92), each differentiable: taken
         whenever a gradient may be asked for.  No weight structure is assumed here, so every entry of the four
         weights receives its gradient.
@@ -514,14 +554,18 @@ class MTAAttentionTriton(nn.Module):
         ``first_visible`` (int32 (B,S)): a band mask, row p sees the keys first_visible[p] .. p.  Applied where the
         reference applies the mask tensor: to the scores ahead of the pre-softmax conv (inside the scores kernel), as
         -inf inside the softmax kernel, and as zeros behind the post-softmax conv; the caller has checked that the
-        kernels this needs exist (``_band_training_supported``)."""
+        kernels this needs exist (``_band_training_supported``).
+
+        ``mask_planes`` (uint8 (1|B, 1|H, S, S), non-zero = attend): a 0 / -inf mask of arbitrary content.  The three
+        elementwise mask steps of the reference run as in-place passes between the operators (``_MaskFill``, and inside
+        ``_ScaledScoresConv``); head mixing and softmax run as two kernels, the mask goes between them."""
         if key_bias is not None:
             hidden = (key_bias == float("-inf"))[:, None, :, None]
             xk = xk.masked_fill(hidden, 0)
             xv = xv.masked_fill(hidden, 0)
         scale = float(torch.rsqrt(torch.tensor(float(xq.size(-1)))))
         scores = _ScaledScoresConv.apply(xq, xk, self.mta_conv_triton.weight, scale, self.causal, self._mark,
-                                         first_visible)
+                                         first_visible, mask_planes)
         group = self.wpsm_triton.group_size
         w_pre = self.wpsm_triton.weight
         # Between two of these stages nothing reads above the diagonal (causal kernels never do, in either direction),
@@ -532,19 +576,25 @@ class MTAAttentionTriton(nn.Module):
         # (the matrix-core variant for groups of 16 takes a key bias in its row-list form only)
         bias_ok = (key_bias is None and first_visible is None) or g_eff <= _FUSED_MAX_GROUP or (
             g_eff == _FUSED_MFMA_GROUP and os.environ.get("MTA_MIX16_NO_ROW_LISTS") != "1")
-        if _one_pass_group(g_eff, scores.dtype, xk.size(-2), w_pre) and bias_ok:
+        if _one_pass_group(g_eff, scores.dtype, xk.size(-2), w_pre) and bias_ok and mask_planes is None:
             self._mark("mix_softmax")
             scores = _MixSoftmax.apply(scores, w_pre, self.causal, group, lower, lower, key_bias, first_visible)
         else:
             self._mark("mix_pre")
             scores = TritonLinearHeadFunction.apply(scores, w_pre, self.wpsm_triton.causal, self.wpsm_triton.output_value,
                                                     group, lower, lower)
+            if mask_planes is not None:
+                self._mark("mask")
+                scores = _MaskFill.apply(scores, mask_planes, True, self.causal)
             self._mark("softmax")
             scores = _MixSoftmax.apply(scores, None, self.causal, None, lower, lower, key_bias, first_visible)
         self._mark("conv_post")
         scores = Conv2dTritonFunction.apply(scores, self.mta_conv_after_sm_triton.weight, self.causal, lower, lower)
         if first_visible is not None:
             scores = _BandZero.apply(scores, first_visible)
+        if mask_planes is not None:
+            self._mark("mask")
+            scores = _MaskFill.apply(scores, mask_planes, False, self.causal)
         self._mark("mix_post")
         post = self.wposm_triton
         # the last stage's output is read by P V: in full by the library GEMM, on and below the diagonal by our kernels
@@ -650,6 +700,12 @@ class MTAAttentionTriton(nn.Module):
                 if wants_grad:
                     return self._forward_stagewise(xq, xk, xv, key_bias=what)
                 return self._forward_hidden_keys(xq, xk, xv, what)
+        if (isinstance(mask, torch.Tensor) and mask.dim() == 4 and xq.size(-2) == xk.size(-2) and xk.size(-2) % 8 == 0):
+            planes = self._mask_planes(mask, xq.size(0), xq.size(-2))
+            if planes is not None:
+                if wants_grad:
+                    return self._forward_stagewise(xq, xk, xv, mask_planes=planes)
+                return self._forward_mask_planes(xq, xk, xv, planes)
         mask = self._update_mask(mask=mask, bsz=xq.size(0), xq=xq, xk_size=xk.size(-2))
         scale = float(torch.rsqrt(torch.tensor(float(xq.size(-1)))))  # a host scalar: the product stays one vectorised pass
         scores = torch.matmul(xq, xk.transpose(2, 3)) * scale
@@ -663,6 +719,46 @@ class MTAAttentionTriton(nn.Module):
         scores = self.wposm_triton(scores)
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         return torch.matmul(scores, xv).transpose(1, 2)
+
+    def _forward_mask_planes(self, xq, xk, xv, visible):
+        """Inference under a 0 / -inf (or boolean) mask of arbitrary content - holes, planes per head - given as uint8
+        visibility planes (1|B, 1|H, S, S): the reference's sequence (mta_attention_triton.py:68-92) on the single-stage
+        kernels, with its three elementwise mask steps as one in-place pass each that reads a byte per position
+        (``mta_mask_fill_fwd``): no mask tensor in the score dtype, no boolean copy of it, no fp32 copy of the scores,
+        and under the causal rule nothing above the diagonal is computed, masked or written."""
+        cz = self.causal
+        fu = not cz   # (fill flags of the causal kernels: nothing above the diagonal is anybody's business)
+        scale = float(torch.rsqrt(torch.tensor(float(xq.size(-1)))))
+        n_keys = xk.size(-2)
+        own_pv = cz and xq.dtype == xv.dtype and ops.causal_pv_supported(xq.dtype, n_keys, xv.size(-1))
+        self._mark("qk")
+        scores = _lower_scores(xq, xk) if cz else None
+        if scores is None:
+            scores = torch.matmul(xq, xk.transpose(2, 3))
+        self._mark("mask")
+        if ops.mask_fill(scores, visible, False, cz, out=scores) is None:
+            raise RuntimeError("mask planes need a number of keys that is a multiple of 8")
+        self._mark("conv_pre")
+        scores = ops.conv2d_causal(scores, self.mta_conv_triton.weight, cz, in_scale=scale, fill_upper=fu)
+        self._mark("mix_pre")
+        scores = ops.headmix(scores, self.wpsm_triton.weight, cz, float("-inf") if cz else 0.0, fill_upper=fu)
+        self._mark("mask")
+        ops.mask_fill(scores, visible, True, cz, out=scores)
+        self._mark("softmax")
+        scores = ops.headmix_softmax(scores, None, None, cz, fill_upper=fu)
+        self._mark("conv_post")
+        scores = ops.conv2d_causal(scores, self.mta_conv_after_sm_triton.weight, cz, fill_upper=fu)
+        self._mark("mask")
+        ops.mask_fill(scores, visible, False, cz, out=scores)
+        self._mark("mix_post")
+        scores = ops.headmix(scores, self.wposm_triton.weight, cz, 0.0, fill_upper=not own_pv)
+        scores = F.dropout(scores, p=self.dropout, training=self.training)
+        self._mark("pv")
+        output = ops.causal_pv(scores, xv, True) if own_pv else None
+        if output is None:
+            output = torch.matmul(scores, xv)
+        self._mark("end")
+        return output.transpose(1, 2)
 
     def _band_training_supported(self, xq, xk, xv) -> bool:
         """Whether the differentiable route takes a band mask: 16-bit data of one dtype, a length the in-place zeroing
@@ -705,9 +801,16 @@ class MTAAttentionTriton(nn.Module):
         answer = (None, None)
         plane = mask[:, 0]
         same_heads = mask.size(1) == 1 or bool((mask == mask[:, :1]).all())
+        # the mask as a byte per position (non-zero = attend), for masks that are none of the forms above: a boolean
+        # mask as it is, an additive one if it holds nothing but 0 and -inf (see _forward_mask_planes)
+        planes = None
         if mask.dtype == torch.bool:
             visible = plane
+            planes = mask.contiguous().view(torch.uint8)
         else:
+            whole = mask == 0
+            if bool(((mask == float("-inf")) | whole).all()):
+                planes = whole.view(torch.uint8)
             visible = plane == 0
             if not bool(((plane == float("-inf")) | visible).all()):
                 visible = None   # other finite values: not a 0 / -inf mask
@@ -730,8 +833,15 @@ class MTAAttentionTriton(nn.Module):
                 lead = visible.int().argmax(-1)
                 if bool(((count >= 1) & (count == rows[None, :] - lead + 1)).all()):
                     answer = ("band", lead.to(torch.int32).expand(bsz, s).contiguous())
-        self._mask_cache = (mask, key, answer)
+        self._mask_cache = (mask, key, answer, planes)
         return answer
+
+    def _mask_planes(self, mask, bsz: int, s: int):
+        """The uint8 visibility planes of a 4-D boolean or 0 / -inf mask ((1|B, 1|H, S, S); None for anything else), from
+        the same look at the mask as ``_structured_mask``."""
+        self._structured_mask(mask, bsz, s)
+        cached = getattr(self, "_mask_cache", None)
+        return cached[3] if cached is not None and cached[0] is mask else None
 
     def _update_mask(self, mask, bsz: int, xq: torch.Tensor, xk_size: int):
         """Additive (B,H,Sq,Sk) mask, 0 = attend, -inf = blocked (mta_attention_triton.py:106-127)."""

@@ -545,6 +545,33 @@ def band_zero_(x: torch.Tensor, first_visible: torch.Tensor) -> Optional[torch.T
     return x
 
 
+def mask_fill(x: torch.Tensor, visible: torch.Tensor, neg_inf: bool, causal: bool,
+              out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """``visible ? x : (-inf if neg_inf else 0)`` for a mask tensor of arbitrary content: ``visible`` is uint8 (or bool),
+    non-zero = attend, of shape (1|N, 1|C, P, Q); with ``causal`` only keys q <= p are read and written.  ``out`` may be
+    ``x`` (in place).  See mta_mask_fill_fwd.  Returns ``None`` when unsupported (Q not a multiple of 8)."""
+    x = _device_tensor(x, "input")
+    if x.dim() != 4 or not x.is_contiguous():
+        raise ValueError(f"expected a contiguous (N,C,P,Q) tensor, got {tuple(x.shape)}")
+    n, c, p, q = x.shape
+    visible = _device_tensor(visible, "visible")
+    if visible.dtype == torch.bool:
+        visible = visible.view(torch.uint8)
+    if (visible.dtype != torch.uint8 or visible.dim() != 4 or not visible.is_contiguous() or visible.shape[2:] != (p, q)
+            or visible.size(0) not in (1, n) or visible.size(1) not in (1, c)):
+        raise ValueError(f"visible must be a contiguous uint8 / bool tensor of shape (1|{n}, 1|{c}, {p}, {q}), got "
+                         f"{visible.dtype} {tuple(visible.shape)}")
+    y = x if out is x else _out_like(x, out)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().mta_mask_fill_fwd(x.data_ptr(), visible.data_ptr(), y.data_ptr(), n, c, p, q, visible.size(0),
+                                           visible.size(1), int(bool(neg_inf)), int(bool(causal)), _code(x, "input"),
+                                           _stream(x))
+    if rc == _lib.MTA_ERR_UNSUPPORTED:
+        return None
+    _lib.check(rc, "mta_mask_fill_fwd")
+    return y
+
+
 def causal_ptx(p: torch.Tensor, x: torch.Tensor, causal: bool) -> Optional[torch.Tensor]:
     """P^T X for P (B,H,S,S), X (B,H,S,D): out[k] = sum_p P[p,k] X[p], over p >= k only when causal (nothing of P above
     the diagonal is read); see mta_causal_ptx_fwd.  Returns ``None`` when unsupported (the caller then uses

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/mta_hip.h but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes signatures out of sync with the header"
-    assert lib.mta_abi_version() == 9
+    assert lib.mta_abi_version() == 10
 
 
 def test_no_torch_symbols_in_the_library():
@@ -103,6 +103,11 @@ def test_triangular_layout_entry_points_validate_and_answer_on_the_host():
     assert lib.mta_causal_pv_tri_fwd(p, p, None, p, 1, 4, 64, 48, 4, 1, None) == -7
     assert lib.mta_band_zero_fwd(None, p, 1, 1, 8, 1, None) == -1 and lib.mta_band_zero_fwd(p, p, 1, 1, 8, 0, None) == -9
     assert lib.mta_band_zero_fwd(p, p, 1, 1, 12, 1, None) == -9 and lib.mta_band_zero_fwd(p, p, 0, 1, 8, 1, None) == -3
+    # the mask pass: null pointers, a mask that is neither one plane nor one per batch entry / head, a width it does not take
+    assert lib.mta_mask_fill_fwd(None, p, p, 1, 1, 8, 8, 1, 1, 0, 1, 1, None) == -1
+    assert lib.mta_mask_fill_fwd(p, p, p, 2, 4, 8, 8, 3, 1, 0, 1, 1, None) == -3
+    assert lib.mta_mask_fill_fwd(p, p, p, 2, 4, 8, 8, 1, 2, 0, 1, 1, None) == -3
+    assert lib.mta_mask_fill_fwd(p, p, p, 1, 1, 8, 12, 1, 1, 0, 1, 1, None) == -9
     # which combinations the softmax stage has a kernel for: (C, S, group, out_planes, io, w, has_w1, has_w2, band, key_bias)
     q = lib.mta_headmix_softmax_tri_supported
     assert q(16, 4096, 4, 0, 1, 1, 1, 1, 0, 0) == 1 and q(16, 4104, 4, 0, 1, 1, 1, 1, 0, 0) == 0   # packed kernel: up to 4096 keys

@@ -424,7 +424,8 @@ def test_mta_use_mask_band_masks_run_through_the_kernels(pkg, kind, dtype):
         got = mod(q.cuda(), k.cuda(), v.cuda(), mask.cuda(), None).cpu()
         assert stages == ["qk_conv", "mix_softmax_mix", "pv", "end"]
         torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
-    # a mask with a hole in a row is no band: the elementwise route (no stage marks), same values as the oracle's
+    # a mask with a hole in a row is no band: the single-stage kernels with three mask passes between them, same values
+    # as the oracle's
     holed = visible.clone()
     holed[0, 0, 700:, 650] = False
     want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3],
@@ -432,7 +433,7 @@ def test_mta_use_mask_band_masks_run_through_the_kernels(pkg, kind, dtype):
     stages = []
     mod._stage_hook = stages.append
     got = mod(q.cuda(), k.cuda(), v.cuda(), holed.cuda(), None).cpu()
-    assert "qk_conv" not in stages
+    assert "qk_conv" not in stages and stages.count("mask") == 3, stages
     torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
 
 
@@ -952,9 +953,10 @@ def test_mta_use_mask_tensor_masks(pkg, name, dtype):
         mod._stage_hook = stages.append
         got = mod(q.cuda(), k.cuda(), v.cuda(), mask.cuda(), None).cpu()
         torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
-        # a 2-D key mask runs through the kernels (per-key bias in the softmax stage, zeroed K and V rows); only a
-        # full mask tensor takes the elementwise route, which calls no stage hook
-        assert (("qk_conv" in stages or "conv_pre" in stages) and "pv" in stages) == name.startswith("key_mask")
+        # a 2-D key mask runs through the kernels as a per-key bias in the softmax stage and zeroed K and V rows; a full
+        # mask tensor with holes runs through the single-stage kernels with three mask passes between them
+        assert "pv" in stages and (stages.count("mask") == 0) == name.startswith("key_mask"), stages
+        assert name.startswith("key_mask") or stages.count("mask") == 3
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -1048,6 +1050,66 @@ def test_mta_use_mask_right_padded_batch(pkg, post):
     got = mod(q.cuda(), k.cuda(), v.cuda(), visible.cuda(), None).cpu()
     assert "qk_conv" in stages and "pv" in stages
     torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("form", ["bool_BHSS", "additive_1HSS", "bool_B1SS"])
+def test_mta_use_mask_arbitrary_planes(pkg, form, causal, dtype):
+    """use_mask=True under masks of arbitrary content - random holes, a plane per head and / or per batch entry, boolean
+    or 0 / -inf - for causal and non-causal modules: the single-stage kernels with the mask read as a byte per position in
+    three passes (``mta_mask_fill_fwd``), against the oracle given the mask tensor.  Every row keeps a visible key (the
+    diagonal)."""
+    print(f"mta use_mask arbitrary planes {form} causal={causal} {dtype}", flush=True)
+    b, h, s, d = 2, 4, 200, 64
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=99)
+    params = _config_like(h, 2, 3, 5, 0.1, dtype, post="random")
+    g = torch.Generator().manual_seed(100)
+    shape = {"bool_BHSS": (b, h, s, s), "additive_1HSS": (1, h, s, s), "bool_B1SS": (b, 1, s, s)}[form]
+    visible = torch.rand(shape, generator=g) > 0.3
+    visible |= torch.eye(s, dtype=torch.bool)
+    if causal:
+        visible &= torch.tril(torch.ones(s, s, dtype=torch.bool))
+    mask = torch.where(visible, 0.0, float("-inf")).to(dtype) if form.startswith("additive") else visible
+    want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3],
+                         mask=torch.where(visible, 0.0, float("-inf")).expand(b, h, s, s).contiguous())
+    assert torch.isfinite(want.float()).all()
+    mod = _mta_module(pkg, h, 3, 5, 3, 3, *params, dtype, causal=causal, use_mask=True, structure="dense")
+    stages = []
+    mod._stage_hook = stages.append
+    got = mod(q.cuda(), k.cuda(), v.cuda(), mask.cuda(), None).cpu()
+    assert stages == ["qk", "mask", "conv_pre", "mix_pre", "mask", "softmax", "conv_post", "mask", "mix_post", "pv", "end"], stages
+    torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+    # an additive mask with a finite value besides 0 and -inf is not such a mask: the reference's own steps
+    if form.startswith("additive"):
+        other = mask.clone()
+        other[0, 0, s - 1, 0] = -2.0
+        del stages[:]
+        mod(q.cuda(), k.cuda(), v.cuda(), other.cuda(), None)
+        assert "mask" not in stages
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_mask_fill_is_the_select(pkg, dtype):
+    """ops.mask_fill against torch.where, bit for bit: 0 and -inf fills, in place and into another tensor, one mask plane
+    for all or one per batch entry / head; with the causal rule nothing above the diagonal is touched."""
+    print(f"mask_fill {dtype}", flush=True)
+    n, c, p = 2, 3, 136
+    g = torch.Generator().manual_seed(101)
+    x = torch.randn(n, c, p, p, generator=g).to(dtype).cuda()
+    low = torch.tril(torch.ones(p, p, dtype=torch.bool, device="cuda"))
+    for shape in ((1, 1, p, p), (n, 1, p, p), (1, c, p, p), (n, c, p, p)):
+        visible = (torch.rand(shape, generator=g) > 0.4).cuda()
+        for neg_inf in (False, True):
+            fill = float("-inf") if neg_inf else 0.0
+            want = torch.where(visible, x, torch.tensor(fill, dtype=dtype, device="cuda"))
+            got = pkg.ops.mask_fill(x, visible, neg_inf, False)
+            assert torch.equal(got, want)
+            poisoned = x.clone()
+            poisoned[..., ~low] = float("nan")
+            got = pkg.ops.mask_fill(poisoned, visible.view(torch.uint8), neg_inf, True, out=poisoned)
+            assert got is poisoned and torch.equal(got[..., low], want[..., low]) and torch.isnan(got[..., ~low]).all()
+    assert pkg.ops.mask_fill(x[..., :100].contiguous(), torch.ones(1, 1, p, 100, dtype=torch.bool, device="cuda"), False, False) is None
 
 
 @pytest.mark.parametrize("kind", ["key_padding", "window"])

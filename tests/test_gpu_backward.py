@@ -698,6 +698,31 @@ def test_mta_module_backward_non_causal_key_padding(pkg, dtype):
         assert not (g.cpu() * ~real).any(), f"grad {name} of a hidden key is not zero"
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [True, False])
+def test_mta_module_backward_arbitrary_mask_planes(pkg, causal, dtype):
+    """Training under a mask of arbitrary content (random holes, a plane per head; boolean): the differentiable operators
+    with the three mask steps as passes over uint8 visibility planes (forward in place; backward: the conv's input
+    gradient and the gradient behind the post-softmax conv zeroed at the hidden positions).  All seven gradients against
+    autograd through the oracle given the mask tensor."""
+    print(f"mta module backward arbitrary mask causal={causal} {dtype}", flush=True)
+    b, h, s, d = 2, 4, 136, 64
+    mod, params = _mta_pair(pkg, h, 3, 5, dtype, seed=421, causal=causal)
+    mod.use_mask = True
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=422)
+    g = torch.Generator().manual_seed(423)
+    visible = (torch.rand(1, h, s, s, generator=g) > 0.3) | torch.eye(s, dtype=torch.bool)
+    if causal:
+        visible &= torch.tril(torch.ones(s, s, dtype=torch.bool))
+    go = _rand((b, s, h, d), 424, dtype)
+    want_out, want_in, want_w = _oracle_grads(q, k, v, params, go, mask=visible.expand(b, h, s, s))
+    stages = []
+    mod._stage_hook = stages.append
+    out, gin, gw = _module_grads(mod, q, k, v, go, mask=visible)
+    assert stages.count("mask") == 3 and "pv" in stages, stages
+    _check_all(dtype, out.cpu(), want_out, [g_.cpu() for g_ in gin + gw], want_in + want_w)
+
+
 def test_mta_module_backward_key_mask_finite_values(pkg):
     """A 2-D additive key mask with finite values besides -inf (B = 1), in training: the values are added ahead of the
     softmax (mta_attention_triton.py:77), only -inf hides a key."""
