@@ -354,7 +354,20 @@ def bench_kernels(torch, mta, O, device, steps, warmup):
     out["mta_forward_bf16_2x16x4096x128_key_padding_mask"] = {
         "ms": ms, "stages": stages,
         "note": "the headline configuration with use_mask=True and a key-padding mask tensor (lengths 4096 and 3000); not a row of the reference's"}
-    del mod, sets, window, padded
+    # ... and under a mask of arbitrary content (a fifth of the keys below the diagonal hidden at random, the diagonal
+    # kept), given as a (1,1,S,S) boolean mask tensor: the single-stage kernels with three mask passes between them
+    gen = torch.Generator(device=device).manual_seed(11)
+    holes = ((torch.rand(s_len, s_len, device=device, generator=gen) > 0.2) | (pos[None, :] == pos[:, None])) & (pos[None, :] <= pos[:, None])
+    holes = holes[None, None]
+    ms = time_steps(torch, lambda i: mod(*sets[i], holes, None), len(sets), min(warmup, 5), max(3, steps // 5))
+    stages = []
+    mod._stage_hook = stages.append
+    mod(*sets[0], holes, None)
+    mod._stage_hook = None
+    out["mta_forward_bf16_2x16x4096x128_random_holes_mask"] = {
+        "ms": ms, "stages": stages,
+        "note": "the headline configuration with use_mask=True and a mask tensor with holes; not a row of the reference's"}
+    del mod, sets, window, padded, holes
     # the first module and shape in training: forward operator by operator (each with its HIP backward kernels; the two
     # matrix products, the softmax and the dropout are torch's) and backward to q, k, v and the four weights
     mod, sets = build_general(torch, mta, O, device, train=True)

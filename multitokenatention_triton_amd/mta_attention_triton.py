@@ -25,8 +25,10 @@ Inference (no input or parameter requires grad, or grad mode is off):
     masks, key padding of a batch) or to "row p sees the keys first[p] .. p" (sliding
     windows, packed documents) go into the same kernels as one value per key or per row
     (a ``causal=False`` module: masks that hide the same keys from every row, the key
-    padding of an encoder batch); any other mask tensor takes the reference's elementwise
-    steps around the kernels.
+    padding of an encoder batch); any other boolean or 0 / -inf mask (holes, a plane per
+    head) runs on the single-stage kernels with the reference's three elementwise mask
+    steps as passes over a byte per position (``mta_mask_fill_fwd``); only a 4-D additive
+    mask with other finite values takes the reference's elementwise steps around the kernels.
 
 Training (something requires grad): the stages run one by one through autograd
 Functions, as in the reference, so that ``backward()`` works: the two conv and the two
@@ -40,8 +42,8 @@ gradients it leaves, the recomputed raw scores) touch the lower triangle only; t
 differentiates the dropout.  ``use_mask=True`` in training: the same two families of masks
 go through these operators -- hidden keys as a key bias inside the softmax kernel and
 zeroed K and V rows, band masks inside the scores and softmax kernels, with the gradients
-around them formed inside the band; any other mask tensor takes the reference's
-elementwise steps between the single operators.
+around them formed inside the band; masks of arbitrary content as mask passes between the
+operators, whose gradients they zero at the same positions.
 
 Weight structure.  By default nothing is assumed about the four weights: every stage runs
 with the dense weight it is given.  Skipping identity stages and applying block-diagonal
