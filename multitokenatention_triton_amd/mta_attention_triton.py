@@ -742,18 +742,29 @@ class MTAAttentionTriton(nn.Module):
             raise RuntimeError("mask planes need a number of keys that is a multiple of 8")
         self._mark("conv_pre")
         scores = ops.conv2d_causal(scores, self.mta_conv_triton.weight, cz, in_scale=scale, fill_upper=fu)
-        self._mark("mix_pre")
-        scores = ops.headmix(scores, self.wpsm_triton.weight, cz, float("-inf") if cz else 0.0, fill_upper=fu)
+        # (a declared or inferred weight structure: identity stages are skipped - the probabilities are 0 at the hidden
+        # positions already, so without a post-softmax conv its mask pass goes too - and block-diagonal head weights are
+        # applied block by block)
+        st = self._current_structure()
+        if not st.pre_head_identity:
+            self._mark("mix_pre")
+            scores = ops.headmix(scores, self.wpsm_triton.weight, cz, float("-inf") if cz else 0.0,
+                                 group_size=st.pre_head_group, fill_upper=fu)
         self._mark("mask")
         ops.mask_fill(scores, visible, True, cz, out=scores)
         self._mark("softmax")
-        scores = ops.headmix_softmax(scores, None, None, cz, fill_upper=fu)
-        self._mark("conv_post")
-        scores = ops.conv2d_causal(scores, self.mta_conv_after_sm_triton.weight, cz, fill_upper=fu)
-        self._mark("mask")
-        ops.mask_fill(scores, visible, False, cz, out=scores)
-        self._mark("mix_post")
-        scores = ops.headmix(scores, self.wposm_triton.weight, cz, 0.0, fill_upper=not own_pv)
+        last = st.post_conv_identity and st.post_head_identity   # (the softmax's output goes to P V)
+        scores = ops.headmix_softmax(scores, None, None, cz, fill_upper=(not own_pv) if last else fu)
+        if not st.post_conv_identity:
+            self._mark("conv_post")
+            scores = ops.conv2d_causal(scores, self.mta_conv_after_sm_triton.weight, cz,
+                                       fill_upper=(not own_pv) if st.post_head_identity else fu)
+            self._mark("mask")
+            ops.mask_fill(scores, visible, False, cz, out=scores)
+        if not st.post_head_identity:
+            self._mark("mix_post")
+            scores = ops.headmix(scores, self.wposm_triton.weight, cz, 0.0, group_size=st.post_head_group,
+                                 fill_upper=not own_pv)
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         self._mark("pv")
         output = ops.causal_pv(scores, xv, True) if own_pv else None
