@@ -242,6 +242,13 @@ int mta_band_zero_fwd(void *x, const void *first_visible, int64_t N, int64_t C, 
 int mta_mask_fill_fwd(const void *x, const void *visible, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
                       int mask_batch, int mask_heads, int neg_inf, int causal, int io_dtype, void *stream);
 
+/* y = x + mask, rounded once to the I/O dtype: the reference's `scores = scores + mask` (mta_attention_triton.py:77-78)
+ * for an additive mask with finite values.  mask: the scores' dtype, (mask_batch, mask_heads, P, Q) with mask_batch 1 or N
+ * and mask_heads 1 or C (broadcast), 16-byte aligned; y may be x.  causal != 0: only keys q <= p are read and written.
+ * Q % 8 == 0; MTA_ERR_UNSUPPORTED otherwise. */
+int mta_mask_add_fwd(const void *x, const void *mask, void *y, int64_t N, int64_t C, int64_t P, int64_t Q,
+                     int mask_batch, int mask_heads, int causal, int io_dtype, void *stream);
+
 /* ---- The three stages of the causal forward (mta_attention_triton.py:68-89 without a post-softmax conv) over
  * score tensors in a TRIANGULAR LAYOUT.  The (B,H,S,S) tensors between the three kernels never leave the library's
  * caller, so their layout is free; this one stores what lies on and below the diagonal only and puts the rows that one

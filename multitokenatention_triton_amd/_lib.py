@@ -34,6 +34,7 @@ SIGNATURES = {
     "mta_causal_pv_band_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),
     "mta_band_zero_fwd": (_int, [_vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "mta_mask_fill_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _vp]),
+    "mta_mask_add_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _vp]),
     "mta_qk_conv_tri_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _f32, _int, _int, _int, _vp]),
     "mta_headmix_softmax_tri_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _int, _int, _vp]),
     "mta_causal_pv_tri_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _vp]),

@@ -25,10 +25,11 @@ Inference (no input or parameter requires grad, or grad mode is off):
     masks, key padding of a batch) or to "row p sees the keys first[p] .. p" (sliding
     windows, packed documents) go into the same kernels as one value per key or per row
     (a ``causal=False`` module: masks that hide the same keys from every row, the key
-    padding of an encoder batch); any other boolean or 0 / -inf mask (holes, a plane per
-    head) runs on the single-stage kernels with the reference's three elementwise mask
-    steps as passes over a byte per position (``mta_mask_fill_fwd``); only a 4-D additive
-    mask with other finite values takes the reference's elementwise steps around the kernels.
+    padding of an encoder batch); any other boolean or additive mask (holes, a plane per
+    head, finite values) runs on the single-stage kernels with the reference's three
+    elementwise mask steps as passes over a byte per position (``mta_mask_fill_fwd``;
+    ``mta_mask_add_fwd`` for finite values); only lengths that are not a multiple of 8 take
+    the reference's elementwise steps around the kernels.
 
 Training (something requires grad): the stages run one by one through autograd
 Functions, as in the reference, so that ``backward()`` works: the two conv and the two
@@ -270,6 +271,23 @@ class _MaskFill(torch.autograd.Function):
             return grad_output, None, None, None
         planes, = ctx.saved_tensors
         return ops.mask_fill(grad_output.contiguous(), planes, False, ctx.causal), None, None, None
+
+
+class _MaskAdd(torch.autograd.Function):
+    """``x + mask`` in place (``mta_mask_add_fwd``): the reference's ``scores + mask`` ahead of the softmax for an additive
+    mask with finite values.  The gradient is handed on as it is: the derivative is 1, and where the mask is -inf the
+    softmax that follows returns exactly 0."""
+
+    @staticmethod
+    def forward(ctx, x, mask, causal):
+        if ops.mask_add(x, mask, causal, out=x) is None:
+            raise RuntimeError("mask planes need a number of keys that is a multiple of 8")
+        ctx.mark_dirty(x)
+        return x
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return grad_output, None, None
 
 
 class _BandZero(torch.autograd.Function):
@@ -542,7 +560,7 @@ class MTAAttentionTriton(nn.Module):
         self._mark("end")
         return output.transpose(1, 2)
 
-    def _forward_stagewise(self, xq, xk, xv, key_bias=None, first_visible=None, mask_planes=None):
+    def _forward_stagewise(self, xq, xk, xv, key_bias=None, first_visible=None, mask_planes=None, mask_additive=None):
         """The reference's own sequence of operators (mta_attention_triton.py:68-92), each differentiable: taken
         whenever a gradient may be asked for.  No weight structure is assumed here, so every entry of the four
         weights receives its gradient.
@@ -587,7 +605,10 @@ class MTAAttentionTriton(nn.Module):
                                                     group, lower, lower)
             if mask_planes is not None:
                 self._mark("mask")
-                scores = _MaskFill.apply(scores, mask_planes, True, self.causal)
+                if mask_additive is None:
+                    scores = _MaskFill.apply(scores, mask_planes, True, self.causal)
+                else:   # (finite values besides 0: the mask in the scores' dtype is added)
+                    scores = _MaskAdd.apply(scores, mask_additive, self.causal)
             self._mark("softmax")
             scores = _MixSoftmax.apply(scores, None, self.causal, None, lower, lower, key_bias, first_visible)
         self._mark("conv_post")
@@ -703,11 +724,15 @@ class MTAAttentionTriton(nn.Module):
                     return self._forward_stagewise(xq, xk, xv, key_bias=what)
                 return self._forward_hidden_keys(xq, xk, xv, what)
         if (isinstance(mask, torch.Tensor) and mask.dim() == 4 and xq.size(-2) == xk.size(-2) and xk.size(-2) % 8 == 0):
-            planes = self._mask_planes(mask, xq.size(0), xq.size(-2))
+            planes, additive = self._mask_planes(mask, xq.size(0), xq.size(-2))
+            if additive is not None:   # (the reference adds the mask in the scores' dtype)
+                additive = additive.to(xq.dtype).contiguous()
+                if additive.data_ptr() % 16 != 0:
+                    planes = None
             if planes is not None:
                 if wants_grad:
-                    return self._forward_stagewise(xq, xk, xv, mask_planes=planes)
-                return self._forward_mask_planes(xq, xk, xv, planes)
+                    return self._forward_stagewise(xq, xk, xv, mask_planes=planes, mask_additive=additive)
+                return self._forward_mask_planes(xq, xk, xv, planes, additive)
         mask = self._update_mask(mask=mask, bsz=xq.size(0), xq=xq, xk_size=xk.size(-2))
         scale = float(torch.rsqrt(torch.tensor(float(xq.size(-1)))))  # a host scalar: the product stays one vectorised pass
         scores = torch.matmul(xq, xk.transpose(2, 3)) * scale
@@ -722,9 +747,10 @@ class MTAAttentionTriton(nn.Module):
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         return torch.matmul(scores, xv).transpose(1, 2)
 
-    def _forward_mask_planes(self, xq, xk, xv, visible):
-        """Inference under a 0 / -inf (or boolean) mask of arbitrary content - holes, planes per head - given as uint8
-        visibility planes (1|B, 1|H, S, S): the reference's sequence (mta_attention_triton.py:68-92) on the single-stage
+    def _forward_mask_planes(self, xq, xk, xv, visible, additive=None):
+        """Inference under a boolean or additive mask of arbitrary content - holes, planes per head - given as uint8
+        visibility planes (1|B, 1|H, S, S), and for an additive mask with finite values besides 0 as that mask in the
+        scores' dtype as well (added ahead of the softmax in place of the -inf fill): the reference's sequence (mta_attention_triton.py:68-92) on the single-stage
         kernels, with its three elementwise mask steps as one in-place pass each that reads a byte per position
         (``mta_mask_fill_fwd``): no mask tensor in the score dtype, no boolean copy of it, no fp32 copy of the scores,
         and under the causal rule nothing above the diagonal is computed, masked or written."""
@@ -751,7 +777,10 @@ class MTAAttentionTriton(nn.Module):
             scores = ops.headmix(scores, self.wpsm_triton.weight, cz, float("-inf") if cz else 0.0,
                                  group_size=st.pre_head_group, fill_upper=fu)
         self._mark("mask")
-        ops.mask_fill(scores, visible, True, cz, out=scores)
+        if additive is None:
+            ops.mask_fill(scores, visible, True, cz, out=scores)
+        elif ops.mask_add(scores, additive, cz, out=scores) is None:
+            raise RuntimeError("mask planes need a number of keys that is a multiple of 8")
         self._mark("softmax")
         last = st.post_conv_identity and st.post_head_identity   # (the softmax's output goes to P V)
         scores = ops.headmix_softmax(scores, None, None, cz, fill_upper=(not own_pv) if last else fu)
@@ -815,15 +844,16 @@ class MTAAttentionTriton(nn.Module):
         plane = mask[:, 0]
         same_heads = mask.size(1) == 1 or bool((mask == mask[:, :1]).all())
         # the mask as a byte per position (non-zero = attend), for masks that are none of the forms above: a boolean
-        # mask as it is, an additive one if it holds nothing but 0 and -inf (see _forward_mask_planes)
-        planes = None
+        # mask as it is, an additive one as "not -inf" (see _forward_mask_planes)
+        planes = additive = None
         if mask.dtype == torch.bool:
             visible = plane
             planes = mask.contiguous().view(torch.uint8)
         else:
-            whole = mask == 0
-            if bool(((mask == float("-inf")) | whole).all()):
-                planes = whole.view(torch.uint8)
+            blocked = mask == float("-inf")
+            planes = (~blocked).view(torch.uint8)
+            if not bool((blocked | (mask == 0)).all()):
+                additive = mask   # finite values besides 0: the mask itself is added ahead of the softmax
             visible = plane == 0
             if not bool(((plane == float("-inf")) | visible).all()):
                 visible = None   # other finite values: not a 0 / -inf mask
@@ -846,15 +876,16 @@ class MTAAttentionTriton(nn.Module):
                 lead = visible.int().argmax(-1)
                 if bool(((count >= 1) & (count == rows[None, :] - lead + 1)).all()):
                     answer = ("band", lead.to(torch.int32).expand(bsz, s).contiguous())
-        self._mask_cache = (mask, key, answer, planes)
+        self._mask_cache = (mask, key, answer, planes, additive)
         return answer
 
     def _mask_planes(self, mask, bsz: int, s: int):
-        """The uint8 visibility planes of a 4-D boolean or 0 / -inf mask ((1|B, 1|H, S, S); None for anything else), from
-        the same look at the mask as ``_structured_mask``."""
+        """(planes, additive) of a 4-D mask (1|B, 1|H, S, S), from the same look at the mask as ``_structured_mask``:
+        its uint8 visibility planes, and the mask itself if it is additive with finite values besides 0 (else None);
+        (None, None) for a mask of another shape."""
         self._structured_mask(mask, bsz, s)
         cached = getattr(self, "_mask_cache", None)
-        return cached[3] if cached is not None and cached[0] is mask else None
+        return (cached[3], cached[4]) if cached is not None and cached[0] is mask else (None, None)
 
     def _update_mask(self, mask, bsz: int, xq: torch.Tensor, xk_size: int):
         """Additive (B,H,Sq,Sk) mask, 0 = attend, -inf = blocked (mta_attention_triton.py:106-127)."""

@@ -561,6 +561,8 @@ def mask_fill(x: torch.Tensor, visible: torch.Tensor, neg_inf: bool, causal: boo
             or visible.size(0) not in (1, n) or visible.size(1) not in (1, c)):
         raise ValueError(f"visible must be a contiguous uint8 / bool tensor of shape (1|{n}, 1|{c}, {p}, {q}), got "
                          f"{visible.dtype} {tuple(visible.shape)}")
+    if visible.data_ptr() % 8 != 0:
+        return None
     y = x if out is x else _out_like(x, out)
     with torch.cuda.device(x.device):
         rc = _lib.load().mta_mask_fill_fwd(x.data_ptr(), visible.data_ptr(), y.data_ptr(), n, c, p, q, visible.size(0),
@@ -569,6 +571,30 @@ def mask_fill(x: torch.Tensor, visible: torch.Tensor, neg_inf: bool, causal: boo
     if rc == _lib.MTA_ERR_UNSUPPORTED:
         return None
     _lib.check(rc, "mta_mask_fill_fwd")
+    return y
+
+
+def mask_add(x: torch.Tensor, mask: torch.Tensor, causal: bool, out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """``x + mask`` in x's dtype for an additive mask of x's dtype and shape (1|N, 1|C, P, Q); with ``causal`` only keys
+    q <= p are read and written.  ``out`` may be ``x``.  See mta_mask_add_fwd.  Returns ``None`` when unsupported."""
+    x = _device_tensor(x, "input")
+    if x.dim() != 4 or not x.is_contiguous():
+        raise ValueError(f"expected a contiguous (N,C,P,Q) tensor, got {tuple(x.shape)}")
+    n, c, p, q = x.shape
+    mask = _device_tensor(mask, "mask")
+    if (mask.dtype != x.dtype or mask.dim() != 4 or not mask.is_contiguous() or mask.shape[2:] != (p, q)
+            or mask.size(0) not in (1, n) or mask.size(1) not in (1, c)):
+        raise ValueError(f"mask must be a contiguous {x.dtype} tensor of shape (1|{n}, 1|{c}, {p}, {q}), got "
+                         f"{mask.dtype} {tuple(mask.shape)}")
+    if mask.data_ptr() % 16 != 0:
+        return None
+    y = x if out is x else _out_like(x, out)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().mta_mask_add_fwd(x.data_ptr(), mask.data_ptr(), y.data_ptr(), n, c, p, q, mask.size(0),
+                                          mask.size(1), int(bool(causal)), _code(x, "input"), _stream(x))
+    if rc == _lib.MTA_ERR_UNSUPPORTED:
+        return None
+    _lib.check(rc, "mta_mask_add_fwd")
     return y
 
 

@@ -108,6 +108,8 @@ def test_triangular_layout_entry_points_validate_and_answer_on_the_host():
     assert lib.mta_mask_fill_fwd(p, p, p, 2, 4, 8, 8, 3, 1, 0, 1, 1, None) == -3
     assert lib.mta_mask_fill_fwd(p, p, p, 2, 4, 8, 8, 1, 2, 0, 1, 1, None) == -3
     assert lib.mta_mask_fill_fwd(p, p, p, 1, 1, 8, 12, 1, 1, 0, 1, 1, None) == -9
+    assert lib.mta_mask_add_fwd(None, p, p, 1, 1, 8, 8, 1, 1, 1, 1, None) == -1
+    assert lib.mta_mask_add_fwd(p, p, p, 2, 4, 8, 8, 3, 1, 1, 1, None) == -3 and lib.mta_mask_add_fwd(p, p, p, 1, 1, 8, 12, 1, 1, 1, 1, None) == -9
     # which combinations the softmax stage has a kernel for: (C, S, group, out_planes, io, w, has_w1, has_w2, band, key_bias)
     q = lib.mta_headmix_softmax_tri_supported
     assert q(16, 4096, 4, 0, 1, 1, 1, 1, 0, 0) == 1 and q(16, 4104, 4, 0, 1, 1, 1, 1, 0, 0) == 0   # packed kernel: up to 4096 keys

@@ -1097,13 +1097,17 @@ def test_mta_use_mask_arbitrary_planes(pkg, form, causal, dtype):
         got2 = mod2(q.cuda(), k.cuda(), v.cuda(), mask.cuda(), None).cpu()
         assert seen == expect, seen
         torch.testing.assert_close(got2.float(), want2.float(), **tol(dtype))
-    # an additive mask with a finite value besides 0 and -inf is not such a mask: the reference's own steps
+    # an additive mask with finite values besides 0 and -inf: the same route, the mask itself added ahead of the softmax
     if form.startswith("additive"):
-        other = mask.clone()
-        other[0, 0, s - 1, 0] = -2.0
+        g2 = torch.Generator().manual_seed(102)
+        other = torch.where(visible, torch.randn(shape, generator=g2) * (torch.rand(shape, generator=g2) > 0.5), float("-inf"))
+        other = other.to(dtype)
+        want3 = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3],
+                              mask=other.expand(b, h, s, s).contiguous())
         del stages[:]
-        mod(q.cuda(), k.cuda(), v.cuda(), other.cuda(), None)
-        assert "mask" not in stages
+        got3 = mod(q.cuda(), k.cuda(), v.cuda(), other.cuda(), None).cpu()
+        assert stages.count("mask") == 3, stages
+        torch.testing.assert_close(got3.float(), want3.float(), **tol(dtype))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
@@ -1127,6 +1131,16 @@ def test_mask_fill_is_the_select(pkg, dtype):
             got = pkg.ops.mask_fill(poisoned, visible.view(torch.uint8), neg_inf, True, out=poisoned)
             assert got is poisoned and torch.equal(got[..., low], want[..., low]) and torch.isnan(got[..., ~low]).all()
     assert pkg.ops.mask_fill(x[..., :100].contiguous(), torch.ones(1, 1, p, 100, dtype=torch.bool, device="cuda"), False, False) is None
+    # the additive pass: x + mask, rounded once, as torch adds two tensors of the dtype; -inf stays -inf
+    for shape in ((1, 1, p, p), (n, c, p, p)):
+        m = torch.randn(shape, generator=g).to(dtype).cuda()
+        m[..., 3] = float("-inf")
+        want = x + m
+        assert torch.equal(pkg.ops.mask_add(x, m, False), want)
+        poisoned = x.clone()
+        poisoned[..., ~low] = float("nan")
+        got = pkg.ops.mask_add(poisoned, m, True, out=poisoned)
+        assert got is poisoned and torch.equal(got[..., low], want[..., low]) and torch.isnan(got[..., ~low]).all()
 
 
 @pytest.mark.parametrize("kind", ["key_padding", "window"])

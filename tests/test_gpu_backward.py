@@ -721,6 +721,13 @@ def test_mta_module_backward_arbitrary_mask_planes(pkg, causal, dtype):
     out, gin, gw = _module_grads(mod, q, k, v, go, mask=visible)
     assert stages.count("mask") == 3 and "pv" in stages, stages
     _check_all(dtype, out.cpu(), want_out, [g_.cpu() for g_ in gin + gw], want_in + want_w)
+    # the same with an additive mask that holds finite values besides 0 and -inf (added ahead of the softmax)
+    additive = torch.where(visible, 0.5 * torch.randn(1, h, s, s, generator=g), float("-inf")).to(dtype)
+    want_out, want_in, want_w = _oracle_grads(q, k, v, params, go, mask=additive.expand(b, h, s, s))
+    del stages[:]
+    out, gin, gw = _module_grads(mod, q, k, v, go, mask=additive)
+    assert stages.count("mask") == 3, stages
+    _check_all(dtype, out.cpu(), want_out, [g_.cpu() for g_ in gin + gw], want_in + want_w)
 
 
 def test_mta_module_backward_key_mask_finite_values(pkg):
