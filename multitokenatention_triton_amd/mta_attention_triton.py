@@ -843,17 +843,9 @@ class MTAAttentionTriton(nn.Module):
         answer = (None, None)
         plane = mask[:, 0]
         same_heads = mask.size(1) == 1 or bool((mask == mask[:, :1]).all())
-        # the mask as a byte per position (non-zero = attend), for masks that are none of the forms above: a boolean
-        # mask as it is, an additive one as "not -inf" (see _forward_mask_planes)
-        planes = additive = None
         if mask.dtype == torch.bool:
             visible = plane
-            planes = mask.contiguous().view(torch.uint8)
         else:
-            blocked = mask == float("-inf")
-            planes = (~blocked).view(torch.uint8)
-            if not bool((blocked | (mask == 0)).all()):
-                additive = mask   # finite values besides 0: the mask itself is added ahead of the softmax
             visible = plane == 0
             if not bool(((plane == float("-inf")) | visible).all()):
                 visible = None   # other finite values: not a 0 / -inf mask
@@ -876,16 +868,28 @@ class MTAAttentionTriton(nn.Module):
                 lead = visible.int().argmax(-1)
                 if bool(((count >= 1) & (count == rows[None, :] - lead + 1)).all()):
                     answer = ("band", lead.to(torch.int32).expand(bsz, s).contiguous())
-        self._mask_cache = (mask, key, answer, planes, additive)
+        self._mask_cache = (mask, key, answer)
         return answer
 
     def _mask_planes(self, mask, bsz: int, s: int):
-        """(planes, additive) of a 4-D mask (1|B, 1|H, S, S), from the same look at the mask as ``_structured_mask``:
-        its uint8 visibility planes, and the mask itself if it is additive with finite values besides 0 (else None);
-        (None, None) for a mask of another shape."""
-        self._structured_mask(mask, bsz, s)
-        cached = getattr(self, "_mask_cache", None)
-        return (cached[3], cached[4]) if cached is not None and cached[0] is mask else (None, None)
+        """(planes, additive) of a 4-D mask (1|B, 1|H, S, S) that is none of the forms ``_structured_mask`` knows: the mask
+        as a byte per position (uint8, non-zero = attend: a boolean mask as it is, an additive one as "not -inf"), and the
+        mask itself if it is additive with finite values besides 0 (else None); (None, None) for a mask of another shape.
+        Kept for the last mask object seen while its version does not change (for an additive mask the planes are a
+        tensor of their own, a byte per mask element)."""
+        if mask.size(0) not in (1, bsz) or mask.size(-2) != s or mask.size(-1) != s or mask.size(1) not in (1, self.n_heads):
+            return None, None
+        cached = getattr(self, "_planes_cache", None)
+        if cached is not None and cached[0] is mask and cached[1] == mask._version:
+            return cached[2]
+        if mask.dtype == torch.bool:
+            answer = (mask.contiguous().view(torch.uint8), None)
+        else:
+            blocked = mask == float("-inf")
+            finite = not bool((blocked | (mask == 0)).all())
+            answer = ((~blocked).view(torch.uint8), mask if finite else None)
+        self._planes_cache = (mask, mask._version, answer)
+        return answer
 
     def _update_mask(self, mask, bsz: int, xq: torch.Tensor, xk_size: int):
         """Additive (B,H,Sq,Sk) mask, 0 = attend, -inf = blocked (mta_attention_triton.py:106-127)."""
