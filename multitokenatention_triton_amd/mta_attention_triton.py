@@ -683,13 +683,16 @@ class MTAAttentionTriton(nn.Module):
         """use_mask=True: an explicit additive mask tensor drives the masking (mta_attention_triton.py:63-64,
         77-83, 96-98); the kernels still apply their own causal rule when ``causal`` is set.
 
-        These masks never become a (B,H,S,S) tensor here (inference, causal module): no mask at all, which the
-        reference turns into the causal rule the kernels apply anyway; a 2-D key mask, which the reference turns into
+        These masks never become a (B,H,S,S) tensor here (causal module, inference and training): no mask at all, which
+        the reference turns into the causal rule the kernels apply anyway; a 2-D key mask, which the reference turns into
         "causal rule + one value per key" (mta_attention_triton.py:118-122); a 4-D mask that says the same per batch
-        entry (key padding for B > 1, which the reference's 2-D form cannot express); and a 4-D band mask.  A hidden key's scores enter the
-        pre-softmax conv as 0 -- which is what a zero K row produces -- its mixed score gets -inf ahead of the softmax
-        (the kernel's per-key bias), its probability is 0, and whatever the post-softmax conv writes into its column,
-        which the reference zeroes, meets a zero V row."""
+        entry (key padding for B > 1, which the reference's 2-D form cannot express); and a 4-D band mask.  A hidden
+        key's scores enter the pre-softmax conv as 0 -- which is what a zero K row produces -- its mixed score gets -inf
+        ahead of the softmax (the kernel's per-key bias), its probability is 0, and whatever the post-softmax conv writes
+        into its column, which the reference zeroes, meets a zero V row.  A ``causal=False`` module knows the hidden-keys
+        form (the same keys hidden from every row).  Any other 4-D mask over square scores whose length is a multiple of
+        8 is read as a byte per position by three mask passes between the single-stage kernels; what is left takes the
+        reference's own steps, at the end of this function."""
         if self.causal and xq.size(-2) == xk.size(-2):
             # (with a gradient wanted: the same masks through the differentiable operators)
             hidden_keys = self._forward_stagewise_hidden_keys if wants_grad else self._forward_hidden_keys
@@ -750,8 +753,8 @@ class MTAAttentionTriton(nn.Module):
     def _forward_mask_planes(self, xq, xk, xv, visible, additive=None):
         """Inference under a boolean or additive mask of arbitrary content - holes, planes per head - given as uint8
         visibility planes (1|B, 1|H, S, S), and for an additive mask with finite values besides 0 as that mask in the
-        scores' dtype as well (added ahead of the softmax in place of the -inf fill): the reference's sequence (mta_attention_triton.py:68-92) on the single-stage
-        kernels, with its three elementwise mask steps as one in-place pass each that reads a byte per position
+        scores' dtype as well (added ahead of the softmax in place of the -inf fill): the reference's sequence
+        (mta_attention_triton.py:68-92) on the single-stage kernels, with its three elementwise mask steps as one in-place pass each that reads a byte per position
         (``mta_mask_fill_fwd``): no mask tensor in the score dtype, no boolean copy of it, no fp32 copy of the scores,
         and under the causal rule nothing above the diagonal is computed, masked or written."""
         cz = self.causal
