@@ -318,11 +318,15 @@ class _MixSoftmax(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, weight, causal, group_size, fill_upper=True, grad_fill_upper=True, key_bias=None,
-                first_visible=None):
+                first_visible=None, zero_planes=None):
         # (key_bias: fp32 (B,Sk) added to the mixed scores, 0 or -inf per key; first_visible: int32 (B,S), a band mask.
         # Constants: the gradient is the softmax's own, taken from the stored probabilities, which are 0 at what is hidden)
         p = ops.headmix_softmax(x, weight, None, causal, group_size=group_size if weight is not None else None,
                                 fill_upper=fill_upper, key_bias=key_bias, first_visible=first_visible)
+        if zero_planes is not None:
+            # (uint8 visibility planes of a mask under which some row sees nothing: that row's NaN becomes zeros, as behind
+            # the reference's masked_fill ahead of its post-softmax conv - and the stored probabilities give it a zero gradient)
+            ops.mask_fill(p, zero_planes, False, causal, out=p)
         ctx.save_for_backward(x if weight is not None else None, weight, p)
         ctx.causal, ctx.group_size, ctx.grad_fill_upper = causal, group_size, grad_fill_upper
         return p
@@ -334,7 +338,7 @@ class _MixSoftmax(torch.autograd.Function):
         ds = ops.softmax_bwd(p, grad_output.to(p.dtype), ctx.causal,
                              fill_upper=weight is None and ctx.grad_fill_upper)
         if weight is None:
-            return ds, None, None, None, None, None, None, None
+            return ds, None, None, None, None, None, None, None, None
         dx = dw = None
         if ctx.needs_input_grad[0]:
             dx = ops.headmix_bwd_input(ds, weight, ctx.causal, ctx.group_size, fill_upper=ctx.grad_fill_upper)
@@ -344,7 +348,7 @@ class _MixSoftmax(torch.autograd.Function):
                 blk = torch.arange(weight.shape[0], device=weight.device) // ctx.group_size
                 dw = dw * (blk[:, None] == blk[None, :])
             dw = dw.to(weight.dtype)
-        return dx, dw, None, None, None, None, None, None
+        return dx, dw, None, None, None, None, None, None, None
 
 
 @dataclass
@@ -560,7 +564,8 @@ class MTAAttentionTriton(nn.Module):
         self._mark("end")
         return output.transpose(1, 2)
 
-    def _forward_stagewise(self, xq, xk, xv, key_bias=None, first_visible=None, mask_planes=None, mask_additive=None):
+    def _forward_stagewise(self, xq, xk, xv, key_bias=None, first_visible=None, mask_planes=None, mask_additive=None,
+                           mask_empty_rows=False):
         """The reference's own sequence of operators (mta_attention_triton.py:68-92), each differentiable: taken
         whenever a gradient may be asked for.  No weight structure is assumed here, so every entry of the four
         weights receives its gradient.
@@ -610,7 +615,8 @@ class MTAAttentionTriton(nn.Module):
                 else:   # (finite values besides 0: the mask in the scores' dtype is added)
                     scores = _MaskAdd.apply(scores, mask_additive, self.causal)
             self._mark("softmax")
-            scores = _MixSoftmax.apply(scores, None, self.causal, None, lower, lower, key_bias, first_visible)
+            scores = _MixSoftmax.apply(scores, None, self.causal, None, lower, lower, key_bias, first_visible,
+                                       mask_planes if mask_empty_rows else None)
         self._mark("conv_post")
         scores = Conv2dTritonFunction.apply(scores, self.mta_conv_after_sm_triton.weight, self.causal, lower, lower)
         if first_visible is not None:
@@ -727,15 +733,16 @@ class MTAAttentionTriton(nn.Module):
                     return self._forward_stagewise(xq, xk, xv, key_bias=what)
                 return self._forward_hidden_keys(xq, xk, xv, what)
         if (isinstance(mask, torch.Tensor) and mask.dim() == 4 and xq.size(-2) == xk.size(-2) and xk.size(-2) % 8 == 0):
-            planes, additive = self._mask_planes(mask, xq.size(0), xq.size(-2))
+            planes, additive, empty_rows = self._mask_planes(mask, xq.size(0), xq.size(-2))
             if additive is not None:   # (the reference adds the mask in the scores' dtype)
                 additive = additive.to(xq.dtype).contiguous()
                 if additive.data_ptr() % 16 != 0:
                     planes = None
             if planes is not None:
                 if wants_grad:
-                    return self._forward_stagewise(xq, xk, xv, mask_planes=planes, mask_additive=additive)
-                return self._forward_mask_planes(xq, xk, xv, planes, additive)
+                    return self._forward_stagewise(xq, xk, xv, mask_planes=planes, mask_additive=additive,
+                                                   mask_empty_rows=empty_rows)
+                return self._forward_mask_planes(xq, xk, xv, planes, additive, empty_rows)
         mask = self._update_mask(mask=mask, bsz=xq.size(0), xq=xq, xk_size=xk.size(-2))
         scale = float(torch.rsqrt(torch.tensor(float(xq.size(-1)))))  # a host scalar: the product stays one vectorised pass
         scores = torch.matmul(xq, xk.transpose(2, 3)) * scale
@@ -750,7 +757,7 @@ class MTAAttentionTriton(nn.Module):
         scores = F.dropout(scores, p=self.dropout, training=self.training)
         return torch.matmul(scores, xv).transpose(1, 2)
 
-    def _forward_mask_planes(self, xq, xk, xv, visible, additive=None):
+    def _forward_mask_planes(self, xq, xk, xv, visible, additive=None, empty_rows=False):
         """Inference under a boolean or additive mask of arbitrary content - holes, planes per head - given as uint8
         visibility planes (1|B, 1|H, S, S), and for an additive mask with finite values besides 0 as that mask in the
         scores' dtype as well (added ahead of the softmax in place of the -inf fill): the reference's sequence
@@ -787,6 +794,11 @@ class MTAAttentionTriton(nn.Module):
         self._mark("softmax")
         last = st.post_conv_identity and st.post_head_identity   # (the softmax's output goes to P V)
         scores = ops.headmix_softmax(scores, None, None, cz, fill_upper=(not own_pv) if last else fu)
+        if empty_rows:
+            # a row that sees nothing comes out of the softmax as NaN; the reference's masked_fill ahead of its
+            # post-softmax conv turns it into zeros (everywhere else the hidden positions hold 0 already)
+            self._mark("mask")
+            ops.mask_fill(scores, visible, False, cz, out=scores)
         if not st.post_conv_identity:
             self._mark("conv_post")
             scores = ops.conv2d_causal(scores, self.mta_conv_after_sm_triton.weight, cz,
@@ -875,22 +887,28 @@ class MTAAttentionTriton(nn.Module):
         return answer
 
     def _mask_planes(self, mask, bsz: int, s: int):
-        """(planes, additive) of a 4-D mask (1|B, 1|H, S, S) that is none of the forms ``_structured_mask`` knows: the mask
-        as a byte per position (uint8, non-zero = attend: a boolean mask as it is, an additive one as "not -inf"), and the
-        mask itself if it is additive with finite values besides 0 (else None); (None, None) for a mask of another shape.
+        """(planes, additive, empty_rows) of a 4-D mask (1|B, 1|H, S, S) that is none of the forms ``_structured_mask``
+        knows: the mask as a byte per position (uint8, non-zero = attend: a boolean mask as it is, an additive one as "not
+        -inf"); the mask itself if it is additive with finite values besides 0 (else None); and whether some query row
+        sees no key at all (the padding rows of a left-padded batch) - the softmax of such a row is NaN, which the
+        reference replaces by zeros ahead of its post-softmax conv (mta_attention_triton.py:81), and so does the route
+        then.  (None, None, False) for a mask of another shape.
         Kept for the last mask object seen while its version does not change (for an additive mask the planes are a
         tensor of their own, a byte per mask element)."""
         if mask.size(0) not in (1, bsz) or mask.size(-2) != s or mask.size(-1) != s or mask.size(1) not in (1, self.n_heads):
-            return None, None
+            return None, None, False
         cached = getattr(self, "_planes_cache", None)
         if cached is not None and cached[0] is mask and cached[1] == mask._version:
             return cached[2]
         if mask.dtype == torch.bool:
-            answer = (mask.contiguous().view(torch.uint8), None)
+            visible, additive = mask.contiguous(), None
         else:
             blocked = mask == float("-inf")
             finite = not bool((blocked | (mask == 0)).all())
-            answer = ((~blocked).view(torch.uint8), mask if finite else None)
+            visible, additive = ~blocked, (mask if finite else None)
+        seen = visible.tril() if self.causal else visible     # (the kernels apply the causal rule on top of the mask)
+        empty_rows = not bool(seen.any(-1).all())
+        answer = (visible.view(torch.uint8), additive, empty_rows)
         self._planes_cache = (mask, mask._version, answer)
         return answer
 

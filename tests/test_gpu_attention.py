@@ -1110,6 +1110,43 @@ def test_mta_use_mask_arbitrary_planes(pkg, form, causal, dtype):
         torch.testing.assert_close(got3.float(), want3.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("post", ["identity", "random"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_mta_use_mask_rows_that_see_nothing(pkg, dtype, post):
+    """A left-padded batch whose mask hides the padding both as keys and as queries: the padding rows see no key at all.
+    Their softmax is NaN; the reference zeroes it ahead of its post-softmax conv (mta_attention_triton.py:81), so their
+    outputs are 0 and no other row is touched - the same here (one more mask pass behind the softmax), in inference and,
+    with finite gradients that are zero for the padding, in training."""
+    print(f"mta use_mask empty rows {dtype} post={post}", flush=True)
+    b, h, s, d = 2, 4, 136, 64
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=103)
+    params = _config_like(h, 2, 3, 5, 0.1, dtype, post=post)
+    pad = torch.tensor([0, 37])
+    keep = torch.arange(s)[None, :] >= pad[:, None]                                   # (B,S): left padding
+    visible = (keep[:, None, :, None] & keep[:, None, None, :] & torch.tril(torch.ones(s, s, dtype=torch.bool))[None, None])
+    want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3],
+                         mask=torch.where(visible, 0.0, float("-inf")).expand(b, h, s, s).contiguous())
+    assert torch.isfinite(want.float()).all() and not want[1, :37].any()
+    for structure in ("dense", "infer"):
+        mod = _mta_module(pkg, h, 3, 5, 3, 3, *params, dtype, use_mask=True, structure=structure)
+        stages = []
+        mod._stage_hook = stages.append
+        got = mod(q.cuda(), k.cuda(), v.cuda(), visible.cuda(), None).cpu()
+        assert stages.count("mask") == (4 if post == "random" or structure == "dense" else 3), stages
+        torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+        assert not got[1, :37].any()
+    # training: the same forward, finite gradients, none for the padding
+    mod = _mta_module(pkg, h, 3, 5, 3, 3, *params, dtype, use_mask=True, structure="dense").requires_grad_(True)
+    qd, kd, vd = [t.clone().cuda().requires_grad_(True) for t in (q, k, v)]
+    out = mod(qd, kd, vd, visible.cuda(), None)
+    torch.testing.assert_close(out.detach().cpu().float(), want.float(), **tol(dtype))
+    out.backward(torch.ones_like(out))
+    for name, g_ in (("xq", qd.grad), ("xk", kd.grad), ("xv", vd.grad)):
+        assert torch.isfinite(g_).all(), name
+        assert not g_[1, :, :37].any(), f"the padding of {name} received a gradient"
+    assert all(torch.isfinite(p_.grad).all() for p_ in mod.parameters())
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_mask_fill_is_the_select(pkg, dtype):
     """ops.mask_fill against torch.where, bit for bit: 0 and -inf fills, in place and into another tensor, one mask plane
