@@ -430,12 +430,16 @@ class MTAAttentionTriton(nn.Module):
             return self._forward_stagewise(xq, xk, xv)
         return self._forward_fused(xq, xk, xv)
 
-    def _forward_fused(self, xq, xk, xv, key_bias=None, first_visible=None):
+    def _forward_fused(self, xq, xk, xv, key_bias=None, first_visible=None, empty_rows=None):
         """Inference route (module docstring).  ``key_bias``: fp32 (B,Sk), added to the mixed scores ahead of the
         softmax -- the caller has zeroed the K and V rows of the keys it hides.  ``first_visible``: int32 (B,S), a band
         mask (row p sees the keys first_visible[p] .. p): applied to the scores inside the first kernel and as -inf
         inside the softmax kernel, and behind a post-softmax conv that is not the identity the hidden stretch of every row
-        is zeroed again; the caller has checked that the first kernel exists."""
+        is zeroed again; the caller has checked that the first kernel exists.  ``empty_rows``: bool (B,S) or None, the
+        rows of the band that see no key (first_visible[p] = p + 1).  Their scores enter the conv as 0 like any hidden
+        score; the softmax leaves NaN in them, which the reference replaces by zeros ahead of its post-softmax conv
+        (mta_attention_triton.py:81): here those rows of the probabilities are cleared ahead of a post-softmax conv
+        that is not the identity, and their rows of the output, where nothing else would, at the end."""
         head_dim = xq.size(-1)
         # the reference multiplies by rsqrt(tensor(head_dim)), an fp32 scalar (mta_attention_triton.py:69-71)
         scale = float(torch.rsqrt(torch.tensor(float(head_dim))))
@@ -476,6 +480,8 @@ class MTAAttentionTriton(nn.Module):
                                              first_visible=first_visible, key_bias=key_bias)
             self._mark("pv")
             output = ops.causal_pv_tri(scores, xv, g_both, first_visible=first_visible)
+            if empty_rows is not None:
+                output.masked_fill_(empty_rows[:, None, :, None], 0)
             self._mark("end")
             return output.transpose(1, 2)
 
@@ -525,6 +531,11 @@ class MTAAttentionTriton(nn.Module):
                 scores = ops.headmix_softmax(scores, None, None, self.causal, key_bias=key_bias,
                                              first_visible=first_visible,
                                              fill_upper=post_conv_identity and w2 is None and not own_pv)
+            if empty_rows is not None and not post_conv_identity:
+                # (the rows that see nothing, NaN out of the softmax: zeros into the conv, whole rows up to the diagonal)
+                rows_all = torch.arange(1, n_keys + 1, device=empty_rows.device, dtype=torch.int32)
+                if ops.band_zero_(scores, torch.where(empty_rows, rows_all[None, :], 0).to(torch.int32)) is None:
+                    raise RuntimeError("band masks need 16-bit scores of a length that is a multiple of 8")
             done = None
             # conv and mix in one pass, the conv result never written: taken where it measures at least as fast as the
             # two kernels (mixing groups of up to 4 heads, kernel sizes with a vector-staged instance: 3x3, 7x7)
@@ -561,6 +572,8 @@ class MTAAttentionTriton(nn.Module):
         output = ops.causal_pv(scores, xv, self.causal, first_visible=first_visible) if own_pv else None
         if output is None:
             output = torch.matmul(scores, xv)
+        if empty_rows is not None:
+            output.masked_fill_(empty_rows[:, None, :, None], 0)
         self._mark("end")
         return output.transpose(1, 2)
 
@@ -720,9 +733,11 @@ class MTAAttentionTriton(nn.Module):
                 if kind == "keys":
                     return hidden_keys(xq, xk, xv, what)
                 if kind == "band" and ops.qk_conv_supported(xq, xk, self.mta_conv_triton.weight):
+                    empty_rows = self._band_empty_rows(mask)
                     if not wants_grad:
-                        return self._forward_fused(xq, xk, xv, first_visible=what)
-                    if self._band_training_supported(xq, xk, xv):
+                        return self._forward_fused(xq, xk, xv, first_visible=what, empty_rows=empty_rows)
+                    # (in training a band with rows that see nothing takes the mask passes below)
+                    if empty_rows is None and self._band_training_supported(xq, xk, xv):
                         return self._forward_stagewise(xq, xk, xv, first_visible=what)
         elif (not self.causal and isinstance(mask, torch.Tensor) and mask.dim() == 4 and xq.size(-2) == xk.size(-2)):
             # no causal rule and a mask that hides the same keys from every row (key padding of an encoder batch): the same
@@ -844,7 +859,7 @@ class MTAAttentionTriton(nn.Module):
         """What a 4-D ``mask`` (bool with True = attend, or additive with 0 / -inf; one plane for all heads) amounts to
         together with the causal rule (a module with ``causal=False``: on its own, and only the first form):
           ("keys", bias)   every row sees the kept keys up to itself and key 0 is kept: fp32 (B,S), 0 / -inf per key;
-          ("band", first)  row p sees exactly the keys first[p] .. p: int32 (B,S);
+          ("band", first)  row p sees exactly the keys first[p] .. p, or none at all (first[p] = p + 1): int32 (B,S);
           (None, None)     anything else (per-head planes, holes that differ between rows, other finite values, a row
                            that sees nothing).
         A few reductions over the mask and one read back; the answer for the last mask object seen is kept while its
@@ -855,7 +870,7 @@ class MTAAttentionTriton(nn.Module):
         cached = getattr(self, "_mask_cache", None)   # (the mask object itself is kept: its identity cannot be reused)
         if cached is not None and cached[0] is mask and cached[1] == key:
             return cached[2]
-        answer = (None, None)
+        answer, empty_rows = (None, None), None
         plane = mask[:, 0]
         same_heads = mask.size(1) == 1 or bool((mask == mask[:, :1]).all())
         if mask.dtype == torch.bool:
@@ -881,10 +896,20 @@ class MTAAttentionTriton(nn.Module):
             else:
                 count = visible.sum(-1)
                 lead = visible.int().argmax(-1)
-                if bool(((count >= 1) & (count == rows[None, :] - lead + 1)).all()):
-                    answer = ("band", lead.to(torch.int32).expand(bsz, s).contiguous())
-        self._mask_cache = (mask, key, answer)
+                empty = count == 0      # rows that see no key (the padding of a left-padded batch): first[p] = p + 1
+                if bool((empty | (count == rows[None, :] - lead + 1)).all()):
+                    first = torch.where(empty, rows[None, :] + 1, lead)
+                    answer = ("band", first.to(torch.int32).expand(bsz, s).contiguous())
+                    if bool(empty.any()):
+                        empty_rows = empty.expand(bsz, s).contiguous()
+        self._mask_cache = (mask, key, answer, empty_rows)
         return answer
+
+    def _band_empty_rows(self, mask):
+        """bool (B,S): the query rows of the band mask last classified that see no key at all, or None if every row sees
+        one."""
+        cached = getattr(self, "_mask_cache", None)
+        return cached[3] if cached is not None and cached[0] is mask else None
 
     def _mask_planes(self, mask, bsz: int, s: int):
         """(planes, additive, empty_rows) of a 4-D mask (1|B, 1|H, S, S) that is none of the forms ``_structured_mask``

@@ -1110,6 +1110,36 @@ def test_mta_use_mask_arbitrary_planes(pkg, form, causal, dtype):
         torch.testing.assert_close(got3.float(), want3.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("case", [(2, 8, 520, 64, 4, 6, 11, "identity", torch.bfloat16), (2, 8, 264, 128, 4, 7, 7, "random", torch.float16),
+                                  (2, 16, 1160, 64, 16, 3, 3, "identity", torch.bfloat16), (1, 16, 520, 128, 16, 7, 7, "random", torch.bfloat16),
+                                  (2, 4, 2304, 64, 2, 6, 11, "identity", torch.float16)])
+def test_mta_use_mask_left_padded_batch(pkg, case):
+    """A left-padded batch (keys ahead of a sequence's start hidden; its padding rows therefore see nothing): a band mask
+    whose empty rows have first[p] = p + 1.  It stays on the band route - the three kernels, or the general route with the
+    empty rows of the probabilities cleared ahead of the post-softmax conv - and the padding rows' outputs are zeros, as
+    the reference's masked_fill behind the softmax leaves them; against the oracle given the mask tensor."""
+    b, h, s, d, group, r1, s1, post, dtype = case
+    print(f"mta use_mask left padding {case}", flush=True)
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=104)
+    params = _config_like(h, group, r1, s1, 0.05, dtype, post=post)
+    pad = torch.tensor([0, s // 3][:b]) if b > 1 else torch.tensor([70])
+    keep = torch.arange(s)[None, :] >= pad[:, None]
+    visible = keep[:, None, None, :] & torch.tril(torch.ones(s, s, dtype=torch.bool))[None, None]     # keys only
+    want = O.mta_forward(q, k, v, params[0].unsqueeze(1), params[1], params[2].unsqueeze(1), params[3],
+                         mask=torch.where(visible, 0.0, float("-inf")).expand(b, h, s, s).contiguous())
+    assert torch.isfinite(want.float()).all()
+    mod = _mta_module(pkg, h, r1, s1, 3, 3, *params, dtype, use_mask=True, structure="infer")
+    stages = []
+    mod._stage_hook = stages.append
+    got = mod(q.cuda(), k.cuda(), v.cuda(), visible.cuda(), None).cpu()
+    assert "qk_conv" in stages and "mask" not in stages, stages
+    if post == "identity":
+        assert stages == ["qk_conv", "mix_softmax_mix", "pv", "end"], stages
+    torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+    last = b - 1
+    assert not got[last, :int(pad[last])].any()
+
+
 @pytest.mark.parametrize("post", ["identity", "random"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_mta_use_mask_rows_that_see_nothing(pkg, dtype, post):
