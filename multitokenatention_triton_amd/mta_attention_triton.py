@@ -324,9 +324,14 @@ class _MixSoftmax(torch.autograd.Function):
         p = ops.headmix_softmax(x, weight, None, causal, group_size=group_size if weight is not None else None,
                                 fill_upper=fill_upper, key_bias=key_bias, first_visible=first_visible)
         if zero_planes is not None:
-            # (uint8 visibility planes of a mask under which some row sees nothing: that row's NaN becomes zeros, as behind
-            # the reference's masked_fill ahead of its post-softmax conv - and the stored probabilities give it a zero gradient)
-            ops.mask_fill(p, zero_planes, False, causal, out=p)
+            # (a mask under which some row sees nothing: that row's NaN becomes zeros, as behind the reference's masked_fill
+            # ahead of its post-softmax conv - and the stored probabilities give it a zero gradient.  Either the mask's uint8
+            # visibility planes, or for a band mask an int32 (B,S) array that is p + 1 for such a row p and 0 elsewhere)
+            if zero_planes.dtype == torch.int32:
+                if ops.band_zero_(p, zero_planes) is None:
+                    raise RuntimeError("band masks need 16-bit scores of a length that is a multiple of 8")
+            else:
+                ops.mask_fill(p, zero_planes, False, causal, out=p)
         ctx.save_for_backward(x if weight is not None else None, weight, p)
         ctx.causal, ctx.group_size, ctx.grad_fill_upper = causal, group_size, grad_fill_upper
         return p
@@ -578,7 +583,7 @@ class MTAAttentionTriton(nn.Module):
         return output.transpose(1, 2)
 
     def _forward_stagewise(self, xq, xk, xv, key_bias=None, first_visible=None, mask_planes=None, mask_additive=None,
-                           mask_empty_rows=False):
+                           mask_empty_rows=False, band_empty_rows=None):
         """The reference's own sequence of operators (mta_attention_triton.py:68-92), each differentiable: taken
         whenever a gradient may be asked for.  No weight structure is assumed here, so every entry of the four
         weights receives its gradient.
@@ -610,13 +615,18 @@ class MTAAttentionTriton(nn.Module):
         # so nothing is written there: only the last stage's output, which torch's GEMM reads in full, and the score
         # gradient that goes into torch's GEMMs (inside _ScaledScoresConv) are filled.
         lower = not self.causal   # value of the fill flags: False (leave alone) when causal
+        # (band_empty_rows: bool (B,S), the rows of the band mask that see no key: their probabilities are cleared)
+        zero_rows = mask_planes if mask_empty_rows else None
+        if band_empty_rows is not None:
+            rows_all = torch.arange(1, xk.size(-2) + 1, device=xq.device, dtype=torch.int32)
+            zero_rows = torch.where(band_empty_rows, rows_all[None, :], 0).to(torch.int32).contiguous()
         g_eff = group or self.n_heads
         # (the matrix-core variant for groups of 16 takes a key bias in its row-list form only)
         bias_ok = (key_bias is None and first_visible is None) or g_eff <= _FUSED_MAX_GROUP or (
             g_eff == _FUSED_MFMA_GROUP and os.environ.get("MTA_MIX16_NO_ROW_LISTS") != "1")
         if _one_pass_group(g_eff, scores.dtype, xk.size(-2), w_pre) and bias_ok and mask_planes is None:
             self._mark("mix_softmax")
-            scores = _MixSoftmax.apply(scores, w_pre, self.causal, group, lower, lower, key_bias, first_visible)
+            scores = _MixSoftmax.apply(scores, w_pre, self.causal, group, lower, lower, key_bias, first_visible, zero_rows)
         else:
             self._mark("mix_pre")
             scores = TritonLinearHeadFunction.apply(scores, w_pre, self.wpsm_triton.causal, self.wpsm_triton.output_value,
@@ -628,8 +638,7 @@ class MTAAttentionTriton(nn.Module):
                 else:   # (finite values besides 0: the mask in the scores' dtype is added)
                     scores = _MaskAdd.apply(scores, mask_additive, self.causal)
             self._mark("softmax")
-            scores = _MixSoftmax.apply(scores, None, self.causal, None, lower, lower, key_bias, first_visible,
-                                       mask_planes if mask_empty_rows else None)
+            scores = _MixSoftmax.apply(scores, None, self.causal, None, lower, lower, key_bias, first_visible, zero_rows)
         self._mark("conv_post")
         scores = Conv2dTritonFunction.apply(scores, self.mta_conv_after_sm_triton.weight, self.causal, lower, lower)
         if first_visible is not None:
@@ -736,9 +745,8 @@ class MTAAttentionTriton(nn.Module):
                     empty_rows = self._band_empty_rows(mask)
                     if not wants_grad:
                         return self._forward_fused(xq, xk, xv, first_visible=what, empty_rows=empty_rows)
-                    # (in training a band with rows that see nothing takes the mask passes below)
-                    if empty_rows is None and self._band_training_supported(xq, xk, xv):
-                        return self._forward_stagewise(xq, xk, xv, first_visible=what)
+                    if self._band_training_supported(xq, xk, xv):
+                        return self._forward_stagewise(xq, xk, xv, first_visible=what, band_empty_rows=empty_rows)
         elif (not self.causal and isinstance(mask, torch.Tensor) and mask.dim() == 4 and xq.size(-2) == xk.size(-2)):
             # no causal rule and a mask that hides the same keys from every row (key padding of an encoder batch): the same
             # key bias and zeroed K and V rows, through the kernels' non-causal form

@@ -730,6 +730,40 @@ def test_mta_module_backward_arbitrary_mask_planes(pkg, causal, dtype):
     _check_all(dtype, out.cpu(), want_out, [g_.cpu() for g_ in gin + gw], want_in + want_w)
 
 
+@pytest.mark.parametrize("case", [(2, 4, 264, 64, 3, 3, torch.bfloat16), (2, 16, 520, 128, 6, 11, torch.float16)])
+def test_mta_module_backward_left_padded_batch(pkg, case):
+    """Training on a left-padded batch (a band mask whose padding rows see no key): the band route of the differentiable
+    operators, the padding rows' probabilities cleared inside the softmax stage.  The reference's own gradients are NaN
+    under such a mask (the softmax of an empty row), so: the forward against the oracle, gradients finite and zero for
+    the padding, and all seven gradients against the mask-pass route (pinned against the oracle above) on the same mask."""
+    b, h, s, d, r1, s1, dtype = case
+    print(f"mta module backward left padding {case}", flush=True)
+    mod, params = _mta_pair(pkg, h, r1, s1, dtype, seed=431)
+    mod.use_mask = True
+    q, k, v = O.seeded_qkv(b, h, s, d, dtype, seed=432)
+    pad = torch.tensor([0, s // 4])
+    keep = torch.arange(s)[None, :] >= pad[:, None]
+    visible = keep[:, None, None, :] & torch.tril(torch.ones(s, s, dtype=torch.bool))[None, None]
+    go = _rand((b, s, h, d), 433, dtype) * keep[:, :, None, None]
+    want_out = O.mta_forward(q.float(), k.float(), v.float(), params[0].float().unsqueeze(1), params[1].float(),
+                             params[2].float().unsqueeze(1), params[3].float(), mask=visible.expand(b, h, s, s))
+    stages = []
+    mod._stage_hook = stages.append
+    out, gin, gw = _module_grads(mod, q, k, v, go, mask=visible)
+    assert "mask" not in stages and "qk_conv" in stages and "pv" in stages, stages
+    _close(out, want_out, dtype, "forward")
+    assert not out[1, :int(pad[1])].any()
+    for name, g_ in zip(_GRAD_NAMES, gin + gw):
+        assert torch.isfinite(g_).all(), name
+    for name, g_ in zip(("xq", "xk", "xv"), gin):
+        assert not g_[1, :, :int(pad[1])].any(), f"the padding of {name} received a gradient"
+    mod._band_training_supported = lambda *a: False      # the mask passes instead
+    del stages[:]
+    out2, gin2, gw2 = _module_grads(mod, q, k, v, go, mask=visible)
+    assert stages.count("mask") >= 3, stages
+    _check_all(dtype, out.cpu(), out2.cpu(), [g_.cpu() for g_ in gin + gw], [g_.cpu() for g_ in gin2 + gw2])
+
+
 def test_mta_module_backward_key_mask_finite_values(pkg):
     """A 2-D additive key mask with finite values besides -inf (B = 1), in training: the values are added ahead of the
     softmax (mta_attention_triton.py:77), only -inf hides a key."""
